@@ -1,0 +1,178 @@
+/*
+ * psn.h -- C ABI of the gfx950 (MI355X) backend for Psionic's quantized GGUF compute path.
+ *
+ * This is the whole drop-in boundary: a thin extern "C" surface doing module load, buffer
+ * alloc, launch and stream sync, which a Rust `-sys` crate binds 1:1.  Plain pointers and
+ * sizes only.  There is no CPU fallback behind it: without a gfx950 device every call that
+ * needs one fails with PSN_E_NO_DEVICE.
+ *
+ * What each entry point replaces.  Psionic's backend crates (psionic-backend-cuda / -metal /
+ * the CPU backend) are not vendored in the reference tree; the tree pins only their existence
+ * and the switch that selects them:
+ *   /root/reference/apps/pylon/docs/2026-06-09-pylon-qwen35-local-inference-roadmap.md:137-150
+ *       (`psionic-openai-server -m <gguf> --backend cpu|cuda|metal`)
+ *   /root/reference/docs/2026-06-10-cs336-distributed-homework-continuation-audit.md:239-241
+ *       (crate names psionic-backend-cuda, psionic-backend-metal)
+ *   /root/reference/docs/muse/muse-glimmer.md:112
+ *       ("kernels for Q4_K, Q5_K, Q6_K, and other GGUF quantizations")
+ * Each declaration below names the op of that CUDA backend it stands in for.
+ *
+ * Conventions
+ *   - every call returns int32_t: PSN_OK (0) or a negative PSN_E_* code; psn_last_error()
+ *     returns a thread-local, NUL-terminated description of the last failure on this thread;
+ *   - handles are created and destroyed by the library; host memory passed in stays the caller's;
+ *   - shape and argument errors are detected on the host before anything is launched;
+ *   - launches are asynchronous on the given stream; only psn_stream_sync and
+ *     psn_event_elapsed_us block.  Calls on distinct streams may come from distinct threads.
+ */
+#ifndef PSN_H
+#define PSN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PSN_ABI_VERSION 1
+
+typedef struct psn_ctx psn_ctx;
+typedef struct psn_stream psn_stream;
+typedef struct psn_buf psn_buf;
+typedef struct psn_module psn_module;
+typedef struct psn_event psn_event;
+
+/* GGUF tensor type ids */
+typedef enum { PSN_Q4_0 = 2, PSN_Q8_0 = 8, PSN_Q4_K = 12, PSN_Q6_K = 14, PSN_Q8_K = 15 } psn_qtype;
+/* how activations enter the dot product */
+typedef enum {
+    PSN_ACT_F32 = 0, /* weights dequantized to fp32, fp32 FMA */
+    PSN_ACT_Q8 = 1   /* x quantized to Q8_0 (Q4_0/Q8_0 weights) or Q8_K (Q4_K/Q6_K), int8 dot */
+} psn_act_scheme;
+typedef enum { PSN_LAYOUT_GGUF = 0 /* raw GGUF blocks, row-major [N][K/block] */ } psn_layout;
+
+enum {
+    PSN_OK = 0,
+    PSN_E_INVALID_ARG = -1, /* null handle, handle of another context, buffer too small */
+    PSN_E_SHAPE = -2,       /* K not a whole number of blocks, N/M/K <= 0, batch outside 1..8 */
+    PSN_E_UNSUPPORTED = -3, /* type / layout / scheme combination without a kernel */
+    PSN_E_NO_DEVICE = -4,   /* no HIP device, or the device is not gfx950 */
+    PSN_E_OOM = -5,
+    PSN_E_MODULE = -6,      /* code object rejected or a kernel symbol is missing */
+    PSN_E_HIP = -7          /* any other HIP runtime failure; text carries the hipError_t */
+};
+
+/* ---- library ------------------------------------------------------------------------- */
+
+int32_t psn_abi_version(void);
+const char *psn_last_error(void);
+const char *psn_error_name(int32_t code);
+
+/* elements / bytes per block of a type; bytes of one row of k elements (PSN_E_SHAPE if ragged) */
+int32_t psn_block_elems(int32_t qtype);
+int32_t psn_block_bytes(int32_t qtype);
+int64_t psn_row_bytes(int32_t qtype, int64_t k);
+
+/* ---- context, module, stream, event, buffer  (the "module load, buffer alloc, launch and
+ *      stream sync" surface; replaces the CUDA backend's context/module/stream/buffer wrappers) -- */
+
+int32_t psn_ctx_create(int32_t device, psn_ctx **out);
+int32_t psn_ctx_destroy(psn_ctx *ctx);
+/* device facts: compute units, bytes of device memory, arch name copied into name[0..n) */
+int32_t psn_ctx_info(psn_ctx *ctx, int32_t *compute_units, int64_t *total_mem, char *name, size_t n);
+
+/* load a gfx950 code object from memory / the one built into the library */
+int32_t psn_module_load(psn_ctx *ctx, const void *code_object, size_t len, psn_module **out);
+int32_t psn_module_load_builtin(psn_ctx *ctx, psn_module **out);
+int32_t psn_module_unload(psn_module *mod);
+/* PSN_OK if the module exports `kernel_name` */
+int32_t psn_module_has_kernel(psn_module *mod, const char *kernel_name);
+
+int32_t psn_stream_create(psn_ctx *ctx, psn_stream **out);
+int32_t psn_stream_sync(psn_stream *s);
+int32_t psn_stream_destroy(psn_stream *s);
+
+int32_t psn_event_create(psn_ctx *ctx, psn_event **out);
+int32_t psn_event_destroy(psn_event *e);
+int32_t psn_event_record(psn_event *e, psn_stream *s);
+/* blocks until `end` has happened */
+int32_t psn_event_elapsed_us(const psn_event *begin, const psn_event *end, double *out_us);
+
+int32_t psn_buf_alloc(psn_ctx *ctx, size_t bytes, psn_buf **out);
+int32_t psn_buf_free(psn_buf *b);
+int64_t psn_buf_size(const psn_buf *b);
+int32_t psn_buf_upload(psn_buf *dst, size_t off, const void *src, size_t n, psn_stream *s);
+int32_t psn_buf_download(const psn_buf *src, size_t off, void *dst, size_t n, psn_stream *s);
+int32_t psn_buf_fill_zero(psn_buf *b, psn_stream *s);
+
+/* ---- weights ---------------------------------------------------------------------------- */
+
+/* Allocates and fills a device copy of an [N][K] quantized tensor from host GGUF blocks
+ * (N * psn_row_bytes(qtype, K) bytes).  Replaces the CUDA backend's tensor upload. */
+int32_t psn_weight_upload(psn_ctx *ctx, int32_t qtype, int64_t N, int64_t K, const void *gguf_blocks,
+                          int32_t layout, psn_stream *s, psn_buf **out);
+
+/* ---- activations ------------------------------------------------------------------------ */
+
+/* Device layout of a quantized activation tensor [batch][K] (all fields row-major over batch):
+ *   act_type PSN_Q8_0: int8 qs[batch][K] at off_qs; float d[batch][K/32] at off_d (the block's
+ *                      fp16 scale widened to fp32); int32 s[batch][K/32] at off_s (sum of qs)
+ *   act_type PSN_Q8_K: int8 qs[batch][K]; float d[batch][K/256]; int16 bsums[batch][K/16]
+ * Values equal field-for-field what the GGUF Q8_0 / Q8_K row quantizers produce. */
+typedef struct psn_actq_info {
+    int64_t off_qs, off_d, off_s, bytes;
+} psn_actq_info;
+int32_t psn_actq_layout(int32_t act_type, int64_t K, int32_t batch, psn_actq_info *out);
+/* the activation type the Q8 scheme pairs with a weight type (PSN_Q8_0 or PSN_Q8_K) */
+int32_t psn_act_type_for(int32_t weight_qtype);
+
+/* x_f32 [batch][K] -> x_q in the layout above.  Replaces the CUDA backend's activation
+ * quantize kernel (the "same activation-quantization scheme" the CPU path uses). */
+int32_t psn_act_quantize(psn_module *mod, psn_stream *s, int32_t act_type, const psn_buf *x_f32, psn_buf *x_q,
+                         int64_t K, int32_t batch);
+
+/* ---- decode matvec ------------------------------------------------------------------------ */
+
+/* y[b][n] = sum_k deq(W)[n][k] * x[b][k], b < batch (1..8), y fp32 [batch][N].
+ * Scheme Q8 quantizes x into a workspace owned by the stream, then runs the int8 kernel.
+ * Replaces the CUDA backend's quantized matvec op (decode path). */
+int32_t psn_qmatvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, const psn_buf *W,
+                    const psn_buf *x_f32, psn_buf *y_f32, int64_t N, int64_t K, int32_t batch);
+
+/* Same contraction from activations already quantized by psn_act_quantize (one quantization
+ * can feed several matrices, e.g. q/k/v or gate/up). */
+int32_t psn_qmatvec_q8(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
+                       const psn_buf *x_q, psn_buf *y_f32, int64_t N, int64_t K, int32_t batch);
+
+/* Launch geometry of one matvec.  psn_qmatvec_plan fills in the library's choice for a shape
+ * (pure host arithmetic, usable without a device); psn_qmatvec_planned runs with a caller-chosen
+ * one (auto-tuners, benchmarks). */
+typedef struct psn_matvec_plan {
+    int32_t lanes_per_row;  /* 8, 16, 32 or 64 lanes share one row */
+    int32_t rows_in_flight; /* 1, 2 or 4 row sets per lane */
+    int32_t batch_tile;     /* compiled batch width: 1, 2, 4 or 8 (>= batch) */
+    int32_t stage_lds;      /* 1: activations staged in LDS (scheme Q8 only) */
+    int32_t blocks;         /* workgroups of 256 threads */
+    int32_t lds_bytes;      /* dynamic LDS the launch asks for */
+} psn_matvec_plan;
+int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t compute_units,
+                         psn_matvec_plan *out);
+/* x is x_q for scheme Q8 (already quantized) and x_f32 for scheme F32 */
+int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const psn_buf *W,
+                            const psn_buf *x, psn_buf *y_f32, int64_t N, int64_t K, int32_t batch,
+                            const psn_matvec_plan *plan);
+
+/* ---- prefill matmul ----------------------------------------------------------------------- */
+
+/* Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k]; X fp16 [M][K], Y fp32 [M][N], weight tiles are
+ * dequantized to fp16 (h = round to nearest even) in LDS and fed to fp16 MFMA with fp32
+ * accumulation.  qtype PSN_Q4_0 or PSN_Q8_0.  Replaces the CUDA backend's quantized prefill
+ * matmul op. */
+int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
+                            const psn_buf *X_f16, psn_buf *Y_f32, int64_t M, int64_t N, int64_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

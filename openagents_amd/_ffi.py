@@ -1,0 +1,98 @@
+"""ctypes declarations of the C ABI in include/psn.h (libpsn_hip.so).
+
+This is the Python stand-in for the Rust `-sys` crate: one declaration per exported symbol,
+no logic.  Loading fails loudly when the library has not been built; nothing here falls back
+to a CPU implementation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libpsn_hip.so")
+
+Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 2, 8, 12, 14, 15
+ACT_F32, ACT_Q8 = 0, 1
+LAYOUT_GGUF = 0
+
+OK = 0
+E_INVALID_ARG, E_SHAPE, E_UNSUPPORTED, E_NO_DEVICE, E_OOM, E_MODULE, E_HIP = -1, -2, -3, -4, -5, -6, -7
+
+
+class ActqInfo(C.Structure):
+    _fields_ = [("off_qs", C.c_int64), ("off_d", C.c_int64), ("off_s", C.c_int64), ("bytes", C.c_int64)]
+
+
+class MatvecPlan(C.Structure):
+    _fields_ = [("lanes_per_row", C.c_int32), ("rows_in_flight", C.c_int32), ("batch_tile", C.c_int32),
+                ("stage_lds", C.c_int32), ("blocks", C.c_int32), ("lds_bytes", C.c_int32)]
+
+    def as_dict(self):
+        return {k: int(getattr(self, k)) for k, _ in self._fields_}
+
+
+_vp, _i32, _i64, _sz = C.c_void_p, C.c_int32, C.c_int64, C.c_size_t
+_pp = C.POINTER(C.c_void_p)
+
+# name -> (restype, argtypes); mirrors include/psn.h declaration by declaration
+SIGNATURES = {
+    "psn_abi_version": (_i32, []),
+    "psn_last_error": (C.c_char_p, []),
+    "psn_error_name": (C.c_char_p, [_i32]),
+    "psn_block_elems": (_i32, [_i32]),
+    "psn_block_bytes": (_i32, [_i32]),
+    "psn_row_bytes": (_i64, [_i32, _i64]),
+    "psn_ctx_create": (_i32, [_i32, _pp]),
+    "psn_ctx_destroy": (_i32, [_vp]),
+    "psn_ctx_info": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_i64), C.c_char_p, _sz]),
+    "psn_module_load": (_i32, [_vp, _vp, _sz, _pp]),
+    "psn_module_load_builtin": (_i32, [_vp, _pp]),
+    "psn_module_unload": (_i32, [_vp]),
+    "psn_module_has_kernel": (_i32, [_vp, C.c_char_p]),
+    "psn_stream_create": (_i32, [_vp, _pp]),
+    "psn_stream_sync": (_i32, [_vp]),
+    "psn_stream_destroy": (_i32, [_vp]),
+    "psn_event_create": (_i32, [_vp, _pp]),
+    "psn_event_destroy": (_i32, [_vp]),
+    "psn_event_record": (_i32, [_vp, _vp]),
+    "psn_event_elapsed_us": (_i32, [_vp, _vp, C.POINTER(C.c_double)]),
+    "psn_buf_alloc": (_i32, [_vp, _sz, _pp]),
+    "psn_buf_free": (_i32, [_vp]),
+    "psn_buf_size": (_i64, [_vp]),
+    "psn_buf_upload": (_i32, [_vp, _sz, _vp, _sz, _vp]),
+    "psn_buf_download": (_i32, [_vp, _sz, _vp, _sz, _vp]),
+    "psn_buf_fill_zero": (_i32, [_vp, _vp]),
+    "psn_weight_upload": (_i32, [_vp, _i32, _i64, _i64, _vp, _i32, _vp, _pp]),
+    "psn_actq_layout": (_i32, [_i32, _i64, _i32, C.POINTER(ActqInfo)]),
+    "psn_act_type_for": (_i32, [_i32]),
+    "psn_act_quantize": (_i32, [_vp, _vp, _i32, _vp, _vp, _i64, _i32]),
+    "psn_qmatvec": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
+    "psn_qmatvec_q8": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
+    "psn_qmatvec_plan": (_i32, [_i32, _i32, _i64, _i64, _i32, _i32, C.POINTER(MatvecPlan)]),
+    "psn_qmatvec_planned": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32, C.POINTER(MatvecPlan)]),
+    "psn_qmatmul_prefill": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i64]),
+}
+
+_lib = None
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def load() -> C.CDLL:
+    """Load libpsn_hip.so from openagents_amd/lib/ and declare every entry point."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise LibraryMissing(f"{LIB_PATH} is missing: build it with `python -m openagents_amd.build` "
+                             "(there is no CPU fallback)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError here means header and library disagree
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib

@@ -1,0 +1,222 @@
+"""Host-side mirror of the backend/operator surface for the quantized GGUF path.
+
+`HipBackend` is what a Psionic backend crate would look like for `--backend hip`
+(the switch is pinned by
+/root/reference/apps/pylon/docs/2026-06-09-pylon-qwen35-local-inference-roadmap.md:137-150;
+the crate names psionic-backend-cuda / -metal by
+/root/reference/docs/2026-06-10-cs336-distributed-homework-continuation-audit.md:239-241):
+buffers, weight upload, activation quantize, quantized matvec (decode) and quantized matmul
+(prefill), all asynchronous on a stream, errors as typed exceptions.  Every method is a thin
+call into the C ABI (include/psn.h); numpy appears only as the host-memory container.
+There is no CPU path: without the library or a gfx950 device construction raises.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _ffi
+from ._ffi import (ACT_F32, ACT_Q8, LAYOUT_GGUF, Q4_0, Q4_K, Q6_K, Q8_0, Q8_K, MatvecPlan)  # noqa: F401
+
+TYPE_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", Q8_K: "Q8_K"}
+
+
+class PsnError(RuntimeError):
+    """A negative return code from the C ABI, with psn_last_error()'s text."""
+
+    def __init__(self, code: int, text: str):
+        lib = _ffi.load()
+        self.code = code
+        self.name = lib.psn_error_name(code).decode()
+        super().__init__(f"{self.name} ({code}): {text}")
+
+
+def _check(rc: int) -> int:
+    if rc < 0:
+        raise PsnError(int(rc), _ffi.load().psn_last_error().decode(errors="replace"))
+    return int(rc)
+
+
+def row_bytes(qtype: int, k: int) -> int:
+    return _check(_ffi.load().psn_row_bytes(qtype, k))
+
+
+def act_type_for(qtype: int) -> int:
+    return _check(_ffi.load().psn_act_type_for(qtype))
+
+
+def actq_layout(act_type: int, k: int, batch: int) -> _ffi.ActqInfo:
+    info = _ffi.ActqInfo()
+    _check(_ffi.load().psn_actq_layout(act_type, k, batch, C.byref(info)))
+    return info
+
+
+def matvec_plan(qtype: int, scheme: int, n: int, k: int, batch: int, compute_units: int = 256) -> MatvecPlan:
+    plan = MatvecPlan()
+    _check(_ffi.load().psn_qmatvec_plan(qtype, scheme, n, k, batch, compute_units, C.byref(plan)))
+    return plan
+
+
+class DeviceBuffer:
+    """Owns one psn_buf."""
+
+    def __init__(self, backend: "HipBackend", nbytes: int):
+        self._b = backend
+        h = C.c_void_p()
+        _check(backend.lib.psn_buf_alloc(backend.ctx, nbytes, C.byref(h)))
+        self.handle = h
+        self.nbytes = nbytes
+
+    @classmethod
+    def _adopt(cls, backend: "HipBackend", handle: C.c_void_p) -> "DeviceBuffer":
+        self = cls.__new__(cls)
+        self._b = backend
+        self.handle = handle
+        self.nbytes = int(backend.lib.psn_buf_size(handle))
+        return self
+
+    def upload(self, arr: np.ndarray, offset: int = 0) -> "DeviceBuffer":
+        a = np.ascontiguousarray(arr)
+        _check(self._b.lib.psn_buf_upload(self.handle, offset, C.c_void_p(a.ctypes.data), a.nbytes, self._b.stream))
+        return self
+
+    def download(self, dtype, shape, offset: int = 0) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        _check(self._b.lib.psn_buf_download(self.handle, offset, C.c_void_p(out.ctypes.data), out.nbytes, self._b.stream))
+        return out
+
+    def free(self):
+        if self.handle is not None and self._b.ctx is not None:
+            _check(self._b.lib.psn_buf_free(self.handle))
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+@dataclass
+class QuantizedTensor:
+    """An [n, k] GGUF-quantized weight resident on the device."""
+    buf: DeviceBuffer
+    qtype: int
+    n: int
+    k: int
+
+    @property
+    def nbytes(self) -> int:
+        return self.n * row_bytes(self.qtype, self.k)
+
+
+class HipBackend:
+    def __init__(self, device: int = 0):
+        self.lib = _ffi.load()
+        self.ctx = None
+        ctx = C.c_void_p()
+        _check(self.lib.psn_ctx_create(device, C.byref(ctx)))
+        self.ctx = ctx
+        mod = C.c_void_p()
+        _check(self.lib.psn_module_load_builtin(ctx, C.byref(mod)))
+        self.module = mod
+        st = C.c_void_p()
+        _check(self.lib.psn_stream_create(ctx, C.byref(st)))
+        self.stream = st
+        cus, mem = C.c_int32(), C.c_int64()
+        name = C.create_string_buffer(64)
+        _check(self.lib.psn_ctx_info(ctx, C.byref(cus), C.byref(mem), name, 64))
+        self.compute_units = int(cus.value)
+        self.total_mem = int(mem.value)
+        self.arch = name.value.decode()
+
+    # -- lifetime ---------------------------------------------------------------------------
+    def close(self):
+        if self.ctx is None:
+            return
+        self.lib.psn_stream_destroy(self.stream)
+        self.lib.psn_module_unload(self.module)
+        self.lib.psn_ctx_destroy(self.ctx)
+        self.ctx = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    # -- buffers ----------------------------------------------------------------------------
+    def alloc(self, nbytes: int) -> DeviceBuffer:
+        return DeviceBuffer(self, nbytes)
+
+    def upload(self, arr: np.ndarray) -> DeviceBuffer:
+        a = np.ascontiguousarray(arr)
+        return DeviceBuffer(self, max(a.nbytes, 1)).upload(a)
+
+    def upload_weight(self, qtype: int, blocks: np.ndarray, n: int, k: int) -> QuantizedTensor:
+        b = np.ascontiguousarray(blocks, dtype=np.uint8)
+        if b.size != n * row_bytes(qtype, k):
+            raise ValueError(f"weight bytes {b.size} != n*row_bytes {n * row_bytes(qtype, k)}")
+        h = C.c_void_p()
+        _check(self.lib.psn_weight_upload(self.ctx, qtype, n, k, C.c_void_p(b.ctypes.data), LAYOUT_GGUF, self.stream, C.byref(h)))
+        return QuantizedTensor(DeviceBuffer._adopt(self, h), qtype, n, k)
+
+    def sync(self):
+        _check(self.lib.psn_stream_sync(self.stream))
+
+    # -- events -----------------------------------------------------------------------------
+    def event(self) -> C.c_void_p:
+        e = C.c_void_p()
+        _check(self.lib.psn_event_create(self.ctx, C.byref(e)))
+        return e
+
+    def record(self, event):
+        _check(self.lib.psn_event_record(event, self.stream))
+
+    def elapsed_us(self, begin, end) -> float:
+        out = C.c_double()
+        _check(self.lib.psn_event_elapsed_us(begin, end, C.byref(out)))
+        return float(out.value)
+
+    def destroy_event(self, event):
+        _check(self.lib.psn_event_destroy(event))
+
+    # -- operators --------------------------------------------------------------------------
+    def quantize_activations(self, x: DeviceBuffer, k: int, batch: int, act_type: int, out: DeviceBuffer | None = None) -> DeviceBuffer:
+        info = actq_layout(act_type, k, batch)
+        out = out or self.alloc(int(info.bytes))
+        _check(self.lib.psn_act_quantize(self.module, self.stream, act_type, x.handle, out.handle, k, batch))
+        return out
+
+    def quantized_matvec(self, w: QuantizedTensor, x: DeviceBuffer, y: DeviceBuffer, batch: int = 1, scheme: int = ACT_Q8):
+        _check(self.lib.psn_qmatvec(self.module, self.stream, w.qtype, LAYOUT_GGUF, scheme, w.buf.handle, x.handle, y.handle, w.n, w.k, batch))
+
+    def quantized_matvec_q8(self, w: QuantizedTensor, xq: DeviceBuffer, y: DeviceBuffer, batch: int = 1):
+        _check(self.lib.psn_qmatvec_q8(self.module, self.stream, w.qtype, LAYOUT_GGUF, w.buf.handle, xq.handle, y.handle, w.n, w.k, batch))
+
+    def quantized_matvec_planned(self, w: QuantizedTensor, x: DeviceBuffer, y: DeviceBuffer, batch: int, scheme: int, plan: MatvecPlan):
+        _check(self.lib.psn_qmatvec_planned(self.module, self.stream, w.qtype, scheme, w.buf.handle, x.handle, y.handle, w.n, w.k, batch, C.byref(plan)))
+
+    def quantized_matmul(self, w: QuantizedTensor, x_f16: DeviceBuffer, y: DeviceBuffer, m: int):
+        _check(self.lib.psn_qmatmul_prefill(self.module, self.stream, w.qtype, LAYOUT_GGUF, w.buf.handle, x_f16.handle, y.handle, m, w.n, w.k))
+
+    # -- convenience for tests and examples: host arrays in, host arrays out ------------------
+    def matvec_host(self, qtype: int, blocks: np.ndarray, x: np.ndarray, n: int, k: int, scheme: int = ACT_Q8,
+                    plan: MatvecPlan | None = None) -> np.ndarray:
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        x2 = x.reshape(1, -1) if x.ndim == 1 else x
+        batch = x2.shape[0]
+        w = self.upload_weight(qtype, blocks, n, k)
+        xb = self.upload(x2)
+        yb = self.alloc(batch * n * 4)
+        if plan is None:
+            self.quantized_matvec(w, xb, yb, batch, scheme)
+        elif scheme == ACT_Q8:
+            xq = self.quantize_activations(xb, k, batch, act_type_for(qtype))
+            self.quantized_matvec_planned(w, xq, yb, batch, scheme, plan)
+        else:
+            self.quantized_matvec_planned(w, xb, yb, batch, scheme, plan)
+        y = yb.download(np.float32, (batch, n))
+        return y[0] if x.ndim == 1 else y

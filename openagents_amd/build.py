@@ -1,0 +1,115 @@
+"""Builds libpsn_hip.so: gfx950 code objects (hipcc --genco) linked into the host C-ABI library.
+
+    python -m openagents_amd.build [--jobs N]
+
+Everything is compiled in-tree into openagents_amd/lib/.  hipcc cross-compiles gfx950 without a
+GPU present.  Device code is always built with packed-fp32 code generation switched off.
+"""
+from __future__ import annotations
+
+import argparse
+import concurrent.futures as cf
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "lib")
+INCLUDE = os.path.join(os.path.dirname(HERE), "include")
+ARCH = "gfx950"
+LIB_NAME = "libpsn_hip.so"
+
+DEVICE_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={ARCH}", "--genco",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+# (output stem, source, extra defines): one code object each, built in parallel
+CODE_OBJECTS = [
+    ("psn_quant", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_QUANT"]),
+    ("psn_mv_q4_0", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q4_0"]),
+    ("psn_mv_q8_0", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q8_0"]),
+    ("psn_mv_q4_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q4_K"]),
+    ("psn_mv_q6_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q6_K"]),
+    ("psn_prefill", "psn_prefill.hip", []),
+    ("psn_decode", "psn_decode.hip", []),
+]
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), p.stdout))
+    return p.stdout
+
+
+def _hipcc():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def lib_path() -> str:
+    return os.path.join(LIB, LIB_NAME)
+
+
+def code_object_paths():
+    return [os.path.join(LIB, f"{stem}.{ARCH}.hsaco") for stem, src, _ in CODE_OBJECTS
+            if os.path.exists(os.path.join(CSRC, src))]
+
+
+def build(jobs: int = 0, verbose: bool = True) -> str:
+    os.makedirs(LIB, exist_ok=True)
+    hipcc = _hipcc()
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    todo = [(stem, src, defs) for stem, src, defs in CODE_OBJECTS if os.path.exists(os.path.join(CSRC, src))]
+
+    def compile_co(item):
+        stem, src, defs = item
+        out = os.path.join(LIB, f"{stem}.{ARCH}.hsaco")
+        _run([hipcc, *DEVICE_FLAGS, *defs, "-I", CSRC, "-o", out, os.path.join(CSRC, src)])
+        return out
+
+    with cf.ThreadPoolExecutor(max_workers=jobs) as ex:
+        outs = list(ex.map(compile_co, todo))
+    if verbose:
+        for o in outs:
+            print("built", os.path.relpath(o, os.path.dirname(HERE)), os.path.getsize(o), "bytes")
+
+    # table of code objects: one .incbin per blob plus {begin, end} pairs the host walks
+    asm = os.path.join(LIB, "psn_blobs.S")
+    with open(asm, "w") as f:
+        f.write("    .section .rodata\n")
+        for i, o in enumerate(outs):
+            f.write(f"    .balign 4096\npsn_blob_{i}_begin:\n    .incbin \"{o}\"\npsn_blob_{i}_end:\n")
+        f.write("    .balign 16\n    .globl psn_builtin_blobs\npsn_builtin_blobs:\n")
+        for i in range(len(outs)):
+            f.write(f"    .quad psn_blob_{i}_begin\n    .quad psn_blob_{i}_end\n")
+        f.write("    .balign 4\n    .globl psn_builtin_blob_count\npsn_builtin_blob_count:\n")
+        f.write(f"    .long {len(outs)}\n")
+        f.write("    .section .note.GNU-stack,\"\",@progbits\n")
+    blob_o = os.path.join(LIB, "psn_blobs.o")
+    _run(["gcc", "-c", "-fPIC", "-o", blob_o, asm])
+
+    host_o = os.path.join(LIB, "psn_host.o")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    _run(["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__",
+          "-I", INCLUDE, "-I", CSRC, "-isystem", os.path.join(rocm, "include"),
+          "-c", "-o", host_o, os.path.join(CSRC, "psn_host.cpp")])
+    out = lib_path()
+    _run(["g++", "-shared", "-fPIC", "-o", out, host_o, blob_o, "-Wl,--no-undefined",
+          "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib")])
+    if verbose:
+        print("built", os.path.relpath(out, os.path.dirname(HERE)), os.path.getsize(out), "bytes")
+    return out
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--jobs", type=int, default=0)
+    args = ap.parse_args(argv)
+    build(args.jobs)
+
+
+if __name__ == "__main__":
+    main(sys.argv[1:])

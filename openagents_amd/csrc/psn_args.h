@@ -1,0 +1,54 @@
+/*
+ * psn_args.h -- kernel argument blocks shared by the host library and the device code.
+ * Every kernel takes exactly one of these structs by value, so the host passes a single
+ * pointer through hipModuleLaunchKernel and the two sides cannot drift apart.
+ */
+#ifndef PSN_ARGS_H
+#define PSN_ARGS_H
+
+#include <stdint.h>
+
+/* Device layout of quantized activations ("actq"), one region per field, row-major over batch:
+ *   Q8_0 activations: int8 qs[B][K]; float d[B][K/32] (the fp16-rounded scale, widened);
+ *                     int32 s[B][K/32] (sum of the block's 32 int8)
+ *   Q8_K activations: int8 qs[B][K]; float d[B][K/256]; int16 bsums[B][K/16]
+ * The three regions live in one allocation at offsets given by psn_actq_layout. */
+struct psn_actq_layout {
+    int64_t off_qs;   /* always 0 */
+    int64_t off_d;
+    int64_t off_s;    /* s (Q8_0) or bsums (Q8_K) */
+    int64_t bytes;    /* total */
+};
+
+struct psn_quantize_args {
+    const float *x;   /* [batch][K] */
+    int8_t *qs;
+    float *d;
+    void *s;
+    int32_t K;
+    int32_t batch;
+};
+
+struct psn_matvec_args {
+    const uint8_t *W;     /* [N][row_bytes] GGUF blocks */
+    const int8_t *xqs;    /* scheme Q8: activation fields (see above) */
+    const float *xd;
+    const void *xs;
+    const float *xf;      /* scheme F32: [batch][K] */
+    float *y;             /* [batch][N] */
+    int32_t N;
+    int32_t K;
+    int32_t batch;        /* live batch columns (<= the kernel's compiled NB) */
+    int32_t pad;
+    int64_t row_bytes;
+};
+
+struct psn_prefill_args {
+    const uint8_t *W;     /* [N][row_bytes] GGUF blocks */
+    const uint16_t *X;    /* fp16 [M][K] */
+    float *Y;             /* [M][N] */
+    int32_t M, N, K, pad;
+    int64_t row_bytes;
+};
+
+#endif

@@ -1,0 +1,662 @@
+/*
+ * psn_host.cpp -- host side of the C ABI in include/psn.h: HIP module load, buffer alloc,
+ * launch and stream sync.  Kernels live in a gfx950 code object (built from psn_matvec.hip and
+ * psn_prefill.hip) that is linked into this library as a byte blob and loaded with
+ * hipModuleLoadData; every launch goes through hipModuleLaunchKernel with one argument struct
+ * (psn_args.h).  No CPU compute path exists here.
+ */
+#include "../../include/psn.h"
+#include "psn_args.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+/* code objects linked into the library (generated table, see build.py) */
+struct psn_blob { const unsigned char *begin, *end; };
+extern "C" {
+extern const psn_blob psn_builtin_blobs[];
+extern const int psn_builtin_blob_count;
+}
+
+/* ------------------------------------------------------------------ errors */
+
+static thread_local char g_err[512] = "";
+
+static int32_t fail(int32_t code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof g_err, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+static int32_t hip_fail(hipError_t e, const char *what) {
+    int32_t code = PSN_E_HIP;
+    if (e == hipErrorOutOfMemory) code = PSN_E_OOM;
+    if (e == hipErrorNoDevice || e == hipErrorInvalidDevice || e == hipErrorInsufficientDriver) code = PSN_E_NO_DEVICE;
+    return fail(code, "%s: hipError %d (%s)", what, (int)e, hipGetErrorString(e));
+}
+
+#define HIP_TRY(expr)                                  \
+    do {                                               \
+        hipError_t e_ = (expr);                        \
+        if (e_ != hipSuccess) return hip_fail(e_, #expr); \
+    } while (0)
+
+extern "C" int32_t psn_abi_version(void) { return PSN_ABI_VERSION; }
+extern "C" const char *psn_last_error(void) { return g_err; }
+extern "C" const char *psn_error_name(int32_t code) {
+    switch (code) {
+        case PSN_OK: return "PSN_OK";
+        case PSN_E_INVALID_ARG: return "PSN_E_INVALID_ARG";
+        case PSN_E_SHAPE: return "PSN_E_SHAPE";
+        case PSN_E_UNSUPPORTED: return "PSN_E_UNSUPPORTED";
+        case PSN_E_NO_DEVICE: return "PSN_E_NO_DEVICE";
+        case PSN_E_OOM: return "PSN_E_OOM";
+        case PSN_E_MODULE: return "PSN_E_MODULE";
+        case PSN_E_HIP: return "PSN_E_HIP";
+        default: return "PSN_E_UNKNOWN";
+    }
+}
+
+/* ------------------------------------------------------------------ formats */
+
+extern "C" int32_t psn_block_elems(int32_t t) {
+    switch (t) {
+        case PSN_Q4_0: case PSN_Q8_0: return 32;
+        case PSN_Q4_K: case PSN_Q6_K: case PSN_Q8_K: return 256;
+        default: return 0;
+    }
+}
+extern "C" int32_t psn_block_bytes(int32_t t) {
+    switch (t) {
+        case PSN_Q4_0: return 18;
+        case PSN_Q8_0: return 34;
+        case PSN_Q4_K: return 144;
+        case PSN_Q6_K: return 210;
+        case PSN_Q8_K: return 292;
+        default: return 0;
+    }
+}
+extern "C" int64_t psn_row_bytes(int32_t t, int64_t k) {
+    const int64_t be = psn_block_elems(t);
+    if (be == 0) return fail(PSN_E_UNSUPPORTED, "unknown tensor type %d", t);
+    if (k <= 0 || k % be) return fail(PSN_E_SHAPE, "K=%lld is not a positive multiple of the block size %lld", (long long)k, (long long)be);
+    return k / be * psn_block_bytes(t);
+}
+static bool is_weight_type(int32_t t) { return t == PSN_Q4_0 || t == PSN_Q8_0 || t == PSN_Q4_K || t == PSN_Q6_K; }
+static const char *fmt_name(int32_t t) {
+    switch (t) {
+        case PSN_Q4_0: return "q4_0";
+        case PSN_Q8_0: return "q8_0";
+        case PSN_Q4_K: return "q4_K";
+        case PSN_Q6_K: return "q6_K";
+        default: return "?";
+    }
+}
+extern "C" int32_t psn_act_type_for(int32_t wt) {
+    if (wt == PSN_Q4_0 || wt == PSN_Q8_0) return PSN_Q8_0;
+    if (wt == PSN_Q4_K || wt == PSN_Q6_K) return PSN_Q8_K;
+    return fail(PSN_E_UNSUPPORTED, "type %d is not a weight type", wt);
+}
+
+static int64_t align_up(int64_t v, int64_t a) { return (v + a - 1) / a * a; }
+
+extern "C" int32_t psn_actq_layout(int32_t act_type, int64_t K, int32_t batch, psn_actq_info *out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_actq_layout: out is null");
+    if (batch < 1 || batch > 8) return fail(PSN_E_SHAPE, "batch=%d outside 1..8", batch);
+    if (act_type != PSN_Q8_0 && act_type != PSN_Q8_K) return fail(PSN_E_UNSUPPORTED, "activation type %d (want Q8_0 or Q8_K)", act_type);
+    const int64_t be = psn_block_elems(act_type);
+    if (K <= 0 || K % be) return fail(PSN_E_SHAPE, "K=%lld is not a positive multiple of %lld", (long long)K, (long long)be);
+    out->off_qs = 0;
+    out->off_d = align_up(batch * K, 256);
+    const int64_t d_bytes = batch * (K / be) * 4;
+    out->off_s = out->off_d + align_up(d_bytes, 256);
+    const int64_t s_bytes = act_type == PSN_Q8_0 ? batch * (K / 32) * 4 : batch * (K / 16) * 2;
+    out->bytes = out->off_s + align_up(s_bytes, 256);
+    return PSN_OK;
+}
+
+/* ------------------------------------------------------------------ handles */
+
+struct psn_ctx {
+    int device;
+    int compute_units;
+    int64_t total_mem;
+    int max_lds;
+    char arch[64];
+};
+struct psn_stream {
+    psn_ctx *ctx;
+    hipStream_t s;
+    void *ws;          /* activation workspace of psn_qmatvec (scheme Q8) */
+    size_t ws_bytes;
+};
+struct psn_buf {
+    psn_ctx *ctx;
+    void *p;
+    size_t bytes;
+};
+struct psn_event {
+    psn_ctx *ctx;
+    hipEvent_t e;
+};
+struct psn_module {
+    psn_ctx *ctx;
+    std::vector<hipModule_t> m;   /* one per code object; kernels are looked up across all */
+    std::mutex mu;
+    std::unordered_map<std::string, hipFunction_t> fn;
+};
+
+static int32_t bind(psn_ctx *c) {
+    if (!c) return fail(PSN_E_INVALID_ARG, "context is null");
+    HIP_TRY(hipSetDevice(c->device));
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_ctx_create(int32_t device, psn_ctx **out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_ctx_create: out is null");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) return fail(PSN_E_NO_DEVICE, "no HIP device visible (hipGetDeviceCount -> %d, count %d)", (int)e, n);
+    if (device < 0 || device >= n) return fail(PSN_E_NO_DEVICE, "device %d out of range (0..%d)", device, n - 1);
+    hipDeviceProp_t p;
+    HIP_TRY(hipGetDeviceProperties(&p, device));
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0)
+        return fail(PSN_E_NO_DEVICE, "device %d is %s; this library carries gfx950 code only", device, p.gcnArchName);
+    HIP_TRY(hipSetDevice(device));
+    psn_ctx *c = new (std::nothrow) psn_ctx();
+    if (!c) return fail(PSN_E_OOM, "host allocation failed");
+    c->device = device;
+    c->compute_units = p.multiProcessorCount;
+    c->total_mem = (int64_t)p.totalGlobalMem;
+    c->max_lds = (int)p.sharedMemPerBlock;
+    snprintf(c->arch, sizeof c->arch, "%s", p.gcnArchName);
+    *out = c;
+    return PSN_OK;
+}
+extern "C" int32_t psn_ctx_destroy(psn_ctx *c) {
+    if (!c) return fail(PSN_E_INVALID_ARG, "context is null");
+    delete c;
+    return PSN_OK;
+}
+extern "C" int32_t psn_ctx_info(psn_ctx *c, int32_t *cus, int64_t *mem, char *name, size_t n) {
+    if (!c) return fail(PSN_E_INVALID_ARG, "context is null");
+    if (cus) *cus = c->compute_units;
+    if (mem) *mem = c->total_mem;
+    if (name && n) snprintf(name, n, "%s", c->arch);
+    return PSN_OK;
+}
+
+static int32_t load_images(psn_ctx *c, const psn_blob *blobs, int n, psn_module **out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_module_load: out is null");
+    *out = nullptr;
+    if (!c) return fail(PSN_E_INVALID_ARG, "context is null");
+    for (int i = 0; i < n; ++i) {
+        const size_t len = (size_t)(blobs[i].end - blobs[i].begin);
+        if (!blobs[i].begin || len < 64) return fail(PSN_E_INVALID_ARG, "psn_module_load: empty code object");
+        if (memcmp(blobs[i].begin, "\x7f" "ELF", 4) != 0 && memcmp(blobs[i].begin, "__CLANG_OFFLOAD_BUNDLE__", 24) != 0)
+            return fail(PSN_E_MODULE, "psn_module_load: not an ELF code object or offload bundle");
+    }
+    int32_t rc = bind(c);
+    if (rc) return rc;
+    psn_module *mod = new (std::nothrow) psn_module();
+    if (!mod) return fail(PSN_E_OOM, "host allocation failed");
+    mod->ctx = c;
+    for (int i = 0; i < n; ++i) {
+        hipModule_t m;
+        hipError_t e = hipModuleLoadData(&m, blobs[i].begin);
+        if (e != hipSuccess) {
+            for (hipModule_t h : mod->m) (void)hipModuleUnload(h);
+            delete mod;
+            return fail(PSN_E_MODULE, "hipModuleLoadData(code object %d): hipError %d (%s)", i, (int)e, hipGetErrorString(e));
+        }
+        mod->m.push_back(m);
+    }
+    *out = mod;
+    return PSN_OK;
+}
+extern "C" int32_t psn_module_load(psn_ctx *c, const void *image, size_t len, psn_module **out) {
+    const psn_blob b = {(const unsigned char *)image, (const unsigned char *)image + (image ? len : 0)};
+    return load_images(c, &b, 1, out);
+}
+extern "C" int32_t psn_module_load_builtin(psn_ctx *c, psn_module **out) {
+    return load_images(c, psn_builtin_blobs, psn_builtin_blob_count, out);
+}
+extern "C" int32_t psn_module_unload(psn_module *mod) {
+    if (!mod) return fail(PSN_E_INVALID_ARG, "module is null");
+    int32_t rc = bind(mod->ctx);
+    if (rc) return rc;
+    hipError_t first = hipSuccess;
+    for (hipModule_t h : mod->m) {
+        hipError_t e = hipModuleUnload(h);
+        if (e != hipSuccess && first == hipSuccess) first = e;
+    }
+    delete mod;
+    if (first != hipSuccess) return hip_fail(first, "hipModuleUnload");
+    return PSN_OK;
+}
+static int32_t get_fn(psn_module *mod, const char *name, hipFunction_t *out) {
+    std::lock_guard<std::mutex> lk(mod->mu);
+    auto it = mod->fn.find(name);
+    if (it != mod->fn.end()) { *out = it->second; return PSN_OK; }
+    hipFunction_t f = nullptr;
+    hipError_t e = hipErrorNotFound;
+    for (hipModule_t h : mod->m) {
+        e = hipModuleGetFunction(&f, h, name);
+        if (e == hipSuccess) break;
+    }
+    if (e != hipSuccess) return fail(PSN_E_MODULE, "kernel '%s' not found in module: hipError %d (%s)", name, (int)e, hipGetErrorString(e));
+    mod->fn.emplace(name, f);
+    *out = f;
+    return PSN_OK;
+}
+extern "C" int32_t psn_module_has_kernel(psn_module *mod, const char *name) {
+    if (!mod || !name) return fail(PSN_E_INVALID_ARG, "module or name is null");
+    int32_t rc = bind(mod->ctx);
+    if (rc) return rc;
+    hipFunction_t f;
+    return get_fn(mod, name, &f);
+}
+
+extern "C" int32_t psn_stream_create(psn_ctx *c, psn_stream **out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_stream_create: out is null");
+    *out = nullptr;
+    int32_t rc = bind(c);
+    if (rc) return rc;
+    hipStream_t s;
+    HIP_TRY(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    psn_stream *st = new (std::nothrow) psn_stream();
+    if (!st) { (void)hipStreamDestroy(s); return fail(PSN_E_OOM, "host allocation failed"); }
+    st->ctx = c;
+    st->s = s;
+    st->ws = nullptr;
+    st->ws_bytes = 0;
+    *out = st;
+    return PSN_OK;
+}
+extern "C" int32_t psn_stream_sync(psn_stream *s) {
+    if (!s) return fail(PSN_E_INVALID_ARG, "stream is null");
+    int32_t rc = bind(s->ctx);
+    if (rc) return rc;
+    HIP_TRY(hipStreamSynchronize(s->s));
+    return PSN_OK;
+}
+extern "C" int32_t psn_stream_destroy(psn_stream *s) {
+    if (!s) return fail(PSN_E_INVALID_ARG, "stream is null");
+    int32_t rc = bind(s->ctx);
+    if (rc) return rc;
+    (void)hipStreamSynchronize(s->s);
+    if (s->ws) (void)hipFree(s->ws);
+    hipError_t e = hipStreamDestroy(s->s);
+    delete s;
+    if (e != hipSuccess) return hip_fail(e, "hipStreamDestroy");
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_event_create(psn_ctx *c, psn_event **out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_event_create: out is null");
+    *out = nullptr;
+    int32_t rc = bind(c);
+    if (rc) return rc;
+    hipEvent_t e;
+    HIP_TRY(hipEventCreate(&e));
+    psn_event *ev = new (std::nothrow) psn_event();
+    if (!ev) { (void)hipEventDestroy(e); return fail(PSN_E_OOM, "host allocation failed"); }
+    ev->ctx = c;
+    ev->e = e;
+    *out = ev;
+    return PSN_OK;
+}
+extern "C" int32_t psn_event_destroy(psn_event *e) {
+    if (!e) return fail(PSN_E_INVALID_ARG, "event is null");
+    int32_t rc = bind(e->ctx);
+    if (rc) return rc;
+    hipError_t r = hipEventDestroy(e->e);
+    delete e;
+    if (r != hipSuccess) return hip_fail(r, "hipEventDestroy");
+    return PSN_OK;
+}
+extern "C" int32_t psn_event_record(psn_event *e, psn_stream *s) {
+    if (!e || !s) return fail(PSN_E_INVALID_ARG, "event or stream is null");
+    if (e->ctx != s->ctx) return fail(PSN_E_INVALID_ARG, "event and stream belong to different contexts");
+    int32_t rc = bind(e->ctx);
+    if (rc) return rc;
+    HIP_TRY(hipEventRecord(e->e, s->s));
+    return PSN_OK;
+}
+extern "C" int32_t psn_event_elapsed_us(const psn_event *b, const psn_event *e, double *out) {
+    if (!b || !e || !out) return fail(PSN_E_INVALID_ARG, "event or out is null");
+    int32_t rc = bind(e->ctx);
+    if (rc) return rc;
+    HIP_TRY(hipEventSynchronize(e->e));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, b->e, e->e));
+    *out = (double)ms * 1000.0;
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_buf_alloc(psn_ctx *c, size_t bytes, psn_buf **out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_buf_alloc: out is null");
+    *out = nullptr;
+    if (bytes == 0) return fail(PSN_E_INVALID_ARG, "psn_buf_alloc: zero bytes");
+    int32_t rc = bind(c);
+    if (rc) return rc;
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, bytes);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+    psn_buf *b = new (std::nothrow) psn_buf();
+    if (!b) { (void)hipFree(p); return fail(PSN_E_OOM, "host allocation failed"); }
+    b->ctx = c;
+    b->p = p;
+    b->bytes = bytes;
+    *out = b;
+    return PSN_OK;
+}
+extern "C" int32_t psn_buf_free(psn_buf *b) {
+    if (!b) return fail(PSN_E_INVALID_ARG, "buffer is null");
+    int32_t rc = bind(b->ctx);
+    if (rc) return rc;
+    hipError_t e = hipFree(b->p);
+    delete b;
+    if (e != hipSuccess) return hip_fail(e, "hipFree");
+    return PSN_OK;
+}
+extern "C" int64_t psn_buf_size(const psn_buf *b) {
+    if (!b) return fail(PSN_E_INVALID_ARG, "buffer is null");
+    return (int64_t)b->bytes;
+}
+static int32_t check_range(const psn_buf *b, size_t off, size_t n, const char *what) {
+    if (!b) return fail(PSN_E_INVALID_ARG, "%s: buffer is null", what);
+    if (off > b->bytes || n > b->bytes - off) return fail(PSN_E_INVALID_ARG, "%s: range [%zu, %zu) outside buffer of %zu bytes", what, off, off + n, b->bytes);
+    return PSN_OK;
+}
+extern "C" int32_t psn_buf_upload(psn_buf *dst, size_t off, const void *src, size_t n, psn_stream *s) {
+    int32_t rc = check_range(dst, off, n, "psn_buf_upload");
+    if (rc) return rc;
+    if (!src || !s) return fail(PSN_E_INVALID_ARG, "psn_buf_upload: src or stream is null");
+    if (s->ctx != dst->ctx) return fail(PSN_E_INVALID_ARG, "psn_buf_upload: stream and buffer belong to different contexts");
+    if ((rc = bind(dst->ctx))) return rc;
+    if (n == 0) return PSN_OK;
+    /* pageable source: the copy is staged, so the caller may reuse src on return */
+    HIP_TRY(hipMemcpyAsync((char *)dst->p + off, src, n, hipMemcpyHostToDevice, s->s));
+    HIP_TRY(hipStreamSynchronize(s->s));
+    return PSN_OK;
+}
+extern "C" int32_t psn_buf_download(const psn_buf *src, size_t off, void *dst, size_t n, psn_stream *s) {
+    int32_t rc = check_range(src, off, n, "psn_buf_download");
+    if (rc) return rc;
+    if (!dst || !s) return fail(PSN_E_INVALID_ARG, "psn_buf_download: dst or stream is null");
+    if (s->ctx != src->ctx) return fail(PSN_E_INVALID_ARG, "psn_buf_download: stream and buffer belong to different contexts");
+    if ((rc = bind(src->ctx))) return rc;
+    if (n == 0) return PSN_OK;
+    HIP_TRY(hipMemcpyAsync(dst, (const char *)src->p + off, n, hipMemcpyDeviceToHost, s->s));
+    HIP_TRY(hipStreamSynchronize(s->s));
+    return PSN_OK;
+}
+extern "C" int32_t psn_buf_fill_zero(psn_buf *b, psn_stream *s) {
+    if (!b || !s) return fail(PSN_E_INVALID_ARG, "buffer or stream is null");
+    int32_t rc = bind(b->ctx);
+    if (rc) return rc;
+    HIP_TRY(hipMemsetAsync(b->p, 0, b->bytes, s->s));
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_weight_upload(psn_ctx *c, int32_t qtype, int64_t N, int64_t K, const void *blocks, int32_t layout,
+                                     psn_stream *s, psn_buf **out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_weight_upload: out is null");
+    *out = nullptr;
+    if (!c || !blocks || !s) return fail(PSN_E_INVALID_ARG, "psn_weight_upload: null argument");
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "psn_weight_upload: type %d is not Q4_0/Q8_0/Q4_K/Q6_K", qtype);
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "psn_weight_upload: layout %d", layout);
+    if (N <= 0) return fail(PSN_E_SHAPE, "N=%lld must be positive", (long long)N);
+    const int64_t rb = psn_row_bytes(qtype, K);
+    if (rb < 0) return (int32_t)rb;
+    psn_buf *b = nullptr;
+    int32_t rc = psn_buf_alloc(c, (size_t)(N * rb), &b);
+    if (rc) return rc;
+    rc = psn_buf_upload(b, 0, blocks, (size_t)(N * rb), s);
+    if (rc) { (void)psn_buf_free(b); return rc; }
+    *out = b;
+    return PSN_OK;
+}
+
+/* ------------------------------------------------------------------ launches */
+
+static int32_t launch(psn_module *mod, psn_stream *s, const char *kernel, unsigned blocks, unsigned threads, unsigned lds,
+                      void *args_struct) {
+    hipFunction_t f;
+    int32_t rc = get_fn(mod, kernel, &f);
+    if (rc) return rc;
+    void *params[] = {args_struct};
+    hipError_t e = hipModuleLaunchKernel(f, blocks, 1, 1, threads, 1, 1, lds, s->s, params, nullptr);
+    if (e != hipSuccess) return fail(PSN_E_HIP, "launch of %s <<<%u,%u,%u>>> failed: hipError %d (%s)", kernel, blocks, threads, lds, (int)e, hipGetErrorString(e));
+    return PSN_OK;
+}
+
+static int32_t check_same_ctx(psn_module *mod, psn_stream *s, const psn_buf *a, const psn_buf *b, const psn_buf *c, const char *what) {
+    if (!mod || !s || !a || !b || !c) return fail(PSN_E_INVALID_ARG, "%s: null handle", what);
+    if (s->ctx != mod->ctx || a->ctx != mod->ctx || b->ctx != mod->ctx || c->ctx != mod->ctx)
+        return fail(PSN_E_INVALID_ARG, "%s: handles belong to different contexts", what);
+    return PSN_OK;
+}
+
+static int32_t quantize_into(psn_module *mod, psn_stream *s, int32_t act_type, const float *x, void *xq, int64_t K, int32_t batch) {
+    psn_actq_info li;
+    int32_t rc = psn_actq_layout(act_type, K, batch, &li);
+    if (rc) return rc;
+    psn_quantize_args qa;
+    qa.x = x;
+    qa.qs = (int8_t *)xq + li.off_qs;
+    qa.d = (float *)((char *)xq + li.off_d);
+    qa.s = (char *)xq + li.off_s;
+    qa.K = (int32_t)K;
+    qa.batch = batch;
+    if (act_type == PSN_Q8_0) {
+        const int64_t threads = K * batch / 4;
+        return launch(mod, s, "psn_quantize_q8_0", (unsigned)((threads + 255) / 256), 256, 0, &qa);
+    }
+    const int64_t waves = K * batch / 256;
+    return launch(mod, s, "psn_quantize_q8_K", (unsigned)((waves + 3) / 4), 256, 0, &qa);
+}
+
+extern "C" int32_t psn_act_quantize(psn_module *mod, psn_stream *s, int32_t act_type, const psn_buf *x, psn_buf *xq, int64_t K, int32_t batch) {
+    int32_t rc = check_same_ctx(mod, s, x, xq, xq, "psn_act_quantize");
+    if (rc) return rc;
+    psn_actq_info li;
+    if ((rc = psn_actq_layout(act_type, K, batch, &li))) return rc;
+    if (K > INT32_MAX / 8) return fail(PSN_E_SHAPE, "K=%lld too large", (long long)K);
+    if ((int64_t)x->bytes < K * batch * 4) return fail(PSN_E_INVALID_ARG, "psn_act_quantize: x holds %zu bytes, need %lld", x->bytes, (long long)(K * batch * 4));
+    if ((int64_t)xq->bytes < li.bytes) return fail(PSN_E_INVALID_ARG, "psn_act_quantize: x_q holds %zu bytes, need %lld", xq->bytes, (long long)li.bytes);
+    if ((rc = bind(mod->ctx))) return rc;
+    return quantize_into(mod, s, act_type, (const float *)x->p, xq->p, K, batch);
+}
+
+static int32_t check_matvec_shape(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch) {
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "matvec: type %d is not Q4_0/Q8_0/Q4_K/Q6_K", qtype);
+    if (scheme != PSN_ACT_F32 && scheme != PSN_ACT_Q8) return fail(PSN_E_UNSUPPORTED, "matvec: activation scheme %d", scheme);
+    if (N <= 0 || N > INT32_MAX / 2) return fail(PSN_E_SHAPE, "N=%lld must be in 1..2^30", (long long)N);
+    if (batch < 1 || batch > 8) return fail(PSN_E_SHAPE, "batch=%d outside 1..8", batch);
+    const int64_t rb = psn_row_bytes(qtype, K);
+    if (rb < 0) return (int32_t)rb;
+    if (K % 256) return fail(PSN_E_SHAPE, "K=%lld: the gfx950 matvec kernels need K to be a multiple of 256", (long long)K);
+    if (K > (1 << 24)) return fail(PSN_E_SHAPE, "K=%lld too large", (long long)K);
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, psn_matvec_plan *out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_plan: out is null");
+    int32_t rc = check_matvec_shape(qtype, scheme, N, K, batch);
+    if (rc) return rc;
+    if (cus <= 0) cus = 256;
+    const int64_t C = K / 256;
+    psn_matvec_plan p;
+    p.lanes_per_row = C <= 8 ? 8 : C <= 16 ? 16 : C <= 32 ? 32 : 64;
+    p.batch_tile = batch <= 1 ? 1 : batch <= 2 ? 2 : batch <= 4 ? 4 : 8;
+    p.stage_lds = 0;
+    p.lds_bytes = 0;
+    /* rows in flight per lane: keep at least ~4 waves per CU, otherwise more bytes per lane */
+    const int64_t S = 64 / p.lanes_per_row;
+    p.rows_in_flight = 1;
+    if (p.batch_tile == 1 && scheme == PSN_ACT_Q8) {
+        const int64_t waves_r2 = (N + 2 * S - 1) / (2 * S);
+        if (waves_r2 >= (int64_t)cus * 8) p.rows_in_flight = 2;
+    }
+    const int64_t rows_per_wave = S * p.rows_in_flight;
+    const int64_t passes = (N + rows_per_wave - 1) / rows_per_wave;
+    int64_t blocks = (passes + 3) / 4;
+    const int64_t cap = (int64_t)cus * 16;
+    if (blocks > cap) blocks = cap;
+    p.blocks = (int32_t)blocks;
+    *out = p;
+    return PSN_OK;
+}
+
+static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t scheme, int64_t K, int32_t batch, int max_lds, int32_t *lds_out) {
+    const int g = p->lanes_per_row, r = p->rows_in_flight, nb = p->batch_tile;
+    if (!(g == 8 || g == 16 || g == 32 || g == 64)) return fail(PSN_E_UNSUPPORTED, "plan: lanes_per_row=%d", g);
+    if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
+    bool ok;
+    if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2 || r == 4)) || ((nb == 2 || nb == 4) && (r == 1 || r == 2)) || (nb == 8 && r == 1);
+    else ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
+    if (!ok) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
+    if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
+    int32_t lds = 0;
+    if (p->stage_lds) {
+        if (scheme != PSN_ACT_Q8) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging exists for scheme Q8 only");
+        psn_actq_info li;
+        int32_t rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li);
+        if (rc) return rc;
+        /* packed copy of the three fields, each rounded to 16 bytes */
+        const int64_t be = psn_block_elems(psn_act_type_for(qtype));
+        const int64_t qs = batch * K, d = align_up(batch * (K / be) * 4, 16);
+        const int64_t sb = psn_act_type_for(qtype) == PSN_Q8_0 ? batch * (K / 32) * 4 : batch * (K / 16) * 2;
+        const int64_t total = qs + d + align_up(sb, 16);
+        if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging needs %lld bytes, device offers %d", (long long)total, max_lds);
+        lds = (int32_t)total;
+    }
+    *lds_out = lds;
+    return PSN_OK;
+}
+
+static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const void *W, const void *x,
+                          float *y, int64_t N, int64_t K, int32_t batch, const psn_matvec_plan *plan) {
+    int32_t lds = 0;
+    int32_t rc = plan_is_valid(plan, qtype, scheme, K, batch, mod->ctx->max_lds, &lds);
+    if (rc) return rc;
+    psn_matvec_args a;
+    memset(&a, 0, sizeof a);
+    a.W = (const uint8_t *)W;
+    a.y = y;
+    a.N = (int32_t)N;
+    a.K = (int32_t)K;
+    a.batch = batch;
+    a.row_bytes = psn_row_bytes(qtype, K);
+    char name[96];
+    if (scheme == PSN_ACT_Q8) {
+        psn_actq_info li;
+        if ((rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li))) return rc;
+        a.xqs = (const int8_t *)x + li.off_qs;
+        a.xd = (const float *)((const char *)x + li.off_d);
+        a.xs = (const char *)x + li.off_s;
+        snprintf(name, sizeof name, "psn_mv_%s_q8_g%d_r%d_b%d%s", fmt_name(qtype), plan->lanes_per_row, plan->rows_in_flight,
+                 plan->batch_tile, plan->stage_lds ? "_lds" : "");
+    } else {
+        a.xf = (const float *)x;
+        snprintf(name, sizeof name, "psn_mv_%s_f32_g%d_r%d_b%d", fmt_name(qtype), plan->lanes_per_row, plan->rows_in_flight, plan->batch_tile);
+    }
+    return launch(mod, s, name, (unsigned)plan->blocks, 256, (unsigned)lds, &a);
+}
+
+static int32_t check_matvec_bufs(int32_t qtype, const psn_buf *W, const psn_buf *y, int64_t N, int64_t K, int32_t batch) {
+    const int64_t need_w = N * psn_row_bytes(qtype, K);
+    if ((int64_t)W->bytes < need_w) return fail(PSN_E_INVALID_ARG, "matvec: W holds %zu bytes, need %lld", W->bytes, (long long)need_w);
+    if ((int64_t)y->bytes < N * batch * 4) return fail(PSN_E_INVALID_ARG, "matvec: y holds %zu bytes, need %lld", y->bytes, (long long)(N * batch * 4));
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const psn_buf *W,
+                                       const psn_buf *x, psn_buf *y, int64_t N, int64_t K, int32_t batch, const psn_matvec_plan *plan) {
+    int32_t rc = check_same_ctx(mod, s, W, x, y, "psn_qmatvec_planned");
+    if (rc) return rc;
+    if (!plan) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_planned: plan is null");
+    if ((rc = check_matvec_shape(qtype, scheme, N, K, batch))) return rc;
+    if ((rc = check_matvec_bufs(qtype, W, y, N, K, batch))) return rc;
+    if (scheme == PSN_ACT_Q8) {
+        psn_actq_info li;
+        if ((rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li))) return rc;
+        if ((int64_t)x->bytes < li.bytes) return fail(PSN_E_INVALID_ARG, "matvec: x_q holds %zu bytes, need %lld", x->bytes, (long long)li.bytes);
+    } else if ((int64_t)x->bytes < K * batch * 4) {
+        return fail(PSN_E_INVALID_ARG, "matvec: x holds %zu bytes, need %lld", x->bytes, (long long)(K * batch * 4));
+    }
+    if ((rc = bind(mod->ctx))) return rc;
+    return run_matvec(mod, s, qtype, scheme, W->p, x->p, (float *)y->p, N, K, batch, plan);
+}
+
+extern "C" int32_t psn_qmatvec_q8(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
+                                  const psn_buf *xq, psn_buf *y, int64_t N, int64_t K, int32_t batch) {
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
+    if (!mod) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_q8: module is null");
+    psn_matvec_plan plan;
+    int32_t rc = psn_qmatvec_plan(qtype, PSN_ACT_Q8, N, K, batch, mod->ctx->compute_units, &plan);
+    if (rc) return rc;
+    return psn_qmatvec_planned(mod, s, qtype, PSN_ACT_Q8, W, xq, y, N, K, batch, &plan);
+}
+
+extern "C" int32_t psn_qmatvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, const psn_buf *W,
+                               const psn_buf *x, psn_buf *y, int64_t N, int64_t K, int32_t batch) {
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
+    int32_t rc = check_same_ctx(mod, s, W, x, y, "psn_qmatvec");
+    if (rc) return rc;
+    if ((rc = check_matvec_shape(qtype, scheme, N, K, batch))) return rc;
+    if ((rc = check_matvec_bufs(qtype, W, y, N, K, batch))) return rc;
+    if ((int64_t)x->bytes < K * batch * 4) return fail(PSN_E_INVALID_ARG, "matvec: x holds %zu bytes, need %lld", x->bytes, (long long)(K * batch * 4));
+    psn_matvec_plan plan;
+    if ((rc = psn_qmatvec_plan(qtype, scheme, N, K, batch, mod->ctx->compute_units, &plan))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    if (scheme == PSN_ACT_F32) return run_matvec(mod, s, qtype, scheme, W->p, x->p, (float *)y->p, N, K, batch, &plan);
+    const int32_t at = psn_act_type_for(qtype);
+    psn_actq_info li;
+    if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;
+    if (s->ws_bytes < (size_t)li.bytes) {
+        /* grow the stream's activation workspace; earlier launches may still read the old one */
+        HIP_TRY(hipStreamSynchronize(s->s));
+        if (s->ws) HIP_TRY(hipFree(s->ws));
+        s->ws = nullptr;
+        s->ws_bytes = 0;
+        const size_t want = (size_t)align_up(li.bytes, 1 << 20);
+        hipError_t e = hipMalloc(&s->ws, want);
+        if (e != hipSuccess) return hip_fail(e, "hipMalloc(workspace)");
+        s->ws_bytes = want;
+    }
+    if ((rc = quantize_into(mod, s, at, (const float *)x->p, s->ws, K, batch))) return rc;
+    return run_matvec(mod, s, qtype, scheme, W->p, s->ws, (float *)y->p, N, K, batch, &plan);
+}
+
+/* ------------------------------------------------------------------ prefill */
+
+extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
+                                       const psn_buf *X, psn_buf *Y, int64_t M, int64_t N, int64_t K) {
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "prefill: layout %d", layout);
+    int32_t rc = check_same_ctx(mod, s, W, X, Y, "psn_qmatmul_prefill");
+    if (rc) return rc;
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) return fail(PSN_E_UNSUPPORTED, "prefill: type %d (Q4_0 and Q8_0 have kernels)", qtype);
+    if (M <= 0 || N <= 0 || M > (1 << 20) || N > (1 << 24)) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld out of range", (long long)M, (long long)N);
+    const int64_t rb = psn_row_bytes(qtype, K);
+    if (rb < 0) return (int32_t)rb;
+    if (K % 256 || K > (1 << 24)) return fail(PSN_E_SHAPE, "prefill: K=%lld must be a multiple of 256", (long long)K);
+    if ((int64_t)W->bytes < N * rb) return fail(PSN_E_INVALID_ARG, "prefill: W holds %zu bytes, need %lld", W->bytes, (long long)(N * rb));
+    if ((int64_t)X->bytes < M * K * 2) return fail(PSN_E_INVALID_ARG, "prefill: X holds %zu bytes, need %lld", X->bytes, (long long)(M * K * 2));
+    if ((int64_t)Y->bytes < M * N * 4) return fail(PSN_E_INVALID_ARG, "prefill: Y holds %zu bytes, need %lld", Y->bytes, (long long)(M * N * 4));
+    if ((rc = bind(mod->ctx))) return rc;
+    return fail(PSN_E_UNSUPPORTED, "prefill: kernel not built into this library yet");
+}

@@ -1,0 +1,625 @@
+/*
+ * psn_matvec.hip -- gfx950 decode kernels: activation quantizers and the batch-1..8 quantized
+ * matvec y[b][n] = sum_k deq(W)[n][k] * x[b][k] over GGUF Q4_0 / Q8_0 / Q4_K / Q6_K rows.
+ *
+ * The matvec is an HBM stream, so everything is organised around 128-bit loads of the raw GGUF
+ * bytes.  Blocks are 18 / 34 / 144 / 210 bytes, which is not a multiple of 16, but 256 weights
+ * always are a whole number of 16-byte words for Q4_0 (144 B), Q8_0 (272 B) and Q4_K (144 B), so a
+ * lane owns one 256-weight "chunk" of a row: it fetches it with 9 or 17 aligned dwordx4 loads and
+ * re-aligns the 2-byte-shifted halves in registers with v_alignbyte.  Q6_K (210 B) is fetched with
+ * 2-byte-aligned dwordx4 loads, which gfx950 serves in unaligned access mode.
+ *
+ * Work split: G lanes share a row (G = 8..64), a wave therefore holds 64/G rows at a time and R
+ * such row sets are in flight per lane to keep enough bytes outstanding; partial sums are folded
+ * with DPP / ds_swizzle (psn_device.h).  Weights held in registers are re-used for every batch
+ * column.  Scheme Q8 multiplies int8 x int8 with v_dot4_i32_i8 and applies the fp16 block scales in
+ * fp32; scheme F32 dequantizes to fp32 and uses fp32 FMA.
+ */
+#include "psn_args.h"
+#include "psn_device.h"
+
+#define UNROLL _Pragma("unroll")
+
+/* ------------------------------------------------------------------------------------------
+ * Activation quantizers (bit-exact restatements of the Q8_0 / Q8_K row quantizers).
+ * ------------------------------------------------------------------------------------------ */
+
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_QUANT)
+/* Q8_0: 8 lanes per 32-element block, 4 elements per lane.  d = amax/127, q = round-half-away(x/d). */
+extern "C" __global__ void __launch_bounds__(256) psn_quantize_q8_0(const psn_quantize_args a) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   /* one float4 each */
+    const int64_t total4 = (int64_t)a.K * a.batch / 4;
+    const bool live = t < total4;
+    float4 v = live ? reinterpret_cast<const float4 *>(a.x)[t] : make_float4(0.f, 0.f, 0.f, 0.f);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = group_max<8>(amax);
+    const float d = amax / 127.f;
+    const float id = d != 0.f ? 1.f / d : 0.f;
+    const int q0 = (int)roundf(v.x * id), q1 = (int)roundf(v.y * id);
+    const int q2 = (int)roundf(v.z * id), q3 = (int)roundf(v.w * id);
+    const int s = group_sum_i<8>(q0 + q1 + q2 + q3);
+    if (!live) return;
+    reinterpret_cast<u32 *>(a.qs)[t] = (u32)(q0 & 0xff) | ((u32)(q1 & 0xff) << 8) | ((u32)(q2 & 0xff) << 16) | ((u32)q3 << 24);
+    if ((threadIdx.x & 7) == 0) {
+        a.d[t >> 3] = (float)(f16)d;            /* what a reader of the fp16 field would see */
+        reinterpret_cast<int *>(a.s)[t >> 3] = s;
+    }
+}
+
+/* Q8_K: one wave per 256-element super-block.  iscale = -127/(signed element of largest magnitude,
+ * first one on ties), q = min(127, rint(iscale*x)), d = 1/iscale, bsums over groups of 16. */
+extern "C" __global__ void __launch_bounds__(256) psn_quantize_q8_K(const psn_quantize_args a) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;   /* super-block index */
+    const int64_t nsb = (int64_t)a.K * a.batch / 256;
+    if (sb >= nsb) return;                                                        /* whole wave leaves together */
+    const float4 v = reinterpret_cast<const float4 *>(a.x)[sb * 64 + lane];
+    const float e[4] = {v.x, v.y, v.z, v.w};
+    float amax = 0.f;
+    int first = 4;
+    UNROLL for (int i = 3; i >= 0; --i) if (fabsf(e[i]) >= amax) { amax = fabsf(e[i]); first = i; }
+    /* >= scanning downwards leaves the lowest index among equal magnitudes */
+    const float wmax = group_max<64>(amax);
+    const int cand = (amax == wmax) ? lane * 4 + first : 1 << 20;
+    const int idx = group_min_i<64>(cand);
+    const float mine = e[idx & 3];
+    const float vmax = __shfl(mine, idx >> 2, 64);
+    u32 packed = 0;
+    int s4 = 0;
+    float dout = 0.f;
+    if (wmax != 0.f) {
+        const float iscale = -127.f / vmax;
+        UNROLL for (int i = 0; i < 4; ++i) {
+            int q = (int)__builtin_rintf(iscale * e[i]);
+            q = q > 127 ? 127 : q;
+            s4 += q;
+            packed |= (u32)(q & 0xff) << (8 * i);
+        }
+        dout = 1.f / iscale;
+    }
+    const int s16 = group_sum_i<4>(s4);
+    reinterpret_cast<u32 *>(a.qs)[sb * 64 + lane] = packed;
+    if ((lane & 3) == 0) reinterpret_cast<int16_t *>(a.s)[sb * 16 + (lane >> 2)] = (int16_t)s16;
+    if (lane == 0) a.d[sb] = dout;
+}
+#endif
+
+/* ------------------------------------------------------------------------------------------
+ * Shared scaffolding of the chunk-per-lane matvec kernels.
+ * ------------------------------------------------------------------------------------------ */
+
+template <int G, int R>
+struct RowMap {
+    static constexpr int S = 64 / G;          /* rows a wave holds side by side */
+    static constexpr int ROWS = S * R;        /* rows a wave retires per pass */
+    int lane, slot, j, wave, nwaves;
+    PSN_DEV RowMap() {
+        lane = threadIdx.x & 63;
+        slot = lane / G;
+        j = lane % G;
+        const int wpb = blockDim.x >> 6;
+        wave = blockIdx.x * wpb + (threadIdx.x >> 6);
+        nwaves = gridDim.x * wpb;
+    }
+};
+
+template <int G, int R, int NB>
+PSN_DEV void store_rows(const RowMap<G, R> &m, float (&acc)[R][NB], const psn_matvec_args &a, int row0) {
+    UNROLL for (int r = 0; r < R; ++r) {
+        const int row = row0 + r * RowMap<G, R>::S + m.slot;
+        UNROLL for (int nb = 0; nb < NB; ++nb) {
+            const float v = group_sum<G>(acc[r][nb]);
+            if (m.j == 0 && row < a.N && nb < a.batch) a.y[(int64_t)nb * a.N + row] = v;
+        }
+    }
+}
+
+/* Copies the live batch columns of a quantized activation into LDS (same three-region layout,
+ * packed for `batch` columns) and re-points the accessors at it. */
+template <typename ST>
+PSN_DEV void stage_actq(const psn_matvec_args &a, int d_per_col, int s_per_col, const int8_t *&xqs, const float *&xd, const ST *&xs) {
+    extern __shared__ uint4 psn_smem[];
+    const int n_qs = a.batch * a.K / 16;
+    /* field sizes rounded up to whole 16-byte words: the global regions are padded to 256 B */
+    const int n_d = (a.batch * d_per_col * 4 + 15) / 16;
+    const int n_s = (a.batch * s_per_col * (int)sizeof(ST) + 15) / 16;
+    uint4 *l_qs = psn_smem, *l_d = l_qs + n_qs, *l_s = l_d + n_d;
+    const uint4 *g_qs = reinterpret_cast<const uint4 *>(xqs), *g_d = reinterpret_cast<const uint4 *>(xd);
+    const uint4 *g_s = reinterpret_cast<const uint4 *>(xs);
+    for (int i = threadIdx.x; i < n_qs; i += blockDim.x) l_qs[i] = g_qs[i];
+    for (int i = threadIdx.x; i < n_d; i += blockDim.x) l_d[i] = g_d[i];
+    for (int i = threadIdx.x; i < n_s; i += blockDim.x) l_s[i] = g_s[i];
+    __syncthreads();
+    xqs = reinterpret_cast<const int8_t *>(l_qs);
+    xd = reinterpret_cast<const float *>(l_d);
+    xs = reinterpret_cast<const ST *>(l_s);
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Q4_0 x Q8_0-activations.  Chunk = 8 blocks = 144 B = 36 dwords.
+ * Block b of the chunk starts at byte 18b: even blocks start on a dword (fp16 d in the low half,
+ * quants shifted by two bytes), odd blocks start mid-dword (d in the high half, quants aligned).
+ * sum (q-8)*x = sum q*x - 8*sum x uses the activation block sums so nibbles stay unsigned.
+ * ------------------------------------------------------------------------------------------ */
+
+template <int B>
+PSN_DEV void q4_0_block(const u32 (&w)[36], float &d, u32 (&lo)[4], u32 (&hi)[4]) {
+    constexpr int base = 9 * (B >> 1);
+    u32 q[4];
+    if constexpr ((B & 1) == 0) {
+        d = h2f_lo(w[base]);
+        UNROLL for (int i = 0; i < 4; ++i) q[i] = align2(w[base + i + 1], w[base + i]);
+    } else {
+        d = h2f_hi(w[base + 4]);
+        UNROLL for (int i = 0; i < 4; ++i) q[i] = w[base + 5 + i];
+    }
+    UNROLL for (int i = 0; i < 4; ++i) { lo[i] = q[i] & 0x0f0f0f0fu; hi[i] = (q[i] >> 4) & 0x0f0f0f0fu; }
+}
+
+template <int B, int R, int NB>
+PSN_DEV void q4_0_q8_step(const u32 (&w)[R][36], const int8_t *xqs, const float *xd, const int *xs, int K, int nblk,
+                          int blk0, int batch, float (&acc)[R][NB]) {
+    float dw[R];
+    u32 lo[R][4], hi[R][4];
+    UNROLL for (int r = 0; r < R; ++r) q4_0_block<B>(w[r], dw[r], lo[r], hi[r]);
+    UNROLL for (int nb = 0; nb < NB; ++nb) {
+        const int col = nb < batch ? nb : batch - 1;
+        const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)(blk0 + B) * 32);
+        const uint4 x0 = xp[0], x1 = xp[1];
+        const float dx = xd[col * nblk + blk0 + B];
+        const int sx = xs[col * nblk + blk0 + B];
+        UNROLL for (int r = 0; r < R; ++r) {
+            int s = dot4(lo[r][0], x0.x, 0);
+            s = dot4(lo[r][1], x0.y, s);
+            s = dot4(lo[r][2], x0.z, s);
+            s = dot4(lo[r][3], x0.w, s);
+            s = dot4(hi[r][0], x1.x, s);
+            s = dot4(hi[r][1], x1.y, s);
+            s = dot4(hi[r][2], x1.z, s);
+            s = dot4(hi[r][3], x1.w, s);
+            s -= 8 * sx;
+            acc[r][nb] += (float)s * dw[r] * dx;
+        }
+    }
+}
+
+template <int G, int R, int NB, bool XLDS>
+PSN_DEV void mv_q4_0_q8(const psn_matvec_args &a) {
+    const RowMap<G, R> m;
+    const int K = a.K, C = K >> 8, nblk = K >> 5;
+    const int8_t *xqs = a.xqs;
+    const float *xd = a.xd;
+    const int *xs = reinterpret_cast<const int *>(a.xs);
+    if constexpr (XLDS) stage_actq<int>(a, nblk, nblk, xqs, xd, xs);
+    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
+        float acc[R][NB];
+        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+        for (int c = m.j; c < C; c += G) {
+            u32 w[R][36];
+            UNROLL for (int r = 0; r < R; ++r) {
+                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
+                const uint4 *p = reinterpret_cast<const uint4 *>(a.W + (int64_t)row * a.row_bytes) + c * 9;
+                UNROLL for (int i = 0; i < 9; ++i) unpack4(p[i], &w[r][4 * i]);
+            }
+            const int blk0 = c * 8;
+            q4_0_q8_step<0>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+            q4_0_q8_step<1>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+            q4_0_q8_step<2>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+            q4_0_q8_step<3>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+            q4_0_q8_step<4>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+            q4_0_q8_step<5>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+            q4_0_q8_step<6>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+            q4_0_q8_step<7>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
+        }
+        store_rows<G, R, NB>(m, acc, a, row0);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Q8_0 x Q8_0-activations.  Chunk = 8 blocks = 272 B = 68 dwords; block b starts at byte 34b.
+ * ------------------------------------------------------------------------------------------ */
+
+template <int B>
+PSN_DEV void q8_0_block(const u32 (&w)[68], float &d, u32 (&q)[8]) {
+    constexpr int base = 17 * (B >> 1);
+    if constexpr ((B & 1) == 0) {
+        d = h2f_lo(w[base]);
+        UNROLL for (int i = 0; i < 8; ++i) q[i] = align2(w[base + i + 1], w[base + i]);
+    } else {
+        d = h2f_hi(w[base + 8]);
+        UNROLL for (int i = 0; i < 8; ++i) q[i] = w[base + 9 + i];
+    }
+}
+
+template <int B, int R, int NB>
+PSN_DEV void q8_0_q8_step(const u32 (&w)[R][68], const int8_t *xqs, const float *xd, int K, int nblk, int blk0, int batch,
+                          float (&acc)[R][NB]) {
+    float dw[R];
+    u32 q[R][8];
+    UNROLL for (int r = 0; r < R; ++r) q8_0_block<B>(w[r], dw[r], q[r]);
+    UNROLL for (int nb = 0; nb < NB; ++nb) {
+        const int col = nb < batch ? nb : batch - 1;
+        const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)(blk0 + B) * 32);
+        const uint4 x0 = xp[0], x1 = xp[1];
+        const float dx = xd[col * nblk + blk0 + B];
+        UNROLL for (int r = 0; r < R; ++r) {
+            int s = dot4(q[r][0], x0.x, 0);
+            s = dot4(q[r][1], x0.y, s);
+            s = dot4(q[r][2], x0.z, s);
+            s = dot4(q[r][3], x0.w, s);
+            s = dot4(q[r][4], x1.x, s);
+            s = dot4(q[r][5], x1.y, s);
+            s = dot4(q[r][6], x1.z, s);
+            s = dot4(q[r][7], x1.w, s);
+            acc[r][nb] += (float)s * (dw[r] * dx);
+        }
+    }
+}
+
+template <int G, int R, int NB, bool XLDS>
+PSN_DEV void mv_q8_0_q8(const psn_matvec_args &a) {
+    const RowMap<G, R> m;
+    const int K = a.K, C = K >> 8, nblk = K >> 5;
+    const int8_t *xqs = a.xqs;
+    const float *xd = a.xd;
+    const int *xs = reinterpret_cast<const int *>(a.xs);
+    if constexpr (XLDS) stage_actq<int>(a, nblk, nblk, xqs, xd, xs);
+    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
+        float acc[R][NB];
+        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+        for (int c = m.j; c < C; c += G) {
+            u32 w[R][68];
+            UNROLL for (int r = 0; r < R; ++r) {
+                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
+                const uint4 *p = reinterpret_cast<const uint4 *>(a.W + (int64_t)row * a.row_bytes) + c * 17;
+                UNROLL for (int i = 0; i < 17; ++i) unpack4(p[i], &w[r][4 * i]);
+            }
+            const int blk0 = c * 8;
+            q8_0_q8_step<0>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+            q8_0_q8_step<1>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+            q8_0_q8_step<2>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+            q8_0_q8_step<3>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+            q8_0_q8_step<4>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+            q8_0_q8_step<5>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+            q8_0_q8_step<6>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+            q8_0_q8_step<7>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
+        }
+        store_rows<G, R, NB>(m, acc, a, row0);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Q4_K x Q8_K-activations.  Chunk = one 144-byte super-block: dword 0 = d | dmin<<16,
+ * dwords 1..3 = the 12-byte 6-bit scale/min field, dwords 4..35 = 128 nibble bytes.
+ * ------------------------------------------------------------------------------------------ */
+
+PSN_DEV void q4_K_scales(u32 s0, u32 s1, u32 s2, u32 (&sc)[2], u32 (&mn)[2]) {
+    sc[0] = s0 & 0x3f3f3f3fu;
+    mn[0] = s1 & 0x3f3f3f3fu;
+    sc[1] = (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u);
+    mn[1] = ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u);
+}
+PSN_DEV int byte_of(const u32 (&v)[2], int i) { return (int)((v[i >> 2] >> (8 * (i & 3))) & 0xffu); }
+
+template <int G, int R, int NB, bool XLDS>
+PSN_DEV void mv_q4_K_q8(const psn_matvec_args &a) {
+    const RowMap<G, R> m;
+    const int K = a.K, C = K >> 8;
+    const int8_t *xqs = a.xqs;
+    const float *xd = a.xd;
+    const int16_t *xs = reinterpret_cast<const int16_t *>(a.xs);
+    if constexpr (XLDS) stage_actq<int16_t>(a, C, C * 16, xqs, xd, xs);
+    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
+        float acc[R][NB];
+        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+        for (int c = m.j; c < C; c += G) {
+            u32 w[R][36];
+            UNROLL for (int r = 0; r < R; ++r) {
+                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
+                const uint4 *p = reinterpret_cast<const uint4 *>(a.W + (int64_t)row * a.row_bytes) + c * 9;
+                UNROLL for (int i = 0; i < 9; ++i) unpack4(p[i], &w[r][4 * i]);
+            }
+            u32 sc[R][2], mn[R][2];
+            UNROLL for (int r = 0; r < R; ++r) q4_K_scales(w[r][1], w[r][2], w[r][3], sc[r], mn[r]);
+            UNROLL for (int nb = 0; nb < NB; ++nb) {
+                const int col = nb < a.batch ? nb : a.batch - 1;
+                const float dx = xd[col * C + c];
+                /* sums of the activation over the eight 32-element sub-blocks */
+                const uint4 *bp = reinterpret_cast<const uint4 *>(xs + ((int64_t)col * C + c) * 16);
+                u32 bs[8];
+                unpack4(bp[0], &bs[0]);
+                unpack4(bp[1], &bs[4]);
+                int bsum[8];
+                UNROLL for (int i = 0; i < 8; ++i) bsum[i] = (int)(int16_t)(bs[i] & 0xffffu) + ((int)bs[i] >> 16);
+                int isum[R], msum[R];
+                UNROLL for (int r = 0; r < R; ++r) {
+                    isum[r] = 0;
+                    msum[r] = 0;
+                    UNROLL for (int i = 0; i < 8; ++i) msum[r] += byte_of(mn[r], i) * bsum[i];
+                }
+                const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)c * 256);
+                UNROLL for (int ch = 0; ch < 4; ++ch) {         /* 64 weights: low nibbles then high nibbles */
+                    u32 xl[8], xh[8];
+                    unpack4(xp[4 * ch + 0], &xl[0]);
+                    unpack4(xp[4 * ch + 1], &xl[4]);
+                    unpack4(xp[4 * ch + 2], &xh[0]);
+                    unpack4(xp[4 * ch + 3], &xh[4]);
+                    UNROLL for (int r = 0; r < R; ++r) {
+                        int sl = 0, sh = 0;
+                        UNROLL for (int i = 0; i < 8; ++i) {
+                            const u32 q = w[r][4 + 8 * ch + i];
+                            sl = dot4(q & 0x0f0f0f0fu, xl[i], sl);
+                            sh = dot4((q >> 4) & 0x0f0f0f0fu, xh[i], sh);
+                        }
+                        isum[r] += byte_of(sc[r], 2 * ch) * sl + byte_of(sc[r], 2 * ch + 1) * sh;
+                    }
+                }
+                UNROLL for (int r = 0; r < R; ++r) {
+                    const float d = h2f_lo(w[r][0]) * dx, dm = h2f_hi(w[r][0]) * dx;
+                    acc[r][nb] += d * (float)isum[r] - dm * (float)msum[r];
+                }
+            }
+        }
+        store_rows<G, R, NB>(m, acc, a, row0);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Q6_K x Q8_K-activations.  Chunk = one 210-byte super-block at a 2-byte-aligned address:
+ * ql[128] | qh[64] | int8 scales[16] | fp16 d.  13 dwordx4 loads cover bytes 0..207.
+ * sum (q-32)*x = sum q*x - 32*bsum per 16-element group keeps the 6-bit values unsigned.
+ * ------------------------------------------------------------------------------------------ */
+
+struct __attribute__((packed, aligned(2))) u4_a2 { u32 x, y, z, w; };
+
+template <int G, int R, int NB, bool XLDS>
+PSN_DEV void mv_q6_K_q8(const psn_matvec_args &a) {
+    const RowMap<G, R> m;
+    const int K = a.K, C = K >> 8;
+    const int8_t *xqs = a.xqs;
+    const float *xd = a.xd;
+    const int16_t *xs = reinterpret_cast<const int16_t *>(a.xs);
+    if constexpr (XLDS) stage_actq<int16_t>(a, C, C * 16, xqs, xd, xs);
+    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
+        float acc[R][NB];
+        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+        for (int c = m.j; c < C; c += G) {
+            u32 w[R][52];
+            float dw[R];
+            UNROLL for (int r = 0; r < R; ++r) {
+                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
+                const uint8_t *base = a.W + (int64_t)row * a.row_bytes + (int64_t)c * 210;
+                const u4_a2 *p = reinterpret_cast<const u4_a2 *>(base);
+                UNROLL for (int i = 0; i < 13; ++i) {
+                    const u4_a2 v = p[i];
+                    w[r][4 * i] = v.x; w[r][4 * i + 1] = v.y; w[r][4 * i + 2] = v.z; w[r][4 * i + 3] = v.w;
+                }
+                dw[r] = h2f_lo(*reinterpret_cast<const unsigned short *>(base + 208));
+            }
+            UNROLL for (int nb = 0; nb < NB; ++nb) {
+                const int col = nb < a.batch ? nb : a.batch - 1;
+                const float dx = xd[col * C + c];
+                const uint4 *bp = reinterpret_cast<const uint4 *>(xs + ((int64_t)col * C + c) * 16);
+                u32 bs[8];
+                unpack4(bp[0], &bs[0]);
+                unpack4(bp[1], &bs[4]);
+                const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)c * 256);
+                int isum[R];
+                UNROLL for (int r = 0; r < R; ++r) isum[r] = 0;
+                UNROLL for (int h = 0; h < 2; ++h) {
+                    u32 xq[32];                                   /* 128 activations of this half */
+                    UNROLL for (int i = 0; i < 8; ++i) unpack4(xp[8 * h + i], &xq[4 * i]);
+                    UNROLL for (int r = 0; r < R; ++r) {
+                        int part[8];
+                        UNROLL for (int g = 0; g < 8; ++g) part[g] = 0;
+                        UNROLL for (int i = 0; i < 8; ++i) {      /* dword i holds l = 4i..4i+3 */
+                            const u32 A = w[r][16 * h + i], B = w[r][16 * h + 8 + i], H = w[r][32 + 8 * h + i];
+                            const u32 q1 = (A & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
+                            const u32 q2 = (B & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
+                            const u32 q3 = ((A >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u);
+                            const u32 q4 = ((B >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u);
+                            const int is = i >> 2;
+                            part[is + 0] = dot4(q1, xq[i], part[is + 0]);
+                            part[is + 2] = dot4(q2, xq[8 + i], part[is + 2]);
+                            part[is + 4] = dot4(q3, xq[16 + i], part[is + 4]);
+                            part[is + 6] = dot4(q4, xq[24 + i], part[is + 6]);
+                        }
+                        UNROLL for (int g = 0; g < 8; ++g) {
+                            const int gi = 8 * h + g;             /* 16-element group of the super-block */
+                            const u32 sw = w[r][48 + (gi >> 2)];
+                            const int scale = (int)(int8_t)((sw >> (8 * (gi & 3))) & 0xffu);
+                            const u32 bw = bs[gi >> 1];
+                            const int bsum = (gi & 1) ? ((int)bw >> 16) : (int)(int16_t)(bw & 0xffffu);
+                            isum[r] += scale * (part[g] - 32 * bsum);
+                        }
+                    }
+                }
+                UNROLL for (int r = 0; r < R; ++r) acc[r][nb] += dw[r] * dx * (float)isum[r];
+            }
+        }
+        store_rows<G, R, NB>(m, acc, a, row0);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations.
+ * One generic driver; the format supplies "dequantize 32 consecutive weights of my chunk".
+ * ------------------------------------------------------------------------------------------ */
+
+struct FmtQ4_0 {
+    static constexpr int DW = 36, BYTES = 144;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    /* 32 weights of sub-block SB (one GGUF block) in element order */
+    template <int SB>
+    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
+        float d;
+        u32 lo[4], hi[4];
+        q4_0_block<SB>(w, d, lo, hi);
+        const float off = -8.f * d;
+        UNROLL for (int i = 0; i < 4; ++i) UNROLL for (int b = 0; b < 4; ++b) {
+            o[4 * i + b] = __builtin_fmaf((float)((lo[i] >> (8 * b)) & 0xffu), d, off);
+            o[16 + 4 * i + b] = __builtin_fmaf((float)((hi[i] >> (8 * b)) & 0xffu), d, off);
+        }
+    }
+};
+
+struct FmtQ8_0 {
+    static constexpr int DW = 68, BYTES = 272;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 17; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    template <int SB>
+    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
+        float d;
+        u32 q[8];
+        q8_0_block<SB>(w, d, q);
+        UNROLL for (int i = 0; i < 8; ++i) UNROLL for (int b = 0; b < 4; ++b)
+            o[4 * i + b] = (float)(int)(int8_t)((q[i] >> (8 * b)) & 0xffu) * d;
+    }
+};
+
+struct FmtQ4_K {
+    static constexpr int DW = 36, BYTES = 144;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    template <int SB>
+    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
+        u32 sc[2], mn[2];
+        q4_K_scales(w[1], w[2], w[3], sc, mn);
+        const float d = h2f_lo(w[0]) * (float)byte_of(sc, SB);
+        const float mv = h2f_hi(w[0]) * (float)byte_of(mn, SB);
+        constexpr int ch = SB >> 1, sh = (SB & 1) * 4;
+        UNROLL for (int i = 0; i < 8; ++i) UNROLL for (int b = 0; b < 4; ++b)
+            o[4 * i + b] = d * (float)((w[4 + 8 * ch + i] >> (8 * b + sh)) & 0xfu) - mv;
+    }
+};
+
+struct FmtQ6_K {
+    static constexpr int DW = 53, BYTES = 210;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const u4_a2 *q = reinterpret_cast<const u4_a2 *>(p);
+        UNROLL for (int i = 0; i < 13; ++i) {
+            const u4_a2 v = q[i];
+            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+        }
+        w[52] = *reinterpret_cast<const unsigned short *>(p + 208);
+    }
+    template <int SB>
+    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
+        constexpr int h = SB >> 2, quarter = SB & 3;              /* elements 128h + 32*quarter + l */
+        const float d = h2f_lo(w[52]);
+        UNROLL for (int i = 0; i < 8; ++i) {
+            const u32 L = w[16 * h + 8 * (quarter & 1) + i], H = w[32 + 8 * h + i];
+            const u32 nib = (quarter < 2 ? L : (L >> 4)) & 0x0f0f0f0fu;
+            const u32 top = ((H >> (2 * quarter)) & 0x03030303u) << 4;
+            const u32 q = nib | top;
+            const int gi = 8 * h + 2 * quarter + (i >> 2);
+            const float ds = d * (float)(int)(int8_t)((w[48 + (gi >> 2)] >> (8 * (gi & 3))) & 0xffu);
+            UNROLL for (int b = 0; b < 4; ++b) o[4 * i + b] = ds * (float)((int)((q >> (8 * b)) & 0xffu) - 32);
+        }
+    }
+};
+
+template <typename F, int SB, int R, int NB>
+PSN_DEV void f32_step(const u32 (&w)[R][F::DW], const float *xf, int K, int k0, int batch, float (&acc)[R][NB]) {
+    float o[R][32];
+    UNROLL for (int r = 0; r < R; ++r) F::template deq32<SB>(w[r], o[r]);
+    UNROLL for (int nb = 0; nb < NB; ++nb) {
+        const int col = nb < batch ? nb : batch - 1;
+        const float4 *xp = reinterpret_cast<const float4 *>(xf + (int64_t)col * K + k0 + SB * 32);
+        UNROLL for (int i = 0; i < 8; ++i) {
+            const float4 x = xp[i];
+            UNROLL for (int r = 0; r < R; ++r) {
+                acc[r][nb] = __builtin_fmaf(o[r][4 * i + 0], x.x, acc[r][nb]);
+                acc[r][nb] = __builtin_fmaf(o[r][4 * i + 1], x.y, acc[r][nb]);
+                acc[r][nb] = __builtin_fmaf(o[r][4 * i + 2], x.z, acc[r][nb]);
+                acc[r][nb] = __builtin_fmaf(o[r][4 * i + 3], x.w, acc[r][nb]);
+            }
+        }
+    }
+}
+
+template <typename F, int G, int R, int NB>
+PSN_DEV void mv_f32(const psn_matvec_args &a) {
+    const RowMap<G, R> m;
+    const int K = a.K, C = K >> 8;
+    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
+        float acc[R][NB];
+        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+        for (int c = m.j; c < C; c += G) {
+            u32 w[R][F::DW];
+            UNROLL for (int r = 0; r < R; ++r) {
+                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
+                F::load(a.W + (int64_t)row * a.row_bytes + (int64_t)c * F::BYTES, w[r]);
+            }
+            const int k0 = c * 256;
+            f32_step<F, 0>(w, a.xf, K, k0, a.batch, acc);
+            f32_step<F, 1>(w, a.xf, K, k0, a.batch, acc);
+            f32_step<F, 2>(w, a.xf, K, k0, a.batch, acc);
+            f32_step<F, 3>(w, a.xf, K, k0, a.batch, acc);
+            f32_step<F, 4>(w, a.xf, K, k0, a.batch, acc);
+            f32_step<F, 5>(w, a.xf, K, k0, a.batch, acc);
+            f32_step<F, 6>(w, a.xf, K, k0, a.batch, acc);
+            f32_step<F, 7>(w, a.xf, K, k0, a.batch, acc);
+        }
+        store_rows<G, R, NB>(m, acc, a, row0);
+    }
+}
+
+/* ------------------------------------------------------------------------------------------
+ * Entry points.  Name = psn_mv_<fmt>_<scheme>_g<G>_r<R>_b<NB>[_lds]; the host picks one per shape.
+ * ------------------------------------------------------------------------------------------ */
+
+#define PSN_Q8_KERNEL(fmt, G, R, NB)                                                                      \
+    extern "C" __global__ void __launch_bounds__(256) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
+        mv_##fmt##_q8<G, R, NB, false>(a);                                                                \
+    }                                                                                                     \
+    extern "C" __global__ void __launch_bounds__(256) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
+        mv_##fmt##_q8<G, R, NB, true>(a);                                                                 \
+    }
+
+#define PSN_F32_KERNEL(fmt, F, G, R, NB)                                                                  \
+    extern "C" __global__ void __launch_bounds__(256) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
+        mv_f32<F, G, R, NB>(a);                                                                           \
+    }
+
+#define PSN_FOR_G(M, ...) M(__VA_ARGS__, 8) M(__VA_ARGS__, 16) M(__VA_ARGS__, 32) M(__VA_ARGS__, 64)
+
+#define PSN_Q8_ALL_G(fmt, R, NB) \
+    PSN_Q8_KERNEL(fmt, 8, R, NB) PSN_Q8_KERNEL(fmt, 16, R, NB) PSN_Q8_KERNEL(fmt, 32, R, NB) PSN_Q8_KERNEL(fmt, 64, R, NB)
+#define PSN_Q8_ALL(fmt)                                                                    \
+    PSN_Q8_ALL_G(fmt, 1, 1) PSN_Q8_ALL_G(fmt, 2, 1) PSN_Q8_ALL_G(fmt, 4, 1)                \
+    PSN_Q8_ALL_G(fmt, 1, 2) PSN_Q8_ALL_G(fmt, 2, 2)                                        \
+    PSN_Q8_ALL_G(fmt, 1, 4) PSN_Q8_ALL_G(fmt, 2, 4)                                        \
+    PSN_Q8_ALL_G(fmt, 1, 8)
+
+#define PSN_F32_ALL_G(fmt, F, R, NB) \
+    PSN_F32_KERNEL(fmt, F, 8, R, NB) PSN_F32_KERNEL(fmt, F, 16, R, NB) PSN_F32_KERNEL(fmt, F, 32, R, NB) PSN_F32_KERNEL(fmt, F, 64, R, NB)
+#define PSN_F32_ALL(fmt, F)                                                               \
+    PSN_F32_ALL_G(fmt, F, 1, 1) PSN_F32_ALL_G(fmt, F, 2, 1)                                \
+    PSN_F32_ALL_G(fmt, F, 1, 2) PSN_F32_ALL_G(fmt, F, 1, 4) PSN_F32_ALL_G(fmt, F, 1, 8)
+
+/* The build compiles this file once per format (-DPSN_BUILD_ONLY -DPSN_BUILD_<FMT>) so the four
+ * code objects build in parallel; without PSN_BUILD_ONLY everything lands in one. */
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q4_0)
+PSN_Q8_ALL(q4_0)
+PSN_F32_ALL(q4_0, FmtQ4_0)
+#endif
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q8_0)
+PSN_Q8_ALL(q8_0)
+PSN_F32_ALL(q8_0, FmtQ8_0)
+#endif
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q4_K)
+PSN_Q8_ALL(q4_K)
+PSN_F32_ALL(q4_K, FmtQ4_K)
+#endif
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q6_K)
+PSN_Q8_ALL(q6_K)
+PSN_F32_ALL(q6_K, FmtQ6_K)
+#endif

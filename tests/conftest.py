@@ -18,3 +18,12 @@ def orc():
     import oracle
     oracle.lib()
     return oracle
+
+
+@pytest.fixture(scope="session")
+def hip():
+    """The HIP backend through the C ABI.  GPU tests fail (not skip) if it cannot be created."""
+    from openagents_amd.backend import HipBackend
+    be = HipBackend(0)
+    yield be
+    be.close()

@@ -1,0 +1,259 @@
+"""GPU parity: activation quantizers (bit-exact) and the decode matvec (both activation schemes,
+all four weight formats, batch 1..8, every kernel variant) against the CPU oracle, through the C ABI.
+
+Gate (north_star): max_i |y_i - ref_i| / max_j |ref_j| <= 1e-3 on identical seeded inputs with the
+same activation scheme on both sides.  The tests assert the much tighter PARITY_TOL below, which is
+what fp32 accumulation-order differences allow; integer work (quantizers) is bit-exact.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import ggufref as G
+from openagents_amd import _ffi, backend
+
+pytestmark = pytest.mark.gpu
+
+GATE = 1e-3          # the stated bar
+PARITY_TOL = 2e-5    # what is asserted
+FORMATS = ["Q4_0", "Q8_0", "Q4_K", "Q6_K"]
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+_weights_cache = {}
+
+
+def weights(orc, qname, seed, n, k):
+    key = (qname, seed, n, k)
+    if key not in _weights_cache:
+        _weights_cache[key] = orc.quantize(getattr(orc, qname), G.seeded_weights(seed, n, k))
+    return _weights_cache[key]
+
+
+# ------------------------------------------------------------------ activation quantizers
+
+@pytest.mark.parametrize("k,batch", [(256, 1), (4096, 1), (14336, 3), (4096, 8)])
+def test_quantize_q8_0_bit_exact(hip, orc, k, batch):
+    say(f"quantize_q8_0 k={k} batch={batch}")
+    x = G.seeded_acts(100 + k + batch, batch, k)
+    x[0, :32] = 0                                   # an all-zero block
+    x[0, 32:64] = np.float32(0.5) * np.arange(-16, 16)   # exact ties
+    xq = hip.quantize_activations(hip.upload(x), k, batch, _ffi.Q8_0)
+    li = backend.actq_layout(_ffi.Q8_0, k, batch)
+    qs = xq.download(np.int8, (batch, k), li.off_qs)
+    d = xq.download(np.float32, (batch, k // 32), li.off_d)
+    s = xq.download(np.int32, (batch, k // 32), li.off_s)
+    for b in range(batch):
+        ref = orc.quantize(orc.Q8_0, x[b]).reshape(k // 32, 34)
+        ref_d = ref[:, :2].copy().view(np.float16).astype(np.float32).reshape(-1)
+        ref_q = ref[:, 2:].copy().view(np.int8).reshape(-1)
+        assert np.array_equal(qs[b], ref_q)
+        assert np.array_equal(d[b].view(np.uint32), ref_d.view(np.uint32))
+        assert np.array_equal(s[b], ref_q.reshape(-1, 32).astype(np.int32).sum(axis=1))
+
+
+@pytest.mark.parametrize("k,batch", [(256, 1), (4096, 1), (14336, 3), (4096, 8)])
+def test_quantize_q8_K_bit_exact(hip, orc, k, batch):
+    say(f"quantize_q8_K k={k} batch={batch}")
+    x = G.seeded_acts(200 + k + batch, batch, k)
+    if k >= 1024:
+        x[0, 256:512] = 0                           # an all-zero super-block
+        x[0, 512] = 3.0
+        x[0, 700] = -3.0                            # equal magnitudes, opposite sign: the first one wins
+        x[0, 513:700] *= 0.1
+        x[0, 701:768] *= 0.1
+    xq = hip.quantize_activations(hip.upload(x), k, batch, _ffi.Q8_K)
+    li = backend.actq_layout(_ffi.Q8_K, k, batch)
+    qs = xq.download(np.int8, (batch, k), li.off_qs)
+    d = xq.download(np.float32, (batch, k // 256), li.off_d)
+    bs = xq.download(np.int16, (batch, k // 16), li.off_s)
+    for b in range(batch):
+        rd, rq, rbs = G.parse_q8_K(orc.quantize(orc.Q8_K, x[b]), k)
+        assert np.array_equal(qs[b], rq.reshape(-1).astype(np.int8))
+        assert np.array_equal(d[b].astype(np.float64), rd)
+        assert np.array_equal(bs[b], rbs.reshape(-1).astype(np.int16))
+
+
+# ------------------------------------------------------------------ matvec: every kernel variant
+
+def all_plans(scheme, batch):
+    nb = 1 if batch <= 1 else 2 if batch <= 2 else 4 if batch <= 4 else 8
+    if scheme == _ffi.ACT_Q8:
+        rs = {1: (1, 2, 4), 2: (1, 2), 4: (1, 2), 8: (1,)}[nb]
+    else:
+        rs = (1, 2) if nb == 1 else (1,)
+    for g in (8, 16, 32, 64):
+        for r in rs:
+            for lds in ((0, 1) if scheme == _ffi.ACT_Q8 else (0,)):
+                p = _ffi.MatvecPlan()
+                p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks = g, r, nb, lds, 3
+                yield p
+
+
+@pytest.mark.parametrize("qname", FORMATS)
+@pytest.mark.parametrize("scheme", [_ffi.ACT_Q8, _ffi.ACT_F32])
+@pytest.mark.parametrize("batch", [1, 2, 3, 8])
+def test_every_kernel_variant_small(hip, orc, qname, scheme, batch):
+    """n=77 is ragged against every rows-per-pass; k=2560 gives 10 chunks, so 8-lane groups loop
+    twice and 16/32/64-lane groups have idle lanes; 3 workgroups force the grid-stride loop."""
+    t = getattr(orc, qname)
+    n, k = 77, 2560
+    W = weights(orc, qname, 300, n, k)
+    x = G.seeded_acts(301 + batch, batch, k)
+    ref = orc.matvec(t, scheme, W, x, n, k)
+    w = hip.upload_weight(t, W, n, k)
+    xb = hip.upload(x)
+    xin = hip.quantize_activations(xb, k, batch, backend.act_type_for(t)) if scheme == _ffi.ACT_Q8 else xb
+    for p in all_plans(scheme, batch):
+        say(f"variant {qname} scheme={scheme} batch={batch} {p.as_dict()}")
+        yb = hip.upload(np.full((batch, n), np.nan, np.float32))
+        hip.quantized_matvec_planned(w, xin, yb, batch, scheme, p)
+        y = yb.download(np.float32, (batch, n))
+        err = G.max_rel_err(y, ref)
+        assert np.all(np.isfinite(y)) and err < PARITY_TOL, (p.as_dict(), err)
+
+
+# ------------------------------------------------------------------ matvec: BASELINE shapes, default plan
+
+SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
+
+
+@pytest.mark.parametrize("n,k", SHAPES)
+@pytest.mark.parametrize("scheme", [_ffi.ACT_Q8, _ffi.ACT_F32])
+def test_q4_0_llama3_8b_projection_shapes(hip, orc, n, k, scheme):
+    say(f"Q4_0 full shape n={n} k={k} scheme={scheme}")
+    W = weights(orc, "Q4_0", 400, n, k)
+    x = G.seeded_acts(401, 1, k)[0]
+    y = hip.matvec_host(orc.Q4_0, W, x, n, k, scheme)
+    err = G.max_rel_err(y, orc.matvec(orc.Q4_0, scheme, W, x, n, k))
+    say(f"  max_rel_err={err:.3e}")
+    assert err < PARITY_TOL < GATE
+
+
+def test_q8_0_4096x4096_reference_config(hip, orc):
+    say("Q8_0 4096x4096")
+    n = k = 4096
+    W = weights(orc, "Q8_0", 410, n, k)
+    x = G.seeded_acts(411, 1, k)[0]
+    for scheme in (_ffi.ACT_Q8, _ffi.ACT_F32):
+        err = G.max_rel_err(hip.matvec_host(orc.Q8_0, W, x, n, k, scheme), orc.matvec(orc.Q8_0, scheme, W, x, n, k))
+        say(f"  scheme={scheme} max_rel_err={err:.3e}")
+        assert err < PARITY_TOL
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("batch", [1, 2, 4, 8])
+def test_q4_K_small_batch_shapes(hip, orc, n, k, batch):
+    say(f"Q4_K n={n} k={k} batch={batch}")
+    W = weights(orc, "Q4_K", 420, n, k)
+    x = G.seeded_acts(421, batch, k)
+    for scheme in (_ffi.ACT_Q8, _ffi.ACT_F32):
+        err = G.max_rel_err(hip.matvec_host(orc.Q4_K, W, x, n, k, scheme), orc.matvec(orc.Q4_K, scheme, W, x, n, k))
+        say(f"  scheme={scheme} max_rel_err={err:.3e}")
+        assert err < PARITY_TOL
+
+
+def test_q6_K_lm_head_slice(hip, orc):
+    """The 128256 x 4096 LM head is checked on a 16032-row slice against the oracle (the quantizer is
+    the slow part on the CPU) and at full height through linearity in test_q6_K_lm_head_full_height."""
+    n, k = 16032, 4096
+    say(f"Q6_K n={n} k={k}")
+    W = weights(orc, "Q6_K", 430, n, k)
+    x = G.seeded_acts(431, 1, k)[0]
+    for scheme in (_ffi.ACT_Q8, _ffi.ACT_F32):
+        err = G.max_rel_err(hip.matvec_host(orc.Q6_K, W, x, n, k, scheme), orc.matvec(orc.Q6_K, scheme, W, x, n, k))
+        say(f"  scheme={scheme} max_rel_err={err:.3e}")
+        assert err < PARITY_TOL
+
+
+def test_q6_K_lm_head_full_height(hip, orc):
+    """Full 128256 rows: the slice's blocks tiled 8 times, so row r must equal row r mod 16032 of the
+    oracle result -- a size-independent check of the row indexing at the real height."""
+    n0, k, reps = 16032, 4096, 8
+    n = n0 * reps
+    say(f"Q6_K full height n={n} k={k}")
+    W0 = weights(orc, "Q6_K", 430, n0, k)
+    x = G.seeded_acts(432, 1, k)[0]
+    ref = orc.matvec(orc.Q6_K, orc.ACT_Q8, W0, x, n0, k)
+    y = hip.matvec_host(orc.Q6_K, np.tile(W0, (reps, 1)), x, n, k, _ffi.ACT_Q8)
+    assert G.max_rel_err(y, np.tile(ref, reps)) < PARITY_TOL
+
+
+# ------------------------------------------------------------------ edge cases and properties
+
+@pytest.mark.parametrize("qname", FORMATS)
+def test_single_row_and_single_chunk(hip, orc, qname):
+    t = getattr(orc, qname)
+    for n, k in ((1, 256), (1, 4096), (5, 256), (63, 512), (65, 768)):
+        say(f"edge {qname} n={n} k={k}")
+        W = weights(orc, qname, 500, n, k)
+        x = G.seeded_acts(501, 2, k)
+        for scheme in (_ffi.ACT_Q8, _ffi.ACT_F32):
+            err = G.max_rel_err(hip.matvec_host(t, W, x, n, k, scheme), orc.matvec(t, scheme, W, x, n, k))
+            assert err < PARITY_TOL, (n, k, scheme, err)
+
+
+@pytest.mark.parametrize("qname", FORMATS)
+def test_one_hot_activation_returns_dequantized_column(hip, orc, qname):
+    t = getattr(orc, qname)
+    n, k = 96, 1024
+    W = weights(orc, qname, 510, n, k)
+    deq = orc.dequantize(t, W, k)
+    for col in (0, 17, 255, 256, 1023):
+        x = np.zeros(k, np.float32)
+        x[col] = 1.0
+        y = hip.matvec_host(t, W, x, n, k, _ffi.ACT_F32)
+        assert np.array_equal(y, deq[:, col]), (qname, col)
+
+
+def test_zero_activations_and_zero_weights(hip, orc):
+    n, k = 64, 1024
+    for qname in FORMATS:
+        t = getattr(orc, qname)
+        W = weights(orc, qname, 520, n, k)
+        for scheme in (_ffi.ACT_Q8, _ffi.ACT_F32):
+            assert not hip.matvec_host(t, W, np.zeros(k, np.float32), n, k, scheme).any()
+            Z = orc.quantize(t, np.zeros((n, k), np.float32))
+            assert not hip.matvec_host(t, Z, G.seeded_acts(521, 1, k)[0], n, k, scheme).any()
+
+
+def test_batch_columns_are_independent(hip, orc):
+    """Column b of a batch-8 call equals the batch-1 call on x[b] bit-for-bit (same kernel math)."""
+    t, n, k = orc.Q4_K, 200, 4096
+    W = weights(orc, "Q4_K", 530, n, k)
+    x = G.seeded_acts(531, 8, k)
+    y8 = hip.matvec_host(t, W, x, n, k, _ffi.ACT_Q8)
+    ref = orc.matvec(t, orc.ACT_Q8, W, x, n, k)
+    assert G.max_rel_err(y8, ref) < PARITY_TOL
+    for b in (0, 3, 7):
+        assert G.max_rel_err(hip.matvec_host(t, W, x[b], n, k, _ffi.ACT_Q8), ref[b]) < PARITY_TOL
+
+
+def test_shape_and_buffer_errors_surface_as_codes(hip, orc):
+    n, k = 16, 512
+    W = weights(orc, "Q4_0", 540, n, k)
+    w = hip.upload_weight(orc.Q4_0, W, n, k)
+    x = hip.upload(np.zeros(k, np.float32))
+    y = hip.alloc(n * 4)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec(w, x, y, batch=9)
+    assert e.value.code == _ffi.E_SHAPE
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec(w, x, y, batch=2)          # x and y too small for two columns
+    assert e.value.code == _ffi.E_INVALID_ARG
+    small = hip.alloc(8)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec(w, x, small, batch=1)
+    assert e.value.code == _ffi.E_INVALID_ARG
+    bad = backend.QuantizedTensor(w.buf, orc.Q4_0, n, 512 + 32)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec(bad, x, y)
+    assert e.value.code == _ffi.E_SHAPE
+    assert hip.lib.psn_module_has_kernel(hip.module, b"no_such_kernel") == _ffi.E_MODULE
+    hip.quantized_matvec(w, x, y)                        # the handles still work afterwards
+    hip.sync()

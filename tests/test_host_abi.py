@@ -1,0 +1,112 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol the header
+declares, and rejects bad shapes/handles before touching a device."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from openagents_amd import _ffi, backend
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _ffi.load()
+
+
+def header_functions():
+    text = open(os.path.join(ROOT, "include", "psn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(psn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = header_functions()
+    assert len(names) >= 30
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/psn.h but not exported"
+        assert n in _ffi.SIGNATURES, f"{n} has no ctypes signature"
+    assert sorted(_ffi.SIGNATURES) == names
+    assert lib.psn_abi_version() == 1
+
+
+def test_block_geometry(lib):
+    assert [lib.psn_block_bytes(t) for t in (_ffi.Q8_0, _ffi.Q4_0, _ffi.Q4_K, _ffi.Q6_K, _ffi.Q8_K)] == [34, 18, 144, 210, 292]
+    assert [lib.psn_block_elems(t) for t in (_ffi.Q8_0, _ffi.Q4_0, _ffi.Q4_K, _ffi.Q6_K)] == [32, 32, 256, 256]
+    assert backend.row_bytes(_ffi.Q4_0, 4096) == 2304
+    assert backend.row_bytes(_ffi.Q4_K, 14336) == 8064
+    assert backend.row_bytes(_ffi.Q6_K, 4096) == 3360
+    with pytest.raises(backend.PsnError) as e:
+        backend.row_bytes(_ffi.Q4_K, 4096 + 32)
+    assert e.value.code == _ffi.E_SHAPE and "multiple" in str(e.value)
+    with pytest.raises(backend.PsnError) as e:
+        backend.row_bytes(99, 4096)
+    assert e.value.code == _ffi.E_UNSUPPORTED
+
+
+def test_activation_layout(lib):
+    li = backend.actq_layout(_ffi.Q8_0, 4096, 1)
+    assert (li.off_qs, li.off_d, li.off_s) == (0, 4096, 4096 + 512) and li.bytes == 4096 + 512 + 512
+    li = backend.actq_layout(_ffi.Q8_K, 14336, 8)
+    assert li.off_d == 8 * 14336 and li.off_d % 256 == 0 and li.off_s % 256 == 0
+    assert li.bytes >= li.off_s + 8 * (14336 // 16) * 2
+    assert backend.act_type_for(_ffi.Q4_0) == _ffi.Q8_0 and backend.act_type_for(_ffi.Q6_K) == _ffi.Q8_K
+    for bad in (0, 9):
+        with pytest.raises(backend.PsnError) as e:
+            backend.actq_layout(_ffi.Q8_0, 4096, bad)
+        assert e.value.code == _ffi.E_SHAPE
+    with pytest.raises(backend.PsnError) as e:
+        backend.actq_layout(_ffi.Q4_0, 4096, 1)
+    assert e.value.code == _ffi.E_UNSUPPORTED
+
+
+def test_matvec_plan_is_host_arithmetic(lib):
+    for qt in (_ffi.Q4_0, _ffi.Q8_0, _ffi.Q4_K, _ffi.Q6_K):
+        for (n, k) in ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096), (1, 256)):
+            for batch in range(1, 9):
+                for scheme in (_ffi.ACT_F32, _ffi.ACT_Q8):
+                    p = backend.matvec_plan(qt, scheme, n, k, batch)
+                    assert p.lanes_per_row in (8, 16, 32, 64) and p.rows_in_flight in (1, 2, 4)
+                    assert p.batch_tile >= batch and p.batch_tile in (1, 2, 4, 8)
+                    assert 1 <= p.blocks <= 256 * 16
+    for args, code in (((_ffi.Q4_0, 1, 0, 4096, 1), _ffi.E_SHAPE), ((_ffi.Q4_0, 1, 16, 4096 + 32, 1), _ffi.E_SHAPE),
+                       ((_ffi.Q4_0, 1, 16, 4096, 9), _ffi.E_SHAPE), ((_ffi.Q8_K, 1, 16, 4096, 1), _ffi.E_UNSUPPORTED),
+                       ((_ffi.Q4_0, 5, 16, 4096, 1), _ffi.E_UNSUPPORTED)):
+        with pytest.raises(backend.PsnError) as e:
+            backend.matvec_plan(*args)
+        assert e.value.code == code, args
+
+
+def test_null_handles_are_rejected_without_a_device(lib):
+    assert lib.psn_stream_sync(None) == _ffi.E_INVALID_ARG
+    assert lib.psn_buf_free(None) == _ffi.E_INVALID_ARG
+    assert lib.psn_module_unload(None) == _ffi.E_INVALID_ARG
+    assert lib.psn_ctx_destroy(None) == _ffi.E_INVALID_ARG
+    assert lib.psn_qmatvec(None, None, _ffi.Q4_0, 0, 1, None, None, None, 16, 4096, 1) == _ffi.E_INVALID_ARG
+    assert b"null" in lib.psn_last_error()
+    assert lib.psn_qmatvec(None, None, _ffi.Q4_0, 7, 1, None, None, None, 16, 4096, 1) == _ffi.E_UNSUPPORTED
+    h = C.c_void_p()
+    assert lib.psn_buf_alloc(None, 16, C.byref(h)) == _ffi.E_INVALID_ARG and not h.value
+    assert lib.psn_module_load(None, None, 0, C.byref(h)) == _ffi.E_INVALID_ARG
+    assert lib.psn_error_name(-4) == b"PSN_E_NO_DEVICE"
+
+
+def test_context_creation_fails_loudly_without_gfx950(lib):
+    h = C.c_void_p()
+    rc = lib.psn_ctx_create(0, C.byref(h))
+    if rc == 0:                      # running on a GPU box: nothing to assert about absence
+        assert lib.psn_ctx_destroy(h) == 0
+        return
+    assert rc == _ffi.E_NO_DEVICE and not h.value
+    assert lib.psn_last_error()
+    with pytest.raises(backend.PsnError):
+        backend.HipBackend(0)
+
+
+def test_missing_library_is_an_error_not_a_fallback(monkeypatch):
+    monkeypatch.setattr(_ffi, "_lib", None)
+    monkeypatch.setattr(_ffi, "LIB_PATH", "/nonexistent/libpsn_hip.so")
+    with pytest.raises(_ffi.LibraryMissing):
+        _ffi.load()
