@@ -42,6 +42,7 @@ typedef struct psn_stream psn_stream;
 typedef struct psn_buf psn_buf;
 typedef struct psn_module psn_module;
 typedef struct psn_event psn_event;
+typedef struct psn_graph psn_graph;
 
 /* GGUF tensor type ids */
 typedef enum { PSN_Q4_0 = 2, PSN_Q8_0 = 8, PSN_Q4_K = 12, PSN_Q6_K = 14, PSN_Q8_K = 15 } psn_qtype;
@@ -92,6 +93,18 @@ int32_t psn_module_has_kernel(psn_module *mod, const char *kernel_name);
 int32_t psn_stream_create(psn_ctx *ctx, psn_stream **out);
 int32_t psn_stream_sync(psn_stream *s);
 int32_t psn_stream_destroy(psn_stream *s);
+
+/* Stream capture into a replayable graph (hipGraph): everything launched on `s` between begin and
+ * end is recorded instead of run; psn_graph_launch replays it on a stream.  Calls that would have
+ * to allocate or synchronize (a workspace that must grow, uploads, downloads) fail while capturing.
+ * Replaces the CUDA backend's CUDA-graph decode loop. */
+int32_t psn_graph_begin_capture(psn_stream *s);
+int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out);
+int32_t psn_graph_launch(psn_graph *g, psn_stream *s);
+int32_t psn_graph_destroy(psn_graph *g);
+/* Sizes the stream's activation workspace for psn_qmatvec / psn_qmatvec_multi with scheme Q8 up to
+ * [batch][K], so later calls (and captures) never allocate. */
+int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch);
 
 int32_t psn_event_create(psn_ctx *ctx, psn_event **out);
 int32_t psn_event_destroy(psn_event *e);
@@ -145,6 +158,16 @@ int32_t psn_qmatvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layou
 int32_t psn_qmatvec_q8(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
                        const psn_buf *x_q, psn_buf *y_f32, int64_t N, int64_t K, int32_t batch);
 
+/* Several matrices that share K, the format and the activations in ONE launch (q/k/v, gate/up):
+ * y[i] = W[i] x for i < count (1..4), each y[i] fp32 [batch][N[i]].  psn_qmatvec_multi takes fp32
+ * activations (scheme as above), psn_qmatvec_q8_multi already-quantized ones. */
+int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, int32_t count,
+                          const psn_buf *const *W, const psn_buf *x_f32, psn_buf *const *y_f32, const int64_t *N, int64_t K,
+                          int32_t batch);
+int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t count,
+                             const psn_buf *const *W, const psn_buf *x_q, psn_buf *const *y_f32, const int64_t *N, int64_t K,
+                             int32_t batch);
+
 /* Launch geometry of one matvec.  psn_qmatvec_plan fills in the library's choice for a shape
  * (pure host arithmetic, usable without a device); psn_qmatvec_planned runs with a caller-chosen
  * one (auto-tuners, benchmarks). */
@@ -153,15 +176,16 @@ typedef struct psn_matvec_plan {
     int32_t rows_in_flight; /* 1, 2 or 4 row sets per lane */
     int32_t batch_tile;     /* compiled batch width: 1, 2, 4 or 8 (>= batch) */
     int32_t stage_lds;      /* 1: activations staged in LDS (scheme Q8 only) */
-    int32_t blocks;         /* workgroups of 256 threads */
-    int32_t lds_bytes;      /* dynamic LDS the launch asks for */
+    int32_t blocks;         /* workgroups */
+    int32_t threads;        /* threads per workgroup: 256 or 512 */
 } psn_matvec_plan;
 int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t compute_units,
                          psn_matvec_plan *out);
-/* x is x_q for scheme Q8 (already quantized) and x_f32 for scheme F32 */
-int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const psn_buf *W,
-                            const psn_buf *x, psn_buf *y_f32, int64_t N, int64_t K, int32_t batch,
-                            const psn_matvec_plan *plan);
+/* x is x_q for scheme Q8 (already quantized) and x_f32 for scheme F32; N in the plan call is the
+ * total row count when several matrices share the launch */
+int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, int32_t count,
+                            const psn_buf *const *W, const psn_buf *x, psn_buf *const *y_f32, const int64_t *N, int64_t K,
+                            int32_t batch, const psn_matvec_plan *plan);
 
 /* ---- prefill matmul ----------------------------------------------------------------------- */
 

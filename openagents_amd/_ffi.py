@@ -26,7 +26,7 @@ class ActqInfo(C.Structure):
 
 class MatvecPlan(C.Structure):
     _fields_ = [("lanes_per_row", C.c_int32), ("rows_in_flight", C.c_int32), ("batch_tile", C.c_int32),
-                ("stage_lds", C.c_int32), ("blocks", C.c_int32), ("lds_bytes", C.c_int32)]
+                ("stage_lds", C.c_int32), ("blocks", C.c_int32), ("threads", C.c_int32)]
 
     def as_dict(self):
         return {k: int(getattr(self, k)) for k, _ in self._fields_}
@@ -53,6 +53,11 @@ SIGNATURES = {
     "psn_stream_create": (_i32, [_vp, _pp]),
     "psn_stream_sync": (_i32, [_vp]),
     "psn_stream_destroy": (_i32, [_vp]),
+    "psn_graph_begin_capture": (_i32, [_vp]),
+    "psn_graph_end_capture": (_i32, [_vp, _pp]),
+    "psn_graph_launch": (_i32, [_vp, _vp]),
+    "psn_graph_destroy": (_i32, [_vp]),
+    "psn_stream_reserve": (_i32, [_vp, _i64, _i32]),
     "psn_event_create": (_i32, [_vp, _pp]),
     "psn_event_destroy": (_i32, [_vp]),
     "psn_event_record": (_i32, [_vp, _vp]),
@@ -70,7 +75,9 @@ SIGNATURES = {
     "psn_qmatvec": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
     "psn_qmatvec_q8": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
     "psn_qmatvec_plan": (_i32, [_i32, _i32, _i64, _i64, _i32, _i32, C.POINTER(MatvecPlan)]),
-    "psn_qmatvec_planned": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32, C.POINTER(MatvecPlan)]),
+    "psn_qmatvec_multi": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32]),
+    "psn_qmatvec_q8_multi": (_i32, [_vp, _vp, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32]),
+    "psn_qmatvec_planned": (_i32, [_vp, _vp, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32, C.POINTER(MatvecPlan)]),
     "psn_qmatmul_prefill": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i64]),
 }
 

@@ -196,8 +196,51 @@ class HipBackend:
     def quantized_matvec_q8(self, w: QuantizedTensor, xq: DeviceBuffer, y: DeviceBuffer, batch: int = 1):
         _check(self.lib.psn_qmatvec_q8(self.module, self.stream, w.qtype, LAYOUT_GGUF, w.buf.handle, xq.handle, y.handle, w.n, w.k, batch))
 
-    def quantized_matvec_planned(self, w: QuantizedTensor, x: DeviceBuffer, y: DeviceBuffer, batch: int, scheme: int, plan: MatvecPlan):
-        _check(self.lib.psn_qmatvec_planned(self.module, self.stream, w.qtype, scheme, w.buf.handle, x.handle, y.handle, w.n, w.k, batch, C.byref(plan)))
+    @staticmethod
+    def _pack(ws, ys):
+        """ctypes arrays for a list of weights / outputs that share one launch."""
+        ws = list(ws) if isinstance(ws, (list, tuple)) else [ws]
+        ys = list(ys) if isinstance(ys, (list, tuple)) else [ys]
+        if len(ws) != len(ys) or not ws:
+            raise ValueError("need as many outputs as weights")
+        if any((w.qtype, w.k) != (ws[0].qtype, ws[0].k) for w in ws):
+            raise ValueError("matrices sharing a launch must share format and K")
+        n = len(ws)
+        W = (C.c_void_p * n)(*[w.buf.handle for w in ws])
+        Y = (C.c_void_p * n)(*[y.handle for y in ys])
+        N = (C.c_int64 * n)(*[w.n for w in ws])
+        return ws[0], n, W, Y, N
+
+    def quantized_matvec_multi(self, ws, x: DeviceBuffer, ys, batch: int = 1, scheme: int = ACT_Q8):
+        """Several matrices sharing x (q/k/v, gate/up) in one launch; x is fp32."""
+        w0, n, W, Y, N = self._pack(ws, ys)
+        _check(self.lib.psn_qmatvec_multi(self.module, self.stream, w0.qtype, LAYOUT_GGUF, scheme, n, W, x.handle, Y, N, w0.k, batch))
+
+    def quantized_matvec_q8_multi(self, ws, xq: DeviceBuffer, ys, batch: int = 1):
+        w0, n, W, Y, N = self._pack(ws, ys)
+        _check(self.lib.psn_qmatvec_q8_multi(self.module, self.stream, w0.qtype, LAYOUT_GGUF, n, W, xq.handle, Y, N, w0.k, batch))
+
+    def quantized_matvec_planned(self, ws, x: DeviceBuffer, ys, batch: int, scheme: int, plan: MatvecPlan):
+        w0, n, W, Y, N = self._pack(ws, ys)
+        _check(self.lib.psn_qmatvec_planned(self.module, self.stream, w0.qtype, scheme, n, W, x.handle, Y, N, w0.k, batch, C.byref(plan)))
+
+    # -- graphs -----------------------------------------------------------------------------
+    def reserve(self, k: int, batch: int = 1):
+        _check(self.lib.psn_stream_reserve(self.stream, k, batch))
+
+    def begin_capture(self):
+        _check(self.lib.psn_graph_begin_capture(self.stream))
+
+    def end_capture(self) -> C.c_void_p:
+        g = C.c_void_p()
+        _check(self.lib.psn_graph_end_capture(self.stream, C.byref(g)))
+        return g
+
+    def launch_graph(self, graph):
+        _check(self.lib.psn_graph_launch(graph, self.stream))
+
+    def destroy_graph(self, graph):
+        _check(self.lib.psn_graph_destroy(graph))
 
     def quantized_matmul(self, w: QuantizedTensor, x_f16: DeviceBuffer, y: DeviceBuffer, m: int):
         _check(self.lib.psn_qmatmul_prefill(self.module, self.stream, w.qtype, LAYOUT_GGUF, w.buf.handle, x_f16.handle, y.handle, m, w.n, w.k))

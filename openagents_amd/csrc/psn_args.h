@@ -29,17 +29,22 @@ struct psn_quantize_args {
     int32_t batch;
 };
 
+#define PSN_MAX_SEGMENTS 4
+
+/* One launch walks the rows of up to four matrices that share K, the format and x as a single
+ * concatenated row space: segment s owns rows [row_end[s-1], row_end[s]). */
 struct psn_matvec_args {
-    const uint8_t *W;     /* [N][row_bytes] GGUF blocks */
+    const uint8_t *W[PSN_MAX_SEGMENTS];   /* [N_s][row_bytes] GGUF blocks */
+    float *y[PSN_MAX_SEGMENTS];           /* [batch][N_s] */
+    int32_t row_end[PSN_MAX_SEGMENTS];    /* cumulative row counts */
     const int8_t *xqs;    /* scheme Q8: activation fields (see above) */
     const float *xd;
     const void *xs;
     const float *xf;      /* scheme F32: [batch][K] */
-    float *y;             /* [batch][N] */
-    int32_t N;
+    int32_t N;            /* total rows = row_end[nseg-1] */
     int32_t K;
     int32_t batch;        /* live batch columns (<= the kernel's compiled NB) */
-    int32_t pad;
+    int32_t nseg;
     int64_t row_bytes;
 };
 

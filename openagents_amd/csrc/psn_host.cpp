@@ -149,6 +149,11 @@ struct psn_event {
     psn_ctx *ctx;
     hipEvent_t e;
 };
+struct psn_graph {
+    psn_ctx *ctx;
+    hipGraph_t g;
+    hipGraphExec_t exec;
+};
 struct psn_module {
     psn_ctx *ctx;
     std::vector<hipModule_t> m;   /* one per code object; kernels are looked up across all */
@@ -300,6 +305,84 @@ extern "C" int32_t psn_stream_destroy(psn_stream *s) {
     hipError_t e = hipStreamDestroy(s->s);
     delete s;
     if (e != hipSuccess) return hip_fail(e, "hipStreamDestroy");
+    return PSN_OK;
+}
+
+static int32_t is_capturing(psn_stream *s, bool *out) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    HIP_TRY(hipStreamIsCapturing(s->s, &st));
+    *out = st != hipStreamCaptureStatusNone;
+    return PSN_OK;
+}
+static int32_t ensure_workspace(psn_stream *s, int64_t bytes) {
+    if (s->ws_bytes >= (size_t)bytes) return PSN_OK;
+    bool cap = false;
+    int32_t rc = is_capturing(s, &cap);
+    if (rc) return rc;
+    if (cap) return fail(PSN_E_INVALID_ARG, "activation workspace must grow to %lld bytes during capture: call psn_stream_reserve first", (long long)bytes);
+    /* earlier launches may still read the old workspace */
+    HIP_TRY(hipStreamSynchronize(s->s));
+    if (s->ws) HIP_TRY(hipFree(s->ws));
+    s->ws = nullptr;
+    s->ws_bytes = 0;
+    const size_t want = (size_t)align_up(bytes, 1 << 20);
+    hipError_t e = hipMalloc(&s->ws, want);
+    if (e != hipSuccess) return hip_fail(e, "hipMalloc(workspace)");
+    s->ws_bytes = want;
+    return PSN_OK;
+}
+extern "C" int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch) {
+    if (!s) return fail(PSN_E_INVALID_ARG, "stream is null");
+    if (K <= 0 || K % 256) return fail(PSN_E_SHAPE, "K=%lld must be a positive multiple of 256", (long long)K);
+    psn_actq_info a, b;
+    int32_t rc = psn_actq_layout(PSN_Q8_0, K, batch, &a);
+    if (rc) return rc;
+    if ((rc = psn_actq_layout(PSN_Q8_K, K, batch, &b))) return rc;
+    if ((rc = bind(s->ctx))) return rc;
+    return ensure_workspace(s, a.bytes > b.bytes ? a.bytes : b.bytes);
+}
+
+extern "C" int32_t psn_graph_begin_capture(psn_stream *s) {
+    if (!s) return fail(PSN_E_INVALID_ARG, "stream is null");
+    int32_t rc = bind(s->ctx);
+    if (rc) return rc;
+    HIP_TRY(hipStreamBeginCapture(s->s, hipStreamCaptureModeThreadLocal));
+    return PSN_OK;
+}
+extern "C" int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out) {
+    if (!s || !out) return fail(PSN_E_INVALID_ARG, "stream or out is null");
+    *out = nullptr;
+    int32_t rc = bind(s->ctx);
+    if (rc) return rc;
+    hipGraph_t g = nullptr;
+    HIP_TRY(hipStreamEndCapture(s->s, &g));
+    if (!g) return fail(PSN_E_HIP, "hipStreamEndCapture returned no graph (capture was invalidated)");
+    hipGraphExec_t ex = nullptr;
+    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) { (void)hipGraphDestroy(g); return hip_fail(e, "hipGraphInstantiate"); }
+    psn_graph *gr = new (std::nothrow) psn_graph();
+    if (!gr) { (void)hipGraphExecDestroy(ex); (void)hipGraphDestroy(g); return fail(PSN_E_OOM, "host allocation failed"); }
+    gr->ctx = s->ctx;
+    gr->g = g;
+    gr->exec = ex;
+    *out = gr;
+    return PSN_OK;
+}
+extern "C" int32_t psn_graph_launch(psn_graph *g, psn_stream *s) {
+    if (!g || !s) return fail(PSN_E_INVALID_ARG, "graph or stream is null");
+    if (g->ctx != s->ctx) return fail(PSN_E_INVALID_ARG, "graph and stream belong to different contexts");
+    int32_t rc = bind(g->ctx);
+    if (rc) return rc;
+    HIP_TRY(hipGraphLaunch(g->exec, s->s));
+    return PSN_OK;
+}
+extern "C" int32_t psn_graph_destroy(psn_graph *g) {
+    if (!g) return fail(PSN_E_INVALID_ARG, "graph is null");
+    int32_t rc = bind(g->ctx);
+    if (rc) return rc;
+    (void)hipGraphExecDestroy(g->exec);
+    (void)hipGraphDestroy(g->g);
+    delete g;
     return PSN_OK;
 }
 
@@ -493,6 +576,16 @@ static int32_t check_matvec_shape(int32_t qtype, int32_t scheme, int64_t N, int6
     return PSN_OK;
 }
 
+/* bytes of LDS the staged copy of a quantized activation takes (qs padded to 272 B per chunk) */
+static int64_t staged_lds_bytes(int32_t qtype, int64_t K, int32_t batch) {
+    const int32_t at = psn_act_type_for(qtype);
+    const int64_t be = psn_block_elems(at);
+    const int64_t qs = batch * (K / 256) * 272;
+    const int64_t d = align_up(batch * (K / be) * 4, 16);
+    const int64_t sb = at == PSN_Q8_0 ? batch * (K / 32) * 4 : batch * (K / 16) * 2;
+    return qs + d + align_up(sb, 16);
+}
+
 extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, psn_matvec_plan *out) {
     if (!out) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_plan: out is null");
     int32_t rc = check_matvec_shape(qtype, scheme, N, K, batch);
@@ -502,18 +595,16 @@ extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, in
     psn_matvec_plan p;
     p.lanes_per_row = C <= 8 ? 8 : C <= 16 ? 16 : C <= 32 ? 32 : 64;
     p.batch_tile = batch <= 1 ? 1 : batch <= 2 ? 2 : batch <= 4 ? 4 : 8;
-    p.stage_lds = 0;
-    p.lds_bytes = 0;
-    /* rows in flight per lane: keep at least ~4 waves per CU, otherwise more bytes per lane */
+    p.threads = 256;
+    p.stage_lds = (scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 64 * 1024) ? 1 : 0;
+    /* rows in flight per lane: two row sets once the matrix is tall enough to still fill the chip */
     const int64_t S = 64 / p.lanes_per_row;
     p.rows_in_flight = 1;
-    if (p.batch_tile == 1 && scheme == PSN_ACT_Q8) {
-        const int64_t waves_r2 = (N + 2 * S - 1) / (2 * S);
-        if (waves_r2 >= (int64_t)cus * 8) p.rows_in_flight = 2;
-    }
+    if (p.batch_tile == 1 && scheme == PSN_ACT_Q8 && N >= 2 * S * 4 * (int64_t)cus) p.rows_in_flight = 2;
     const int64_t rows_per_wave = S * p.rows_in_flight;
     const int64_t passes = (N + rows_per_wave - 1) / rows_per_wave;
-    int64_t blocks = (passes + 3) / 4;
+    const int64_t wpb = p.threads / 64;
+    int64_t blocks = (passes + wpb - 1) / wpb;
     const int64_t cap = (int64_t)cus * 16;
     if (blocks > cap) blocks = cap;
     p.blocks = (int32_t)blocks;
@@ -525,6 +616,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     const int g = p->lanes_per_row, r = p->rows_in_flight, nb = p->batch_tile;
     if (!(g == 8 || g == 16 || g == 32 || g == 64)) return fail(PSN_E_UNSUPPORTED, "plan: lanes_per_row=%d", g);
     if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
+    if (p->threads != 256 && p->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
     bool ok;
     if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2 || r == 4)) || ((nb == 2 || nb == 4) && (r == 1 || r == 2)) || (nb == 8 && r == 1);
     else ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
@@ -533,14 +625,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     int32_t lds = 0;
     if (p->stage_lds) {
         if (scheme != PSN_ACT_Q8) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging exists for scheme Q8 only");
-        psn_actq_info li;
-        int32_t rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li);
-        if (rc) return rc;
-        /* packed copy of the three fields, each rounded to 16 bytes */
-        const int64_t be = psn_block_elems(psn_act_type_for(qtype));
-        const int64_t qs = batch * K, d = align_up(batch * (K / be) * 4, 16);
-        const int64_t sb = psn_act_type_for(qtype) == PSN_Q8_0 ? batch * (K / 32) * 4 : batch * (K / 16) * 2;
-        const int64_t total = qs + d + align_up(sb, 16);
+        const int64_t total = staged_lds_bytes(qtype, K, batch);
         if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging needs %lld bytes, device offers %d", (long long)total, max_lds);
         lds = (int32_t)total;
     }
@@ -548,18 +633,33 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     return PSN_OK;
 }
 
-static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const void *W, const void *x,
-                          float *y, int64_t N, int64_t K, int32_t batch, const psn_matvec_plan *plan) {
+struct seg_list {
+    int32_t count;
+    const void *W[PSN_MAX_SEGMENTS];
+    float *y[PSN_MAX_SEGMENTS];
+    int64_t N[PSN_MAX_SEGMENTS];
+    int64_t total;
+};
+
+static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const seg_list &sg, const void *x,
+                          int64_t K, int32_t batch, const psn_matvec_plan *plan) {
     int32_t lds = 0;
     int32_t rc = plan_is_valid(plan, qtype, scheme, K, batch, mod->ctx->max_lds, &lds);
     if (rc) return rc;
     psn_matvec_args a;
     memset(&a, 0, sizeof a);
-    a.W = (const uint8_t *)W;
-    a.y = y;
-    a.N = (int32_t)N;
+    int64_t end = 0;
+    for (int i = 0; i < PSN_MAX_SEGMENTS; ++i) {
+        const int j = i < sg.count ? i : sg.count - 1;
+        if (i < sg.count) end += sg.N[i];
+        a.W[i] = (const uint8_t *)sg.W[j];
+        a.y[i] = sg.y[j];
+        a.row_end[i] = (int32_t)end;
+    }
+    a.N = (int32_t)sg.total;
     a.K = (int32_t)K;
     a.batch = batch;
+    a.nseg = sg.count;
     a.row_bytes = psn_row_bytes(qtype, K);
     char name[96];
     if (scheme == PSN_ACT_Q8) {
@@ -574,72 +674,101 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
         a.xf = (const float *)x;
         snprintf(name, sizeof name, "psn_mv_%s_f32_g%d_r%d_b%d", fmt_name(qtype), plan->lanes_per_row, plan->rows_in_flight, plan->batch_tile);
     }
-    return launch(mod, s, name, (unsigned)plan->blocks, 256, (unsigned)lds, &a);
+    return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)lds, &a);
 }
 
-static int32_t check_matvec_bufs(int32_t qtype, const psn_buf *W, const psn_buf *y, int64_t N, int64_t K, int32_t batch) {
-    const int64_t need_w = N * psn_row_bytes(qtype, K);
-    if ((int64_t)W->bytes < need_w) return fail(PSN_E_INVALID_ARG, "matvec: W holds %zu bytes, need %lld", W->bytes, (long long)need_w);
-    if ((int64_t)y->bytes < N * batch * 4) return fail(PSN_E_INVALID_ARG, "matvec: y holds %zu bytes, need %lld", y->bytes, (long long)(N * batch * 4));
+/* validates handles, shapes and buffer sizes of a (multi-)matvec and flattens it into a seg_list */
+static int32_t gather_segments(const char *what, psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, int32_t count,
+                               const psn_buf *const *W, const psn_buf *x, psn_buf *const *y, const int64_t *N, int64_t K,
+                               int32_t batch, seg_list *out) {
+    if (!mod || !s || !W || !x || !y || !N) return fail(PSN_E_INVALID_ARG, "%s: null handle", what);
+    if (count < 1 || count > PSN_MAX_SEGMENTS) return fail(PSN_E_SHAPE, "%s: count=%d outside 1..%d", what, count, PSN_MAX_SEGMENTS);
+    if (s->ctx != mod->ctx || x->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "%s: handles belong to different contexts", what);
+    out->count = count;
+    out->total = 0;
+    for (int i = 0; i < count; ++i) {
+        if (!W[i] || !y[i]) return fail(PSN_E_INVALID_ARG, "%s: null buffer for matrix %d", what, i);
+        if (W[i]->ctx != mod->ctx || y[i]->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "%s: handles belong to different contexts", what);
+        int32_t rc = check_matvec_shape(qtype, scheme, N[i], K, batch);
+        if (rc) return rc;
+        const int64_t need_w = N[i] * psn_row_bytes(qtype, K);
+        if ((int64_t)W[i]->bytes < need_w) return fail(PSN_E_INVALID_ARG, "%s: W[%d] holds %zu bytes, need %lld", what, i, W[i]->bytes, (long long)need_w);
+        if ((int64_t)y[i]->bytes < N[i] * batch * 4) return fail(PSN_E_INVALID_ARG, "%s: y[%d] holds %zu bytes, need %lld", what, i, y[i]->bytes, (long long)(N[i] * batch * 4));
+        out->W[i] = W[i]->p;
+        out->y[i] = (float *)y[i]->p;
+        out->N[i] = N[i];
+        out->total += N[i];
+    }
+    if (out->total > INT32_MAX / 2) return fail(PSN_E_SHAPE, "%s: %lld rows in one launch", what, (long long)out->total);
     return PSN_OK;
 }
 
-extern "C" int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const psn_buf *W,
-                                       const psn_buf *x, psn_buf *y, int64_t N, int64_t K, int32_t batch, const psn_matvec_plan *plan) {
-    int32_t rc = check_same_ctx(mod, s, W, x, y, "psn_qmatvec_planned");
+static int32_t check_x_q8(const char *what, int32_t qtype, const psn_buf *x, int64_t K, int32_t batch) {
+    psn_actq_info li;
+    int32_t rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li);
     if (rc) return rc;
+    if ((int64_t)x->bytes < li.bytes) return fail(PSN_E_INVALID_ARG, "%s: x_q holds %zu bytes, need %lld", what, x->bytes, (long long)li.bytes);
+    return PSN_OK;
+}
+static int32_t check_x_f32(const char *what, const psn_buf *x, int64_t K, int32_t batch) {
+    if ((int64_t)x->bytes < K * batch * 4) return fail(PSN_E_INVALID_ARG, "%s: x holds %zu bytes, need %lld", what, x->bytes, (long long)(K * batch * 4));
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, int32_t count,
+                                       const psn_buf *const *W, const psn_buf *x, psn_buf *const *y, const int64_t *N, int64_t K,
+                                       int32_t batch, const psn_matvec_plan *plan) {
     if (!plan) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_planned: plan is null");
-    if ((rc = check_matvec_shape(qtype, scheme, N, K, batch))) return rc;
-    if ((rc = check_matvec_bufs(qtype, W, y, N, K, batch))) return rc;
-    if (scheme == PSN_ACT_Q8) {
-        psn_actq_info li;
-        if ((rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li))) return rc;
-        if ((int64_t)x->bytes < li.bytes) return fail(PSN_E_INVALID_ARG, "matvec: x_q holds %zu bytes, need %lld", x->bytes, (long long)li.bytes);
-    } else if ((int64_t)x->bytes < K * batch * 4) {
-        return fail(PSN_E_INVALID_ARG, "matvec: x holds %zu bytes, need %lld", x->bytes, (long long)(K * batch * 4));
-    }
+    seg_list sg;
+    int32_t rc = gather_segments("psn_qmatvec_planned", mod, s, qtype, scheme, count, W, x, y, N, K, batch, &sg);
+    if (rc) return rc;
+    if ((rc = scheme == PSN_ACT_Q8 ? check_x_q8("psn_qmatvec_planned", qtype, x, K, batch) : check_x_f32("psn_qmatvec_planned", x, K, batch))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
-    return run_matvec(mod, s, qtype, scheme, W->p, x->p, (float *)y->p, N, K, batch, plan);
+    return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, plan);
+}
+
+extern "C" int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t count,
+                                        const psn_buf *const *W, const psn_buf *xq, psn_buf *const *y, const int64_t *N, int64_t K,
+                                        int32_t batch) {
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
+    seg_list sg;
+    int32_t rc = gather_segments("psn_qmatvec_q8_multi", mod, s, qtype, PSN_ACT_Q8, count, W, xq, y, N, K, batch, &sg);
+    if (rc) return rc;
+    if ((rc = check_x_q8("psn_qmatvec_q8_multi", qtype, xq, K, batch))) return rc;
+    psn_matvec_plan plan;
+    if ((rc = psn_qmatvec_plan(qtype, PSN_ACT_Q8, sg.total, K, batch, mod->ctx->compute_units, &plan))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, xq->p, K, batch, &plan);
 }
 
 extern "C" int32_t psn_qmatvec_q8(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
                                   const psn_buf *xq, psn_buf *y, int64_t N, int64_t K, int32_t batch) {
+    return psn_qmatvec_q8_multi(mod, s, qtype, layout, 1, &W, xq, &y, &N, K, batch);
+}
+
+extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, int32_t count,
+                                     const psn_buf *const *W, const psn_buf *x, psn_buf *const *y, const int64_t *N, int64_t K,
+                                     int32_t batch) {
     if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
-    if (!mod) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_q8: module is null");
-    psn_matvec_plan plan;
-    int32_t rc = psn_qmatvec_plan(qtype, PSN_ACT_Q8, N, K, batch, mod->ctx->compute_units, &plan);
+    seg_list sg;
+    int32_t rc = gather_segments("psn_qmatvec", mod, s, qtype, scheme, count, W, x, y, N, K, batch, &sg);
     if (rc) return rc;
-    return psn_qmatvec_planned(mod, s, qtype, PSN_ACT_Q8, W, xq, y, N, K, batch, &plan);
+    if ((rc = check_x_f32("psn_qmatvec", x, K, batch))) return rc;
+    psn_matvec_plan plan;
+    if ((rc = psn_qmatvec_plan(qtype, scheme, sg.total, K, batch, mod->ctx->compute_units, &plan))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    if (scheme == PSN_ACT_F32) return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
+    const int32_t at = psn_act_type_for(qtype);
+    psn_actq_info li;
+    if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;
+    if ((rc = ensure_workspace(s, li.bytes))) return rc;
+    if ((rc = quantize_into(mod, s, at, (const float *)x->p, s->ws, K, batch))) return rc;
+    return run_matvec(mod, s, qtype, scheme, sg, s->ws, K, batch, &plan);
 }
 
 extern "C" int32_t psn_qmatvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, const psn_buf *W,
                                const psn_buf *x, psn_buf *y, int64_t N, int64_t K, int32_t batch) {
-    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
-    int32_t rc = check_same_ctx(mod, s, W, x, y, "psn_qmatvec");
-    if (rc) return rc;
-    if ((rc = check_matvec_shape(qtype, scheme, N, K, batch))) return rc;
-    if ((rc = check_matvec_bufs(qtype, W, y, N, K, batch))) return rc;
-    if ((int64_t)x->bytes < K * batch * 4) return fail(PSN_E_INVALID_ARG, "matvec: x holds %zu bytes, need %lld", x->bytes, (long long)(K * batch * 4));
-    psn_matvec_plan plan;
-    if ((rc = psn_qmatvec_plan(qtype, scheme, N, K, batch, mod->ctx->compute_units, &plan))) return rc;
-    if ((rc = bind(mod->ctx))) return rc;
-    if (scheme == PSN_ACT_F32) return run_matvec(mod, s, qtype, scheme, W->p, x->p, (float *)y->p, N, K, batch, &plan);
-    const int32_t at = psn_act_type_for(qtype);
-    psn_actq_info li;
-    if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;
-    if (s->ws_bytes < (size_t)li.bytes) {
-        /* grow the stream's activation workspace; earlier launches may still read the old one */
-        HIP_TRY(hipStreamSynchronize(s->s));
-        if (s->ws) HIP_TRY(hipFree(s->ws));
-        s->ws = nullptr;
-        s->ws_bytes = 0;
-        const size_t want = (size_t)align_up(li.bytes, 1 << 20);
-        hipError_t e = hipMalloc(&s->ws, want);
-        if (e != hipSuccess) return hip_fail(e, "hipMalloc(workspace)");
-        s->ws_bytes = want;
-    }
-    if ((rc = quantize_into(mod, s, at, (const float *)x->p, s->ws, K, batch))) return rc;
-    return run_matvec(mod, s, qtype, scheme, W->p, s->ws, (float *)y->p, N, K, batch, &plan);
+    return psn_qmatvec_multi(mod, s, qtype, layout, scheme, 1, &W, x, &y, &N, K, batch);
 }
 
 /* ------------------------------------------------------------------ prefill */

@@ -1,6 +1,8 @@
 /*
  * psn_matvec.hip -- gfx950 decode kernels: activation quantizers and the batch-1..8 quantized
  * matvec y[b][n] = sum_k deq(W)[n][k] * x[b][k] over GGUF Q4_0 / Q8_0 / Q4_K / Q6_K rows.
+ * One launch can serve up to four matrices that share x (q/k/v, gate/up): their rows are walked
+ * as one concatenated row space ("segments").
  *
  * The matvec is an HBM stream, so everything is organised around 128-bit loads of the raw GGUF
  * bytes.  Blocks are 18 / 34 / 144 / 210 bytes, which is not a multiple of 16, but 256 weights
@@ -103,36 +105,83 @@ struct RowMap {
     }
 };
 
+/* row of the concatenated row space -> (segment, local row) */
+PSN_DEV int seg_of(const psn_matvec_args &a, int row) {
+    int s = 0;
+    if (a.nseg > 1 && row >= a.row_end[0]) s = 1;
+    if (a.nseg > 2 && row >= a.row_end[1]) s = 2;
+    if (a.nseg > 3 && row >= a.row_end[2]) s = 3;
+    return s;
+}
+PSN_DEV const uint8_t *row_ptr(const psn_matvec_args &a, int row) {
+    const int s = seg_of(a, row);
+    const int local = row - (s ? a.row_end[s - 1] : 0);
+    return a.W[s] + (int64_t)local * a.row_bytes;
+}
+
 template <int G, int R, int NB>
 PSN_DEV void store_rows(const RowMap<G, R> &m, float (&acc)[R][NB], const psn_matvec_args &a, int row0) {
     UNROLL for (int r = 0; r < R; ++r) {
         const int row = row0 + r * RowMap<G, R>::S + m.slot;
+        const int s = seg_of(a, row);
+        const int base = s ? a.row_end[s - 1] : 0;
+        const int nseg_rows = a.row_end[s] - base;
         UNROLL for (int nb = 0; nb < NB; ++nb) {
             const float v = group_sum<G>(acc[r][nb]);
-            if (m.j == 0 && row < a.N && nb < a.batch) a.y[(int64_t)nb * a.N + row] = v;
+            if (m.j == 0 && row < a.N && nb < a.batch) a.y[s][(int64_t)nb * nseg_rows + (row - base)] = v;
         }
     }
 }
 
-/* Copies the live batch columns of a quantized activation into LDS (same three-region layout,
- * packed for `batch` columns) and re-points the accessors at it. */
+/* Quantized activations as the kernels see them: either the global three-field layout or a copy
+ * staged in LDS.  In LDS every 256-byte chunk of qs is followed by 16 bytes of padding, so lanes
+ * that own neighbouring chunks start 68 dwords apart and their 128-bit reads fall into disjoint
+ * banks (a 64-dword stride would put all of them on the same ones). */
 template <typename ST>
-PSN_DEV void stage_actq(const psn_matvec_args &a, int d_per_col, int s_per_col, const int8_t *&xqs, const float *&xd, const ST *&xs) {
+struct ActQ {
+    const int8_t *qs;
+    const float *d;
+    const ST *s;
+    int chunk_stride;   /* bytes between consecutive 256-element chunks of qs */
+    int col_stride;     /* bytes between batch columns of qs */
+    PSN_DEV const uint4 *chunk(int col, int c) const {
+        return reinterpret_cast<const uint4 *>(qs + (int64_t)col * col_stride + (int64_t)c * chunk_stride);
+    }
+};
+
+template <typename ST>
+PSN_DEV ActQ<ST> act_global(const psn_matvec_args &a) {
+    ActQ<ST> x;
+    x.qs = a.xqs;
+    x.d = a.xd;
+    x.s = reinterpret_cast<const ST *>(a.xs);
+    x.chunk_stride = 256;
+    x.col_stride = a.K;
+    return x;
+}
+
+/* d_per_col floats and s_per_col ST values per batch column */
+template <typename ST>
+PSN_DEV ActQ<ST> act_stage_lds(const psn_matvec_args &a, int d_per_col, int s_per_col) {
     extern __shared__ uint4 psn_smem[];
-    const int n_qs = a.batch * a.K / 16;
-    /* field sizes rounded up to whole 16-byte words: the global regions are padded to 256 B */
-    const int n_d = (a.batch * d_per_col * 4 + 15) / 16;
+    const int C = a.K >> 8;
+    const int n_qs = a.batch * C * 16;                       /* source words */
+    const int n_d = (a.batch * d_per_col * 4 + 15) / 16;     /* the global fields are padded to 256 B */
     const int n_s = (a.batch * s_per_col * (int)sizeof(ST) + 15) / 16;
-    uint4 *l_qs = psn_smem, *l_d = l_qs + n_qs, *l_s = l_d + n_d;
-    const uint4 *g_qs = reinterpret_cast<const uint4 *>(xqs), *g_d = reinterpret_cast<const uint4 *>(xd);
-    const uint4 *g_s = reinterpret_cast<const uint4 *>(xs);
-    for (int i = threadIdx.x; i < n_qs; i += blockDim.x) l_qs[i] = g_qs[i];
+    uint4 *l_qs = psn_smem, *l_d = l_qs + a.batch * C * 17, *l_s = l_d + n_d;
+    const uint4 *g_qs = reinterpret_cast<const uint4 *>(a.xqs), *g_d = reinterpret_cast<const uint4 *>(a.xd);
+    const uint4 *g_s = reinterpret_cast<const uint4 *>(a.xs);
+    for (int i = threadIdx.x; i < n_qs; i += blockDim.x) l_qs[(i >> 4) * 17 + (i & 15)] = g_qs[i];
     for (int i = threadIdx.x; i < n_d; i += blockDim.x) l_d[i] = g_d[i];
     for (int i = threadIdx.x; i < n_s; i += blockDim.x) l_s[i] = g_s[i];
     __syncthreads();
-    xqs = reinterpret_cast<const int8_t *>(l_qs);
-    xd = reinterpret_cast<const float *>(l_d);
-    xs = reinterpret_cast<const ST *>(l_s);
+    ActQ<ST> x;
+    x.qs = reinterpret_cast<const int8_t *>(l_qs);
+    x.d = reinterpret_cast<const float *>(l_d);
+    x.s = reinterpret_cast<const ST *>(l_s);
+    x.chunk_stride = 272;
+    x.col_stride = C * 272;
+    return x;
 }
 
 /* ------------------------------------------------------------------------------------------
@@ -156,69 +205,6 @@ PSN_DEV void q4_0_block(const u32 (&w)[36], float &d, u32 (&lo)[4], u32 (&hi)[4]
     UNROLL for (int i = 0; i < 4; ++i) { lo[i] = q[i] & 0x0f0f0f0fu; hi[i] = (q[i] >> 4) & 0x0f0f0f0fu; }
 }
 
-template <int B, int R, int NB>
-PSN_DEV void q4_0_q8_step(const u32 (&w)[R][36], const int8_t *xqs, const float *xd, const int *xs, int K, int nblk,
-                          int blk0, int batch, float (&acc)[R][NB]) {
-    float dw[R];
-    u32 lo[R][4], hi[R][4];
-    UNROLL for (int r = 0; r < R; ++r) q4_0_block<B>(w[r], dw[r], lo[r], hi[r]);
-    UNROLL for (int nb = 0; nb < NB; ++nb) {
-        const int col = nb < batch ? nb : batch - 1;
-        const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)(blk0 + B) * 32);
-        const uint4 x0 = xp[0], x1 = xp[1];
-        const float dx = xd[col * nblk + blk0 + B];
-        const int sx = xs[col * nblk + blk0 + B];
-        UNROLL for (int r = 0; r < R; ++r) {
-            int s = dot4(lo[r][0], x0.x, 0);
-            s = dot4(lo[r][1], x0.y, s);
-            s = dot4(lo[r][2], x0.z, s);
-            s = dot4(lo[r][3], x0.w, s);
-            s = dot4(hi[r][0], x1.x, s);
-            s = dot4(hi[r][1], x1.y, s);
-            s = dot4(hi[r][2], x1.z, s);
-            s = dot4(hi[r][3], x1.w, s);
-            s -= 8 * sx;
-            acc[r][nb] += (float)s * dw[r] * dx;
-        }
-    }
-}
-
-template <int G, int R, int NB, bool XLDS>
-PSN_DEV void mv_q4_0_q8(const psn_matvec_args &a) {
-    const RowMap<G, R> m;
-    const int K = a.K, C = K >> 8, nblk = K >> 5;
-    const int8_t *xqs = a.xqs;
-    const float *xd = a.xd;
-    const int *xs = reinterpret_cast<const int *>(a.xs);
-    if constexpr (XLDS) stage_actq<int>(a, nblk, nblk, xqs, xd, xs);
-    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
-        float acc[R][NB];
-        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
-        for (int c = m.j; c < C; c += G) {
-            u32 w[R][36];
-            UNROLL for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
-                const uint4 *p = reinterpret_cast<const uint4 *>(a.W + (int64_t)row * a.row_bytes) + c * 9;
-                UNROLL for (int i = 0; i < 9; ++i) unpack4(p[i], &w[r][4 * i]);
-            }
-            const int blk0 = c * 8;
-            q4_0_q8_step<0>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-            q4_0_q8_step<1>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-            q4_0_q8_step<2>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-            q4_0_q8_step<3>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-            q4_0_q8_step<4>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-            q4_0_q8_step<5>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-            q4_0_q8_step<6>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-            q4_0_q8_step<7>(w, xqs, xd, xs, K, nblk, blk0, a.batch, acc);
-        }
-        store_rows<G, R, NB>(m, acc, a, row0);
-    }
-}
-
-/* ------------------------------------------------------------------------------------------
- * Q8_0 x Q8_0-activations.  Chunk = 8 blocks = 272 B = 68 dwords; block b starts at byte 34b.
- * ------------------------------------------------------------------------------------------ */
-
 template <int B>
 PSN_DEV void q8_0_block(const u32 (&w)[68], float &d, u32 (&q)[8]) {
     constexpr int base = 17 * (B >> 1);
@@ -231,62 +217,115 @@ PSN_DEV void q8_0_block(const u32 (&w)[68], float &d, u32 (&q)[8]) {
     }
 }
 
-template <int B, int R, int NB>
-PSN_DEV void q8_0_q8_step(const u32 (&w)[R][68], const int8_t *xqs, const float *xd, int K, int nblk, int blk0, int batch,
-                          float (&acc)[R][NB]) {
-    float dw[R];
-    u32 q[R][8];
-    UNROLL for (int r = 0; r < R; ++r) q8_0_block<B>(w[r], dw[r], q[r]);
-    UNROLL for (int nb = 0; nb < NB; ++nb) {
-        const int col = nb < batch ? nb : batch - 1;
-        const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)(blk0 + B) * 32);
-        const uint4 x0 = xp[0], x1 = xp[1];
-        const float dx = xd[col * nblk + blk0 + B];
-        UNROLL for (int r = 0; r < R; ++r) {
-            int s = dot4(q[r][0], x0.x, 0);
-            s = dot4(q[r][1], x0.y, s);
-            s = dot4(q[r][2], x0.z, s);
-            s = dot4(q[r][3], x0.w, s);
-            s = dot4(q[r][4], x1.x, s);
-            s = dot4(q[r][5], x1.y, s);
-            s = dot4(q[r][6], x1.z, s);
-            s = dot4(q[r][7], x1.w, s);
-            acc[r][nb] += (float)s * (dw[r] * dx);
-        }
+struct FmtQ4_0 {
+    static constexpr int DW = 36, BYTES = 144;
+    typedef int ActSum;
+    static PSN_DEV int d_per_col(int K) { return K >> 5; }
+    static PSN_DEV int s_per_col(int K) { return K >> 5; }
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
     }
-}
-
-template <int G, int R, int NB, bool XLDS>
-PSN_DEV void mv_q8_0_q8(const psn_matvec_args &a) {
-    const RowMap<G, R> m;
-    const int K = a.K, C = K >> 8, nblk = K >> 5;
-    const int8_t *xqs = a.xqs;
-    const float *xd = a.xd;
-    const int *xs = reinterpret_cast<const int *>(a.xs);
-    if constexpr (XLDS) stage_actq<int>(a, nblk, nblk, xqs, xd, xs);
-    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
-        float acc[R][NB];
-        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
-        for (int c = m.j; c < C; c += G) {
-            u32 w[R][68];
+    template <int B, int R, int NB>
+    static PSN_DEV void step(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
+        float dw[R];
+        u32 lo[R][4], hi[R][4];
+        UNROLL for (int r = 0; r < R; ++r) q4_0_block<B>(w[r], dw[r], lo[r], hi[r]);
+        const int nblk = K >> 5;
+        UNROLL for (int nb = 0; nb < NB; ++nb) {
+            const int col = nb < batch ? nb : batch - 1;
+            const uint4 *xp = x.chunk(col, c) + 2 * B;
+            const uint4 x0 = xp[0], x1 = xp[1];
+            const float dx = x.d[col * nblk + c * 8 + B];
+            const int sx = x.s[col * nblk + c * 8 + B];
             UNROLL for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
-                const uint4 *p = reinterpret_cast<const uint4 *>(a.W + (int64_t)row * a.row_bytes) + c * 17;
-                UNROLL for (int i = 0; i < 17; ++i) unpack4(p[i], &w[r][4 * i]);
+                int s = dot4(lo[r][0], x0.x, 0);
+                s = dot4(lo[r][1], x0.y, s);
+                s = dot4(lo[r][2], x0.z, s);
+                s = dot4(lo[r][3], x0.w, s);
+                s = dot4(hi[r][0], x1.x, s);
+                s = dot4(hi[r][1], x1.y, s);
+                s = dot4(hi[r][2], x1.z, s);
+                s = dot4(hi[r][3], x1.w, s);
+                s -= 8 * sx;
+                acc[r][nb] += (float)s * dw[r] * dx;
             }
-            const int blk0 = c * 8;
-            q8_0_q8_step<0>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
-            q8_0_q8_step<1>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
-            q8_0_q8_step<2>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
-            q8_0_q8_step<3>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
-            q8_0_q8_step<4>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
-            q8_0_q8_step<5>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
-            q8_0_q8_step<6>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
-            q8_0_q8_step<7>(w, xqs, xd, K, nblk, blk0, a.batch, acc);
         }
-        store_rows<G, R, NB>(m, acc, a, row0);
     }
-}
+    template <int R, int NB>
+    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
+        step<0>(w, x, K, c, batch, acc); step<1>(w, x, K, c, batch, acc);
+        step<2>(w, x, K, c, batch, acc); step<3>(w, x, K, c, batch, acc);
+        step<4>(w, x, K, c, batch, acc); step<5>(w, x, K, c, batch, acc);
+        step<6>(w, x, K, c, batch, acc); step<7>(w, x, K, c, batch, acc);
+    }
+    /* 32 weights of GGUF block SB of the chunk, fp32, element order (scheme F32) */
+    template <int SB>
+    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
+        float d;
+        u32 lo[4], hi[4];
+        q4_0_block<SB>(w, d, lo, hi);
+        const float off = -8.f * d;
+        UNROLL for (int i = 0; i < 4; ++i) UNROLL for (int b = 0; b < 4; ++b) {
+            o[4 * i + b] = __builtin_fmaf((float)((lo[i] >> (8 * b)) & 0xffu), d, off);
+            o[16 + 4 * i + b] = __builtin_fmaf((float)((hi[i] >> (8 * b)) & 0xffu), d, off);
+        }
+    }
+};
+
+/* ------------------------------------------------------------------------------------------
+ * Q8_0 x Q8_0-activations.  Chunk = 8 blocks = 272 B = 68 dwords; block b starts at byte 34b.
+ * ------------------------------------------------------------------------------------------ */
+
+struct FmtQ8_0 {
+    static constexpr int DW = 68, BYTES = 272;
+    typedef int ActSum;
+    static PSN_DEV int d_per_col(int K) { return K >> 5; }
+    static PSN_DEV int s_per_col(int K) { return K >> 5; }
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 17; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    template <int B, int R, int NB>
+    static PSN_DEV void step(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
+        float dw[R];
+        u32 q[R][8];
+        UNROLL for (int r = 0; r < R; ++r) q8_0_block<B>(w[r], dw[r], q[r]);
+        const int nblk = K >> 5;
+        UNROLL for (int nb = 0; nb < NB; ++nb) {
+            const int col = nb < batch ? nb : batch - 1;
+            const uint4 *xp = x.chunk(col, c) + 2 * B;
+            const uint4 x0 = xp[0], x1 = xp[1];
+            const float dx = x.d[col * nblk + c * 8 + B];
+            UNROLL for (int r = 0; r < R; ++r) {
+                int s = dot4(q[r][0], x0.x, 0);
+                s = dot4(q[r][1], x0.y, s);
+                s = dot4(q[r][2], x0.z, s);
+                s = dot4(q[r][3], x0.w, s);
+                s = dot4(q[r][4], x1.x, s);
+                s = dot4(q[r][5], x1.y, s);
+                s = dot4(q[r][6], x1.z, s);
+                s = dot4(q[r][7], x1.w, s);
+                acc[r][nb] += (float)s * (dw[r] * dx);
+            }
+        }
+    }
+    template <int R, int NB>
+    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
+        step<0>(w, x, K, c, batch, acc); step<1>(w, x, K, c, batch, acc);
+        step<2>(w, x, K, c, batch, acc); step<3>(w, x, K, c, batch, acc);
+        step<4>(w, x, K, c, batch, acc); step<5>(w, x, K, c, batch, acc);
+        step<6>(w, x, K, c, batch, acc); step<7>(w, x, K, c, batch, acc);
+    }
+    template <int SB>
+    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
+        float d;
+        u32 q[8];
+        q8_0_block<SB>(w, d, q);
+        UNROLL for (int i = 0; i < 8; ++i) UNROLL for (int b = 0; b < 4; ++b)
+            o[4 * i + b] = (float)(int)(int8_t)((q[i] >> (8 * b)) & 0xffu) * d;
+    }
+};
 
 /* ------------------------------------------------------------------------------------------
  * Q4_K x Q8_K-activations.  Chunk = one 144-byte super-block: dword 0 = d | dmin<<16,
@@ -301,192 +340,58 @@ PSN_DEV void q4_K_scales(u32 s0, u32 s1, u32 s2, u32 (&sc)[2], u32 (&mn)[2]) {
 }
 PSN_DEV int byte_of(const u32 (&v)[2], int i) { return (int)((v[i >> 2] >> (8 * (i & 3))) & 0xffu); }
 
-template <int G, int R, int NB, bool XLDS>
-PSN_DEV void mv_q4_K_q8(const psn_matvec_args &a) {
-    const RowMap<G, R> m;
-    const int K = a.K, C = K >> 8;
-    const int8_t *xqs = a.xqs;
-    const float *xd = a.xd;
-    const int16_t *xs = reinterpret_cast<const int16_t *>(a.xs);
-    if constexpr (XLDS) stage_actq<int16_t>(a, C, C * 16, xqs, xd, xs);
-    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
-        float acc[R][NB];
-        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
-        for (int c = m.j; c < C; c += G) {
-            u32 w[R][36];
-            UNROLL for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
-                const uint4 *p = reinterpret_cast<const uint4 *>(a.W + (int64_t)row * a.row_bytes) + c * 9;
-                UNROLL for (int i = 0; i < 9; ++i) unpack4(p[i], &w[r][4 * i]);
-            }
-            u32 sc[R][2], mn[R][2];
-            UNROLL for (int r = 0; r < R; ++r) q4_K_scales(w[r][1], w[r][2], w[r][3], sc[r], mn[r]);
-            UNROLL for (int nb = 0; nb < NB; ++nb) {
-                const int col = nb < a.batch ? nb : a.batch - 1;
-                const float dx = xd[col * C + c];
-                /* sums of the activation over the eight 32-element sub-blocks */
-                const uint4 *bp = reinterpret_cast<const uint4 *>(xs + ((int64_t)col * C + c) * 16);
-                u32 bs[8];
-                unpack4(bp[0], &bs[0]);
-                unpack4(bp[1], &bs[4]);
-                int bsum[8];
-                UNROLL for (int i = 0; i < 8; ++i) bsum[i] = (int)(int16_t)(bs[i] & 0xffffu) + ((int)bs[i] >> 16);
-                int isum[R], msum[R];
-                UNROLL for (int r = 0; r < R; ++r) {
-                    isum[r] = 0;
-                    msum[r] = 0;
-                    UNROLL for (int i = 0; i < 8; ++i) msum[r] += byte_of(mn[r], i) * bsum[i];
-                }
-                const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)c * 256);
-                UNROLL for (int ch = 0; ch < 4; ++ch) {         /* 64 weights: low nibbles then high nibbles */
-                    u32 xl[8], xh[8];
-                    unpack4(xp[4 * ch + 0], &xl[0]);
-                    unpack4(xp[4 * ch + 1], &xl[4]);
-                    unpack4(xp[4 * ch + 2], &xh[0]);
-                    unpack4(xp[4 * ch + 3], &xh[4]);
-                    UNROLL for (int r = 0; r < R; ++r) {
-                        int sl = 0, sh = 0;
-                        UNROLL for (int i = 0; i < 8; ++i) {
-                            const u32 q = w[r][4 + 8 * ch + i];
-                            sl = dot4(q & 0x0f0f0f0fu, xl[i], sl);
-                            sh = dot4((q >> 4) & 0x0f0f0f0fu, xh[i], sh);
-                        }
-                        isum[r] += byte_of(sc[r], 2 * ch) * sl + byte_of(sc[r], 2 * ch + 1) * sh;
-                    }
-                }
-                UNROLL for (int r = 0; r < R; ++r) {
-                    const float d = h2f_lo(w[r][0]) * dx, dm = h2f_hi(w[r][0]) * dx;
-                    acc[r][nb] += d * (float)isum[r] - dm * (float)msum[r];
-                }
-            }
-        }
-        store_rows<G, R, NB>(m, acc, a, row0);
-    }
-}
-
-/* ------------------------------------------------------------------------------------------
- * Q6_K x Q8_K-activations.  Chunk = one 210-byte super-block at a 2-byte-aligned address:
- * ql[128] | qh[64] | int8 scales[16] | fp16 d.  13 dwordx4 loads cover bytes 0..207.
- * sum (q-32)*x = sum q*x - 32*bsum per 16-element group keeps the 6-bit values unsigned.
- * ------------------------------------------------------------------------------------------ */
-
-struct __attribute__((packed, aligned(2))) u4_a2 { u32 x, y, z, w; };
-
-template <int G, int R, int NB, bool XLDS>
-PSN_DEV void mv_q6_K_q8(const psn_matvec_args &a) {
-    const RowMap<G, R> m;
-    const int K = a.K, C = K >> 8;
-    const int8_t *xqs = a.xqs;
-    const float *xd = a.xd;
-    const int16_t *xs = reinterpret_cast<const int16_t *>(a.xs);
-    if constexpr (XLDS) stage_actq<int16_t>(a, C, C * 16, xqs, xd, xs);
-    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
-        float acc[R][NB];
-        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
-        for (int c = m.j; c < C; c += G) {
-            u32 w[R][52];
-            float dw[R];
-            UNROLL for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
-                const uint8_t *base = a.W + (int64_t)row * a.row_bytes + (int64_t)c * 210;
-                const u4_a2 *p = reinterpret_cast<const u4_a2 *>(base);
-                UNROLL for (int i = 0; i < 13; ++i) {
-                    const u4_a2 v = p[i];
-                    w[r][4 * i] = v.x; w[r][4 * i + 1] = v.y; w[r][4 * i + 2] = v.z; w[r][4 * i + 3] = v.w;
-                }
-                dw[r] = h2f_lo(*reinterpret_cast<const unsigned short *>(base + 208));
-            }
-            UNROLL for (int nb = 0; nb < NB; ++nb) {
-                const int col = nb < a.batch ? nb : a.batch - 1;
-                const float dx = xd[col * C + c];
-                const uint4 *bp = reinterpret_cast<const uint4 *>(xs + ((int64_t)col * C + c) * 16);
-                u32 bs[8];
-                unpack4(bp[0], &bs[0]);
-                unpack4(bp[1], &bs[4]);
-                const uint4 *xp = reinterpret_cast<const uint4 *>(xqs + (int64_t)col * K + (int64_t)c * 256);
-                int isum[R];
-                UNROLL for (int r = 0; r < R; ++r) isum[r] = 0;
-                UNROLL for (int h = 0; h < 2; ++h) {
-                    u32 xq[32];                                   /* 128 activations of this half */
-                    UNROLL for (int i = 0; i < 8; ++i) unpack4(xp[8 * h + i], &xq[4 * i]);
-                    UNROLL for (int r = 0; r < R; ++r) {
-                        int part[8];
-                        UNROLL for (int g = 0; g < 8; ++g) part[g] = 0;
-                        UNROLL for (int i = 0; i < 8; ++i) {      /* dword i holds l = 4i..4i+3 */
-                            const u32 A = w[r][16 * h + i], B = w[r][16 * h + 8 + i], H = w[r][32 + 8 * h + i];
-                            const u32 q1 = (A & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
-                            const u32 q2 = (B & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
-                            const u32 q3 = ((A >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u);
-                            const u32 q4 = ((B >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u);
-                            const int is = i >> 2;
-                            part[is + 0] = dot4(q1, xq[i], part[is + 0]);
-                            part[is + 2] = dot4(q2, xq[8 + i], part[is + 2]);
-                            part[is + 4] = dot4(q3, xq[16 + i], part[is + 4]);
-                            part[is + 6] = dot4(q4, xq[24 + i], part[is + 6]);
-                        }
-                        UNROLL for (int g = 0; g < 8; ++g) {
-                            const int gi = 8 * h + g;             /* 16-element group of the super-block */
-                            const u32 sw = w[r][48 + (gi >> 2)];
-                            const int scale = (int)(int8_t)((sw >> (8 * (gi & 3))) & 0xffu);
-                            const u32 bw = bs[gi >> 1];
-                            const int bsum = (gi & 1) ? ((int)bw >> 16) : (int)(int16_t)(bw & 0xffffu);
-                            isum[r] += scale * (part[g] - 32 * bsum);
-                        }
-                    }
-                }
-                UNROLL for (int r = 0; r < R; ++r) acc[r][nb] += dw[r] * dx * (float)isum[r];
-            }
-        }
-        store_rows<G, R, NB>(m, acc, a, row0);
-    }
-}
-
-/* ------------------------------------------------------------------------------------------
- * Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations.
- * One generic driver; the format supplies "dequantize 32 consecutive weights of my chunk".
- * ------------------------------------------------------------------------------------------ */
-
-struct FmtQ4_0 {
-    static constexpr int DW = 36, BYTES = 144;
-    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
-        const uint4 *q = reinterpret_cast<const uint4 *>(p);
-        UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
-    }
-    /* 32 weights of sub-block SB (one GGUF block) in element order */
-    template <int SB>
-    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
-        float d;
-        u32 lo[4], hi[4];
-        q4_0_block<SB>(w, d, lo, hi);
-        const float off = -8.f * d;
-        UNROLL for (int i = 0; i < 4; ++i) UNROLL for (int b = 0; b < 4; ++b) {
-            o[4 * i + b] = __builtin_fmaf((float)((lo[i] >> (8 * b)) & 0xffu), d, off);
-            o[16 + 4 * i + b] = __builtin_fmaf((float)((hi[i] >> (8 * b)) & 0xffu), d, off);
-        }
-    }
-};
-
-struct FmtQ8_0 {
-    static constexpr int DW = 68, BYTES = 272;
-    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
-        const uint4 *q = reinterpret_cast<const uint4 *>(p);
-        UNROLL for (int i = 0; i < 17; ++i) unpack4(q[i], &w[4 * i]);
-    }
-    template <int SB>
-    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
-        float d;
-        u32 q[8];
-        q8_0_block<SB>(w, d, q);
-        UNROLL for (int i = 0; i < 8; ++i) UNROLL for (int b = 0; b < 4; ++b)
-            o[4 * i + b] = (float)(int)(int8_t)((q[i] >> (8 * b)) & 0xffu) * d;
-    }
-};
-
 struct FmtQ4_K {
     static constexpr int DW = 36, BYTES = 144;
+    typedef int16_t ActSum;
+    static PSN_DEV int d_per_col(int K) { return K >> 8; }
+    static PSN_DEV int s_per_col(int K) { return K >> 4; }
     static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    template <int R, int NB>
+    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int16_t> &x, int K, int c, int batch, float (&acc)[R][NB]) {
+        const int C = K >> 8;
+        u32 sc[R][2], mn[R][2];
+        UNROLL for (int r = 0; r < R; ++r) q4_K_scales(w[r][1], w[r][2], w[r][3], sc[r], mn[r]);
+        UNROLL for (int nb = 0; nb < NB; ++nb) {
+            const int col = nb < batch ? nb : batch - 1;
+            const float dx = x.d[col * C + c];
+            /* sums of the activation over the eight 32-element sub-blocks */
+            const uint4 *bp = reinterpret_cast<const uint4 *>(x.s + ((int64_t)col * C + c) * 16);
+            u32 bs[8];
+            unpack4(bp[0], &bs[0]);
+            unpack4(bp[1], &bs[4]);
+            int bsum[8];
+            UNROLL for (int i = 0; i < 8; ++i) bsum[i] = (int)(int16_t)(bs[i] & 0xffffu) + ((int)bs[i] >> 16);
+            int isum[R], msum[R];
+            UNROLL for (int r = 0; r < R; ++r) {
+                isum[r] = 0;
+                msum[r] = 0;
+                UNROLL for (int i = 0; i < 8; ++i) msum[r] += byte_of(mn[r], i) * bsum[i];
+            }
+            const uint4 *xp = x.chunk(col, c);
+            UNROLL for (int ch = 0; ch < 4; ++ch) {         /* 64 weights: low nibbles then high nibbles */
+                u32 xl[8], xh[8];
+                unpack4(xp[4 * ch + 0], &xl[0]);
+                unpack4(xp[4 * ch + 1], &xl[4]);
+                unpack4(xp[4 * ch + 2], &xh[0]);
+                unpack4(xp[4 * ch + 3], &xh[4]);
+                UNROLL for (int r = 0; r < R; ++r) {
+                    int sl = 0, sh = 0;
+                    UNROLL for (int i = 0; i < 8; ++i) {
+                        const u32 q = w[r][4 + 8 * ch + i];
+                        sl = dot4(q & 0x0f0f0f0fu, xl[i], sl);
+                        sh = dot4((q >> 4) & 0x0f0f0f0fu, xh[i], sh);
+                    }
+                    isum[r] += byte_of(sc[r], 2 * ch) * sl + byte_of(sc[r], 2 * ch + 1) * sh;
+                }
+            }
+            UNROLL for (int r = 0; r < R; ++r) {
+                const float d = h2f_lo(w[r][0]) * dx, dm = h2f_hi(w[r][0]) * dx;
+                acc[r][nb] += d * (float)isum[r] - dm * (float)msum[r];
+            }
+        }
     }
     template <int SB>
     static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
@@ -500,8 +405,19 @@ struct FmtQ4_K {
     }
 };
 
+/* ------------------------------------------------------------------------------------------
+ * Q6_K x Q8_K-activations.  Chunk = one 210-byte super-block at a 2-byte-aligned address:
+ * ql[128] | qh[64] | int8 scales[16] | fp16 d.  13 dwordx4 loads cover bytes 0..207.
+ * sum (q-32)*x = sum q*x - 32*bsum per 16-element group keeps the 6-bit values unsigned.
+ * ------------------------------------------------------------------------------------------ */
+
+struct __attribute__((packed, aligned(2))) u4_a2 { u32 x, y, z, w; };
+
 struct FmtQ6_K {
     static constexpr int DW = 53, BYTES = 210;
+    typedef int16_t ActSum;
+    static PSN_DEV int d_per_col(int K) { return K >> 8; }
+    static PSN_DEV int s_per_col(int K) { return K >> 4; }
     static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
         const u4_a2 *q = reinterpret_cast<const u4_a2 *>(p);
         UNROLL for (int i = 0; i < 13; ++i) {
@@ -509,6 +425,50 @@ struct FmtQ6_K {
             w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
         }
         w[52] = *reinterpret_cast<const unsigned short *>(p + 208);
+    }
+    template <int R, int NB>
+    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int16_t> &x, int K, int c, int batch, float (&acc)[R][NB]) {
+        const int C = K >> 8;
+        UNROLL for (int nb = 0; nb < NB; ++nb) {
+            const int col = nb < batch ? nb : batch - 1;
+            const float dx = x.d[col * C + c];
+            const uint4 *bp = reinterpret_cast<const uint4 *>(x.s + ((int64_t)col * C + c) * 16);
+            u32 bs[8];
+            unpack4(bp[0], &bs[0]);
+            unpack4(bp[1], &bs[4]);
+            const uint4 *xp = x.chunk(col, c);
+            int isum[R];
+            UNROLL for (int r = 0; r < R; ++r) isum[r] = 0;
+            UNROLL for (int h = 0; h < 2; ++h) {
+                u32 xq[32];                                   /* 128 activations of this half */
+                UNROLL for (int i = 0; i < 8; ++i) unpack4(xp[8 * h + i], &xq[4 * i]);
+                UNROLL for (int r = 0; r < R; ++r) {
+                    int part[8];
+                    UNROLL for (int g = 0; g < 8; ++g) part[g] = 0;
+                    UNROLL for (int i = 0; i < 8; ++i) {      /* dword i holds l = 4i..4i+3 */
+                        const u32 A = w[r][16 * h + i], B = w[r][16 * h + 8 + i], H = w[r][32 + 8 * h + i];
+                        const u32 q1 = (A & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
+                        const u32 q2 = (B & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
+                        const u32 q3 = ((A >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u);
+                        const u32 q4 = ((B >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u);
+                        const int is = i >> 2;
+                        part[is + 0] = dot4(q1, xq[i], part[is + 0]);
+                        part[is + 2] = dot4(q2, xq[8 + i], part[is + 2]);
+                        part[is + 4] = dot4(q3, xq[16 + i], part[is + 4]);
+                        part[is + 6] = dot4(q4, xq[24 + i], part[is + 6]);
+                    }
+                    UNROLL for (int g = 0; g < 8; ++g) {
+                        const int gi = 8 * h + g;             /* 16-element group of the super-block */
+                        const u32 sw = w[r][48 + (gi >> 2)];
+                        const int scale = (int)(int8_t)((sw >> (8 * (gi & 3))) & 0xffu);
+                        const u32 bw = bs[gi >> 1];
+                        const int bsum = (gi & 1) ? ((int)bw >> 16) : (int)(int16_t)(bw & 0xffffu);
+                        isum[r] += scale * (part[g] - 32 * bsum);
+                    }
+                }
+            }
+            UNROLL for (int r = 0; r < R; ++r) acc[r][nb] += h2f_lo(w[r][52]) * dx * (float)isum[r];
+        }
     }
     template <int SB>
     static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
@@ -526,6 +486,44 @@ struct FmtQ6_K {
     }
 };
 
+/* ------------------------------------------------------------------------------------------
+ * Drivers.
+ * ------------------------------------------------------------------------------------------ */
+
+template <typename F, int G, int R>
+PSN_DEV void load_rows(const psn_matvec_args &a, const RowMap<G, R> &m, int row0, int c, u32 (&w)[R][F::DW]) {
+    UNROLL for (int r = 0; r < R; ++r) {
+        const int row = min(row0 + r * m.S + m.slot, a.N - 1);     /* rows past the end re-read the last one */
+        F::load(row_ptr(a, row) + (int64_t)c * F::BYTES, w[r]);
+    }
+}
+
+/* Scheme Q8.  The first chunk's weight loads are issued before the activations are staged, so
+ * the staging (an L2 round trip plus a barrier) hides under the HBM latency of the weights. */
+template <typename F, int G, int R, int NB, bool XLDS>
+PSN_DEV void mv_q8(const psn_matvec_args &a) {
+    typedef typename F::ActSum ST;
+    const RowMap<G, R> m;
+    const int K = a.K, C = K >> 8;
+    const int stride = m.nwaves * m.ROWS;
+    int row0 = m.wave * m.ROWS;
+    u32 w[R][F::DW];
+    bool pre = row0 < a.N && m.j < C;
+    if (pre) load_rows<F, G, R>(a, m, row0, m.j, w);
+    const ActQ<ST> x = XLDS ? act_stage_lds<ST>(a, F::d_per_col(K), F::s_per_col(K)) : act_global<ST>(a);
+    for (; row0 < a.N; row0 += stride) {
+        float acc[R][NB];
+        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+        for (int c = m.j; c < C; c += G) {
+            if (!pre) load_rows<F, G, R>(a, m, row0, c, w);
+            pre = false;
+            F::template compute<R, NB>(w, x, K, c, a.batch, acc);
+        }
+        store_rows<G, R, NB>(m, acc, a, row0);
+    }
+}
+
+/* Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations. */
 template <typename F, int SB, int R, int NB>
 PSN_DEV void f32_step(const u32 (&w)[R][F::DW], const float *xf, int K, int k0, int batch, float (&acc)[R][NB]) {
     float o[R][32];
@@ -554,10 +552,7 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
         UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
         for (int c = m.j; c < C; c += G) {
             u32 w[R][F::DW];
-            UNROLL for (int r = 0; r < R; ++r) {
-                const int row = min(row0 + r * m.S + m.slot, a.N - 1);
-                F::load(a.W + (int64_t)row * a.row_bytes + (int64_t)c * F::BYTES, w[r]);
-            }
+            load_rows<F, G, R>(a, m, row0, c, w);
             const int k0 = c * 256;
             f32_step<F, 0>(w, a.xf, K, k0, a.batch, acc);
             f32_step<F, 1>(w, a.xf, K, k0, a.batch, acc);
@@ -574,30 +569,29 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
 
 /* ------------------------------------------------------------------------------------------
  * Entry points.  Name = psn_mv_<fmt>_<scheme>_g<G>_r<R>_b<NB>[_lds]; the host picks one per shape.
+ * Workgroups are 256 or 512 threads.
  * ------------------------------------------------------------------------------------------ */
 
-#define PSN_Q8_KERNEL(fmt, G, R, NB)                                                                      \
-    extern "C" __global__ void __launch_bounds__(256) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
-        mv_##fmt##_q8<G, R, NB, false>(a);                                                                \
+#define PSN_Q8_KERNEL(fmt, F, G, R, NB)                                                                   \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
+        mv_q8<F, G, R, NB, false>(a);                                                                     \
     }                                                                                                     \
-    extern "C" __global__ void __launch_bounds__(256) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
-        mv_##fmt##_q8<G, R, NB, true>(a);                                                                 \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
+        mv_q8<F, G, R, NB, true>(a);                                                                      \
     }
 
 #define PSN_F32_KERNEL(fmt, F, G, R, NB)                                                                  \
-    extern "C" __global__ void __launch_bounds__(256) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
         mv_f32<F, G, R, NB>(a);                                                                           \
     }
 
-#define PSN_FOR_G(M, ...) M(__VA_ARGS__, 8) M(__VA_ARGS__, 16) M(__VA_ARGS__, 32) M(__VA_ARGS__, 64)
-
-#define PSN_Q8_ALL_G(fmt, R, NB) \
-    PSN_Q8_KERNEL(fmt, 8, R, NB) PSN_Q8_KERNEL(fmt, 16, R, NB) PSN_Q8_KERNEL(fmt, 32, R, NB) PSN_Q8_KERNEL(fmt, 64, R, NB)
-#define PSN_Q8_ALL(fmt)                                                                    \
-    PSN_Q8_ALL_G(fmt, 1, 1) PSN_Q8_ALL_G(fmt, 2, 1) PSN_Q8_ALL_G(fmt, 4, 1)                \
-    PSN_Q8_ALL_G(fmt, 1, 2) PSN_Q8_ALL_G(fmt, 2, 2)                                        \
-    PSN_Q8_ALL_G(fmt, 1, 4) PSN_Q8_ALL_G(fmt, 2, 4)                                        \
-    PSN_Q8_ALL_G(fmt, 1, 8)
+#define PSN_Q8_ALL_G(fmt, F, R, NB) \
+    PSN_Q8_KERNEL(fmt, F, 8, R, NB) PSN_Q8_KERNEL(fmt, F, 16, R, NB) PSN_Q8_KERNEL(fmt, F, 32, R, NB) PSN_Q8_KERNEL(fmt, F, 64, R, NB)
+#define PSN_Q8_ALL(fmt, F)                                                                 \
+    PSN_Q8_ALL_G(fmt, F, 1, 1) PSN_Q8_ALL_G(fmt, F, 2, 1) PSN_Q8_ALL_G(fmt, F, 4, 1)       \
+    PSN_Q8_ALL_G(fmt, F, 1, 2) PSN_Q8_ALL_G(fmt, F, 2, 2)                                  \
+    PSN_Q8_ALL_G(fmt, F, 1, 4) PSN_Q8_ALL_G(fmt, F, 2, 4)                                  \
+    PSN_Q8_ALL_G(fmt, F, 1, 8)
 
 #define PSN_F32_ALL_G(fmt, F, R, NB) \
     PSN_F32_KERNEL(fmt, F, 8, R, NB) PSN_F32_KERNEL(fmt, F, 16, R, NB) PSN_F32_KERNEL(fmt, F, 32, R, NB) PSN_F32_KERNEL(fmt, F, 64, R, NB)
@@ -608,18 +602,18 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
 /* The build compiles this file once per format (-DPSN_BUILD_ONLY -DPSN_BUILD_<FMT>) so the four
  * code objects build in parallel; without PSN_BUILD_ONLY everything lands in one. */
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q4_0)
-PSN_Q8_ALL(q4_0)
+PSN_Q8_ALL(q4_0, FmtQ4_0)
 PSN_F32_ALL(q4_0, FmtQ4_0)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q8_0)
-PSN_Q8_ALL(q8_0)
+PSN_Q8_ALL(q8_0, FmtQ8_0)
 PSN_F32_ALL(q8_0, FmtQ8_0)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q4_K)
-PSN_Q8_ALL(q4_K)
+PSN_Q8_ALL(q4_K, FmtQ4_K)
 PSN_F32_ALL(q4_K, FmtQ4_K)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q6_K)
-PSN_Q8_ALL(q6_K)
+PSN_Q8_ALL(q6_K, FmtQ6_K)
 PSN_F32_ALL(q6_K, FmtQ6_K)
 #endif

@@ -92,6 +92,7 @@ def all_plans(scheme, batch):
             for lds in ((0, 1) if scheme == _ffi.ACT_Q8 else (0,)):
                 p = _ffi.MatvecPlan()
                 p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks = g, r, nb, lds, 3
+                p.threads = 512 if (g // 8 + r + lds) % 2 else 256
                 yield p
 
 
@@ -257,3 +258,88 @@ def test_shape_and_buffer_errors_surface_as_codes(hip, orc):
     assert hip.lib.psn_module_has_kernel(hip.module, b"no_such_kernel") == _ffi.E_MODULE
     hip.quantized_matvec(w, x, y)                        # the handles still work afterwards
     hip.sync()
+
+
+# ------------------------------------------------------------------ several matrices per launch, graphs
+
+@pytest.mark.parametrize("qname", FORMATS)
+@pytest.mark.parametrize("scheme", [_ffi.ACT_Q8, _ffi.ACT_F32])
+def test_multi_matrix_every_variant_ragged_segments(hip, orc, qname, scheme):
+    """Segment boundaries (77 | 82 | 212 | 215) fall inside a wave's row set for every G and R."""
+    t = getattr(orc, qname)
+    k, ns, batch = 1024, [77, 5, 130, 3], 2
+    Ws = [weights(orc, qname, 600 + i, n, k) for i, n in enumerate(ns)]
+    x = G.seeded_acts(601, batch, k)
+    refs = [orc.matvec(t, scheme, W, x, n, k) for W, n in zip(Ws, ns)]
+    ws = [hip.upload_weight(t, W, n, k) for W, n in zip(Ws, ns)]
+    xb = hip.upload(x)
+    xin = hip.quantize_activations(xb, k, batch, backend.act_type_for(t)) if scheme == _ffi.ACT_Q8 else xb
+    for count in (2, 4):
+        for p in all_plans(scheme, batch):
+            say(f"multi {qname} scheme={scheme} count={count} {p.as_dict()}")
+            ys = [hip.upload(np.full((batch, n), np.nan, np.float32)) for n in ns[:count]]
+            hip.quantized_matvec_planned(ws[:count], xin, ys, batch, scheme, p)
+            for y, ref, n in zip(ys, refs, ns):
+                err = G.max_rel_err(y.download(np.float32, (batch, n)), ref)
+                assert err < PARITY_TOL, (count, p.as_dict(), n, err)
+
+
+def test_qkv_and_gate_up_shapes_in_one_launch(hip, orc):
+    say("multi: Q4_0 q/k/v 4096+1024+1024 x 4096 and Q4_K gate/up 2 x 14336 x 4096")
+    k = 4096
+    x = G.seeded_acts(611, 1, k)
+    for qname, ns in (("Q4_0", [4096, 1024, 1024]), ("Q4_K", [14336, 14336])):
+        t = getattr(orc, qname)
+        Ws = [weights(orc, qname, 400 if qname == "Q4_0" else 420, n, k) for n in ns]
+        ws = [hip.upload_weight(t, W, n, k) for W, n in zip(Ws, ns)]
+        ys = [hip.alloc(n * 4) for n in ns]
+        hip.quantized_matvec_multi(ws, hip.upload(x), ys, 1, _ffi.ACT_Q8)
+        for W, n, y in zip(Ws, ns, ys):
+            err = G.max_rel_err(y.download(np.float32, (1, n)), orc.matvec(t, orc.ACT_Q8, W, x, n, k))
+            assert err < PARITY_TOL, (qname, n, err)
+    with pytest.raises(ValueError):
+        hip.quantized_matvec_multi([ws[0], hip.upload_weight(orc.Q4_K, weights(orc, "Q4_K", 1, 8, 512), 8, 512)], hip.upload(x), ys, 1)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_multi([ws[0]] * 5, hip.upload(x), [ys[0]] * 5, 1)
+    assert e.value.code == _ffi.E_SHAPE
+
+
+def test_graph_replay_matches_eager(hip, orc):
+    """A captured decode-like chain (quantize, fused q/k/v, second quantize, o) replayed several
+    times with fresh activations between replays; every replay must equal the eager result."""
+    t, k = orc.Q4_0, 2048
+    ns = [2048, 512, 512]
+    Ws = [weights(orc, "Q4_0", 620 + i, n, k) for i, n in enumerate(ns)]
+    Wo = weights(orc, "Q4_0", 629, k, 2048)
+    ws = [hip.upload_weight(t, W, n, k) for W, n in zip(Ws, ns)]
+    wo = hip.upload_weight(t, Wo, k, 2048)
+    xb = hip.alloc(k * 4)
+    ys = [hip.alloc(n * 4) for n in ns]
+    yo = hip.alloc(k * 4)
+    hip.reserve(k, 1)
+    hip.begin_capture()
+    hip.quantized_matvec_multi(ws, xb, ys, 1, _ffi.ACT_Q8)
+    hip.quantized_matvec(wo, ys[0], yo, 1, _ffi.ACT_Q8)       # o-projection fed by q's output
+    graph = hip.end_capture()
+    try:
+        for rep in range(4):
+            x = G.seeded_acts(630 + rep, 1, k)
+            xb.upload(x)
+            hip.launch_graph(graph)
+            got = [y.download(np.float32, (1, n)) for y, n in zip(ys, ns)]
+            got_o = yo.download(np.float32, (1, k))
+            for W, n, g in zip(Ws, ns, got):
+                assert G.max_rel_err(g, orc.matvec(t, orc.ACT_Q8, W, x, n, k)) < PARITY_TOL
+            assert G.max_rel_err(got_o, orc.matvec(t, orc.ACT_Q8, Wo, got[0], k, 2048)) < PARITY_TOL
+            hip.quantized_matvec(wo, ys[0], yo, 1, _ffi.ACT_Q8)  # eager work between replays
+            hip.sync()
+            assert np.array_equal(yo.download(np.float32, (1, k)), got_o)
+    finally:
+        hip.destroy_graph(graph)
+    small = hip.alloc(8)
+    hip.begin_capture()
+    with pytest.raises(backend.PsnError):
+        big = backend.QuantizedTensor(ws[0].buf, t, 8, 1 << 20)      # would need a larger workspace mid-capture
+        hip.quantized_matvec(big, small, small, 1, _ffi.ACT_Q8)
+    g2 = hip.end_capture()
+    hip.destroy_graph(g2)
