@@ -175,14 +175,15 @@ typedef struct psn_matvec_plan {
     int32_t lanes_per_row;  /* 8, 16, 32 or 64 lanes share one row */
     int32_t rows_in_flight; /* 1, 2 or 4 row sets per lane */
     int32_t batch_tile;     /* compiled batch width: 1, 2, 4 or 8 (>= batch) */
-    int32_t stage_lds;      /* 1: activations staged in LDS (scheme Q8 only) */
+    int32_t stage_lds;      /* scheme Q8 only. 0: quantized x read from global memory; 1: staged in LDS;
+                               2: x is fp32 and every workgroup quantizes it while staging */
     int32_t blocks;         /* workgroups */
     int32_t threads;        /* threads per workgroup: 256 or 512 */
 } psn_matvec_plan;
 int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t compute_units,
                          psn_matvec_plan *out);
-/* x is x_q for scheme Q8 (already quantized) and x_f32 for scheme F32; N in the plan call is the
- * total row count when several matrices share the launch */
+/* x is x_f32 for scheme F32 and for stage_lds == 2, x_q (already quantized) otherwise; N in the
+ * plan call is the total row count when several matrices share the launch */
 int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, int32_t count,
                             const psn_buf *const *W, const psn_buf *x, psn_buf *const *y_f32, const int64_t *N, int64_t K,
                             int32_t batch, const psn_matvec_plan *plan);

@@ -256,7 +256,7 @@ class HipBackend:
         yb = self.alloc(batch * n * 4)
         if plan is None:
             self.quantized_matvec(w, xb, yb, batch, scheme)
-        elif scheme == ACT_Q8:
+        elif scheme == ACT_Q8 and plan.stage_lds != 2:
             xq = self.quantize_activations(xb, k, batch, act_type_for(qtype))
             self.quantized_matvec_planned(w, xq, yb, batch, scheme, plan)
         else:

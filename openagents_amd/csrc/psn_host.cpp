@@ -593,19 +593,21 @@ extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, in
     if (cus <= 0) cus = 256;
     const int64_t C = K / 256;
     psn_matvec_plan p;
-    p.lanes_per_row = C <= 8 ? 8 : C <= 16 ? 16 : C <= 32 ? 32 : 64;
     p.batch_tile = batch <= 1 ? 1 : batch <= 2 ? 2 : batch <= 4 ? 4 : 8;
-    p.threads = 256;
-    p.stage_lds = (scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 64 * 1024) ? 1 : 0;
-    /* rows in flight per lane: two row sets once the matrix is tall enough to still fill the chip */
-    const int64_t S = 64 / p.lanes_per_row;
     p.rows_in_flight = 1;
-    if (p.batch_tile == 1 && scheme == PSN_ACT_Q8 && N >= 2 * S * 4 * (int64_t)cus) p.rows_in_flight = 2;
-    const int64_t rows_per_wave = S * p.rows_in_flight;
-    const int64_t passes = (N + rows_per_wave - 1) / rows_per_wave;
+    p.stage_lds = (scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 64 * 1024) ? 1 : 0;
+    /* long rows amortize the activation staging over bigger workgroups */
+    p.threads = K > 8192 ? 512 : 256;
+    /* lanes per row: the row's chunk count rounded up to a power of two, widened (idle lanes, more
+     * waves) while the launch would otherwise leave compute units without a workgroup */
+    int g = C <= 8 ? 8 : C <= 16 ? 16 : C <= 32 ? 32 : 64;
     const int64_t wpb = p.threads / 64;
+    while (g < 64 && (N + (64 / g) - 1) / (64 / g) < (int64_t)cus * wpb) g *= 2;
+    p.lanes_per_row = g;
+    const int64_t rows_per_wave = (64 / g) * p.rows_in_flight;
+    const int64_t passes = (N + rows_per_wave - 1) / rows_per_wave;
     int64_t blocks = (passes + wpb - 1) / wpb;
-    const int64_t cap = (int64_t)cus * 16;
+    const int64_t cap = (int64_t)cus * (p.threads == 256 ? 4 : 2);
     if (blocks > cap) blocks = cap;
     p.blocks = (int32_t)blocks;
     *out = p;
@@ -623,6 +625,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     if (!ok) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
     int32_t lds = 0;
+    if (p->stage_lds < 0 || p->stage_lds > 2) return fail(PSN_E_UNSUPPORTED, "plan: stage_lds=%d", p->stage_lds);
     if (p->stage_lds) {
         if (scheme != PSN_ACT_Q8) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging exists for scheme Q8 only");
         const int64_t total = staged_lds_bytes(qtype, K, batch);
@@ -662,7 +665,10 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
     a.nseg = sg.count;
     a.row_bytes = psn_row_bytes(qtype, K);
     char name[96];
-    if (scheme == PSN_ACT_Q8) {
+    if (scheme == PSN_ACT_Q8 && plan->stage_lds == 2) {
+        a.xf = (const float *)x;
+        snprintf(name, sizeof name, "psn_mv_%s_q8_g%d_r%d_b%d_xf", fmt_name(qtype), plan->lanes_per_row, plan->rows_in_flight, plan->batch_tile);
+    } else if (scheme == PSN_ACT_Q8) {
         psn_actq_info li;
         if ((rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li))) return rc;
         a.xqs = (const int8_t *)x + li.off_qs;
@@ -722,7 +728,8 @@ extern "C" int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t q
     seg_list sg;
     int32_t rc = gather_segments("psn_qmatvec_planned", mod, s, qtype, scheme, count, W, x, y, N, K, batch, &sg);
     if (rc) return rc;
-    if ((rc = scheme == PSN_ACT_Q8 ? check_x_q8("psn_qmatvec_planned", qtype, x, K, batch) : check_x_f32("psn_qmatvec_planned", x, K, batch))) return rc;
+    const bool x_is_q8 = scheme == PSN_ACT_Q8 && plan->stage_lds != 2;
+    if ((rc = x_is_q8 ? check_x_q8("psn_qmatvec_planned", qtype, x, K, batch) : check_x_f32("psn_qmatvec_planned", x, K, batch))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
     return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, plan);
 }
@@ -758,6 +765,11 @@ extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qty
     if ((rc = psn_qmatvec_plan(qtype, scheme, sg.total, K, batch, mod->ctx->compute_units, &plan))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
     if (scheme == PSN_ACT_F32) return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
+    if (plan.stage_lds) {
+        /* one launch: every workgroup quantizes x while staging it */
+        plan.stage_lds = 2;
+        return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
+    }
     const int32_t at = psn_act_type_for(qtype);
     psn_actq_info li;
     if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;

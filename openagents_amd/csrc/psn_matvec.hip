@@ -23,52 +23,42 @@
 #define UNROLL _Pragma("unroll")
 
 /* ------------------------------------------------------------------------------------------
- * Activation quantizers (bit-exact restatements of the Q8_0 / Q8_K row quantizers).
+ * Activation quantizers (bit-exact restatements of the Q8_0 / Q8_K row quantizers).  The same
+ * math runs as stand-alone kernels and inside the matvec's staging step.
  * ------------------------------------------------------------------------------------------ */
 
-#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_QUANT)
-/* Q8_0: 8 lanes per 32-element block, 4 elements per lane.  d = amax/127, q = round-half-away(x/d). */
-extern "C" __global__ void __launch_bounds__(256) psn_quantize_q8_0(const psn_quantize_args a) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   /* one float4 each */
-    const int64_t total4 = (int64_t)a.K * a.batch / 4;
-    const bool live = t < total4;
-    float4 v = live ? reinterpret_cast<const float4 *>(a.x)[t] : make_float4(0.f, 0.f, 0.f, 0.f);
+/* Q8_0: the four elements a lane owns of a 32-element block shared by 8 adjacent lanes.
+ * d = amax/127, q = round-half-away(x/d); returns the packed int8x4, the fp16-rounded scale
+ * (widened) and the block's sum of q. */
+PSN_DEV void q8_0_quant4(const float4 v, u32 &packed, float &d_out, int &sum) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = group_max<8>(amax);
     const float d = amax / 127.f;
     const float id = d != 0.f ? 1.f / d : 0.f;
     const int q0 = (int)roundf(v.x * id), q1 = (int)roundf(v.y * id);
     const int q2 = (int)roundf(v.z * id), q3 = (int)roundf(v.w * id);
-    const int s = group_sum_i<8>(q0 + q1 + q2 + q3);
-    if (!live) return;
-    reinterpret_cast<u32 *>(a.qs)[t] = (u32)(q0 & 0xff) | ((u32)(q1 & 0xff) << 8) | ((u32)(q2 & 0xff) << 16) | ((u32)q3 << 24);
-    if ((threadIdx.x & 7) == 0) {
-        a.d[t >> 3] = (float)(f16)d;            /* what a reader of the fp16 field would see */
-        reinterpret_cast<int *>(a.s)[t >> 3] = s;
-    }
+    sum = group_sum_i<8>(q0 + q1 + q2 + q3);
+    packed = (u32)(q0 & 0xff) | ((u32)(q1 & 0xff) << 8) | ((u32)(q2 & 0xff) << 16) | ((u32)q3 << 24);
+    d_out = (float)(f16)d;            /* what a reader of the fp16 field would see */
 }
 
-/* Q8_K: one wave per 256-element super-block.  iscale = -127/(signed element of largest magnitude,
- * first one on ties), q = min(127, rint(iscale*x)), d = 1/iscale, bsums over groups of 16. */
-extern "C" __global__ void __launch_bounds__(256) psn_quantize_q8_K(const psn_quantize_args a) {
-    const int lane = threadIdx.x & 63;
-    const int64_t sb = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;   /* super-block index */
-    const int64_t nsb = (int64_t)a.K * a.batch / 256;
-    if (sb >= nsb) return;                                                        /* whole wave leaves together */
-    const float4 v = reinterpret_cast<const float4 *>(a.x)[sb * 64 + lane];
+/* Q8_K: one wave owns a 256-element super-block, four elements per lane.
+ * iscale = -127/(signed element of largest magnitude, first one on ties), q = min(127, rint(iscale*x)),
+ * d = 1/iscale; s16 = sum of q over the lane's 16-element group (valid in every lane of the quad). */
+PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out, int &s16) {
     const float e[4] = {v.x, v.y, v.z, v.w};
     float amax = 0.f;
     int first = 4;
-    UNROLL for (int i = 3; i >= 0; --i) if (fabsf(e[i]) >= amax) { amax = fabsf(e[i]); first = i; }
     /* >= scanning downwards leaves the lowest index among equal magnitudes */
+    UNROLL for (int i = 3; i >= 0; --i) if (fabsf(e[i]) >= amax) { amax = fabsf(e[i]); first = i; }
     const float wmax = group_max<64>(amax);
     const int cand = (amax == wmax) ? lane * 4 + first : 1 << 20;
     const int idx = group_min_i<64>(cand);
     const float mine = e[idx & 3];
     const float vmax = __shfl(mine, idx >> 2, 64);
-    u32 packed = 0;
+    packed = 0;
     int s4 = 0;
-    float dout = 0.f;
+    d_out = 0.f;
     if (wmax != 0.f) {
         const float iscale = -127.f / vmax;
         UNROLL for (int i = 0; i < 4; ++i) {
@@ -77,12 +67,42 @@ extern "C" __global__ void __launch_bounds__(256) psn_quantize_q8_K(const psn_qu
             s4 += q;
             packed |= (u32)(q & 0xff) << (8 * i);
         }
-        dout = 1.f / iscale;
+        d_out = 1.f / iscale;
     }
-    const int s16 = group_sum_i<4>(s4);
+    s16 = group_sum_i<4>(s4);
+}
+
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_QUANT)
+extern "C" __global__ void __launch_bounds__(256) psn_quantize_q8_0(const psn_quantize_args a) {
+    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   /* one float4 each */
+    const int64_t total4 = (int64_t)a.K * a.batch / 4;
+    const bool live = t < total4;
+    const float4 v = live ? reinterpret_cast<const float4 *>(a.x)[t] : make_float4(0.f, 0.f, 0.f, 0.f);
+    u32 packed;
+    float d;
+    int s;
+    q8_0_quant4(v, packed, d, s);
+    if (!live) return;
+    reinterpret_cast<u32 *>(a.qs)[t] = packed;
+    if ((threadIdx.x & 7) == 0) {
+        a.d[t >> 3] = d;
+        reinterpret_cast<int *>(a.s)[t >> 3] = s;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(256) psn_quantize_q8_K(const psn_quantize_args a) {
+    const int lane = threadIdx.x & 63;
+    const int64_t sb = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;   /* super-block index */
+    const int64_t nsb = (int64_t)a.K * a.batch / 256;
+    if (sb >= nsb) return;                                                        /* whole wave leaves together */
+    const float4 v = reinterpret_cast<const float4 *>(a.x)[sb * 64 + lane];
+    u32 packed;
+    float d;
+    int s16;
+    q8_K_quant_wave(v, lane, packed, d, s16);
     reinterpret_cast<u32 *>(a.qs)[sb * 64 + lane] = packed;
     if ((lane & 3) == 0) reinterpret_cast<int16_t *>(a.s)[sb * 16 + (lane >> 2)] = (int16_t)s16;
-    if (lane == 0) a.d[sb] = dout;
+    if (lane == 0) a.d[sb] = d;
 }
 #endif
 
@@ -179,6 +199,52 @@ PSN_DEV ActQ<ST> act_stage_lds(const psn_matvec_args &a, int d_per_col, int s_pe
     x.qs = reinterpret_cast<const int8_t *>(l_qs);
     x.d = reinterpret_cast<const float *>(l_d);
     x.s = reinterpret_cast<const ST *>(l_s);
+    x.chunk_stride = 272;
+    x.col_stride = C * 272;
+    return x;
+}
+
+/* Same LDS layout, but filled by quantizing the fp32 activations on the way in: every workgroup
+ * redoes the (tiny) quantization instead of a separate launch doing it once.  ST = int selects
+ * Q8_0 activations, ST = int16_t selects Q8_K. */
+template <typename ST>
+PSN_DEV ActQ<ST> act_stage_quantize(const psn_matvec_args &a, int d_per_col, int s_per_col) {
+    extern __shared__ uint4 psn_smem[];
+    const int C = a.K >> 8;
+    const int n_d = (a.batch * d_per_col * 4 + 15) / 16;
+    uint4 *l_qs4 = psn_smem, *l_d4 = l_qs4 + a.batch * C * 17, *l_s4 = l_d4 + n_d;
+    u32 *l_qs = reinterpret_cast<u32 *>(l_qs4);
+    float *l_d = reinterpret_cast<float *>(l_d4);
+    ST *l_s = reinterpret_cast<ST *>(l_s4);
+    const float4 *x4 = reinterpret_cast<const float4 *>(a.xf);
+    const int lane = threadIdx.x & 63;
+    if constexpr (sizeof(ST) == 4) {
+        const int total4 = a.batch * C * 64;                  /* float4 words; a multiple of 64, so waves stay whole */
+        for (int i = threadIdx.x; i < total4; i += blockDim.x) {
+            u32 packed;
+            float d;
+            int sum;
+            q8_0_quant4(x4[i], packed, d, sum);
+            l_qs[(i >> 6) * 68 + (i & 63)] = packed;          /* chunk index i/64 already runs over batch */
+            if ((lane & 7) == 0) { l_d[i >> 3] = d; l_s[i >> 3] = sum; }
+        }
+    } else {
+        const int nsb = a.batch * C;
+        for (int sb = threadIdx.x >> 6; sb < nsb; sb += blockDim.x >> 6) {
+            u32 packed;
+            float d;
+            int s16;
+            q8_K_quant_wave(x4[sb * 64 + lane], lane, packed, d, s16);
+            l_qs[sb * 68 + lane] = packed;
+            if ((lane & 3) == 0) l_s[sb * 16 + (lane >> 2)] = (ST)s16;
+            if (lane == 0) l_d[sb] = d;
+        }
+    }
+    __syncthreads();
+    ActQ<ST> x;
+    x.qs = reinterpret_cast<const int8_t *>(l_qs4);
+    x.d = l_d;
+    x.s = l_s;
     x.chunk_stride = 272;
     x.col_stride = C * 272;
     return x;
@@ -500,7 +566,9 @@ PSN_DEV void load_rows(const psn_matvec_args &a, const RowMap<G, R> &m, int row0
 
 /* Scheme Q8.  The first chunk's weight loads are issued before the activations are staged, so
  * the staging (an L2 round trip plus a barrier) hides under the HBM latency of the weights. */
-template <typename F, int G, int R, int NB, bool XLDS>
+/* XSRC: 0 = quantized activations read from global memory, 1 = staged into LDS,
+ * 2 = fp32 activations quantized into LDS by the workgroup itself. */
+template <typename F, int G, int R, int NB, int XSRC>
 PSN_DEV void mv_q8(const psn_matvec_args &a) {
     typedef typename F::ActSum ST;
     const RowMap<G, R> m;
@@ -510,7 +578,9 @@ PSN_DEV void mv_q8(const psn_matvec_args &a) {
     u32 w[R][F::DW];
     bool pre = row0 < a.N && m.j < C;
     if (pre) load_rows<F, G, R>(a, m, row0, m.j, w);
-    const ActQ<ST> x = XLDS ? act_stage_lds<ST>(a, F::d_per_col(K), F::s_per_col(K)) : act_global<ST>(a);
+    const ActQ<ST> x = XSRC == 2   ? act_stage_quantize<ST>(a, F::d_per_col(K), F::s_per_col(K))
+                       : XSRC == 1 ? act_stage_lds<ST>(a, F::d_per_col(K), F::s_per_col(K))
+                                   : act_global<ST>(a);
     for (; row0 < a.N; row0 += stride) {
         float acc[R][NB];
         UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
@@ -568,16 +638,20 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
 }
 
 /* ------------------------------------------------------------------------------------------
- * Entry points.  Name = psn_mv_<fmt>_<scheme>_g<G>_r<R>_b<NB>[_lds]; the host picks one per shape.
+ * Entry points.  Name = psn_mv_<fmt>_<scheme>_g<G>_r<R>_b<NB>[_lds|_xf]; the host picks one per shape
+ * (_lds: quantized activations staged in LDS; _xf: fp32 activations quantized while staging).
  * Workgroups are 256 or 512 threads.
  * ------------------------------------------------------------------------------------------ */
 
 #define PSN_Q8_KERNEL(fmt, F, G, R, NB)                                                                   \
     extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
-        mv_q8<F, G, R, NB, false>(a);                                                                     \
+        mv_q8<F, G, R, NB, 0>(a);                                                                         \
     }                                                                                                     \
     extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
-        mv_q8<F, G, R, NB, true>(a);                                                                      \
+        mv_q8<F, G, R, NB, 1>(a);                                                                         \
+    }                                                                                                     \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_xf(const psn_matvec_args a) { \
+        mv_q8<F, G, R, NB, 2>(a);                                                                         \
     }
 
 #define PSN_F32_KERNEL(fmt, F, G, R, NB)                                                                  \

@@ -89,7 +89,7 @@ def all_plans(scheme, batch):
         rs = (1, 2) if nb == 1 else (1,)
     for g in (8, 16, 32, 64):
         for r in rs:
-            for lds in ((0, 1) if scheme == _ffi.ACT_Q8 else (0,)):
+            for lds in ((0, 1, 2) if scheme == _ffi.ACT_Q8 else (0,)):
                 p = _ffi.MatvecPlan()
                 p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks = g, r, nb, lds, 3
                 p.threads = 512 if (g // 8 + r + lds) % 2 else 256
@@ -109,11 +109,11 @@ def test_every_kernel_variant_small(hip, orc, qname, scheme, batch):
     ref = orc.matvec(t, scheme, W, x, n, k)
     w = hip.upload_weight(t, W, n, k)
     xb = hip.upload(x)
-    xin = hip.quantize_activations(xb, k, batch, backend.act_type_for(t)) if scheme == _ffi.ACT_Q8 else xb
+    xq = hip.quantize_activations(xb, k, batch, backend.act_type_for(t)) if scheme == _ffi.ACT_Q8 else xb
     for p in all_plans(scheme, batch):
         say(f"variant {qname} scheme={scheme} batch={batch} {p.as_dict()}")
         yb = hip.upload(np.full((batch, n), np.nan, np.float32))
-        hip.quantized_matvec_planned(w, xin, yb, batch, scheme, p)
+        hip.quantized_matvec_planned(w, xb if p.stage_lds == 2 else xq, yb, batch, scheme, p)
         y = yb.download(np.float32, (batch, n))
         err = G.max_rel_err(y, ref)
         assert np.all(np.isfinite(y)) and err < PARITY_TOL, (p.as_dict(), err)
@@ -273,12 +273,12 @@ def test_multi_matrix_every_variant_ragged_segments(hip, orc, qname, scheme):
     refs = [orc.matvec(t, scheme, W, x, n, k) for W, n in zip(Ws, ns)]
     ws = [hip.upload_weight(t, W, n, k) for W, n in zip(Ws, ns)]
     xb = hip.upload(x)
-    xin = hip.quantize_activations(xb, k, batch, backend.act_type_for(t)) if scheme == _ffi.ACT_Q8 else xb
+    xq = hip.quantize_activations(xb, k, batch, backend.act_type_for(t)) if scheme == _ffi.ACT_Q8 else xb
     for count in (2, 4):
         for p in all_plans(scheme, batch):
             say(f"multi {qname} scheme={scheme} count={count} {p.as_dict()}")
             ys = [hip.upload(np.full((batch, n), np.nan, np.float32)) for n in ns[:count]]
-            hip.quantized_matvec_planned(ws[:count], xin, ys, batch, scheme, p)
+            hip.quantized_matvec_planned(ws[:count], xb if p.stage_lds == 2 else xq, ys, batch, scheme, p)
             for y, ref, n in zip(ys, refs, ns):
                 err = G.max_rel_err(y.download(np.float32, (batch, n)), ref)
                 assert err < PARITY_TOL, (count, p.as_dict(), n, err)
