@@ -118,6 +118,8 @@ int64_t psn_buf_size(const psn_buf *b);
 int32_t psn_buf_upload(psn_buf *dst, size_t off, const void *src, size_t n, psn_stream *s);
 int32_t psn_buf_download(const psn_buf *src, size_t off, void *dst, size_t n, psn_stream *s);
 int32_t psn_buf_fill_zero(psn_buf *b, psn_stream *s);
+/* device-to-device copy of n bytes, asynchronous on s */
+int32_t psn_buf_copy(psn_buf *dst, size_t dst_off, const psn_buf *src, size_t src_off, size_t n, psn_stream *s);
 
 /* ---- weights ---------------------------------------------------------------------------- */
 
@@ -169,11 +171,12 @@ int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t qtype, int3
                              int32_t batch);
 
 /* Launch geometry of one matvec.  psn_qmatvec_plan fills in the library's choice for a shape
- * (pure host arithmetic, usable without a device); psn_qmatvec_planned runs with a caller-chosen
- * one (auto-tuners, benchmarks). */
+ * (pure host arithmetic, usable without a device; x_is_f32 != 0 asks for the plan psn_qmatvec uses
+ * when it quantizes fp32 activations inside the matvec launch); psn_qmatvec_planned runs with a
+ * caller-chosen one (auto-tuners, benchmarks). */
 typedef struct psn_matvec_plan {
     int32_t lanes_per_row;  /* 8, 16, 32 or 64 lanes share one row */
-    int32_t rows_in_flight; /* 1, 2 or 4 row sets per lane */
+    int32_t rows_in_flight; /* row sets per lane: 1, 2 or 4 at batch_tile 1 (2 for scheme F32), else 1 */
     int32_t batch_tile;     /* compiled batch width: 1, 2, 4 or 8 (>= batch) */
     int32_t stage_lds;      /* scheme Q8 only. 0: quantized x read from global memory; 1: staged in LDS;
                                2: x is fp32 and every workgroup quantizes it while staging */
@@ -181,7 +184,7 @@ typedef struct psn_matvec_plan {
     int32_t threads;        /* threads per workgroup: 256 or 512 */
 } psn_matvec_plan;
 int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t compute_units,
-                         psn_matvec_plan *out);
+                         int32_t x_is_f32, psn_matvec_plan *out);
 /* x is x_f32 for scheme F32 and for stage_lds == 2, x_q (already quantized) otherwise; N in the
  * plan call is the total row count when several matrices share the launch */
 int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, int32_t count,

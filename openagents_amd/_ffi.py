@@ -68,13 +68,14 @@ SIGNATURES = {
     "psn_buf_upload": (_i32, [_vp, _sz, _vp, _sz, _vp]),
     "psn_buf_download": (_i32, [_vp, _sz, _vp, _sz, _vp]),
     "psn_buf_fill_zero": (_i32, [_vp, _vp]),
+    "psn_buf_copy": (_i32, [_vp, _sz, _vp, _sz, _sz, _vp]),
     "psn_weight_upload": (_i32, [_vp, _i32, _i64, _i64, _vp, _i32, _vp, _pp]),
     "psn_actq_layout": (_i32, [_i32, _i64, _i32, C.POINTER(ActqInfo)]),
     "psn_act_type_for": (_i32, [_i32]),
     "psn_act_quantize": (_i32, [_vp, _vp, _i32, _vp, _vp, _i64, _i32]),
     "psn_qmatvec": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
     "psn_qmatvec_q8": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
-    "psn_qmatvec_plan": (_i32, [_i32, _i32, _i64, _i64, _i32, _i32, C.POINTER(MatvecPlan)]),
+    "psn_qmatvec_plan": (_i32, [_i32, _i32, _i64, _i64, _i32, _i32, _i32, C.POINTER(MatvecPlan)]),
     "psn_qmatvec_multi": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32]),
     "psn_qmatvec_q8_multi": (_i32, [_vp, _vp, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32]),
     "psn_qmatvec_planned": (_i32, [_vp, _vp, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32, C.POINTER(MatvecPlan)]),

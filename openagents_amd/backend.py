@@ -53,9 +53,9 @@ def actq_layout(act_type: int, k: int, batch: int) -> _ffi.ActqInfo:
     return info
 
 
-def matvec_plan(qtype: int, scheme: int, n: int, k: int, batch: int, compute_units: int = 256) -> MatvecPlan:
+def matvec_plan(qtype: int, scheme: int, n: int, k: int, batch: int, compute_units: int = 256, x_is_f32: bool = False) -> MatvecPlan:
     plan = MatvecPlan()
-    _check(_ffi.load().psn_qmatvec_plan(qtype, scheme, n, k, batch, compute_units, C.byref(plan)))
+    _check(_ffi.load().psn_qmatvec_plan(qtype, scheme, n, k, batch, compute_units, int(x_is_f32), C.byref(plan)))
     return plan
 
 
@@ -162,6 +162,9 @@ class HipBackend:
         h = C.c_void_p()
         _check(self.lib.psn_weight_upload(self.ctx, qtype, n, k, C.c_void_p(b.ctypes.data), LAYOUT_GGUF, self.stream, C.byref(h)))
         return QuantizedTensor(DeviceBuffer._adopt(self, h), qtype, n, k)
+
+    def copy(self, dst: DeviceBuffer, src: DeviceBuffer, nbytes: int, dst_off: int = 0, src_off: int = 0):
+        _check(self.lib.psn_buf_copy(dst.handle, dst_off, src.handle, src_off, nbytes, self.stream))
 
     def sync(self):
         _check(self.lib.psn_stream_sync(self.stream))

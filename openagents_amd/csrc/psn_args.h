@@ -46,6 +46,7 @@ struct psn_matvec_args {
     int32_t batch;        /* live batch columns (<= the kernel's compiled NB) */
     int32_t nseg;
     int64_t row_bytes;
+    uint64_t *timeline;   /* development builds (-DPSN_TIMELINE): per-wave clock stamps; otherwise unused, null */
 };
 
 struct psn_prefill_args {

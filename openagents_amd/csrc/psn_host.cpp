@@ -494,6 +494,18 @@ extern "C" int32_t psn_buf_fill_zero(psn_buf *b, psn_stream *s) {
     return PSN_OK;
 }
 
+extern "C" int32_t psn_buf_copy(psn_buf *dst, size_t dst_off, const psn_buf *src, size_t src_off, size_t n, psn_stream *s) {
+    int32_t rc = check_range(dst, dst_off, n, "psn_buf_copy(dst)");
+    if (rc) return rc;
+    if ((rc = check_range(src, src_off, n, "psn_buf_copy(src)"))) return rc;
+    if (!s) return fail(PSN_E_INVALID_ARG, "psn_buf_copy: stream is null");
+    if (s->ctx != dst->ctx || src->ctx != dst->ctx) return fail(PSN_E_INVALID_ARG, "psn_buf_copy: handles belong to different contexts");
+    if ((rc = bind(dst->ctx))) return rc;
+    if (n == 0) return PSN_OK;
+    HIP_TRY(hipMemcpyAsync((char *)dst->p + dst_off, (const char *)src->p + src_off, n, hipMemcpyDeviceToDevice, s->s));
+    return PSN_OK;
+}
+
 extern "C" int32_t psn_weight_upload(psn_ctx *c, int32_t qtype, int64_t N, int64_t K, const void *blocks, int32_t layout,
                                      psn_stream *s, psn_buf **out) {
     if (!out) return fail(PSN_E_INVALID_ARG, "psn_weight_upload: out is null");
@@ -586,8 +598,7 @@ static int64_t staged_lds_bytes(int32_t qtype, int64_t K, int32_t batch) {
     return qs + d + align_up(sb, 16);
 }
 
-extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, psn_matvec_plan *out) {
-    if (!out) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_plan: out is null");
+static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, bool fuse_quantize, psn_matvec_plan *out) {
     int32_t rc = check_matvec_shape(qtype, scheme, N, K, batch);
     if (rc) return rc;
     if (cus <= 0) cus = 256;
@@ -595,23 +606,40 @@ extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, in
     psn_matvec_plan p;
     p.batch_tile = batch <= 1 ? 1 : batch <= 2 ? 2 : batch <= 4 ? 4 : 8;
     p.rows_in_flight = 1;
-    p.stage_lds = (scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 64 * 1024) ? 1 : 0;
-    /* long rows amortize the activation staging over bigger workgroups */
-    p.threads = K > 8192 ? 512 : 256;
+    const bool lds_fits = scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 64 * 1024;
+    p.stage_lds = lds_fits ? (fuse_quantize ? 2 : 1) : 0;
     /* lanes per row: the row's chunk count rounded up to a power of two, widened (idle lanes, more
-     * waves) while the launch would otherwise leave compute units without a workgroup */
+     * waves) until the launch offers about four waves per compute unit */
     int g = C <= 8 ? 8 : C <= 16 ? 16 : C <= 32 ? 32 : 64;
-    const int64_t wpb = p.threads / 64;
-    while (g < 64 && (N + (64 / g) - 1) / (64 / g) < (int64_t)cus * wpb) g *= 2;
+    while (g < 64 && (N + (64 / g) - 1) / (64 / g) < (int64_t)cus * 4) g *= 2;
+    int64_t waves = (N + (64 / g) - 1) / (64 / g);
+    int64_t blocks;
+    if (p.stage_lds == 2) {
+        /* Every workgroup re-quantizes x while staging it, a cost proportional to K: keep to about
+         * eight waves per compute unit in as few workgroups as stream well (measured on MI355X). */
+        while (g < 64 && waves * 2 <= (int64_t)cus * 8) { g *= 2; waves = (N + (64 / g) - 1) / (64 / g); }
+        const bool small_groups = K <= 8192 && waves >= (int64_t)cus * 16;
+        p.threads = small_groups ? 256 : 512;
+        const int64_t wpb = p.threads / 64;
+        blocks = (waves + wpb - 1) / wpb;
+        const int64_t cap = small_groups ? 2 * (int64_t)cus : (int64_t)cus;
+        if (blocks > cap) blocks = cap;
+    } else {
+        /* small workgroups, one pass per wave where the chip can hold them */
+        p.threads = 256;
+        blocks = (waves + 3) / 4;
+        if (blocks > 4 * (int64_t)cus) blocks = 4 * (int64_t)cus;
+    }
     p.lanes_per_row = g;
-    const int64_t rows_per_wave = (64 / g) * p.rows_in_flight;
-    const int64_t passes = (N + rows_per_wave - 1) / rows_per_wave;
-    int64_t blocks = (passes + wpb - 1) / wpb;
-    const int64_t cap = (int64_t)cus * (p.threads == 256 ? 4 : 2);
-    if (blocks > cap) blocks = cap;
     p.blocks = (int32_t)blocks;
     *out = p;
     return PSN_OK;
+}
+
+extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus,
+                                    int32_t x_is_f32, psn_matvec_plan *out) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_plan: out is null");
+    return make_plan(qtype, scheme, N, K, batch, cus, x_is_f32 != 0 && scheme == PSN_ACT_Q8, out);
 }
 
 static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t scheme, int64_t K, int32_t batch, int max_lds, int32_t *lds_out) {
@@ -620,7 +648,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
     if (p->threads != 256 && p->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
     bool ok;
-    if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2 || r == 4)) || ((nb == 2 || nb == 4) && (r == 1 || r == 2)) || (nb == 8 && r == 1);
+    if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2 || r == 4)) || (nb > 1 && r == 1);
     else ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
     if (!ok) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
@@ -743,7 +771,7 @@ extern "C" int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t 
     if (rc) return rc;
     if ((rc = check_x_q8("psn_qmatvec_q8_multi", qtype, xq, K, batch))) return rc;
     psn_matvec_plan plan;
-    if ((rc = psn_qmatvec_plan(qtype, PSN_ACT_Q8, sg.total, K, batch, mod->ctx->compute_units, &plan))) return rc;
+    if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, batch, mod->ctx->compute_units, false, &plan))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
     return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, xq->p, K, batch, &plan);
 }
@@ -762,14 +790,11 @@ extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qty
     if (rc) return rc;
     if ((rc = check_x_f32("psn_qmatvec", x, K, batch))) return rc;
     psn_matvec_plan plan;
-    if ((rc = psn_qmatvec_plan(qtype, scheme, sg.total, K, batch, mod->ctx->compute_units, &plan))) return rc;
+    if ((rc = make_plan(qtype, scheme, sg.total, K, batch, mod->ctx->compute_units, true, &plan))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
     if (scheme == PSN_ACT_F32) return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
-    if (plan.stage_lds) {
-        /* one launch: every workgroup quantizes x while staging it */
-        plan.stage_lds = 2;
-        return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
-    }
+    /* one launch when the staged copy fits LDS: every workgroup quantizes x while staging it */
+    if (plan.stage_lds == 2) return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
     const int32_t at = psn_act_type_for(qtype);
     psn_actq_info li;
     if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;

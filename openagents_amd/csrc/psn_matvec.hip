@@ -22,6 +22,14 @@
 
 #define UNROLL _Pragma("unroll")
 
+/* build-time experiment switches */
+#ifndef PSN_DOUBLE_BUFFER
+#define PSN_DOUBLE_BUFFER 0
+#endif
+#ifndef PSN_KERNEL_ATTR
+#define PSN_KERNEL_ATTR
+#endif
+
 /* ------------------------------------------------------------------------------------------
  * Activation quantizers (bit-exact restatements of the Q8_0 / Q8_K row quantizers).  The same
  * math runs as stand-alone kernels and inside the matvec's staging step.
@@ -169,92 +177,160 @@ struct ActQ {
     }
 };
 
-template <typename ST>
-PSN_DEV ActQ<ST> act_global(const psn_matvec_args &a) {
-    ActQ<ST> x;
-    x.qs = a.xqs;
-    x.d = a.xd;
-    x.s = reinterpret_cast<const ST *>(a.xs);
-    x.chunk_stride = 256;
-    x.col_stride = a.K;
-    return x;
-}
+/* Brings the activations to where the dot products read them, in two halves so that the weight
+ * loads of the first chunk can be issued in between: issue() starts the (small) activation loads,
+ * finish() waits for them only -- loads return in order, the weights stay in flight -- writes LDS
+ * and crosses the workgroup barrier.
+ *   XSRC 0: quantized activations stay in global memory (no LDS);
+ *   XSRC 1: quantized activations copied into LDS;
+ *   XSRC 2: fp32 activations quantized into LDS by the workgroup itself (every workgroup redoes the
+ *           tiny quantization instead of a separate launch doing it once).
+ * ST = int selects Q8_0 activations (d and s per 32), ST = int16_t Q8_K (d per 256, bsums per 16).
+ * Up to SLOTS 16-byte words per thread are held in registers; larger inputs (long K, batch > 1 on
+ * small workgroups) take the plain copy loop in finish(). */
+template <typename ST, int XSRC>
+struct Stager {
+    static constexpr int SLOTS = 8;
+    uint4 t[SLOTS];
+    uint4 td, ts;
+    int n_qs, n_d, n_s, C;
+    bool in_regs;
 
-/* d_per_col floats and s_per_col ST values per batch column */
-template <typename ST>
-PSN_DEV ActQ<ST> act_stage_lds(const psn_matvec_args &a, int d_per_col, int s_per_col) {
-    extern __shared__ uint4 psn_smem[];
-    const int C = a.K >> 8;
-    const int n_qs = a.batch * C * 16;                       /* source words */
-    const int n_d = (a.batch * d_per_col * 4 + 15) / 16;     /* the global fields are padded to 256 B */
-    const int n_s = (a.batch * s_per_col * (int)sizeof(ST) + 15) / 16;
-    uint4 *l_qs = psn_smem, *l_d = l_qs + a.batch * C * 17, *l_s = l_d + n_d;
-    const uint4 *g_qs = reinterpret_cast<const uint4 *>(a.xqs), *g_d = reinterpret_cast<const uint4 *>(a.xd);
-    const uint4 *g_s = reinterpret_cast<const uint4 *>(a.xs);
-    for (int i = threadIdx.x; i < n_qs; i += blockDim.x) l_qs[(i >> 4) * 17 + (i & 15)] = g_qs[i];
-    for (int i = threadIdx.x; i < n_d; i += blockDim.x) l_d[i] = g_d[i];
-    for (int i = threadIdx.x; i < n_s; i += blockDim.x) l_s[i] = g_s[i];
-    __syncthreads();
-    ActQ<ST> x;
-    x.qs = reinterpret_cast<const int8_t *>(l_qs);
-    x.d = reinterpret_cast<const float *>(l_d);
-    x.s = reinterpret_cast<const ST *>(l_s);
-    x.chunk_stride = 272;
-    x.col_stride = C * 272;
-    return x;
-}
-
-/* Same LDS layout, but filled by quantizing the fp32 activations on the way in: every workgroup
- * redoes the (tiny) quantization instead of a separate launch doing it once.  ST = int selects
- * Q8_0 activations, ST = int16_t selects Q8_K. */
-template <typename ST>
-PSN_DEV ActQ<ST> act_stage_quantize(const psn_matvec_args &a, int d_per_col, int s_per_col) {
-    extern __shared__ uint4 psn_smem[];
-    const int C = a.K >> 8;
-    const int n_d = (a.batch * d_per_col * 4 + 15) / 16;
-    uint4 *l_qs4 = psn_smem, *l_d4 = l_qs4 + a.batch * C * 17, *l_s4 = l_d4 + n_d;
-    u32 *l_qs = reinterpret_cast<u32 *>(l_qs4);
-    float *l_d = reinterpret_cast<float *>(l_d4);
-    ST *l_s = reinterpret_cast<ST *>(l_s4);
-    const float4 *x4 = reinterpret_cast<const float4 *>(a.xf);
-    const int lane = threadIdx.x & 63;
-    if constexpr (sizeof(ST) == 4) {
-        const int total4 = a.batch * C * 64;                  /* float4 words; a multiple of 64, so waves stay whole */
-        for (int i = threadIdx.x; i < total4; i += blockDim.x) {
-            u32 packed;
-            float d;
-            int sum;
-            q8_0_quant4(x4[i], packed, d, sum);
-            l_qs[(i >> 6) * 68 + (i & 63)] = packed;          /* chunk index i/64 already runs over batch */
-            if ((lane & 7) == 0) { l_d[i >> 3] = d; l_s[i >> 3] = sum; }
-        }
-    } else {
-        const int nsb = a.batch * C;
-        for (int sb = threadIdx.x >> 6; sb < nsb; sb += blockDim.x >> 6) {
-            u32 packed;
-            float d;
-            int s16;
-            q8_K_quant_wave(x4[sb * 64 + lane], lane, packed, d, s16);
-            l_qs[sb * 68 + lane] = packed;
-            if ((lane & 3) == 0) l_s[sb * 16 + (lane >> 2)] = (ST)s16;
-            if (lane == 0) l_d[sb] = d;
+    PSN_DEV void issue(const psn_matvec_args &a, int d_per_col, int s_per_col) {
+        C = a.K >> 8;
+        n_qs = a.batch * C * 16;                                   /* 16-byte words of int8 */
+        n_d = (a.batch * d_per_col * 4 + 15) / 16;                 /* the global fields are padded to 256 B */
+        n_s = (a.batch * s_per_col * (int)sizeof(ST) + 15) / 16;
+        in_regs = false;
+        UNROLL for (int i = 0; i < SLOTS; ++i) t[i] = make_uint4(0, 0, 0, 0);
+        td = ts = make_uint4(0, 0, 0, 0);
+        if constexpr (XSRC == 1) {
+            in_regs = n_qs <= SLOTS * (int)blockDim.x && n_d <= (int)blockDim.x && n_s <= (int)blockDim.x;
+            if (in_regs) {
+                const uint4 *g_qs = reinterpret_cast<const uint4 *>(a.xqs);
+                UNROLL for (int i = 0; i < SLOTS; ++i) {
+                    const int idx = threadIdx.x + i * blockDim.x;
+                    if (idx < n_qs) t[i] = g_qs[idx];
+                }
+                if ((int)threadIdx.x < n_d) td = reinterpret_cast<const uint4 *>(a.xd)[threadIdx.x];
+                if ((int)threadIdx.x < n_s) ts = reinterpret_cast<const uint4 *>(a.xs)[threadIdx.x];
+            }
+        } else if constexpr (XSRC == 2) {
+            const float4 *x4 = reinterpret_cast<const float4 *>(a.xf);
+            if constexpr (sizeof(ST) == 4) {
+                const int total4 = a.batch * C * 64;               /* float4 words: whole waves, whole blocks */
+                in_regs = total4 <= SLOTS * (int)blockDim.x;
+                if (in_regs) {
+                    UNROLL for (int i = 0; i < SLOTS; ++i) {
+                        const int idx = threadIdx.x + i * blockDim.x;
+                        if (idx < total4) { const float4 v = x4[idx]; t[i] = make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)); }
+                    }
+                }
+            } else {
+                const int nsb = a.batch * C, wpb = blockDim.x >> 6, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+                in_regs = nsb <= SLOTS * wpb;
+                if (in_regs) {
+                    UNROLL for (int i = 0; i < SLOTS; ++i) {
+                        const int sb = wid + i * wpb;
+                        if (sb < nsb) { const float4 v = x4[sb * 64 + lane]; t[i] = make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)); }
+                    }
+                }
+            }
         }
     }
-    __syncthreads();
-    ActQ<ST> x;
-    x.qs = reinterpret_cast<const int8_t *>(l_qs4);
-    x.d = l_d;
-    x.s = l_s;
-    x.chunk_stride = 272;
-    x.col_stride = C * 272;
-    return x;
-}
+
+    PSN_DEV ActQ<ST> finish(const psn_matvec_args &a) {
+        ActQ<ST> x;
+        if constexpr (XSRC == 0) {
+            x.qs = a.xqs;
+            x.d = a.xd;
+            x.s = reinterpret_cast<const ST *>(a.xs);
+            x.chunk_stride = 256;
+            x.col_stride = a.K;
+            return x;
+        } else {
+            extern __shared__ uint4 psn_smem[];
+            uint4 *l_qs4 = psn_smem, *l_d4 = l_qs4 + a.batch * C * 17, *l_s4 = l_d4 + n_d;
+            if constexpr (XSRC == 1) {
+                const uint4 *g_qs = reinterpret_cast<const uint4 *>(a.xqs), *g_d = reinterpret_cast<const uint4 *>(a.xd);
+                const uint4 *g_s = reinterpret_cast<const uint4 *>(a.xs);
+                if (in_regs) {
+                    UNROLL for (int i = 0; i < SLOTS; ++i) {
+                        const int idx = threadIdx.x + i * blockDim.x;
+                        if (idx < n_qs) l_qs4[(idx >> 4) * 17 + (idx & 15)] = t[i];
+                    }
+                    if ((int)threadIdx.x < n_d) l_d4[threadIdx.x] = td;
+                    if ((int)threadIdx.x < n_s) l_s4[threadIdx.x] = ts;
+                } else {
+                    for (int i = threadIdx.x; i < n_qs; i += blockDim.x) l_qs4[(i >> 4) * 17 + (i & 15)] = g_qs[i];
+                    for (int i = threadIdx.x; i < n_d; i += blockDim.x) l_d4[i] = g_d[i];
+                    for (int i = threadIdx.x; i < n_s; i += blockDim.x) l_s4[i] = g_s[i];
+                }
+            } else {
+                u32 *l_qs = reinterpret_cast<u32 *>(l_qs4);
+                float *l_d = reinterpret_cast<float *>(l_d4);
+                ST *l_s = reinterpret_cast<ST *>(l_s4);
+                const float4 *x4 = reinterpret_cast<const float4 *>(a.xf);
+                const int lane = threadIdx.x & 63;
+                if constexpr (sizeof(ST) == 4) {
+                    const int total4 = a.batch * C * 64;
+                    auto one = [&](int i, const float4 v) {
+                        u32 packed;
+                        float d;
+                        int sum;
+                        q8_0_quant4(v, packed, d, sum);
+                        l_qs[(i >> 6) * 68 + (i & 63)] = packed;      /* chunk index i/64 already runs over batch */
+                        if ((lane & 7) == 0) { l_d[i >> 3] = d; l_s[i >> 3] = sum; }
+                    };
+                    if (in_regs) {
+                        UNROLL for (int k = 0; k < SLOTS; ++k) {
+                            const int i = threadIdx.x + k * blockDim.x;
+                            if (i < total4) one(i, make_float4(__uint_as_float(t[k].x), __uint_as_float(t[k].y), __uint_as_float(t[k].z), __uint_as_float(t[k].w)));
+                        }
+                    } else {
+                        for (int i = threadIdx.x; i < total4; i += blockDim.x) one(i, x4[i]);
+                    }
+                } else {
+                    const int nsb = a.batch * C, wpb = blockDim.x >> 6, wid = threadIdx.x >> 6;
+                    auto one = [&](int sb, const float4 v) {
+                        u32 packed;
+                        float d;
+                        int s16;
+                        q8_K_quant_wave(v, lane, packed, d, s16);
+                        l_qs[sb * 68 + lane] = packed;
+                        if ((lane & 3) == 0) l_s[sb * 16 + (lane >> 2)] = (ST)s16;
+                        if (lane == 0) l_d[sb] = d;
+                    };
+                    if (in_regs) {
+                        UNROLL for (int k = 0; k < SLOTS; ++k) {
+                            const int sb = wid + k * wpb;
+                            if (sb < nsb) one(sb, make_float4(__uint_as_float(t[k].x), __uint_as_float(t[k].y), __uint_as_float(t[k].z), __uint_as_float(t[k].w)));
+                        }
+                    } else {
+                        for (int sb = wid; sb < nsb; sb += wpb) one(sb, x4[sb * 64 + lane]);
+                    }
+                }
+            }
+            __syncthreads();
+            x.qs = reinterpret_cast<const int8_t *>(l_qs4);
+            x.d = reinterpret_cast<const float *>(l_d4);
+            x.s = reinterpret_cast<const ST *>(l_s4);
+            x.chunk_stride = 272;
+            x.col_stride = C * 272;
+            return x;
+        }
+    }
+};
 
 /* ------------------------------------------------------------------------------------------
- * Q4_0 x Q8_0-activations.  Chunk = 8 blocks = 144 B = 36 dwords.
- * Block b of the chunk starts at byte 18b: even blocks start on a dword (fp16 d in the low half,
- * quants shifted by two bytes), odd blocks start mid-dword (d in the high half, quants aligned).
- * sum (q-8)*x = sum q*x - 8*sum x uses the activation block sums so nibbles stay unsigned.
+ * Formats.  Each supplies: DW/BYTES (a lane's 256-weight chunk), load() of the chunk's dwords,
+ * XR + load_x() (the matching 256 activations with their scales, as registers) and dot()
+ * (the chunk's contribution to the row's sum); deq32() serves the F32 scheme.
+ *
+ * Q4_0: chunk = 8 blocks = 144 B = 36 dwords.  Block b starts at byte 18b: even blocks start on
+ * a dword (fp16 d in the low half, quants shifted by two bytes), odd blocks start mid-dword (d in
+ * the high half, quants aligned).  sum (q-8)*x = sum q*x - 8*sum x uses the activation block sums
+ * so nibbles stay unsigned.
  * ------------------------------------------------------------------------------------------ */
 
 template <int B>
@@ -283,8 +359,31 @@ PSN_DEV void q8_0_block(const u32 (&w)[68], float &d, u32 (&q)[8]) {
     }
 }
 
+/* activations of one chunk for the 32-element-block formats: 64 dwords of int8, 8 scales, 8 sums */
+PSN_DEV void load_x_q8_0(const ActQ<int> &x, int K, int col, int c, u32 (&xr)[80]) {
+    const uint4 *xp = x.chunk(col, c);
+    UNROLL for (int i = 0; i < 16; ++i) unpack4(xp[i], &xr[4 * i]);
+    const int nblk = K >> 5;
+    const uint4 *dp = reinterpret_cast<const uint4 *>(x.d + col * nblk + c * 8);
+    const uint4 *sp = reinterpret_cast<const uint4 *>(x.s + col * nblk + c * 8);
+    unpack4(dp[0], &xr[64]);
+    unpack4(dp[1], &xr[68]);
+    unpack4(sp[0], &xr[72]);
+    unpack4(sp[1], &xr[76]);
+}
+/* ... and for the super-block formats: 64 dwords of int8, one scale, 16 int16 group sums */
+PSN_DEV void load_x_q8_K(const ActQ<int16_t> &x, int K, int col, int c, u32 (&xr)[73]) {
+    const int C = K >> 8;
+    const uint4 *xp = x.chunk(col, c);
+    UNROLL for (int i = 0; i < 16; ++i) unpack4(xp[i], &xr[4 * i]);
+    xr[64] = __float_as_uint(x.d[col * C + c]);
+    const uint4 *bp = reinterpret_cast<const uint4 *>(x.s + ((int64_t)col * C + c) * 16);
+    unpack4(bp[0], &xr[65]);
+    unpack4(bp[1], &xr[69]);
+}
+
 struct FmtQ4_0 {
-    static constexpr int DW = 36, BYTES = 144;
+    static constexpr int DW = 36, BYTES = 144, XR = 80;
     typedef int ActSum;
     static PSN_DEV int d_per_col(int K) { return K >> 5; }
     static PSN_DEV int s_per_col(int K) { return K >> 5; }
@@ -292,38 +391,23 @@ struct FmtQ4_0 {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
     }
-    template <int B, int R, int NB>
-    static PSN_DEV void step(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
-        float dw[R];
-        u32 lo[R][4], hi[R][4];
-        UNROLL for (int r = 0; r < R; ++r) q4_0_block<B>(w[r], dw[r], lo[r], hi[r]);
-        const int nblk = K >> 5;
-        UNROLL for (int nb = 0; nb < NB; ++nb) {
-            const int col = nb < batch ? nb : batch - 1;
-            const uint4 *xp = x.chunk(col, c) + 2 * B;
-            const uint4 x0 = xp[0], x1 = xp[1];
-            const float dx = x.d[col * nblk + c * 8 + B];
-            const int sx = x.s[col * nblk + c * 8 + B];
-            UNROLL for (int r = 0; r < R; ++r) {
-                int s = dot4(lo[r][0], x0.x, 0);
-                s = dot4(lo[r][1], x0.y, s);
-                s = dot4(lo[r][2], x0.z, s);
-                s = dot4(lo[r][3], x0.w, s);
-                s = dot4(hi[r][0], x1.x, s);
-                s = dot4(hi[r][1], x1.y, s);
-                s = dot4(hi[r][2], x1.z, s);
-                s = dot4(hi[r][3], x1.w, s);
-                s -= 8 * sx;
-                acc[r][nb] += (float)s * dw[r] * dx;
-            }
-        }
+    static PSN_DEV void load_x(const ActQ<int> &x, int K, int col, int c, u32 (&xr)[XR]) { load_x_q8_0(x, K, col, c, xr); }
+    template <int B>
+    static PSN_DEV float block(const u32 (&w)[DW], const u32 (&xr)[XR]) {
+        float dw;
+        u32 lo[4], hi[4];
+        q4_0_block<B>(w, dw, lo, hi);
+        int s = 0;
+        UNROLL for (int i = 0; i < 4; ++i) s = dot4(lo[i], xr[8 * B + i], s);
+        UNROLL for (int i = 0; i < 4; ++i) s = dot4(hi[i], xr[8 * B + 4 + i], s);
+        s -= 8 * (int)xr[72 + B];
+        return (float)s * dw * __uint_as_float(xr[64 + B]);
     }
-    template <int R, int NB>
-    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
-        step<0>(w, x, K, c, batch, acc); step<1>(w, x, K, c, batch, acc);
-        step<2>(w, x, K, c, batch, acc); step<3>(w, x, K, c, batch, acc);
-        step<4>(w, x, K, c, batch, acc); step<5>(w, x, K, c, batch, acc);
-        step<6>(w, x, K, c, batch, acc); step<7>(w, x, K, c, batch, acc);
+    static PSN_DEV float dot(const u32 (&w)[DW], const u32 (&xr)[XR]) {
+        float acc = block<0>(w, xr);
+        acc += block<1>(w, xr); acc += block<2>(w, xr); acc += block<3>(w, xr);
+        acc += block<4>(w, xr); acc += block<5>(w, xr); acc += block<6>(w, xr); acc += block<7>(w, xr);
+        return acc;
     }
     /* 32 weights of GGUF block SB of the chunk, fp32, element order (scheme F32) */
     template <int SB>
@@ -339,12 +423,9 @@ struct FmtQ4_0 {
     }
 };
 
-/* ------------------------------------------------------------------------------------------
- * Q8_0 x Q8_0-activations.  Chunk = 8 blocks = 272 B = 68 dwords; block b starts at byte 34b.
- * ------------------------------------------------------------------------------------------ */
-
+/* Q8_0: chunk = 8 blocks = 272 B = 68 dwords; block b starts at byte 34b. */
 struct FmtQ8_0 {
-    static constexpr int DW = 68, BYTES = 272;
+    static constexpr int DW = 68, BYTES = 272, XR = 80;
     typedef int ActSum;
     static PSN_DEV int d_per_col(int K) { return K >> 5; }
     static PSN_DEV int s_per_col(int K) { return K >> 5; }
@@ -352,36 +433,21 @@ struct FmtQ8_0 {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 17; ++i) unpack4(q[i], &w[4 * i]);
     }
-    template <int B, int R, int NB>
-    static PSN_DEV void step(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
-        float dw[R];
-        u32 q[R][8];
-        UNROLL for (int r = 0; r < R; ++r) q8_0_block<B>(w[r], dw[r], q[r]);
-        const int nblk = K >> 5;
-        UNROLL for (int nb = 0; nb < NB; ++nb) {
-            const int col = nb < batch ? nb : batch - 1;
-            const uint4 *xp = x.chunk(col, c) + 2 * B;
-            const uint4 x0 = xp[0], x1 = xp[1];
-            const float dx = x.d[col * nblk + c * 8 + B];
-            UNROLL for (int r = 0; r < R; ++r) {
-                int s = dot4(q[r][0], x0.x, 0);
-                s = dot4(q[r][1], x0.y, s);
-                s = dot4(q[r][2], x0.z, s);
-                s = dot4(q[r][3], x0.w, s);
-                s = dot4(q[r][4], x1.x, s);
-                s = dot4(q[r][5], x1.y, s);
-                s = dot4(q[r][6], x1.z, s);
-                s = dot4(q[r][7], x1.w, s);
-                acc[r][nb] += (float)s * (dw[r] * dx);
-            }
-        }
+    static PSN_DEV void load_x(const ActQ<int> &x, int K, int col, int c, u32 (&xr)[XR]) { load_x_q8_0(x, K, col, c, xr); }
+    template <int B>
+    static PSN_DEV float block(const u32 (&w)[DW], const u32 (&xr)[XR]) {
+        float dw;
+        u32 q[8];
+        q8_0_block<B>(w, dw, q);
+        int s = 0;
+        UNROLL for (int i = 0; i < 8; ++i) s = dot4(q[i], xr[8 * B + i], s);
+        return (float)s * (dw * __uint_as_float(xr[64 + B]));
     }
-    template <int R, int NB>
-    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int> &x, int K, int c, int batch, float (&acc)[R][NB]) {
-        step<0>(w, x, K, c, batch, acc); step<1>(w, x, K, c, batch, acc);
-        step<2>(w, x, K, c, batch, acc); step<3>(w, x, K, c, batch, acc);
-        step<4>(w, x, K, c, batch, acc); step<5>(w, x, K, c, batch, acc);
-        step<6>(w, x, K, c, batch, acc); step<7>(w, x, K, c, batch, acc);
+    static PSN_DEV float dot(const u32 (&w)[DW], const u32 (&xr)[XR]) {
+        float acc = block<0>(w, xr);
+        acc += block<1>(w, xr); acc += block<2>(w, xr); acc += block<3>(w, xr);
+        acc += block<4>(w, xr); acc += block<5>(w, xr); acc += block<6>(w, xr); acc += block<7>(w, xr);
+        return acc;
     }
     template <int SB>
     static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
@@ -393,11 +459,9 @@ struct FmtQ8_0 {
     }
 };
 
-/* ------------------------------------------------------------------------------------------
- * Q4_K x Q8_K-activations.  Chunk = one 144-byte super-block: dword 0 = d | dmin<<16,
- * dwords 1..3 = the 12-byte 6-bit scale/min field, dwords 4..35 = 128 nibble bytes.
- * ------------------------------------------------------------------------------------------ */
-
+/* Q4_K: chunk = one 144-byte super-block: dword 0 = d | dmin<<16, dwords 1..3 = the 12-byte
+ * 6-bit scale/min field, dwords 4..35 = 128 nibble bytes (64 weights per 32 bytes: low nibbles
+ * then high nibbles). */
 PSN_DEV void q4_K_scales(u32 s0, u32 s1, u32 s2, u32 (&sc)[2], u32 (&mn)[2]) {
     sc[0] = s0 & 0x3f3f3f3fu;
     mn[0] = s1 & 0x3f3f3f3fu;
@@ -407,7 +471,7 @@ PSN_DEV void q4_K_scales(u32 s0, u32 s1, u32 s2, u32 (&sc)[2], u32 (&mn)[2]) {
 PSN_DEV int byte_of(const u32 (&v)[2], int i) { return (int)((v[i >> 2] >> (8 * (i & 3))) & 0xffu); }
 
 struct FmtQ4_K {
-    static constexpr int DW = 36, BYTES = 144;
+    static constexpr int DW = 36, BYTES = 144, XR = 73;
     typedef int16_t ActSum;
     static PSN_DEV int d_per_col(int K) { return K >> 8; }
     static PSN_DEV int s_per_col(int K) { return K >> 4; }
@@ -415,49 +479,28 @@ struct FmtQ4_K {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
     }
-    template <int R, int NB>
-    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int16_t> &x, int K, int c, int batch, float (&acc)[R][NB]) {
-        const int C = K >> 8;
-        u32 sc[R][2], mn[R][2];
-        UNROLL for (int r = 0; r < R; ++r) q4_K_scales(w[r][1], w[r][2], w[r][3], sc[r], mn[r]);
-        UNROLL for (int nb = 0; nb < NB; ++nb) {
-            const int col = nb < batch ? nb : batch - 1;
-            const float dx = x.d[col * C + c];
-            /* sums of the activation over the eight 32-element sub-blocks */
-            const uint4 *bp = reinterpret_cast<const uint4 *>(x.s + ((int64_t)col * C + c) * 16);
-            u32 bs[8];
-            unpack4(bp[0], &bs[0]);
-            unpack4(bp[1], &bs[4]);
-            int bsum[8];
-            UNROLL for (int i = 0; i < 8; ++i) bsum[i] = (int)(int16_t)(bs[i] & 0xffffu) + ((int)bs[i] >> 16);
-            int isum[R], msum[R];
-            UNROLL for (int r = 0; r < R; ++r) {
-                isum[r] = 0;
-                msum[r] = 0;
-                UNROLL for (int i = 0; i < 8; ++i) msum[r] += byte_of(mn[r], i) * bsum[i];
-            }
-            const uint4 *xp = x.chunk(col, c);
-            UNROLL for (int ch = 0; ch < 4; ++ch) {         /* 64 weights: low nibbles then high nibbles */
-                u32 xl[8], xh[8];
-                unpack4(xp[4 * ch + 0], &xl[0]);
-                unpack4(xp[4 * ch + 1], &xl[4]);
-                unpack4(xp[4 * ch + 2], &xh[0]);
-                unpack4(xp[4 * ch + 3], &xh[4]);
-                UNROLL for (int r = 0; r < R; ++r) {
-                    int sl = 0, sh = 0;
-                    UNROLL for (int i = 0; i < 8; ++i) {
-                        const u32 q = w[r][4 + 8 * ch + i];
-                        sl = dot4(q & 0x0f0f0f0fu, xl[i], sl);
-                        sh = dot4((q >> 4) & 0x0f0f0f0fu, xh[i], sh);
-                    }
-                    isum[r] += byte_of(sc[r], 2 * ch) * sl + byte_of(sc[r], 2 * ch + 1) * sh;
-                }
-            }
-            UNROLL for (int r = 0; r < R; ++r) {
-                const float d = h2f_lo(w[r][0]) * dx, dm = h2f_hi(w[r][0]) * dx;
-                acc[r][nb] += d * (float)isum[r] - dm * (float)msum[r];
-            }
+    static PSN_DEV void load_x(const ActQ<int16_t> &x, int K, int col, int c, u32 (&xr)[XR]) { load_x_q8_K(x, K, col, c, xr); }
+    static PSN_DEV float dot(const u32 (&w)[DW], const u32 (&xr)[XR]) {
+        u32 sc[2], mn[2];
+        q4_K_scales(w[1], w[2], w[3], sc, mn);
+        int isum = 0, msum = 0;
+        /* the eight 32-element sub-block sums of the activation are pairs of 16-element group sums */
+        UNROLL for (int i = 0; i < 8; ++i) {
+            const u32 b = xr[65 + i];
+            msum += byte_of(mn, i) * ((int)(int16_t)(b & 0xffffu) + ((int)b >> 16));
         }
+        UNROLL for (int ch = 0; ch < 4; ++ch) {
+            int sl = 0, sh = 0;
+            UNROLL for (int i = 0; i < 8; ++i) {
+                const u32 q = w[4 + 8 * ch + i];
+                sl = dot4(q & 0x0f0f0f0fu, xr[16 * ch + i], sl);
+                sh = dot4((q >> 4) & 0x0f0f0f0fu, xr[16 * ch + 8 + i], sh);
+            }
+            isum += byte_of(sc, 2 * ch) * sl + byte_of(sc, 2 * ch + 1) * sh;
+        }
+        const float dx = __uint_as_float(xr[64]);
+        const float d = h2f_lo(w[0]) * dx, dm = h2f_hi(w[0]) * dx;
+        return d * (float)isum - dm * (float)msum;
     }
     template <int SB>
     static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
@@ -471,16 +514,13 @@ struct FmtQ4_K {
     }
 };
 
-/* ------------------------------------------------------------------------------------------
- * Q6_K x Q8_K-activations.  Chunk = one 210-byte super-block at a 2-byte-aligned address:
- * ql[128] | qh[64] | int8 scales[16] | fp16 d.  13 dwordx4 loads cover bytes 0..207.
- * sum (q-32)*x = sum q*x - 32*bsum per 16-element group keeps the 6-bit values unsigned.
- * ------------------------------------------------------------------------------------------ */
-
+/* Q6_K: chunk = one 210-byte super-block at a 2-byte-aligned address: ql[128] | qh[64] |
+ * int8 scales[16] | fp16 d.  13 dwordx4 loads cover bytes 0..207.  sum (q-32)*x =
+ * sum q*x - 32*bsum per 16-element group keeps the 6-bit values unsigned. */
 struct __attribute__((packed, aligned(2))) u4_a2 { u32 x, y, z, w; };
 
 struct FmtQ6_K {
-    static constexpr int DW = 53, BYTES = 210;
+    static constexpr int DW = 53, BYTES = 210, XR = 73;
     typedef int16_t ActSum;
     static PSN_DEV int d_per_col(int K) { return K >> 8; }
     static PSN_DEV int s_per_col(int K) { return K >> 4; }
@@ -492,49 +532,34 @@ struct FmtQ6_K {
         }
         w[52] = *reinterpret_cast<const unsigned short *>(p + 208);
     }
-    template <int R, int NB>
-    static PSN_DEV void compute(const u32 (&w)[R][DW], const ActQ<int16_t> &x, int K, int c, int batch, float (&acc)[R][NB]) {
-        const int C = K >> 8;
-        UNROLL for (int nb = 0; nb < NB; ++nb) {
-            const int col = nb < batch ? nb : batch - 1;
-            const float dx = x.d[col * C + c];
-            const uint4 *bp = reinterpret_cast<const uint4 *>(x.s + ((int64_t)col * C + c) * 16);
-            u32 bs[8];
-            unpack4(bp[0], &bs[0]);
-            unpack4(bp[1], &bs[4]);
-            const uint4 *xp = x.chunk(col, c);
-            int isum[R];
-            UNROLL for (int r = 0; r < R; ++r) isum[r] = 0;
-            UNROLL for (int h = 0; h < 2; ++h) {
-                u32 xq[32];                                   /* 128 activations of this half */
-                UNROLL for (int i = 0; i < 8; ++i) unpack4(xp[8 * h + i], &xq[4 * i]);
-                UNROLL for (int r = 0; r < R; ++r) {
-                    int part[8];
-                    UNROLL for (int g = 0; g < 8; ++g) part[g] = 0;
-                    UNROLL for (int i = 0; i < 8; ++i) {      /* dword i holds l = 4i..4i+3 */
-                        const u32 A = w[r][16 * h + i], B = w[r][16 * h + 8 + i], H = w[r][32 + 8 * h + i];
-                        const u32 q1 = (A & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
-                        const u32 q2 = (B & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
-                        const u32 q3 = ((A >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u);
-                        const u32 q4 = ((B >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u);
-                        const int is = i >> 2;
-                        part[is + 0] = dot4(q1, xq[i], part[is + 0]);
-                        part[is + 2] = dot4(q2, xq[8 + i], part[is + 2]);
-                        part[is + 4] = dot4(q3, xq[16 + i], part[is + 4]);
-                        part[is + 6] = dot4(q4, xq[24 + i], part[is + 6]);
-                    }
-                    UNROLL for (int g = 0; g < 8; ++g) {
-                        const int gi = 8 * h + g;             /* 16-element group of the super-block */
-                        const u32 sw = w[r][48 + (gi >> 2)];
-                        const int scale = (int)(int8_t)((sw >> (8 * (gi & 3))) & 0xffu);
-                        const u32 bw = bs[gi >> 1];
-                        const int bsum = (gi & 1) ? ((int)bw >> 16) : (int)(int16_t)(bw & 0xffffu);
-                        isum[r] += scale * (part[g] - 32 * bsum);
-                    }
-                }
+    static PSN_DEV void load_x(const ActQ<int16_t> &x, int K, int col, int c, u32 (&xr)[XR]) { load_x_q8_K(x, K, col, c, xr); }
+    static PSN_DEV float dot(const u32 (&w)[DW], const u32 (&xr)[XR]) {
+        int isum = 0;
+        UNROLL for (int h = 0; h < 2; ++h) {
+            int part[8];
+            UNROLL for (int g = 0; g < 8; ++g) part[g] = 0;
+            UNROLL for (int i = 0; i < 8; ++i) {      /* dword i holds l = 4i..4i+3 */
+                const u32 A = w[16 * h + i], B = w[16 * h + 8 + i], H = w[32 + 8 * h + i];
+                const u32 q1 = (A & 0x0f0f0f0fu) | ((H << 4) & 0x30303030u);
+                const u32 q2 = (B & 0x0f0f0f0fu) | ((H << 2) & 0x30303030u);
+                const u32 q3 = ((A >> 4) & 0x0f0f0f0fu) | (H & 0x30303030u);
+                const u32 q4 = ((B >> 4) & 0x0f0f0f0fu) | ((H >> 2) & 0x30303030u);
+                const int is = i >> 2;
+                part[is + 0] = dot4(q1, xr[32 * h + i], part[is + 0]);
+                part[is + 2] = dot4(q2, xr[32 * h + 8 + i], part[is + 2]);
+                part[is + 4] = dot4(q3, xr[32 * h + 16 + i], part[is + 4]);
+                part[is + 6] = dot4(q4, xr[32 * h + 24 + i], part[is + 6]);
             }
-            UNROLL for (int r = 0; r < R; ++r) acc[r][nb] += h2f_lo(w[r][52]) * dx * (float)isum[r];
+            UNROLL for (int g = 0; g < 8; ++g) {
+                const int gi = 8 * h + g;             /* 16-element group of the super-block */
+                const u32 sw = w[48 + (gi >> 2)];
+                const int scale = (int)(int8_t)((sw >> (8 * (gi & 3))) & 0xffu);
+                const u32 bw = xr[65 + (gi >> 1)];
+                const int bsum = (gi & 1) ? ((int)bw >> 16) : (int)(int16_t)(bw & 0xffffu);
+                isum += scale * (part[g] - 32 * bsum);
+            }
         }
+        return h2f_lo(w[52]) * __uint_as_float(xr[64]) * (float)isum;
     }
     template <int SB>
     static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
@@ -556,6 +581,17 @@ struct FmtQ6_K {
  * Drivers.
  * ------------------------------------------------------------------------------------------ */
 
+/* Development aid: with -DPSN_TIMELINE lane 0 of every wave records the 100 MHz steady clock at five
+ * points of the kernel (8 slots per wave).  Compiled out of the shipped code objects. */
+#ifdef PSN_TIMELINE
+#define PSN_STAMP(a, m, slot)                                                                     \
+    do {                                                                                          \
+        if ((a).timeline && (m).lane == 0) (a).timeline[(int64_t)(m).wave * 8 + (slot)] = __builtin_readsteadycounter(); \
+    } while (0)
+#else
+#define PSN_STAMP(a, m, slot) do { } while (0)
+#endif
+
 template <typename F, int G, int R>
 PSN_DEV void load_rows(const psn_matvec_args &a, const RowMap<G, R> &m, int row0, int c, u32 (&w)[R][F::DW]) {
     UNROLL for (int r = 0; r < R; ++r) {
@@ -564,33 +600,77 @@ PSN_DEV void load_rows(const psn_matvec_args &a, const RowMap<G, R> &m, int row0
     }
 }
 
-/* Scheme Q8.  The first chunk's weight loads are issued before the activations are staged, so
- * the staging (an L2 round trip plus a barrier) hides under the HBM latency of the weights. */
-/* XSRC: 0 = quantized activations read from global memory, 1 = staged into LDS,
- * 2 = fp32 activations quantized into LDS by the workgroup itself. */
+/* Scheme Q8.  A wave walks its work as (row set, chunk iteration) items.  Order of events: the
+ * small activation loads are issued, then the first item's weight loads, then the activations are
+ * staged (waiting only for their own loads) while the weights are still in flight.  With one row
+ * set and one batch column per lane (R = NB = 1) the weights are double-buffered: the next item's
+ * loads are issued before the current item is consumed, and the lane's activation chunk stays in
+ * registers for as long as the chunk index does not change. */
 template <typename F, int G, int R, int NB, int XSRC>
 PSN_DEV void mv_q8(const psn_matvec_args &a) {
     typedef typename F::ActSum ST;
+    constexpr bool DB = PSN_DOUBLE_BUFFER && (R == 1 && NB == 1);
     const RowMap<G, R> m;
-    const int K = a.K, C = K >> 8;
-    const int stride = m.nwaves * m.ROWS;
-    int row0 = m.wave * m.ROWS;
-    u32 w[R][F::DW];
-    bool pre = row0 < a.N && m.j < C;
-    if (pre) load_rows<F, G, R>(a, m, row0, m.j, w);
-    const ActQ<ST> x = XSRC == 2   ? act_stage_quantize<ST>(a, F::d_per_col(K), F::s_per_col(K))
-                       : XSRC == 1 ? act_stage_lds<ST>(a, F::d_per_col(K), F::s_per_col(K))
-                                   : act_global<ST>(a);
-    for (; row0 < a.N; row0 += stride) {
-        float acc[R][NB];
-        UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
-        for (int c = m.j; c < C; c += G) {
-            if (!pre) load_rows<F, G, R>(a, m, row0, c, w);
-            pre = false;
-            F::template compute<R, NB>(w, x, K, c, a.batch, acc);
+    const int K = a.K, C = K >> 8, iters = (C + G - 1) / G, stride = m.nwaves * m.ROWS;
+    int row0 = m.wave * m.ROWS, it = 0;
+    PSN_STAMP(a, m, 0);
+    Stager<ST, XSRC> st;
+    st.issue(a, F::d_per_col(K), F::s_per_col(K));
+    u32 wa[R][F::DW], wb[DB ? R : 1][DB ? F::DW : 1];
+    load_rows<F, G, R>(a, m, min(row0, a.N - 1), min(m.j, C - 1), wa);
+    PSN_STAMP(a, m, 1);
+    const ActQ<ST> x = st.finish(a);
+    PSN_STAMP(a, m, 2);
+    u32 xr[F::XR];
+    int xc = -1;
+    float acc[R][NB];
+    UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+
+    auto advance = [&](int &r0, int &i) {
+        if (++i == iters) { i = 0; r0 += stride; }
+    };
+    auto consume = [&](const u32 (&w)[R][F::DW], int r0, int i) {
+        const int c = m.j + i * G;
+        if (c < C) {
+            UNROLL for (int nb = 0; nb < NB; ++nb) {
+                const int col = nb < a.batch ? nb : a.batch - 1;
+                if (NB > 1 || xc != c) { F::load_x(x, K, col, c, xr); xc = c; }
+                UNROLL for (int r = 0; r < R; ++r) acc[r][nb] += F::dot(w[r], xr);
+            }
         }
-        store_rows<G, R, NB>(m, acc, a, row0);
+        if (i == iters - 1) {
+            PSN_STAMP(a, m, 3);
+            store_rows<G, R, NB>(m, acc, a, r0);
+            UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
+        }
+    };
+
+    if constexpr (DB) {
+        /* Prefetches are unconditional (indices clamped into range) so that the loads sit in
+         * straight-line code and the compiler can wait for exactly the older buffer. */
+        while (row0 < a.N) {
+            int r1 = row0, i1 = it;
+            advance(r1, i1);
+            load_rows<F, G, R>(a, m, r1, min(m.j + i1 * G, C - 1), wb);
+            consume(wa, row0, it);
+            if (r1 >= a.N) break;
+            int r2 = r1, i2 = i1;
+            advance(r2, i2);
+            load_rows<F, G, R>(a, m, r2, min(m.j + i2 * G, C - 1), wa);
+            consume(wb, r1, i1);
+            row0 = r2;
+            it = i2;
+        }
+    } else {
+        bool pre = true;
+        while (row0 < a.N) {
+            if (!pre) load_rows<F, G, R>(a, m, row0, min(m.j + it * G, C - 1), wa);
+            pre = false;
+            consume(wa, row0, it);
+            advance(row0, it);
+        }
     }
+    PSN_STAMP(a, m, 4);
 }
 
 /* Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations. */
@@ -644,13 +724,13 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
  * ------------------------------------------------------------------------------------------ */
 
 #define PSN_Q8_KERNEL(fmt, F, G, R, NB)                                                                   \
-    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
+    extern "C" __global__ void PSN_KERNEL_ATTR __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
         mv_q8<F, G, R, NB, 0>(a);                                                                         \
     }                                                                                                     \
-    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
+    extern "C" __global__ void PSN_KERNEL_ATTR __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
         mv_q8<F, G, R, NB, 1>(a);                                                                         \
     }                                                                                                     \
-    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_xf(const psn_matvec_args a) { \
+    extern "C" __global__ void PSN_KERNEL_ATTR __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_xf(const psn_matvec_args a) { \
         mv_q8<F, G, R, NB, 2>(a);                                                                         \
     }
 
@@ -663,9 +743,7 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
     PSN_Q8_KERNEL(fmt, F, 8, R, NB) PSN_Q8_KERNEL(fmt, F, 16, R, NB) PSN_Q8_KERNEL(fmt, F, 32, R, NB) PSN_Q8_KERNEL(fmt, F, 64, R, NB)
 #define PSN_Q8_ALL(fmt, F)                                                                 \
     PSN_Q8_ALL_G(fmt, F, 1, 1) PSN_Q8_ALL_G(fmt, F, 2, 1) PSN_Q8_ALL_G(fmt, F, 4, 1)       \
-    PSN_Q8_ALL_G(fmt, F, 1, 2) PSN_Q8_ALL_G(fmt, F, 2, 2)                                  \
-    PSN_Q8_ALL_G(fmt, F, 1, 4) PSN_Q8_ALL_G(fmt, F, 2, 4)                                  \
-    PSN_Q8_ALL_G(fmt, F, 1, 8)
+    PSN_Q8_ALL_G(fmt, F, 1, 2) PSN_Q8_ALL_G(fmt, F, 1, 4) PSN_Q8_ALL_G(fmt, F, 1, 8)
 
 #define PSN_F32_ALL_G(fmt, F, R, NB) \
     PSN_F32_KERNEL(fmt, F, 8, R, NB) PSN_F32_KERNEL(fmt, F, 16, R, NB) PSN_F32_KERNEL(fmt, F, 32, R, NB) PSN_F32_KERNEL(fmt, F, 64, R, NB)
