@@ -29,6 +29,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by
+# what the same counter reads for a 256 MiB device-to-device copy: x1.9998 and x1.0000).  The
+# figures and the commands are in profiles/matvec_q4_0_llama3_8b_step.md.
+MEASURED_TRAFFIC_BYTES = {"qkv": 14.45e6 + 24.0 * 1024, "o": 9.74e6 + 16.0 * 1024,
+                          "gate_up": 66.38e6 + 114.2 * 1024, "down": 33.67e6 + 17.0 * 1024}
 HIDDEN, KV, FFN, LAYERS = 4096, 1024, 14336, 32
 BPW_Q4_0 = 18.0 / 32.0
 
@@ -150,7 +155,8 @@ def main(argv=None):
     dom_bytes = sum(algo_bytes(ns, k) for name, ns, k in LAUNCHES if name in dom_names) / len(dom_names)
     achieved = dom_bytes / dom_us / 1e3
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "kernel": dom_kernel,
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": int(sum(MEASURED_TRAFFIC_BYTES[n] for n in dom_names) / len(dom_names)), "kernel": dom_kernel,
                 "avg_launch_us": round(dom_us, 3), "algo_bytes_per_launch": int(dom_bytes),
                 "launches_per_step": args.layers * len(dom_names),
                 "note": "average over the " + ", ".join(dom_names) + " launches, which share this kernel ("
