@@ -199,6 +199,12 @@ int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32
  * matmul op. */
 int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
                             const psn_buf *X_f16, psn_buf *Y_f32, int64_t M, int64_t N, int64_t K);
+/* The workgroup tile (rows of Y x columns of Y) the library picks for a shape: 64x64, 64x128,
+ * 128x128, 128x256, 256x128 or 256x256 (host arithmetic only) ... */
+int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m, int32_t *tile_n);
+/* ... and the same matmul with a caller-chosen tile (auto-tuners, benchmarks). */
+int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X_f16,
+                                  psn_buf *Y_f32, int64_t M, int64_t N, int64_t K, int32_t tile_m, int32_t tile_n);
 
 #ifdef __cplusplus
 }

@@ -810,19 +810,79 @@ extern "C" int32_t psn_qmatvec(psn_module *mod, psn_stream *s, int32_t qtype, in
 
 /* ------------------------------------------------------------------ prefill */
 
+static const int k_prefill_tiles[][2] = {{64, 64}, {64, 128}, {128, 128}, {128, 256}, {256, 128}, {256, 256}};
+
+static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X,
+                             psn_buf *Y, int64_t M, int64_t N, int64_t K) {
+    int32_t rc = check_same_ctx(mod, s, W, X, Y, what);
+    if (rc) return rc;
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) return fail(PSN_E_UNSUPPORTED, "%s: type %d (Q4_0 and Q8_0 have kernels)", what, qtype);
+    if (M <= 0 || N <= 0 || M > (1 << 20) || N > (1 << 24)) return fail(PSN_E_SHAPE, "%s: M=%lld N=%lld out of range", what, (long long)M, (long long)N);
+    const int64_t rb = psn_row_bytes(qtype, K);
+    if (rb < 0) return (int32_t)rb;
+    if (K % 256 || K > (1 << 24)) return fail(PSN_E_SHAPE, "%s: K=%lld must be a multiple of 256", what, (long long)K);
+    if ((int64_t)W->bytes < N * rb) return fail(PSN_E_INVALID_ARG, "%s: W holds %zu bytes, need %lld", what, W->bytes, (long long)(N * rb));
+    if ((int64_t)X->bytes < M * K * 2) return fail(PSN_E_INVALID_ARG, "%s: X holds %zu bytes, need %lld", what, X->bytes, (long long)(M * K * 2));
+    if ((int64_t)Y->bytes < M * N * 4) return fail(PSN_E_INVALID_ARG, "%s: Y holds %zu bytes, need %lld", what, Y->bytes, (long long)(M * N * 4));
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n) {
+    if (!tile_m || !tile_n) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: out is null");
+    if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if (cus <= 0) cus = 256;
+    /* Score = operand re-use of the tile (bm*bn/(bm+bn), what bounds LDS traffic per MFMA) times how
+     * evenly the tiles fill the chip's workgroup slots; padding rows of a partial tile count as waste. */
+    double best = -1.0;
+    int bi = 0;
+    for (int i = 0; i < 6; ++i) {
+        const int bm = k_prefill_tiles[i][0], bn = k_prefill_tiles[i][1];
+        const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn, tiles = mt * nt;
+        const int lds = 2 * (bm + bn) * 128;
+        const int64_t slots = (int64_t)cus * (160 * 1024 / lds);
+        const int64_t rounds = (tiles + slots - 1) / slots;
+        const double fill = (double)tiles / (double)(rounds * slots);
+        const double useful = (double)(M * N) / (double)(mt * bm * nt * bn);
+        const double score = (double)bm * bn / (bm + bn) * fill * useful;
+        if (score > best) { best = score; bi = i; }
+    }
+    *tile_m = k_prefill_tiles[bi][0];
+    *tile_n = k_prefill_tiles[bi][1];
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X,
+                                             psn_buf *Y, int64_t M, int64_t N, int64_t K, int32_t bm, int32_t bn) {
+    int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
+    if (rc) return rc;
+    bool known = false;
+    for (int i = 0; i < 6; ++i) known = known || (k_prefill_tiles[i][0] == bm && k_prefill_tiles[i][1] == bn);
+    if (!known) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel with a %dx%d tile", bm, bn);
+    const int lds = 2 * (bm + bn) * 128;
+    if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);
+    if ((rc = bind(mod->ctx))) return rc;
+    psn_prefill_args a;
+    memset(&a, 0, sizeof a);
+    a.W = (const uint8_t *)W->p;
+    a.X = (const uint16_t *)X->p;
+    a.Y = (float *)Y->p;
+    a.M = (int32_t)M;
+    a.N = (int32_t)N;
+    a.K = (int32_t)K;
+    a.row_bytes = psn_row_bytes(qtype, K);
+    const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
+    const int64_t blocks = 8 * ((nt + 7) / 8) * mt;               /* the kernel spreads N tiles over 8 XCDs */
+    char name[96];
+    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d", fmt_name(qtype), bm, bn);
+    return launch(mod, s, name, (unsigned)blocks, 256, (unsigned)lds, &a);
+}
+
 extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
                                        const psn_buf *X, psn_buf *Y, int64_t M, int64_t N, int64_t K) {
     if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "prefill: layout %d", layout);
-    int32_t rc = check_same_ctx(mod, s, W, X, Y, "psn_qmatmul_prefill");
+    int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
-    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) return fail(PSN_E_UNSUPPORTED, "prefill: type %d (Q4_0 and Q8_0 have kernels)", qtype);
-    if (M <= 0 || N <= 0 || M > (1 << 20) || N > (1 << 24)) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld out of range", (long long)M, (long long)N);
-    const int64_t rb = psn_row_bytes(qtype, K);
-    if (rb < 0) return (int32_t)rb;
-    if (K % 256 || K > (1 << 24)) return fail(PSN_E_SHAPE, "prefill: K=%lld must be a multiple of 256", (long long)K);
-    if ((int64_t)W->bytes < N * rb) return fail(PSN_E_INVALID_ARG, "prefill: W holds %zu bytes, need %lld", W->bytes, (long long)(N * rb));
-    if ((int64_t)X->bytes < M * K * 2) return fail(PSN_E_INVALID_ARG, "prefill: X holds %zu bytes, need %lld", X->bytes, (long long)(M * K * 2));
-    if ((int64_t)Y->bytes < M * N * 4) return fail(PSN_E_INVALID_ARG, "prefill: Y holds %zu bytes, need %lld", Y->bytes, (long long)(M * N * 4));
-    if ((rc = bind(mod->ctx))) return rc;
-    return fail(PSN_E_UNSUPPORTED, "prefill: kernel not built into this library yet");
+    int32_t bm = 0, bn = 0;
+    if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn))) return rc;
+    return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn);
 }

@@ -1,0 +1,213 @@
+/*
+ * psn_prefill.hip -- gfx950 quantized prefill matmul  Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k]
+ * for GGUF Q4_0 / Q8_0 weights, fp16 activations, fp32 accumulation on v_mfma_f32_32x32x16_f16.
+ *
+ * A workgroup of 256 threads owns a BM x BN tile of Y and walks K in steps of 64.  Per step
+ *   - the X tile (BM x 64 fp16) goes global -> LDS with 16-byte direct-to-LDS loads;
+ *   - the W tile is dequantized from registers: every thread keeps one 256-weight chunk of one
+ *     weight row (the same 144- or 272-byte chunk the decode kernels fetch) and turns two GGUF
+ *     blocks of it into 64 fp16 values, bit-exactly h(d * q): (0x6400 | q) is the fp16 1024 + q,
+ *     subtracting the bias is exact, and the fp16 multiply by the block's fp16 scale rounds once;
+ *   - each wave multiplies its (BM/WM) x (BN/WN) part with 32x32x16 MFMAs, operands read from LDS
+ *     as 16-byte fragments (8 consecutive k per lane for both A = X rows and B = W rows).
+ * LDS rows are 128 bytes (64 fp16); the eight 16-byte chunks of a row are stored XOR-swizzled by
+ * (row & 7) so that the 32 rows a fragment read touches fall into distinct banks.  Two LDS
+ * buffers alternate; one barrier per K step.
+ *
+ * Workgroup -> tile mapping is XCD-aware: workgroup b runs on XCD b % 8, and all M tiles of one
+ * N tile are placed on the same XCD back to back, so a weight panel streams from HBM into one L2.
+ */
+#include "psn_args.h"
+#include "psn_device.h"
+
+#define UNROLL _Pragma("unroll")
+
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+
+/* byte offset of 16-byte chunk `chunk` (0..7) of tile row `row` */
+PSN_DEV int tile_off(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
+
+PSN_DEV u32 h2_bits(half2_t v) { return __builtin_bit_cast(u32, v); }
+PSN_DEV half2_t bits_h2(u32 v) { return __builtin_bit_cast(half2_t, v); }
+
+/* four bytes of v (already masked to the wanted 0..255 values) -> four fp16 (1024 + byte) in element
+ * order, minus `bias`, times the block scale */
+PSN_DEV void bytes_to_h4(u32 v, u32 keep, half2_t bias, half2_t d2, u32 &lo, u32 &hi) {
+    const u32 t01 = __builtin_amdgcn_perm(0x64646464u, v, 0x04010400u) & keep;   /* [b0, 0x64, b1, 0x64] */
+    const u32 t23 = __builtin_amdgcn_perm(0x64646464u, v, 0x04030402u) & keep;   /* [b2, 0x64, b3, 0x64] */
+    lo = h2_bits((bits_h2(t01) - bias) * d2);
+    hi = h2_bits((bits_h2(t23) - bias) * d2);
+}
+
+struct PfQ4_0 {
+    static constexpr int DW = 36, BYTES = 144;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    /* GGUF block B of the chunk -> 32 fp16 in element order (16 dwords) */
+    template <int B>
+    static PSN_DEV void deq_block(const u32 (&w)[DW], u32 (&o)[16]) {
+        constexpr int base = 9 * (B >> 1);
+        u32 q[4], dbits;
+        if constexpr ((B & 1) == 0) {
+            dbits = w[base] & 0xffffu;
+            UNROLL for (int i = 0; i < 4; ++i) q[i] = align2(w[base + i + 1], w[base + i]);
+        } else {
+            dbits = w[base + 4] >> 16;
+            UNROLL for (int i = 0; i < 4; ++i) q[i] = w[base + 5 + i];
+        }
+        const half2_t d2 = bits_h2(dbits | (dbits << 16));
+        const half2_t bias = bits_h2(0x64086408u);               /* 1032 = 1024 + 8 */
+        UNROLL for (int i = 0; i < 4; ++i) {
+            bytes_to_h4(q[i], 0x640f640fu, bias, d2, o[2 * i], o[2 * i + 1]);              /* elements 4i..4i+3 */
+            bytes_to_h4(q[i] >> 4, 0x640f640fu, bias, d2, o[8 + 2 * i], o[8 + 2 * i + 1]); /* elements 16+4i.. */
+        }
+    }
+};
+
+struct PfQ8_0 {
+    static constexpr int DW = 68, BYTES = 272;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 17; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    template <int B>
+    static PSN_DEV void deq_block(const u32 (&w)[DW], u32 (&o)[16]) {
+        constexpr int base = 17 * (B >> 1);
+        u32 q[8], dbits;
+        if constexpr ((B & 1) == 0) {
+            dbits = w[base] & 0xffffu;
+            UNROLL for (int i = 0; i < 8; ++i) q[i] = align2(w[base + i + 1], w[base + i]);
+        } else {
+            dbits = w[base + 8] >> 16;
+            UNROLL for (int i = 0; i < 8; ++i) q[i] = w[base + 9 + i];
+        }
+        const half2_t d2 = bits_h2(dbits | (dbits << 16));
+        const half2_t bias = bits_h2(0x64806480u);               /* 1152 = 1024 + 128 */
+        UNROLL for (int i = 0; i < 8; ++i)
+            bytes_to_h4(q[i] ^ 0x80808080u, 0x64ff64ffu, bias, d2, o[2 * i], o[2 * i + 1]);   /* int8 + 128 */
+    }
+};
+
+/* 64 dequantized fp16 (blocks 2P and 2P+1 of the chunk) into one swizzled tile row */
+template <typename WF, int P>
+PSN_DEV void stage_w_row(const u32 (&w)[WF::DW], char *tile, int row) {
+    u32 o[32];
+    u32 (&o0)[16] = *reinterpret_cast<u32 (*)[16]>(&o[0]);
+    u32 (&o1)[16] = *reinterpret_cast<u32 (*)[16]>(&o[16]);
+    WF::template deq_block<2 * P>(w, o0);
+    WF::template deq_block<2 * P + 1>(w, o1);
+    UNROLL for (int c = 0; c < 8; ++c)
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, c)) = make_uint4(o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]);
+}
+
+template <typename WF, int BM, int BN, int WM, int WN>
+PSN_DEV void prefill_body(const psn_prefill_args &a) {
+    static_assert(WM * WN == 4, "four waves");
+    static_assert(BN == 64 || BN == 128 || BN == 256, "BN");
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;     /* 32x32 MFMA tiles per wave */
+    constexpr int KCH = 256 / BN;                           /* 256-wide K chunks held in registers per round */
+    constexpr int XBYTES = BM * 128, WBYTES = BN * 128;
+    extern __shared__ uint4 psn_smem[];
+    char *smem = reinterpret_cast<char *>(psn_smem);
+    char *xs[2] = {smem, smem + XBYTES};
+    char *ws[2] = {smem + 2 * XBYTES, smem + 2 * XBYTES + WBYTES};
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
+
+    /* XCD-aware tile choice: workgroups b, b+8, b+16, ... share an XCD; give them the M tiles of one
+     * N tile in a row so that a weight panel is fetched into a single L2 */
+    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_xcd_n = (nt + 7) >> 3;
+    const int tile_n = xcd + 8 * (local / mt), tile_m = local % mt;
+    if (local / mt >= per_xcd_n || tile_n >= nt) return;          /* whole workgroup leaves together */
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    float16_t acc[TM][TN];
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int wrow = tid % BN, wsel = tid / BN;                  /* weight row and which chunk of the round */
+    const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
+    u32 w[WF::DW];
+
+    auto stage_x = [&](char *tile, int k0) {
+        /* slot s = 16-byte word s of the tile in LDS order: row s/8, position s%8 holds chunk (s%8)^(row&7) */
+        UNROLL for (int i = 0; i < BM * 8 / 256; ++i) {
+            const int s = i * 256 + tid, row = s >> 3, chunk = (s & 7) ^ (row & 7);
+            const uint16_t *src = a.X + (int64_t)min(m0 + row, M - 1) * K + k0 + chunk * 8;
+            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + (i * 256 + wave * 64) * 16), 16, 0, 0);
+        }
+    };
+    auto compute = [&](const char *xt, const char *wt) {
+        UNROLL for (int kk = 0; kk < 4; ++kk) {
+            half8_t af[TM], bf[TN];
+            const int chunk = 2 * kk + (lane >> 5);
+            UNROLL for (int i = 0; i < TM; ++i)
+                af[i] = *reinterpret_cast<const half8_t *>(xt + tile_off(wm * (BM / WM) + 32 * i + (lane & 31), chunk));
+            UNROLL for (int j = 0; j < TN; ++j)
+                bf[j] = *reinterpret_cast<const half8_t *>(wt + tile_off(wn * (BN / WN) + 32 * j + (lane & 31), chunk));
+            UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        }
+    };
+
+    const int rounds = (C + KCH - 1) / KCH;
+    int buf = 0;
+    for (int r = 0; r < rounds; ++r) {
+        const int chunk = r * KCH + wsel;
+        if (chunk < C) {
+            WF::load(wbase + (int64_t)chunk * WF::BYTES, w);
+        } else {
+            UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = 0;      /* scale 0: contributes nothing */
+        }
+        UNROLL for (int sub = 0; sub < 4 * KCH; ++sub) {
+            const int k0 = (r * KCH * 4 + sub) * 64;
+            if (k0 < K) {                                          /* uniform */
+                stage_x(xs[buf], k0);
+                if (wsel == sub / 4) {
+                    switch (sub % 4) {
+                        case 0: stage_w_row<WF, 0>(w, ws[buf], wrow); break;
+                        case 1: stage_w_row<WF, 1>(w, ws[buf], wrow); break;
+                        case 2: stage_w_row<WF, 2>(w, ws[buf], wrow); break;
+                        default: stage_w_row<WF, 3>(w, ws[buf], wrow); break;
+                    }
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                compute(xs[buf], ws[buf]);
+                buf ^= 1;
+            }
+        }
+    }
+
+    /* 32x32 accumulator: lane holds column (lane & 31); register r is row 8*(r/4) + 4*(lane/32) + r%4 */
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
+        UNROLL for (int r = 0; r < 16; ++r) {
+            const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (row < M && col < N) a.Y[(int64_t)row * N + col] = acc[i][j][r];
+        }
+    }
+}
+
+#define PSN_PREFILL_KERNEL(fmt, WF, BM, BN, WM, WN)                                                          \
+    extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_m##BM##_n##BN(const psn_prefill_args a) { \
+        prefill_body<WF, BM, BN, WM, WN>(a);                                                                 \
+    }
+
+#define PSN_PREFILL_ALL(fmt, WF)               \
+    PSN_PREFILL_KERNEL(fmt, WF, 64, 64, 2, 2)    \
+    PSN_PREFILL_KERNEL(fmt, WF, 64, 128, 2, 2)   \
+    PSN_PREFILL_KERNEL(fmt, WF, 128, 128, 2, 2)  \
+    PSN_PREFILL_KERNEL(fmt, WF, 128, 256, 2, 2)  \
+    PSN_PREFILL_KERNEL(fmt, WF, 256, 128, 2, 2)  \
+    PSN_PREFILL_KERNEL(fmt, WF, 256, 256, 2, 2)
+
+PSN_PREFILL_ALL(q4_0, PfQ4_0)
+PSN_PREFILL_ALL(q8_0, PfQ8_0)

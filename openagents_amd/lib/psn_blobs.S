@@ -19,6 +19,10 @@ psn_blob_3_end:
 psn_blob_4_begin:
     .incbin "/root/repo/openagents_amd/lib/psn_mv_q6_K.gfx950.hsaco"
 psn_blob_4_end:
+    .balign 4096
+psn_blob_5_begin:
+    .incbin "/root/repo/openagents_amd/lib/psn_prefill.gfx950.hsaco"
+psn_blob_5_end:
     .balign 16
     .globl psn_builtin_blobs
 psn_builtin_blobs:
@@ -32,8 +36,10 @@ psn_builtin_blobs:
     .quad psn_blob_3_end
     .quad psn_blob_4_begin
     .quad psn_blob_4_end
+    .quad psn_blob_5_begin
+    .quad psn_blob_5_end
     .balign 4
     .globl psn_builtin_blob_count
 psn_builtin_blob_count:
-    .long 5
+    .long 6
     .section .note.GNU-stack,"",@progbits

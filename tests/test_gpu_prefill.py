@@ -1,0 +1,131 @@
+"""GPU parity of the quantized prefill matmul (Q4_0 / Q8_0 weights, fp16 activations, fp16 MFMA with
+fp32 accumulation) against the CPU oracle, through the C ABI.
+
+Oracle definition: Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k] with h = round-to-nearest-even to fp16 and
+fp32 accumulation.  The kernel forms h(d*q) bit-exactly, so only the accumulation order differs.
+Gate (north_star): max|y - ref| / max|ref| <= 1e-3; asserted: PARITY_TOL.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import ggufref as G
+from openagents_amd import _ffi, backend
+
+pytestmark = pytest.mark.gpu
+
+GATE = 1e-3
+PARITY_TOL = 2e-5
+TILES = [(64, 64), (64, 128), (128, 128), (128, 256), (256, 128), (256, 256)]
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+_cache = {}
+
+
+def weights(orc, qname, seed, n, k):
+    key = (qname, seed, n, k)
+    if key not in _cache:
+        _cache[key] = orc.quantize(getattr(orc, qname), G.seeded_weights(seed, n, k))
+    return _cache[key]
+
+
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
+@pytest.mark.parametrize("tile", TILES)
+def test_every_tile_ragged_shapes(hip, orc, qname, tile):
+    """m and n are ragged against every tile; k = 768 and 1280 exercise the partial last round of the
+    256-wide register chunks for the 64- and 128-column tiles."""
+    t = getattr(orc, qname)
+    for m, n, k in ((1, 70, 768), (37, 300, 1280), (200, 129, 512), (333, 515, 1024)):
+        say(f"prefill {qname} tile={tile} m={m} n={n} k={k}")
+        W = weights(orc, qname, 800, n, k)
+        X = G.seeded_acts(801 + m, m, k).astype(np.float16)
+        ref = orc.prefill(t, W, X, n, k)
+        y = hip.matmul_host(t, W, X, n, k, tile)
+        err = G.max_rel_err(y, ref)
+        assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, m, n, k, err)
+
+
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
+def test_prefill_m1_matches_matvec_f32_scheme(hip, orc, qname):
+    """One row of the prefill is the F32-scheme matvec on the same fp16 activations, up to the fp16
+    rounding of the weights (about 1.5e-4 of the output scale)."""
+    t = getattr(orc, qname)
+    n, k = 512, 4096
+    W = weights(orc, qname, 810, n, k)
+    X = G.seeded_acts(811, 1, k).astype(np.float16)
+    y = hip.matmul_host(t, W, X, n, k)
+    mv = hip.matvec_host(t, W, X[0].astype(np.float32), n, k, _ffi.ACT_F32)
+    assert G.max_rel_err(y[0], mv) < GATE
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
+def test_prefill_baseline_shapes_m64(hip, orc, qname, n, k):
+    say(f"prefill {qname} m=64 n={n} k={k} (full oracle)")
+    t = getattr(orc, qname)
+    W = weights(orc, qname, 820, n, k)
+    X = G.seeded_acts(821, 64, k).astype(np.float16)
+    y = hip.matmul_host(t, W, X, n, k)
+    err = G.max_rel_err(y, orc.prefill(t, W, X, n, k))
+    say(f"  max_rel_err={err:.3e}")
+    assert err < PARITY_TOL
+
+
+@pytest.mark.parametrize("m", [512, 2048])
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+def test_prefill_baseline_shapes_large_m_sampled(hip, orc, m, n, k):
+    """The GPU computes the full [m, n] product; the oracle re-computes a sample of 96 activation rows x
+    160 weight rows (tile corners, edges and random interior rows) that the full result must match."""
+    t = orc.Q4_0
+    say(f"prefill Q4_0 m={m} n={n} k={k} (sampled oracle)")
+    W = weights(orc, "Q4_0", 820, n, k)
+    X = G.seeded_acts(830 + m, m, k).astype(np.float16)
+    y = hip.matmul_host(t, W, X, n, k)
+    rng = np.random.default_rng(m + n)
+    mi = np.unique(np.concatenate([[0, 31, 32, 63, 64, 127, 128, 255, 256, m - 1], rng.integers(0, m, 86)]))
+    ni = np.unique(np.concatenate([[0, 31, 32, 63, 64, 127, 128, 255, 256, n - 1], rng.integers(0, n, 150)]))
+    ref = orc.prefill(t, W[ni], X[mi], len(ni), k)
+    err = G.max_rel_err(y[np.ix_(mi, ni)], ref)
+    say(f"  max_rel_err={err:.3e}")
+    assert err < PARITY_TOL
+    assert np.all(np.isfinite(y))
+
+
+def test_prefill_linearity_and_zero(hip, orc):
+    """Size-independent properties at a full shape: Y(X1 + X2) = Y(X1) + Y(X2) when X1, X2 have disjoint
+    supports (exact in fp16), and zero activations give exactly zero."""
+    t, n, k, m = orc.Q8_0, 4096, 4096, 128
+    W = weights(orc, "Q8_0", 840, n, k)
+    X = G.seeded_acts(841, m, k).astype(np.float16)
+    X1, X2 = X.copy(), X.copy()
+    X1[:, k // 2:] = 0
+    X2[:, :k // 2] = 0
+    y, y1, y2 = (hip.matmul_host(t, W, A, n, k) for A in (X, X1, X2))
+    assert G.max_rel_err(y, y1 + y2) < PARITY_TOL
+    assert not hip.matmul_host(t, W, np.zeros((m, k), np.float16), n, k).any()
+
+
+def test_prefill_errors(hip, orc):
+    n, k = 64, 512
+    W = weights(orc, "Q4_0", 850, n, k)
+    w = hip.upload_weight(orc.Q4_0, W, n, k)
+    x = hip.upload(np.zeros((4, k), np.float16))
+    y = hip.alloc(4 * n * 4)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matmul(w, x, y, 4, tile=(96, 96))
+    assert e.value.code == _ffi.E_UNSUPPORTED
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matmul(w, x, y, 8)                      # X and Y too small for 8 rows
+    assert e.value.code == _ffi.E_INVALID_ARG
+    wk = hip.upload_weight(orc.Q4_K, weights(orc, "Q4_K", 851, n, k), n, k)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matmul(wk, x, y, 4)
+    assert e.value.code == _ffi.E_UNSUPPORTED
+    hip.quantized_matmul(w, x, y, 4)
+    hip.sync()
