@@ -210,6 +210,27 @@ int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype,
                                   psn_buf *Y_f32, int64_t M, int64_t N, int64_t K, int32_t tile_m, int32_t tile_n,
                                   int32_t ksplit);
 
+/* ---- decode-step glue (what sits between the matvecs of a Llama-style layer) ----------------
+ * These replace the CUDA backend's RMSNorm / rotary / attention / activation ops only as far as a
+ * whole token step needs them to be measured on the device; all vectors are fp32, the KV cache is
+ * fp16 [positions][n_kv_heads][head_dim].  Positions are immediate arguments: a captured graph
+ * replays the position it was captured at. */
+
+/* x += delta (skipped when delta is NULL), then y = x * rsqrt(mean(x^2) + eps) * weight; n % 4 == 0 */
+int32_t psn_add_rmsnorm(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
+                        int64_t n, float eps);
+/* rotary embedding (pairs (2i, 2i+1), angle pos * theta_base^(-2i/head_dim)) of q in place and of k,
+ * then k and v are stored as fp16 at row `pos` of the caches */
+int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q, psn_buf *k, const psn_buf *v, psn_buf *k_cache,
+                          psn_buf *v_cache, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t pos, float theta_base);
+/* softmax(q K^T / sqrt(head_dim)) V over cache positions 0 .. n_ctx-1, grouped-query (n_heads a multiple
+ * of n_kv_heads, at most 8 per group), head_dim 128; workspace holds n_heads * ceil(n_ctx/64) * 130 floats */
+int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
+                             psn_buf *workspace, psn_buf *out, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
+                             int32_t n_ctx);
+/* out = silu(gate) * up; n % 4 == 0 */
+int32_t psn_swiglu(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, int64_t n);
+
 #ifdef __cplusplus
 }
 #endif

@@ -234,6 +234,22 @@ class HipBackend:
         w0, n, W, Y, N = self._pack(ws, ys)
         _check(self.lib.psn_qmatvec_planned(self.module, self.stream, w0.qtype, scheme, n, W, x.handle, Y, N, w0.k, batch, C.byref(plan)))
 
+    # -- decode-step glue --------------------------------------------------------------------
+    def add_rmsnorm(self, x: DeviceBuffer, delta, weight: DeviceBuffer, y: DeviceBuffer, n: int, eps: float = 1e-5):
+        _check(self.lib.psn_add_rmsnorm(self.module, self.stream, x.handle, delta.handle if delta is not None else None,
+                                        weight.handle, y.handle, n, eps))
+
+    def rope_kv_store(self, q, k, v, k_cache, v_cache, n_heads: int, n_kv_heads: int, head_dim: int, pos: int, theta_base: float):
+        _check(self.lib.psn_rope_kv_store(self.module, self.stream, q.handle, k.handle, v.handle, k_cache.handle, v_cache.handle,
+                                          n_heads, n_kv_heads, head_dim, pos, theta_base))
+
+    def attention_decode(self, q, k_cache, v_cache, workspace, out, n_heads: int, n_kv_heads: int, head_dim: int, n_ctx: int):
+        _check(self.lib.psn_attention_decode(self.module, self.stream, q.handle, k_cache.handle, v_cache.handle, workspace.handle,
+                                             out.handle, n_heads, n_kv_heads, head_dim, n_ctx))
+
+    def swiglu(self, gate, up, out, n: int):
+        _check(self.lib.psn_swiglu(self.module, self.stream, gate.handle, up.handle, out.handle, n))
+
     # -- graphs -----------------------------------------------------------------------------
     def reserve(self, k: int, batch: int = 1):
         _check(self.lib.psn_stream_reserve(self.stream, k, batch))

@@ -63,4 +63,39 @@ struct psn_fill_args {
     int64_t n16;          /* number of 16-byte words to zero */
 };
 
+/* decode-step glue kernels (psn_decode.hip) */
+struct psn_norm_args {
+    float *x;             /* [n], updated in place when delta != null */
+    const float *delta;   /* optional residual to add first */
+    const float *weight;  /* [n] */
+    float *y;             /* [n] normalized output */
+    int32_t n;
+    float eps;
+};
+struct psn_rope_args {
+    float *q;             /* [n_heads][head_dim], rotated in place */
+    float *k;             /* [n_kv_heads][head_dim] */
+    const float *v;       /* [n_kv_heads][head_dim] */
+    void *k_cache;        /* fp16 [positions][n_kv_heads][head_dim] */
+    void *v_cache;
+    int32_t n_heads, n_kv_heads, head_dim, pos;
+    float theta_base;
+    int32_t pad;
+};
+struct psn_attn_args {
+    const float *q;       /* [n_heads][128] */
+    const void *k_cache;
+    const void *v_cache;
+    float *partial;       /* [n_heads][n_splits][130] */
+    float *out;           /* [n_heads][128] */
+    int32_t n_heads, n_kv_heads, n_ctx, n_splits;
+    float scale;
+    int32_t pad;
+};
+struct psn_swiglu_args {
+    const float *gate, *up;
+    float *out;
+    int32_t n, pad;
+};
+
 #endif

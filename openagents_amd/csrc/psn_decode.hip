@@ -1,0 +1,171 @@
+/*
+ * psn_decode.hip -- the small kernels that sit between the quantized matvecs of a Llama-style
+ * decode step: residual add + RMSNorm, rotary embedding + KV-cache append, grouped-query attention
+ * over the cache (split over the context, then combined), and SwiGLU.  They exist so that a whole
+ * token step can run on the device and the matvec share of it can be measured; none of them is a
+ * bandwidth-critical kernel (the KV cache read, 8 MB per layer at context 2048, is the largest).
+ */
+#include "psn_args.h"
+#include "psn_device.h"
+
+#define UNROLL _Pragma("unroll")
+
+/* sum over a workgroup of up to 1024 threads; every thread gets the result */
+PSN_DEV float block_sum(float v, float *scratch) {
+    v = group_sum<64>(v);
+    const int wave = threadIdx.x >> 6, nw = (blockDim.x + 63) >> 6;
+    __syncthreads();                                   /* scratch may still be read from a previous call */
+    if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; ++i) t += scratch[i];
+    return t;
+}
+
+/* x += delta (if delta != null);  y = x * rsqrt(mean(x^2) + eps) * weight.   One workgroup, n % 4 == 0. */
+extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_norm_args a) {
+    __shared__ float red[16];
+    const int n4 = a.n >> 2;
+    float4 *x4 = reinterpret_cast<float4 *>(a.x);
+    const float4 *d4 = reinterpret_cast<const float4 *>(a.delta);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+        float4 v = x4[i];
+        if (d4) {
+            const float4 d = d4[i];
+            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
+            x4[i] = v;
+        }
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_sum(ss, red);
+    const float scale = 1.0f / sqrtf(ss / (float)a.n + a.eps);
+    const float4 *w4 = reinterpret_cast<const float4 *>(a.weight);
+    float4 *y4 = reinterpret_cast<float4 *>(a.y);
+    for (int i = threadIdx.x; i < n4; i += blockDim.x) {
+        const float4 v = x4[i], w = w4[i];
+        y4[i] = make_float4(v.x * scale * w.x, v.y * scale * w.y, v.z * scale * w.z, v.w * scale * w.w);
+    }
+}
+
+/* Rotary embedding of q (in place) and k at position pos, pairs (2i, 2i+1), angle pos * base^(-2i/d);
+ * k and v are appended to the fp16 cache row of that position.  One thread per pair. */
+extern "C" __global__ void __launch_bounds__(256) psn_rope_kv_store(const psn_rope_args a) {
+    const int half = a.head_dim >> 1;
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    const int nq = a.n_heads * half, nk = a.n_kv_heads * half;
+    if (t >= nq + nk) return;
+    const bool is_q = t < nq;
+    const int idx = is_q ? t : t - nq;
+    const int head = idx / half, i = idx % half;
+    const float freq = powf(a.theta_base, -2.0f * (float)i / (float)a.head_dim);
+    float sn, cs;
+    sincosf((float)a.pos * freq, &sn, &cs);
+    float *src = (is_q ? a.q : a.k) + head * a.head_dim + 2 * i;
+    const float x0 = src[0], x1 = src[1];
+    const float r0 = x0 * cs - x1 * sn, r1 = x0 * sn + x1 * cs;
+    if (is_q) {
+        src[0] = r0;
+        src[1] = r1;
+    } else {
+        const int64_t row = ((int64_t)a.pos * a.n_kv_heads + head) * a.head_dim + 2 * i;
+        reinterpret_cast<f16 *>(a.k_cache)[row] = (f16)r0;
+        reinterpret_cast<f16 *>(a.k_cache)[row + 1] = (f16)r1;
+        const float *v = a.v + head * a.head_dim + 2 * i;
+        reinterpret_cast<f16 *>(a.v_cache)[row] = (f16)v[0];
+        reinterpret_cast<f16 *>(a.v_cache)[row + 1] = (f16)v[1];
+    }
+}
+
+/* Attention of one new token over cache positions 0 .. n_ctx-1, head_dim 128, up to 8 query heads
+ * per kv head.  Workgroup = one wave = (kv head, 64 consecutive positions): lane p scores its
+ * position against all query heads of the group (one K row of 256 bytes in registers), then lanes
+ * switch to two output dims each and accumulate exp(score - max) * V.  Writes the unnormalized
+ * partial output plus (max, sum) per head and split. */
+extern "C" __global__ void __launch_bounds__(64) psn_attn_partial(const psn_attn_args a) {
+    constexpr int D = 128, MAXG = 8;
+    __shared__ float qs[MAXG][D];
+    __shared__ float es[MAXG][64];
+    const int lane = threadIdx.x;
+    const int kvh = blockIdx.x % a.n_kv_heads, split = blockIdx.x / a.n_kv_heads;
+    const int group = a.n_heads / a.n_kv_heads;
+    for (int i = lane; i < group * D; i += 64) qs[i / D][i % D] = a.q[(kvh * group + i / D) * D + (i % D)];
+    __syncthreads();
+    const int p = split * 64 + lane;
+    const bool live = p < a.n_ctx;
+    float s[MAXG];
+    UNROLL for (int g = 0; g < MAXG; ++g) s[g] = 0.f;
+    {
+        const uint4 *krow = reinterpret_cast<const uint4 *>(reinterpret_cast<const f16 *>(a.k_cache) + ((int64_t)(live ? p : 0) * a.n_kv_heads + kvh) * D);
+        UNROLL for (int c = 0; c < 16; ++c) {
+            const uint4 kv = krow[c];
+            const u32 kw[4] = {kv.x, kv.y, kv.z, kv.w};
+            UNROLL for (int j = 0; j < 4; ++j) {
+                const float k0 = h2f_lo(kw[j]), k1 = h2f_hi(kw[j]);
+                UNROLL for (int g = 0; g < MAXG; ++g)
+                    if (g < group) s[g] += k0 * qs[g][8 * c + 2 * j] + k1 * qs[g][8 * c + 2 * j + 1];
+            }
+        }
+    }
+    float mx[MAXG], sum[MAXG];
+    UNROLL for (int g = 0; g < MAXG; ++g) {
+        if (g < group) {
+            const float sc = live ? s[g] * a.scale : -INFINITY;
+            const float m = group_max<64>(sc);
+            const float e = live ? __expf(sc - m) : 0.f;
+            mx[g] = m;
+            sum[g] = group_sum<64>(e);
+            es[g][lane] = e;
+        }
+    }
+    __syncthreads();
+    float o0[MAXG], o1[MAXG];
+    UNROLL for (int g = 0; g < MAXG; ++g) o0[g] = o1[g] = 0.f;
+    const int np = min(64, a.n_ctx - split * 64);
+    const u32 *vbase = reinterpret_cast<const u32 *>(reinterpret_cast<const f16 *>(a.v_cache) + ((int64_t)split * 64 * a.n_kv_heads + kvh) * D) + lane;
+    const int64_t vstride = (int64_t)a.n_kv_heads * D / 2;       /* dwords between positions */
+    for (int i = 0; i < np; ++i) {
+        const u32 vv = vbase[i * vstride];
+        const float v0 = h2f_lo(vv), v1 = h2f_hi(vv);
+        UNROLL for (int g = 0; g < MAXG; ++g)
+            if (g < group) { const float e = es[g][i]; o0[g] += e * v0; o1[g] += e * v1; }
+    }
+    UNROLL for (int g = 0; g < MAXG; ++g) {
+        if (g < group) {
+            const int head = kvh * group + g;
+            float *dst = a.partial + ((int64_t)head * a.n_splits + split) * (D + 2);
+            dst[2 * lane] = o0[g];
+            dst[2 * lane + 1] = o1[g];
+            if (lane == 0) { dst[D] = mx[g]; dst[D + 1] = sum[g]; }
+        }
+    }
+}
+
+/* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One workgroup of 128 threads per head. */
+extern "C" __global__ void __launch_bounds__(128) psn_attn_combine(const psn_attn_args a) {
+    constexpr int D = 128;
+    const int head = blockIdx.x, d = threadIdx.x;
+    const float *base = a.partial + (int64_t)head * a.n_splits * (D + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < a.n_splits; ++s) M = fmaxf(M, base[s * (D + 2) + D]);
+    float num = 0.f, den = 0.f;
+    for (int s = 0; s < a.n_splits; ++s) {
+        const float w = __expf(base[s * (D + 2) + D] - M);
+        num += base[s * (D + 2) + d] * w;
+        den += base[s * (D + 2) + D + 1] * w;
+    }
+    a.out[head * D + d] = num / den;
+}
+
+/* out = silu(gate) * up */
+extern "C" __global__ void __launch_bounds__(256) psn_swiglu(const psn_swiglu_args a) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.n / 4) return;
+    const float4 g = reinterpret_cast<const float4 *>(a.gate)[i], u = reinterpret_cast<const float4 *>(a.up)[i];
+    float4 o;
+    o.x = g.x / (1.f + __expf(-g.x)) * u.x;
+    o.y = g.y / (1.f + __expf(-g.y)) * u.y;
+    o.z = g.z / (1.f + __expf(-g.z)) * u.z;
+    o.w = g.w / (1.f + __expf(-g.w)) * u.w;
+    reinterpret_cast<float4 *>(a.out)[i] = o;
+}

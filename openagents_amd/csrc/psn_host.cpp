@@ -905,3 +905,105 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp))) return rc;
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp);
 }
+
+/* ------------------------------------------------------------------ decode-step glue */
+
+static int32_t need(const psn_buf *b, int64_t bytes, const char *what, const char *name) {
+    if (!b) return fail(PSN_E_INVALID_ARG, "%s: %s is null", what, name);
+    if ((int64_t)b->bytes < bytes) return fail(PSN_E_INVALID_ARG, "%s: %s holds %zu bytes, need %lld", what, name, b->bytes, (long long)bytes);
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_add_rmsnorm(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
+                                   int64_t n, float eps) {
+    int32_t rc = check_same_ctx(mod, s, x, weight, y, "psn_add_rmsnorm");
+    if (rc) return rc;
+    if (n <= 0 || n % 4 || n > (1 << 24)) return fail(PSN_E_SHAPE, "psn_add_rmsnorm: n=%lld must be a positive multiple of 4", (long long)n);
+    if ((rc = need(x, n * 4, "psn_add_rmsnorm", "x")) || (rc = need(weight, n * 4, "psn_add_rmsnorm", "weight")) ||
+        (rc = need(y, n * 4, "psn_add_rmsnorm", "y")) || (delta && (rc = need(delta, n * 4, "psn_add_rmsnorm", "delta"))))
+        return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    psn_norm_args a;
+    a.x = (float *)x->p;
+    a.delta = delta ? (const float *)delta->p : nullptr;
+    a.weight = (const float *)weight->p;
+    a.y = (float *)y->p;
+    a.n = (int32_t)n;
+    a.eps = eps;
+    const unsigned threads = n >= 4096 ? 1024 : n >= 1024 ? 256 : 64;
+    return launch(mod, s, "psn_add_rmsnorm", 1, threads, 0, &a);
+}
+
+extern "C" int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q, psn_buf *k, const psn_buf *v, psn_buf *k_cache,
+                                     psn_buf *v_cache, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t pos, float theta_base) {
+    int32_t rc = check_same_ctx(mod, s, q, k, v, "psn_rope_kv_store");
+    if (rc) return rc;
+    if (n_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || head_dim % 2 || pos < 0) return fail(PSN_E_SHAPE, "psn_rope_kv_store: bad head geometry or position");
+    const int64_t row = (int64_t)n_kv_heads * head_dim * 2;
+    if ((rc = need(q, (int64_t)n_heads * head_dim * 4, "psn_rope_kv_store", "q")) || (rc = need(k, row * 2, "psn_rope_kv_store", "k")) ||
+        (rc = need(v, row * 2, "psn_rope_kv_store", "v")) || (rc = need(k_cache, (pos + 1) * row, "psn_rope_kv_store", "k_cache")) ||
+        (rc = need(v_cache, (pos + 1) * row, "psn_rope_kv_store", "v_cache")))
+        return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    psn_rope_args a;
+    memset(&a, 0, sizeof a);
+    a.q = (float *)q->p;
+    a.k = (float *)k->p;
+    a.v = (const float *)v->p;
+    a.k_cache = k_cache->p;
+    a.v_cache = v_cache->p;
+    a.n_heads = n_heads;
+    a.n_kv_heads = n_kv_heads;
+    a.head_dim = head_dim;
+    a.pos = pos;
+    a.theta_base = theta_base;
+    const int pairs = (n_heads + n_kv_heads) * head_dim / 2;
+    return launch(mod, s, "psn_rope_kv_store", (unsigned)((pairs + 255) / 256), 256, 0, &a);
+}
+
+extern "C" int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
+                                        psn_buf *workspace, psn_buf *out, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx) {
+    int32_t rc = check_same_ctx(mod, s, q, k_cache, v_cache, "psn_attention_decode");
+    if (rc) return rc;
+    if (head_dim != 128) return fail(PSN_E_UNSUPPORTED, "psn_attention_decode: head_dim=%d (128 has a kernel)", head_dim);
+    if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || n_heads / n_kv_heads > 8)
+        return fail(PSN_E_SHAPE, "psn_attention_decode: %d query heads over %d kv heads (need a multiple, at most 8 per group)", n_heads, n_kv_heads);
+    if (n_ctx <= 0) return fail(PSN_E_SHAPE, "psn_attention_decode: n_ctx=%d", n_ctx);
+    const int32_t splits = (n_ctx + 63) / 64;
+    const int64_t row = (int64_t)n_kv_heads * head_dim * 2;
+    if ((rc = need(q, (int64_t)n_heads * 512, "psn_attention_decode", "q")) || (rc = need(out, (int64_t)n_heads * 512, "psn_attention_decode", "out")) ||
+        (rc = need(k_cache, n_ctx * row, "psn_attention_decode", "k_cache")) || (rc = need(v_cache, n_ctx * row, "psn_attention_decode", "v_cache")) ||
+        (rc = need(workspace, (int64_t)n_heads * splits * 130 * 4, "psn_attention_decode", "workspace")))
+        return rc;
+    if (workspace->ctx != mod->ctx || out->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "psn_attention_decode: handles belong to different contexts");
+    if ((rc = bind(mod->ctx))) return rc;
+    psn_attn_args a;
+    memset(&a, 0, sizeof a);
+    a.q = (const float *)q->p;
+    a.k_cache = k_cache->p;
+    a.v_cache = v_cache->p;
+    a.partial = (float *)workspace->p;
+    a.out = (float *)out->p;
+    a.n_heads = n_heads;
+    a.n_kv_heads = n_kv_heads;
+    a.n_ctx = n_ctx;
+    a.n_splits = splits;
+    a.scale = 0.08838834764831845f;                 /* 1/sqrt(128) */
+    if ((rc = launch(mod, s, "psn_attn_partial", (unsigned)(n_kv_heads * splits), 64, 0, &a))) return rc;
+    return launch(mod, s, "psn_attn_combine", (unsigned)n_heads, 128, 0, &a);
+}
+
+extern "C" int32_t psn_swiglu(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, int64_t n) {
+    int32_t rc = check_same_ctx(mod, s, gate, up, out, "psn_swiglu");
+    if (rc) return rc;
+    if (n <= 0 || n % 4 || n > (1 << 28)) return fail(PSN_E_SHAPE, "psn_swiglu: n=%lld must be a positive multiple of 4", (long long)n);
+    if ((rc = need(gate, n * 4, "psn_swiglu", "gate")) || (rc = need(up, n * 4, "psn_swiglu", "up")) || (rc = need(out, n * 4, "psn_swiglu", "out"))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    psn_swiglu_args a;
+    a.gate = (const float *)gate->p;
+    a.up = (const float *)up->p;
+    a.out = (float *)out->p;
+    a.n = (int32_t)n;
+    a.pad = 0;
+    return launch(mod, s, "psn_swiglu", (unsigned)((n / 4 + 255) / 256), 256, 0, &a);
+}

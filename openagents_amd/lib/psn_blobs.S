@@ -23,6 +23,10 @@ psn_blob_4_end:
 psn_blob_5_begin:
     .incbin "/root/repo/openagents_amd/lib/psn_prefill.gfx950.hsaco"
 psn_blob_5_end:
+    .balign 4096
+psn_blob_6_begin:
+    .incbin "/root/repo/openagents_amd/lib/psn_decode.gfx950.hsaco"
+psn_blob_6_end:
     .balign 16
     .globl psn_builtin_blobs
 psn_builtin_blobs:
@@ -38,8 +42,10 @@ psn_builtin_blobs:
     .quad psn_blob_4_end
     .quad psn_blob_5_begin
     .quad psn_blob_5_end
+    .quad psn_blob_6_begin
+    .quad psn_blob_6_end
     .balign 4
     .globl psn_builtin_blob_count
 psn_builtin_blob_count:
-    .long 6
+    .long 7
     .section .note.GNU-stack,"",@progbits

@@ -1,0 +1,186 @@
+"""GPU parity of the decode-step glue kernels and of a whole (small) token step against a numpy
+restatement of the textbook Llama layer, with the CPU oracle doing the quantized matvecs.
+
+The reference here is plain numpy (fp64 where it matters): RMSNorm, rotary pairs (2i, 2i+1) with
+theta = 500000, grouped-query softmax attention over an fp16 cache, SwiGLU.  Sizes are reduced
+(hidden 512, 4 query / 2 kv heads of dim 128, FFN 1024, vocab 768, 3 layers, context 150); the
+8B-shaped step is exercised by `python -m openagents_amd.decode`, whose logits only have to be finite.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+import ggufref as G
+from openagents_amd import _ffi
+from openagents_amd.decode import DecodeStep, LayerWeights, LlamaShape, ModelWeights
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def rmsnorm_ref(x, w, eps):
+    x = x.astype(np.float64)
+    return (x / np.sqrt(np.mean(x * x) + eps) * w).astype(np.float32)
+
+
+def rope_ref(vec, n_heads, head_dim, pos, theta):
+    v = vec.astype(np.float64).reshape(n_heads, head_dim // 2, 2)
+    i = np.arange(head_dim // 2)
+    ang = pos * theta ** (-2.0 * i / head_dim)
+    c, s = np.cos(ang), np.sin(ang)
+    out = np.empty_like(v)
+    out[:, :, 0] = v[:, :, 0] * c - v[:, :, 1] * s
+    out[:, :, 1] = v[:, :, 0] * s + v[:, :, 1] * c
+    return out.reshape(-1).astype(np.float32)
+
+
+def attention_ref(q, kc, vc, n_heads, n_kv, d, n_ctx):
+    q = q.astype(np.float64).reshape(n_heads, d)
+    k = kc[:n_ctx].astype(np.float64).reshape(n_ctx, n_kv, d)
+    v = vc[:n_ctx].astype(np.float64).reshape(n_ctx, n_kv, d)
+    out = np.empty((n_heads, d))
+    for h in range(n_heads):
+        g = h // (n_heads // n_kv)
+        s = k[:, g, :] @ q[h] / np.sqrt(d)
+        p = np.exp(s - s.max())
+        out[h] = (p / p.sum()) @ v[:, g, :]
+    return out.reshape(-1).astype(np.float32)
+
+
+def test_add_rmsnorm(hip):
+    rng = np.random.default_rng(900)
+    for n in (256, 4096, 14336):
+        x = rng.standard_normal(n, dtype=np.float32) * 3
+        dl = rng.standard_normal(n, dtype=np.float32)
+        w = rng.standard_normal(n, dtype=np.float32)
+        xb, db, wb, yb = hip.upload(x), hip.upload(dl), hip.upload(w), hip.alloc(n * 4)
+        hip.add_rmsnorm(xb, None, wb, yb, n, 1e-5)
+        assert G.max_rel_err(yb.download(np.float32, (n,)), rmsnorm_ref(x, w, 1e-5)) < 1e-5
+        assert np.array_equal(xb.download(np.float32, (n,)), x)
+        hip.add_rmsnorm(xb, db, wb, yb, n, 1e-5)
+        assert np.array_equal(xb.download(np.float32, (n,)), x + dl)
+        assert G.max_rel_err(yb.download(np.float32, (n,)), rmsnorm_ref(x + dl, w, 1e-5)) < 1e-5
+
+
+def test_rope_and_cache_append(hip):
+    rng = np.random.default_rng(901)
+    nh, nkv, d, ctx = 8, 2, 128, 40
+    for pos in (0, 1, 17, 39):
+        q = rng.standard_normal(nh * d, dtype=np.float32)
+        k = rng.standard_normal(nkv * d, dtype=np.float32)
+        v = rng.standard_normal(nkv * d, dtype=np.float32)
+        qb, kb, vb = hip.upload(q), hip.upload(k), hip.upload(v)
+        kc, vc = hip.upload(np.zeros((ctx, nkv * d), np.float16)), hip.upload(np.zeros((ctx, nkv * d), np.float16))
+        hip.rope_kv_store(qb, kb, vb, kc, vc, nh, nkv, d, pos, 500000.0)
+        assert G.max_rel_err(qb.download(np.float32, (nh * d,)), rope_ref(q, nh, d, pos, 500000.0)) < 2e-5
+        kcache = kc.download(np.float16, (ctx, nkv * d))
+        vcache = vc.download(np.float16, (ctx, nkv * d))
+        assert G.max_rel_err(kcache[pos].astype(np.float32), rope_ref(k, nkv, d, pos, 500000.0)) < 1e-3   # fp16 storage
+        assert np.array_equal(vcache[pos], v.astype(np.float16))
+        assert not np.delete(kcache, pos, axis=0).any() and not np.delete(vcache, pos, axis=0).any()
+
+
+@pytest.mark.parametrize("nh,nkv", [(4, 2), (32, 8), (8, 1)])
+def test_attention_decode(hip, nh, nkv):
+    rng = np.random.default_rng(902)
+    d = 128
+    for n_ctx in (1, 63, 64, 65, 150, 2048):
+        say(f"attention heads={nh}/{nkv} ctx={n_ctx}")
+        q = rng.standard_normal(nh * d, dtype=np.float32)
+        kc = rng.standard_normal((n_ctx, nkv * d), dtype=np.float32).astype(np.float16)
+        vc = rng.standard_normal((n_ctx, nkv * d), dtype=np.float32).astype(np.float16)
+        ws = hip.alloc(nh * ((n_ctx + 63) // 64) * 130 * 4)
+        out = hip.alloc(nh * d * 4)
+        hip.attention_decode(hip.upload(q), hip.upload(kc), hip.upload(vc), ws, out, nh, nkv, d, n_ctx)
+        got = out.download(np.float32, (nh * d,))
+        assert G.max_rel_err(got, attention_ref(q, kc, vc, nh, nkv, d, n_ctx)) < 2e-5
+
+
+def test_swiglu(hip):
+    rng = np.random.default_rng(903)
+    n = 14336
+    g = rng.standard_normal(n, dtype=np.float32) * 4
+    u = rng.standard_normal(n, dtype=np.float32)
+    out = hip.alloc(n * 4)
+    hip.swiglu(hip.upload(g), hip.upload(u), out, n)
+    ref = (g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u).astype(np.float32)
+    assert G.max_rel_err(out.download(np.float32, (n,)), ref) < 1e-5
+
+
+def test_whole_small_decode_step_eager_and_graph(hip, orc):
+    s = LlamaShape(hidden=512, n_heads=4, n_kv_heads=2, head_dim=128, ffn=1024, vocab=768, n_layers=3)
+    ctx, pos = 150, 149
+    rng = np.random.default_rng(904)
+
+    def qmat(t, n, k):
+        return orc.quantize(t, (rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.05)))
+
+    host_layers, dev_layers = [], []
+    for _ in range(s.n_layers):
+        h = {"wq": qmat(orc.Q4_K, s.hidden, s.hidden), "wk": qmat(orc.Q4_K, s.kv_dim, s.hidden), "wv": qmat(orc.Q4_K, s.kv_dim, s.hidden),
+             "wo": qmat(orc.Q4_K, s.hidden, s.hidden), "w_gate": qmat(orc.Q4_K, s.ffn, s.hidden), "w_up": qmat(orc.Q4_K, s.ffn, s.hidden),
+             "w_down": qmat(orc.Q4_K, s.hidden, s.ffn),
+             "attn_norm": (1 + 0.1 * rng.standard_normal(s.hidden)).astype(np.float32), "ffn_norm": (1 + 0.1 * rng.standard_normal(s.hidden)).astype(np.float32)}
+        host_layers.append(h)
+        dims = {"wq": (s.hidden, s.hidden), "wk": (s.kv_dim, s.hidden), "wv": (s.kv_dim, s.hidden), "wo": (s.hidden, s.hidden),
+                "w_gate": (s.ffn, s.hidden), "w_up": (s.ffn, s.hidden), "w_down": (s.hidden, s.ffn)}
+        dev_layers.append(LayerWeights(**{n: hip.upload_weight(orc.Q4_K, h[n], *dims[n]) for n in dims},
+                                       attn_norm=hip.upload(h["attn_norm"]), ffn_norm=hip.upload(h["ffn_norm"])))
+    final_norm = (1 + 0.1 * rng.standard_normal(s.hidden)).astype(np.float32)
+    head = qmat(orc.Q6_K, s.vocab, s.hidden)
+    weights = ModelWeights(dev_layers, hip.upload(final_norm), hip.upload_weight(orc.Q6_K, head, s.vocab, s.hidden))
+    step = DecodeStep(hip, s, weights, ctx)
+    kv0 = [(rng.standard_normal((ctx, s.kv_dim), dtype=np.float32).astype(np.float16), rng.standard_normal((ctx, s.kv_dim), dtype=np.float32).astype(np.float16))
+           for _ in range(s.n_layers)]
+    x0 = rng.standard_normal(s.hidden, dtype=np.float32)
+
+    # ---- numpy + oracle reference
+    mv = lambda t, W, x, n, k: orc.matvec(t, orc.ACT_Q8, W, x, n, k)
+    x = x0.copy()
+    for li, h in enumerate(host_layers):
+        kc, vc = kv0[li][0].copy(), kv0[li][1].copy()
+        xn = rmsnorm_ref(x, h["attn_norm"], s.eps)
+        q = rope_ref(mv(orc.Q4_K, h["wq"], xn, s.hidden, s.hidden), s.n_heads, s.head_dim, pos, s.rope_theta)
+        k = rope_ref(mv(orc.Q4_K, h["wk"], xn, s.kv_dim, s.hidden), s.n_kv_heads, s.head_dim, pos, s.rope_theta)
+        v = mv(orc.Q4_K, h["wv"], xn, s.kv_dim, s.hidden)
+        kc[pos], vc[pos] = k.astype(np.float16), v.astype(np.float16)
+        att = attention_ref(q, kc, vc, s.n_heads, s.n_kv_heads, s.head_dim, pos + 1)
+        x = x + mv(orc.Q4_K, h["wo"], att, s.hidden, s.hidden)
+        xn = rmsnorm_ref(x, h["ffn_norm"], s.eps)
+        g, u = mv(orc.Q4_K, h["w_gate"], xn, s.ffn, s.hidden), mv(orc.Q4_K, h["w_up"], xn, s.ffn, s.hidden)
+        act = (g.astype(np.float64) / (1 + np.exp(-g.astype(np.float64))) * u).astype(np.float32)
+        x = x + mv(orc.Q4_K, h["w_down"], act, s.hidden, s.ffn)
+    ref_logits = mv(orc.Q6_K, head, rmsnorm_ref(x, final_norm, s.eps), s.vocab, s.hidden)
+
+    def reset():
+        for li in range(s.n_layers):
+            step.k_cache[li].upload(kv0[li][0])
+            step.v_cache[li].upload(kv0[li][1])
+        step.x.upload(x0)
+
+    reset()
+    step.enqueue(pos)
+    eager = step.logits.download(np.float32, (s.vocab,))
+    # activations are re-quantized to int8 after every op, so tiny differences can flip a rounding
+    # now and then; the logits must still agree to well inside the 1e-3 gate
+    err = G.max_rel_err(eager, ref_logits)
+    say(f"small decode step: logits max_rel_err={err:.3e}")
+    assert err < 1e-3
+    assert int(np.argmax(eager)) == int(np.argmax(ref_logits))
+
+    graph = step.capture(pos)
+    try:
+        for _ in range(3):
+            reset()
+            hip.launch_graph(graph)
+            replay = step.logits.download(np.float32, (s.vocab,))
+            assert np.array_equal(replay, eager)
+            hip.swiglu(step.gate, step.up, step.act, s.ffn)      # eager work between replays
+            hip.sync()
+    finally:
+        hip.destroy_graph(graph)

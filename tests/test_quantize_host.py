@@ -17,3 +17,26 @@ def test_numpy_q4_0_and_q8_0_match_oracle_bit_for_bit(orc):
     x = G.seeded_acts(701, 4, 4096)
     assert np.array_equal(quantize.quantize_q8_0(x), orc.quantize(orc.Q8_0, x))
     assert np.array_equal(quantize.quantize_q4_0(x), orc.quantize(orc.Q4_0, x))
+
+
+def test_numpy_k_quant_producers_are_valid_and_close(orc):
+    """The simple Q4_K / Q6_K producers (no scale search) must emit blocks the oracle's dequantizer
+    reads back close to the input: the element-index parsers pin the byte layout, the error bounds
+    pin the scale/min arithmetic."""
+    w = G.seeded_weights(710, 16, 1024)
+    w[0, :256] = 0
+    w[1, :32] = np.abs(w[1, :32])                       # an all-positive sub-block: min stays 0
+    r4 = quantize.quantize_q4_K(w)
+    d, dmin, sc, mn, q = G.parse_q4_K(r4, 1024)
+    assert sc.max() <= 63 and mn.max() <= 63 and q.max() <= 15 and np.all(d >= 0) and np.all(dmin >= 0)
+    y4 = orc.dequantize(orc.Q4_K, r4, 1024)
+    assert np.sqrt(np.mean((y4 - w) ** 2)) / np.sqrt(np.mean(w ** 2)) < 0.10
+    step = (d[:, :, None] * sc).repeat(32, axis=2).reshape(16, 1024)
+    assert np.all(np.abs(y4 - w) <= step + 1e-6)
+    assert not y4[0, :256].any()
+    r6 = quantize.quantize_q6_K(w)
+    d6, s6, q6 = G.parse_q6_K(r6, 1024)
+    assert q6.min() >= -32 and q6.max() <= 31
+    y6 = orc.dequantize(orc.Q6_K, r6, 1024)
+    assert np.sqrt(np.mean((y6 - w) ** 2)) / np.sqrt(np.mean(w ** 2)) < 0.03
+    assert not y6[0, :256].any()
