@@ -77,82 +77,97 @@ extern "C" __global__ void __launch_bounds__(256) psn_rope_kv_store(const psn_ro
     }
 }
 
-/* Attention of one new token over cache positions 0 .. n_ctx-1, head_dim 128, up to 8 query heads
- * per kv head.  Workgroup = one wave = (kv head, 64 consecutive positions): lane p scores its
- * position against all query heads of the group (one K row of 256 bytes in registers), then lanes
- * switch to two output dims each and accumulate exp(score - max) * V.  Writes the unnormalized
- * partial output plus (max, sum) per head and split. */
-extern "C" __global__ void __launch_bounds__(64) psn_attn_partial(const psn_attn_args a) {
-    constexpr int D = 128, MAXG = 8;
-    __shared__ float qs[MAXG][D];
-    __shared__ float es[MAXG][64];
-    const int lane = threadIdx.x;
+/* Attention of one new token over cache positions 0 .. n_ctx-1, head_dim 128.  Workgroup = (kv head,
+ * 64 consecutive positions), one wave per query head of the group (up to 8).  A wave first scores
+ * its head: lane p takes position p (one K row of 256 bytes in registers, the query read from LDS
+ * as broadcasts); then the lanes switch to two output dims each and accumulate
+ * exp(score - max) * V, the weights handed from lane to lane with v_readlane.  Everything the wave
+ * needs from the cache -- its K row and its two dims of all 64 V rows -- is requested up front,
+ * so the kernel pays one memory round trip.  Rows past the context re-read the last valid one and
+ * get weight 0.  Writes the unnormalized partial output plus (max, sum) per head and split. */
+extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_attn_args a) {
+    constexpr int D = 128;
+    __shared__ float qs[8][D];
+    const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
     const int kvh = blockIdx.x % a.n_kv_heads, split = blockIdx.x / a.n_kv_heads;
-    const int group = a.n_heads / a.n_kv_heads;
-    for (int i = lane; i < group * D; i += 64) qs[i / D][i % D] = a.q[(kvh * group + i / D) * D + (i % D)];
-    __syncthreads();
+    const int group = a.n_heads / a.n_kv_heads;                  /* == blockDim.x / 64 */
+    const int head = kvh * group + g;
     const int p = split * 64 + lane;
     const bool live = p < a.n_ctx;
-    float s[MAXG];
-    UNROLL for (int g = 0; g < MAXG; ++g) s[g] = 0.f;
+    const int last = a.n_ctx - 1 - split * 64;                   /* last valid position of this split, >= 0 */
+    uint4 kreg[16];
     {
-        const uint4 *krow = reinterpret_cast<const uint4 *>(reinterpret_cast<const f16 *>(a.k_cache) + ((int64_t)(live ? p : 0) * a.n_kv_heads + kvh) * D);
-        UNROLL for (int c = 0; c < 16; ++c) {
-            const uint4 kv = krow[c];
-            const u32 kw[4] = {kv.x, kv.y, kv.z, kv.w};
-            UNROLL for (int j = 0; j < 4; ++j) {
-                const float k0 = h2f_lo(kw[j]), k1 = h2f_hi(kw[j]);
-                UNROLL for (int g = 0; g < MAXG; ++g)
-                    if (g < group) s[g] += k0 * qs[g][8 * c + 2 * j] + k1 * qs[g][8 * c + 2 * j + 1];
-            }
-        }
+        const uint4 *krow = reinterpret_cast<const uint4 *>(reinterpret_cast<const f16 *>(a.k_cache) + ((int64_t)(split * 64 + min(lane, last)) * a.n_kv_heads + kvh) * D);
+        UNROLL for (int c = 0; c < 16; ++c) kreg[c] = krow[c];
     }
-    float mx[MAXG], sum[MAXG];
-    UNROLL for (int g = 0; g < MAXG; ++g) {
-        if (g < group) {
-            const float sc = live ? s[g] * a.scale : -INFINITY;
-            const float m = group_max<64>(sc);
-            const float e = live ? __expf(sc - m) : 0.f;
-            mx[g] = m;
-            sum[g] = group_sum<64>(e);
-            es[g][lane] = e;
-        }
+    u32 vreg[64];
+    {
+        const u32 *vbase = reinterpret_cast<const u32 *>(reinterpret_cast<const f16 *>(a.v_cache) + ((int64_t)split * 64 * a.n_kv_heads + kvh) * D) + lane;
+        const int64_t vstride = (int64_t)a.n_kv_heads * D / 2;   /* dwords between positions */
+        UNROLL for (int i = 0; i < 64; ++i) vreg[i] = vbase[(int64_t)min(i, last) * vstride];
     }
+    qs[g][lane] = a.q[head * D + lane];
+    qs[g][lane + 64] = a.q[head * D + lane + 64];
     __syncthreads();
-    float o0[MAXG], o1[MAXG];
-    UNROLL for (int g = 0; g < MAXG; ++g) o0[g] = o1[g] = 0.f;
-    const int np = min(64, a.n_ctx - split * 64);
-    const u32 *vbase = reinterpret_cast<const u32 *>(reinterpret_cast<const f16 *>(a.v_cache) + ((int64_t)split * 64 * a.n_kv_heads + kvh) * D) + lane;
-    const int64_t vstride = (int64_t)a.n_kv_heads * D / 2;       /* dwords between positions */
-    for (int i = 0; i < np; ++i) {
-        const u32 vv = vbase[i * vstride];
-        const float v0 = h2f_lo(vv), v1 = h2f_hi(vv);
-        UNROLL for (int g = 0; g < MAXG; ++g)
-            if (g < group) { const float e = es[g][i]; o0[g] += e * v0; o1[g] += e * v1; }
+    float s = 0.f;
+    UNROLL for (int c = 0; c < 16; ++c) {
+        const u32 kw[4] = {kreg[c].x, kreg[c].y, kreg[c].z, kreg[c].w};
+        const float4 qa = *reinterpret_cast<const float4 *>(&qs[g][8 * c]), qb = *reinterpret_cast<const float4 *>(&qs[g][8 * c + 4]);
+        s += h2f_lo(kw[0]) * qa.x + h2f_hi(kw[0]) * qa.y + h2f_lo(kw[1]) * qa.z + h2f_hi(kw[1]) * qa.w;
+        s += h2f_lo(kw[2]) * qb.x + h2f_hi(kw[2]) * qb.y + h2f_lo(kw[3]) * qb.z + h2f_hi(kw[3]) * qb.w;
     }
-    UNROLL for (int g = 0; g < MAXG; ++g) {
-        if (g < group) {
-            const int head = kvh * group + g;
-            float *dst = a.partial + ((int64_t)head * a.n_splits + split) * (D + 2);
-            dst[2 * lane] = o0[g];
-            dst[2 * lane + 1] = o1[g];
-            if (lane == 0) { dst[D] = mx[g]; dst[D + 1] = sum[g]; }
-        }
+    const float sc = live ? s * a.scale : -INFINITY;
+    const float m = group_max<64>(sc);
+    const float e = live ? __expf(sc - m) : 0.f;                 /* lane i holds the weight of position i */
+    const float sum = group_sum<64>(e);
+    float o0 = 0.f, o1 = 0.f;
+    UNROLL for (int i = 0; i < 64; ++i) {
+        const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), i));
+        o0 += w * h2f_lo(vreg[i]);
+        o1 += w * h2f_hi(vreg[i]);
     }
+    float *dst = a.partial + ((int64_t)head * a.n_splits + split) * (D + 2);
+    dst[2 * lane] = o0;
+    dst[2 * lane + 1] = o1;
+    if (lane == 0) { dst[D] = m; dst[D + 1] = sum; }
 }
 
-/* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One workgroup of 128 threads per head. */
+/* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One workgroup of 128 threads per
+ * head: the per-split (max, sum) pairs are fetched in parallel, the weights go through LDS, and the
+ * partial outputs are summed eight loads at a time. */
 extern "C" __global__ void __launch_bounds__(128) psn_attn_combine(const psn_attn_args a) {
     constexpr int D = 128;
+    __shared__ float wts[128];
+    __shared__ float red[4];
     const int head = blockIdx.x, d = threadIdx.x;
     const float *base = a.partial + (int64_t)head * a.n_splits * (D + 2);
-    float M = -INFINITY;
-    for (int s = 0; s < a.n_splits; ++s) M = fmaxf(M, base[s * (D + 2) + D]);
     float num = 0.f, den = 0.f;
-    for (int s = 0; s < a.n_splits; ++s) {
-        const float w = __expf(base[s * (D + 2) + D] - M);
-        num += base[s * (D + 2) + d] * w;
-        den += base[s * (D + 2) + D + 1] * w;
+    /* global max first (splits are few: a strided pass per thread, then a block reduce) */
+    float m = -INFINITY;
+    for (int s = d; s < a.n_splits; s += 128) m = fmaxf(m, base[(int64_t)s * (D + 2) + D]);
+    m = group_max<64>(m);
+    if ((d & 63) == 0) red[d >> 6] = m;
+    __syncthreads();
+    const float M = fmaxf(red[0], red[1]);
+    for (int s0 = 0; s0 < a.n_splits; s0 += 128) {
+        const int s = s0 + d;
+        float w = 0.f, l = 0.f;
+        if (s < a.n_splits) {
+            w = __expf(base[(int64_t)s * (D + 2) + D] - M);
+            l = base[(int64_t)s * (D + 2) + D + 1] * w;
+        }
+        __syncthreads();                                          /* wts from the previous round is consumed */
+        wts[d] = w;
+        l = group_sum<64>(l);
+        if ((d & 63) == 0) red[2 + (d >> 6)] = l;
+        __syncthreads();
+        den += red[2] + red[3];
+        const int cnt = min(128, a.n_splits - s0);
+        for (int i0 = 0; i0 < cnt; i0 += 8) {
+            float o[8];
+            UNROLL for (int u = 0; u < 8; ++u) o[u] = base[(int64_t)(s0 + min(i0 + u, cnt - 1)) * (D + 2) + d];
+            UNROLL for (int u = 0; u < 8; ++u) if (i0 + u < cnt) num += o[u] * wts[i0 + u];
+        }
     }
     a.out[head * D + d] = num / den;
 }

@@ -989,7 +989,7 @@ extern "C" int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const ps
     a.n_ctx = n_ctx;
     a.n_splits = splits;
     a.scale = 0.08838834764831845f;                 /* 1/sqrt(128) */
-    if ((rc = launch(mod, s, "psn_attn_partial", (unsigned)(n_kv_heads * splits), 64, 0, &a))) return rc;
+    if ((rc = launch(mod, s, "psn_attn_partial", (unsigned)(n_kv_heads * splits), (unsigned)(64 * (n_heads / n_kv_heads)), 0, &a))) return rc;
     return launch(mod, s, "psn_attn_combine", (unsigned)n_heads, 128, 0, &a);
 }
 
