@@ -30,8 +30,8 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by
-# what the same counter reads for a 256 MiB device-to-device copy: x1.9998 and x1.0000).  The
-# figures and the commands are in profiles/matvec_q4_0_llama3_8b_step.md.
+# what the same counter reads for a 256 MiB device-to-device copy: x1.9998 and x1.0000; the copies
+# are what --calibrate-copy adds to a run).
 MEASURED_TRAFFIC_BYTES = {"qkv": 14.45e6 + 24.0 * 1024, "o": 9.74e6 + 16.0 * 1024,
                           "gate_up": 66.38e6 + 114.2 * 1024, "down": 33.67e6 + 17.0 * 1024}
 HIDDEN, KV, FFN, LAYERS = 4096, 1024, 14336, 32
@@ -70,7 +70,7 @@ def main(argv=None):
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this build drives one GPU; --gpus N with N > 1 is not supported "
-              "(the path shards by rows across GPUs, see DESIGN.md, but nothing here launches a second rank)", file=sys.stderr)
+              "(the path would shard by weight rows across GPUs, but nothing here launches a second rank)", file=sys.stderr)
         return 2
 
     from openagents_amd import _ffi

@@ -110,3 +110,10 @@ def test_missing_library_is_an_error_not_a_fallback(monkeypatch):
     monkeypatch.setattr(_ffi, "LIB_PATH", "/nonexistent/libpsn_hip.so")
     with pytest.raises(_ffi.LibraryMissing):
         _ffi.load()
+
+
+def test_integration_doc_binding_lists_every_entry_point():
+    """The Rust `-sys` text a maintainer would paste must not drift from the header."""
+    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    rust = set(re.findall(r"pub fn (psn_[a-z0-9_]+)\(", doc))
+    assert rust == set(header_functions())
