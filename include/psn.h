@@ -181,7 +181,11 @@ typedef struct psn_matvec_plan {
     int32_t stage_lds;      /* scheme Q8 only. 0: quantized x read from global memory; 1: staged in LDS;
                                2: x is fp32 and every workgroup quantizes it while staging */
     int32_t blocks;         /* workgroups */
-    int32_t threads;        /* threads per workgroup: 256 or 512 */
+    int32_t threads;        /* threads per workgroup: 256 or 512 (256, 512 or 768 with `stream`) */
+    int32_t stream;         /* 1: weights land in per-wave LDS buffers by direct-to-LDS loads (scheme Q8,
+                               batch 1, Q4_0/Q8_0/Q4_K, rows of at most lanes_per_row chunks, every matrix a
+                               multiple of 64/lanes_per_row rows, stage_lds 1 or 2); 0: register kernels */
+    int32_t reserved;
 } psn_matvec_plan;
 int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t compute_units,
                          int32_t x_is_f32, psn_matvec_plan *out);

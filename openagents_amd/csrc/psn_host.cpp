@@ -598,7 +598,9 @@ static int64_t staged_lds_bytes(int32_t qtype, int64_t K, int32_t batch) {
     return qs + d + align_up(sb, 16);
 }
 
-static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, bool fuse_quantize, psn_matvec_plan *out) {
+/* n_rows: the row counts of the matrices sharing the launch (count of them), or null when unknown */
+static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, bool fuse_quantize,
+                         const int64_t *n_rows, int32_t count, psn_matvec_plan *out) {
     int32_t rc = check_matvec_shape(qtype, scheme, N, K, batch);
     if (rc) return rc;
     if (cus <= 0) cus = 256;
@@ -606,8 +608,13 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
     psn_matvec_plan p;
     p.batch_tile = batch <= 1 ? 1 : batch <= 2 ? 2 : batch <= 4 ? 4 : 8;
     p.rows_in_flight = 1;
-    const bool lds_fits = scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 64 * 1024;
-    p.stage_lds = lds_fits ? (fuse_quantize ? 2 : 1) : 0;
+    p.stream = 0;
+    p.reserved = 0;
+    /* the staged activations may take the whole 160 KB of a compute unit's LDS (batch 8 at K = 14336
+     * needs 140 KB); re-quantizing inside the launch only pays up to batch 2 -- beyond that every
+     * workgroup would redo batch x K of quantization, and one extra launch is cheaper (measured) */
+    const bool lds_fits = scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 160 * 1024;
+    p.stage_lds = lds_fits ? ((fuse_quantize && batch <= 2) ? 2 : 1) : 0;
     /* lanes per row: the row's chunk count rounded up to a power of two, widened (idle lanes, more
      * waves) until the launch offers about four waves per compute unit */
     int g = C <= 8 ? 8 : C <= 16 ? 16 : C <= 32 ? 32 : 64;
@@ -624,11 +631,26 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
         blocks = (waves + wpb - 1) / wpb;
         const int64_t cap = small_groups ? 2 * (int64_t)cus : (int64_t)cus;
         if (blocks > cap) blocks = cap;
+        /* tall matrices with short rows: the direct-to-LDS streaming kernel wins once every wave has
+         * several passes to pipeline (measured: 2 x 14336 x 4096 Q4_0, 15.3 us against 16.4 us) */
+        bool can_stream = small_groups && batch == 1 && qtype != PSN_Q6_K && C <= g && n_rows != nullptr;
+        for (int i = 0; can_stream && i < count; ++i) can_stream = n_rows[i] % (64 / g) == 0;
+        if (can_stream) {
+            p.stream = 1;
+            p.threads = 512;
+            blocks = 2 * (int64_t)cus;
+        }
     } else {
         /* small workgroups, one pass per wave where the chip can hold them */
         p.threads = 256;
         blocks = (waves + 3) / 4;
         if (blocks > 4 * (int64_t)cus) blocks = 4 * (int64_t)cus;
+        if (staged_lds_bytes(qtype, K, batch) > 40 * 1024) {
+            /* a big staged copy limits how many workgroups fit a compute unit: fewer, larger ones */
+            p.threads = 512;
+            blocks = (waves + 7) / 8;
+            if (blocks > (int64_t)cus) blocks = cus;
+        }
     }
     p.lanes_per_row = g;
     p.blocks = (int32_t)blocks;
@@ -639,14 +661,14 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
 extern "C" int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus,
                                     int32_t x_is_f32, psn_matvec_plan *out) {
     if (!out) return fail(PSN_E_INVALID_ARG, "psn_qmatvec_plan: out is null");
-    return make_plan(qtype, scheme, N, K, batch, cus, x_is_f32 != 0 && scheme == PSN_ACT_Q8, out);
+    return make_plan(qtype, scheme, N, K, batch, cus, x_is_f32 != 0 && scheme == PSN_ACT_Q8, &N, 1, out);
 }
 
 static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t scheme, int64_t K, int32_t batch, int max_lds, int32_t *lds_out) {
     const int g = p->lanes_per_row, r = p->rows_in_flight, nb = p->batch_tile;
     if (!(g == 8 || g == 16 || g == 32 || g == 64)) return fail(PSN_E_UNSUPPORTED, "plan: lanes_per_row=%d", g);
     if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
-    if (p->threads != 256 && p->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
+    if (p->threads != 256 && p->threads != 512 && !(p->stream && p->threads == 768)) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
     bool ok;
     if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2 || r == 4)) || (nb > 1 && r == 1);
     else ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
@@ -693,6 +715,36 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
     a.nseg = sg.count;
     a.row_bytes = psn_row_bytes(qtype, K);
     char name[96];
+    if (plan->stream) {
+        const int g = plan->lanes_per_row, rows = 64 / g;
+        const int64_t C = K / 256;
+        if (scheme != PSN_ACT_Q8 || batch != 1 || plan->batch_tile != 1 || plan->rows_in_flight != 1)
+            return fail(PSN_E_UNSUPPORTED, "plan: the streaming kernels serve scheme Q8 at batch 1");
+        if (qtype == PSN_Q6_K) return fail(PSN_E_UNSUPPORTED, "plan: no streaming kernel for Q6_K (rows are not 16-byte multiples)");
+        if (C > g) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs rows of at most lanes_per_row chunks (K <= %d)", g * 256);
+        if (plan->stage_lds != 1 && plan->stage_lds != 2) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs stage_lds 1 or 2");
+        if (plan->threads != 256 && plan->threads != 512 && plan->threads != 768) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d", plan->threads);
+        for (int i = 0; i < sg.count; ++i)
+            if (sg.N[i] % rows) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs every matrix to hold a multiple of %d rows", rows);
+        const int32_t at = psn_act_type_for(qtype);
+        const int64_t be = psn_block_elems(at);
+        const int64_t n_d = ((K / be) * 4 + 15) / 16, n_s = ((at == PSN_Q8_0 ? (K / 32) * 4 : (K / 16) * 2) + 15) / 16;
+        const int64_t stage = (C * 272 + (n_d + n_s) * 16 + 1023) / 1024 * 1024;
+        const int64_t wbuf = (rows * a.row_bytes + 1023) / 1024 * 1024;
+        const int64_t total = stage + (plan->threads / 64) * wbuf;
+        if (total > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs %lld bytes of LDS, device offers %d", (long long)total, mod->ctx->max_lds);
+        if (plan->stage_lds == 2) {
+            a.xf = (const float *)x;
+        } else {
+            psn_actq_info li;
+            if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;
+            a.xqs = (const int8_t *)x + li.off_qs;
+            a.xd = (const float *)((const char *)x + li.off_d);
+            a.xs = (const char *)x + li.off_s;
+        }
+        snprintf(name, sizeof name, "psn_mvs_%s_q8_g%d_%s", fmt_name(qtype), g, plan->stage_lds == 2 ? "xf" : "lds");
+        return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)total, &a);
+    }
     if (scheme == PSN_ACT_Q8 && plan->stage_lds == 2) {
         a.xf = (const float *)x;
         snprintf(name, sizeof name, "psn_mv_%s_q8_g%d_r%d_b%d_xf", fmt_name(qtype), plan->lanes_per_row, plan->rows_in_flight, plan->batch_tile);
@@ -771,7 +823,7 @@ extern "C" int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t 
     if (rc) return rc;
     if ((rc = check_x_q8("psn_qmatvec_q8_multi", qtype, xq, K, batch))) return rc;
     psn_matvec_plan plan;
-    if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, batch, mod->ctx->compute_units, false, &plan))) return rc;
+    if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, batch, mod->ctx->compute_units, false, sg.N, sg.count, &plan))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
     return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, xq->p, K, batch, &plan);
 }
@@ -790,7 +842,7 @@ extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qty
     if (rc) return rc;
     if ((rc = check_x_f32("psn_qmatvec", x, K, batch))) return rc;
     psn_matvec_plan plan;
-    if ((rc = make_plan(qtype, scheme, sg.total, K, batch, mod->ctx->compute_units, true, &plan))) return rc;
+    if ((rc = make_plan(qtype, scheme, sg.total, K, batch, mod->ctx->compute_units, true, sg.N, sg.count, &plan))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
     if (scheme == PSN_ACT_F32) return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
     /* one launch when the staged copy fits LDS: every workgroup quantizes x while staging it */

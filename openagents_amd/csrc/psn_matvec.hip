@@ -188,7 +188,7 @@ struct ActQ {
  * ST = int selects Q8_0 activations (d and s per 32), ST = int16_t Q8_K (d per 256, bsums per 16).
  * Up to SLOTS 16-byte words per thread are held in registers; larger inputs (long K, batch > 1 on
  * small workgroups) take the plain copy loop in finish(). */
-template <typename ST, int XSRC>
+template <typename ST, int XSRC, bool REGS = true>
 struct Stager {
     static constexpr int SLOTS = 8;
     uint4 t[SLOTS];
@@ -202,6 +202,7 @@ struct Stager {
         n_d = (a.batch * d_per_col * 4 + 15) / 16;                 /* the global fields are padded to 256 B */
         n_s = (a.batch * s_per_col * (int)sizeof(ST) + 15) / 16;
         in_regs = false;
+        if constexpr (!REGS) return;                               /* finish() does plain copy loops */
         UNROLL for (int i = 0; i < SLOTS; ++i) t[i] = make_uint4(0, 0, 0, 0);
         td = ts = make_uint4(0, 0, 0, 0);
         if constexpr (XSRC == 1) {
@@ -673,6 +674,94 @@ PSN_DEV void mv_q8(const psn_matvec_args &a) {
     PSN_STAMP(a, m, 4);
 }
 
+/* Scheme Q8, streaming variant (batch 1, rows of at most G chunks).  The weights do not pass through
+ * registers on their way in: each wave owns an LDS buffer that holds the 64/G rows of one pass and
+ * fills it with 16-byte direct-to-LDS loads (lanes fetch consecutive 16-byte words, so every load
+ * instruction covers 1 KB of contiguous row bytes).  Per pass: wait for the buffer, copy the lane's
+ * chunk into registers, immediately start the next pass's loads into the same buffer, then do the
+ * dot products -- the memory latency of pass p+1 runs under the arithmetic of pass p without a
+ * second register set.  The lane's activation chunk is read from the staged copy once and kept.
+ * One workgroup per compute unit (LDS-limited); waves stride over the passes. */
+template <typename F, int G, int XSRC>
+PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
+    typedef typename F::ActSum ST;
+    constexpr int S = 64 / G;                                /* rows per pass; every matrix holds a multiple of S rows */
+    extern __shared__ uint4 psn_smem[];
+    const int lane = threadIdx.x & 63, slot = lane / G, j = lane % G;
+    const int wpb = blockDim.x >> 6;
+    const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   /* wave-uniform, and the compiler should know it */
+    const int K = a.K, C = K >> 8, N = a.N;
+    const int rb = (int)a.row_bytes;                         /* bytes per row; a multiple of 16 */
+    const int span = S * rb, nloads = (span + 1023) >> 10;   /* bytes and 1 KB load instructions per pass */
+    const int wbuf = nloads << 10;
+    const int npass = N / S;
+    const int stride = gridDim.x * wpb;
+    int p = blockIdx.x * wpb + wib;
+
+    /* where the wave buffers start: right behind the staged activations (same arithmetic as the host) */
+    const int n_d = (F::d_per_col(K) * 4 + 15) / 16, n_s = (F::s_per_col(K) * (int)sizeof(ST) + 15) / 16;
+    const int stage_bytes = ((C * 272 + (n_d + n_s) * 16 + 1023) >> 10) << 10;
+    char *buf = reinterpret_cast<char *>(psn_smem) + stage_bytes + wib * wbuf;
+
+    /* a pass never straddles two matrices, so its rows are one contiguous range of one of them;
+     * all of this is scalar arithmetic on kernel arguments */
+    /* The four base pointers are pinned in scalar registers (the empty asm keeps the compiler from
+     * turning the selects below back into an indexed load from a private copy of the arguments). */
+    const uint8_t *W0 = a.W[0], *W1 = a.W[1], *W2 = a.W[2], *W3 = a.W[3];
+    float *Y0 = a.y[0], *Y1 = a.y[1], *Y2 = a.y[2], *Y3 = a.y[3];
+    int E0 = a.row_end[0], E1 = a.row_end[1], E2 = a.row_end[2];
+    asm volatile("" : "+s"(W0), "+s"(W1), "+s"(W2), "+s"(W3), "+s"(Y0), "+s"(Y1), "+s"(Y2), "+s"(Y3), "+s"(E0), "+s"(E1), "+s"(E2));
+    const int nseg = a.nseg;
+    auto pass_base = [&](int pass, const uint8_t *&w, float *&y) {
+        const int row0 = pass * S;
+        const uint8_t *wb = W0;
+        float *yb = Y0;
+        int first = 0;
+        if (nseg > 1 && row0 >= E0) { wb = W1; yb = Y1; first = E0; }
+        if (nseg > 2 && row0 >= E1) { wb = W2; yb = Y2; first = E1; }
+        if (nseg > 3 && row0 >= E2) { wb = W3; yb = Y3; first = E2; }
+        w = wb + (int64_t)(row0 - first) * rb;
+        y = yb + (row0 - first);
+    };
+    /* straight-line issue: up to F::DW / 4 (+1 when G > chunks leaves a ragged tail) predicated loads */
+    auto issue = [&](const uint8_t *w) {
+        const uint8_t *src = w + lane * 16;
+        UNROLL for (int i = 0; i < F::DW / 4 + 1; ++i)
+            if (i * 1024 + lane * 16 < span)
+                __builtin_amdgcn_global_load_lds((const void *)(src + i * 1024), (__attribute__((address_space(3))) void *)(buf + i * 1024), 16, 0, 0);
+    };
+
+    Stager<ST, XSRC, false> st;                                  /* staged after the first loads are on their way */
+    st.issue(a, F::d_per_col(K), F::s_per_col(K));
+    const uint8_t *wsrc = nullptr;
+    float *ydst = nullptr;
+    if (p < npass) {
+        pass_base(p, wsrc, ydst);
+        issue(wsrc);
+    }
+    const ActQ<ST> x = st.finish(a);
+    u32 xr[F::XR];
+    UNROLL for (int i = 0; i < F::XR; ++i) xr[i] = 0;
+    if (j < C) F::load_x(x, K, 0, j, xr);
+    while (p < npass) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 /* this pass's rows are in the buffer */
+        u32 w[F::DW];
+        UNROLL for (int i = 0; i < F::DW; ++i) w[i] = 0;
+        if (j < C) F::load(reinterpret_cast<const uint8_t *>(buf) + slot * rb + j * F::BYTES, w);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");               /* ... and in registers: the buffer is free */
+        float *ycur = ydst;
+        const int pn = p + stride;
+        if (pn < npass) {
+            pass_base(pn, wsrc, ydst);
+            issue(wsrc);
+        }
+        float acc = (j < C) ? F::dot(w, xr) : 0.f;
+        acc = group_sum<G>(acc);
+        if (j == 0) ycur[slot] = acc;
+        p = pn;
+    }
+}
+
 /* Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations. */
 template <typename F, int SB, int R, int NB>
 PSN_DEV void f32_step(const u32 (&w)[R][F::DW], const float *xf, int K, int k0, int batch, float (&acc)[R][NB]) {
@@ -734,6 +823,15 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
         mv_q8<F, G, R, NB, 2>(a);                                                                         \
     }
 
+#define PSN_STREAM_KERNEL(fmt, F, G)                                                                      \
+    extern "C" __global__ void __launch_bounds__(768) psn_mvs_##fmt##_q8_g##G##_lds(const psn_matvec_args a) { \
+        mv_q8_stream<F, G, 1>(a);                                                                         \
+    }                                                                                                     \
+    extern "C" __global__ void __launch_bounds__(768) psn_mvs_##fmt##_q8_g##G##_xf(const psn_matvec_args a) {  \
+        mv_q8_stream<F, G, 2>(a);                                                                         \
+    }
+#define PSN_STREAM_ALL(fmt, F) PSN_STREAM_KERNEL(fmt, F, 8) PSN_STREAM_KERNEL(fmt, F, 16) PSN_STREAM_KERNEL(fmt, F, 32) PSN_STREAM_KERNEL(fmt, F, 64)
+
 #define PSN_F32_KERNEL(fmt, F, G, R, NB)                                                                  \
     extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
         mv_f32<F, G, R, NB>(a);                                                                           \
@@ -756,14 +854,17 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q4_0)
 PSN_Q8_ALL(q4_0, FmtQ4_0)
 PSN_F32_ALL(q4_0, FmtQ4_0)
+PSN_STREAM_ALL(q4_0, FmtQ4_0)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q8_0)
 PSN_Q8_ALL(q8_0, FmtQ8_0)
 PSN_F32_ALL(q8_0, FmtQ8_0)
+PSN_STREAM_ALL(q8_0, FmtQ8_0)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q4_K)
 PSN_Q8_ALL(q4_K, FmtQ4_K)
 PSN_F32_ALL(q4_K, FmtQ4_K)
+PSN_STREAM_ALL(q4_K, FmtQ4_K)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q6_K)
 PSN_Q8_ALL(q6_K, FmtQ6_K)

@@ -343,3 +343,52 @@ def test_graph_replay_matches_eager(hip, orc):
         hip.quantized_matvec(big, small, small, 1, _ffi.ACT_Q8)
     g2 = hip.end_capture()
     hip.destroy_graph(g2)
+
+
+# ------------------------------------------------------------------ streaming (direct-to-LDS) kernels
+
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K"])
+def test_streaming_kernels_every_variant(hip, orc, qname):
+    """Weights land in per-wave LDS buffers; rows per pass = 64 / lanes_per_row, so the matrices hold
+    multiples of 8 rows.  k = 2048 fills 8-lane groups exactly, k = 2560 (10 chunks) leaves idle lanes
+    and a ragged last 1 KB load; few workgroups force several passes per wave."""
+    t = getattr(orc, qname)
+    for k, ns in ((2048, [80]), (2560, [80, 8, 136, 16]), (4096, [1024, 256, 256]), (14336, [64])):
+        Ws = [weights(orc, qname, 900 + i, n, k) for i, n in enumerate(ns)]
+        x = G.seeded_acts(901, 1, k)
+        refs = [orc.matvec(t, orc.ACT_Q8, W, x, n, k) for W, n in zip(Ws, ns)]
+        ws = [hip.upload_weight(t, W, n, k) for W, n in zip(Ws, ns)]
+        xb = hip.upload(x)
+        xq = hip.quantize_activations(xb, k, 1, backend.act_type_for(t))
+        for g in (8, 16, 32, 64):
+            if k // 256 > g:
+                continue
+            for stage in (1, 2):
+                for threads, blocks in ((256, 2), (512, 1), (768, 3)):
+                    p = _ffi.MatvecPlan()
+                    p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream = g, 1, 1, stage, blocks, threads, 1
+                    say(f"stream {qname} k={k} ns={ns} {p.as_dict()}")
+                    ys = [hip.upload(np.full((1, n), np.nan, np.float32)) for n in ns]
+                    try:
+                        hip.quantized_matvec_planned(ws, xb if stage == 2 else xq, ys, 1, _ffi.ACT_Q8, p)
+                    except backend.PsnError as e:              # 12 waves x 17 KB of Q8_0 rows do not fit 160 KB
+                        assert e.code == _ffi.E_UNSUPPORTED and "LDS" in str(e) and qname == "Q8_0" and threads == 768
+                        continue
+                    for y, ref, n in zip(ys, refs, ns):
+                        err = G.max_rel_err(y.download(np.float32, (1, n)), ref)
+                        assert err < PARITY_TOL, (p.as_dict(), k, n, err)
+
+
+def test_streaming_plan_is_refused_where_it_cannot_run(hip, orc):
+    k = 2048
+    W = weights(orc, "Q6_K", 910, 80, k)
+    w6 = hip.upload_weight(orc.Q6_K, W, 80, k)
+    w4 = hip.upload_weight(orc.Q4_0, weights(orc, "Q4_0", 911, 84, k), 84, k)
+    x = hip.upload(np.zeros(k, np.float32))
+    y = hip.alloc(84 * 4)
+    p = _ffi.MatvecPlan()
+    p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream = 8, 1, 1, 2, 4, 256, 1
+    for w in (w6, w4):                                   # Q6_K has no streaming kernel; 84 rows is not a multiple of 8
+        with pytest.raises(backend.PsnError) as e:
+            hip.quantized_matvec_planned(w, x, y, 1, _ffi.ACT_Q8, p)
+        assert e.value.code == _ffi.E_UNSUPPORTED
