@@ -176,7 +176,7 @@ int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t qtype, int3
  * caller-chosen one (auto-tuners, benchmarks). */
 typedef struct psn_matvec_plan {
     int32_t lanes_per_row;  /* 8, 16, 32 or 64 lanes share one row */
-    int32_t rows_in_flight; /* row sets per lane: 1, 2 or 4 at batch_tile 1 (2 for scheme F32), else 1 */
+    int32_t rows_in_flight; /* row sets per lane: 1 or 2 at batch_tile 1, else 1 */
     int32_t batch_tile;     /* compiled batch width: 1, 2, 4 or 8 (>= batch) */
     int32_t stage_lds;      /* scheme Q8 only. 0: quantized x read from global memory; 1: staged in LDS;
                                2: x is fp32 and every workgroup quantizes it while staging */

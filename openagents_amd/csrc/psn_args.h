@@ -46,6 +46,8 @@ struct psn_matvec_args {
     int32_t batch;        /* live batch columns (<= the kernel's compiled NB) */
     int32_t nseg;
     int64_t row_bytes;
+    int32_t threads;      /* launch geometry, passed in so that kernels never read the dispatch packet */
+    int32_t blocks;
     uint64_t *timeline;   /* development builds (-DPSN_TIMELINE): per-wave clock stamps; otherwise unused, null */
 };
 

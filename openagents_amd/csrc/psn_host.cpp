@@ -670,7 +670,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
     if (p->threads != 256 && p->threads != 512 && !(p->stream && p->threads == 768)) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
     bool ok;
-    if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2 || r == 4)) || (nb > 1 && r == 1);
+    if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
     else ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
     if (!ok) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
@@ -714,6 +714,8 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
     a.batch = batch;
     a.nseg = sg.count;
     a.row_bytes = psn_row_bytes(qtype, K);
+    a.threads = plan->threads;
+    a.blocks = plan->blocks;
     char name[96];
     if (plan->stream) {
         const int g = plan->lanes_per_row, rows = 64 / g;

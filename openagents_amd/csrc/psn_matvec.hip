@@ -123,43 +123,70 @@ struct RowMap {
     static constexpr int S = 64 / G;          /* rows a wave holds side by side */
     static constexpr int ROWS = S * R;        /* rows a wave retires per pass */
     int lane, slot, j, wave, nwaves;
-    PSN_DEV RowMap() {
+    PSN_DEV RowMap(const psn_matvec_args &a) {
         lane = threadIdx.x & 63;
         slot = lane / G;
         j = lane % G;
-        const int wpb = blockDim.x >> 6;
+        const int wpb = a.threads >> 6;
         wave = blockIdx.x * wpb + (threadIdx.x >> 6);
-        nwaves = gridDim.x * wpb;
+        nwaves = a.blocks * wpb;
     }
 };
 
-/* row of the concatenated row space -> (segment, local row) */
-PSN_DEV int seg_of(const psn_matvec_args &a, int row) {
-    int s = 0;
-    if (a.nseg > 1 && row >= a.row_end[0]) s = 1;
-    if (a.nseg > 2 && row >= a.row_end[1]) s = 2;
-    if (a.nseg > 3 && row >= a.row_end[2]) s = 3;
-    return s;
+/* The per-matrix base pointers and row boundaries of a launch, pinned in scalar registers (plain
+ * locals of the kernel body, declared by this macro).  Lanes pick theirs with compares and selects;
+ * the empty asm keeps the compiler from folding the selects back into an indexed (vector-memory)
+ * load from a private copy of the kernel arguments, which would put memory round trips in front of
+ * the first weight load.  Unused segments repeat the last one (row_end == N), so no count check is
+ * needed.  seg_row_ptr(row): start of that row's blocks; seg_out_ptr(row, nrows): where its
+ * batch-column-0 output goes and how many rows its matrix has. */
+#define PSN_DECLARE_SEGMENTS(a)                                                                             \
+    const uint8_t *sgW0 = (a).W[0], *sgW1 = (a).W[1], *sgW2 = (a).W[2], *sgW3 = (a).W[3];                   \
+    float *sgY0 = (a).y[0], *sgY1 = (a).y[1], *sgY2 = (a).y[2], *sgY3 = (a).y[3];                           \
+    int sgE0 = (a).row_end[0], sgE1 = (a).row_end[1], sgE2 = (a).row_end[2], sgE3 = (a).row_end[3];         \
+    asm volatile("" : "+s"(sgW0), "+s"(sgW1), "+s"(sgW2), "+s"(sgW3), "+s"(sgY0), "+s"(sgY1), "+s"(sgY2),   \
+                 "+s"(sgY3), "+s"(sgE0), "+s"(sgE1), "+s"(sgE2), "+s"(sgE3));                               \
+    const int64_t sg_row_bytes = (a).row_bytes
+#define seg_row_ptr(row) seg_row_ptr_fn((row), sg_row_bytes, sgW0, sgW1, sgW2, sgW3, sgE0, sgE1, sgE2)
+#define seg_out_ptr(row, nrows) seg_out_ptr_fn((row), (nrows), sgY0, sgY1, sgY2, sgY3, sgE0, sgE1, sgE2, sgE3)
+
+PSN_DEV const uint8_t *seg_row_ptr_fn(int row, int64_t row_bytes, const uint8_t *w0, const uint8_t *w1, const uint8_t *w2,
+                                      const uint8_t *w3, int e0, int e1, int e2) {
+    const uint8_t *w = w0;
+    int first = 0;
+    if (row >= e0) { w = w1; first = e0; }
+    if (row >= e1) { w = w2; first = e1; }
+    if (row >= e2) { w = w3; first = e2; }
+    return w + (int64_t)(row - first) * row_bytes;
 }
-PSN_DEV const uint8_t *row_ptr(const psn_matvec_args &a, int row) {
-    const int s = seg_of(a, row);
-    const int local = row - (s ? a.row_end[s - 1] : 0);
-    return a.W[s] + (int64_t)local * a.row_bytes;
+PSN_DEV float *seg_out_ptr_fn(int row, int &rows_of_matrix, float *y0, float *y1, float *y2, float *y3, int e0, int e1, int e2, int e3) {
+    float *y = y0;
+    int first = 0, end = e0;
+    if (row >= e0) { y = y1; first = e0; end = e1; }
+    if (row >= e1) { y = y2; first = e1; end = e2; }
+    if (row >= e2) { y = y3; first = e2; end = e3; }
+    rows_of_matrix = end - first;
+    return y + (row - first);
 }
 
-template <int G, int R, int NB>
-PSN_DEV void store_rows(const RowMap<G, R> &m, float (&acc)[R][NB], const psn_matvec_args &a, int row0) {
-    UNROLL for (int r = 0; r < R; ++r) {
-        const int row = row0 + r * RowMap<G, R>::S + m.slot;
-        const int s = seg_of(a, row);
-        const int base = s ? a.row_end[s - 1] : 0;
-        const int nseg_rows = a.row_end[s] - base;
-        UNROLL for (int nb = 0; nb < NB; ++nb) {
-            const float v = group_sum<G>(acc[r][nb]);
-            if (m.j == 0 && row < a.N && nb < a.batch) a.y[s][(int64_t)nb * nseg_rows + (row - base)] = v;
-        }
+/* folds the G-lane partial sums of R row sets x NB batch columns and stores them */
+#define PSN_STORE_ROWS(m, acc, a, row0)                                                                     \
+    UNROLL for (int r_ = 0; r_ < R; ++r_) {                                                                 \
+        const int row_ = (row0) + r_ * (m).S + (m).slot;                                                    \
+        int nrows_;                                                                                         \
+        float *dst_ = seg_out_ptr(min(row_, (a).N - 1), nrows_);                                            \
+        UNROLL for (int nb_ = 0; nb_ < NB; ++nb_) {                                                         \
+            const float v_ = group_sum<G>((acc)[r_][nb_]);                                                  \
+            if ((m).j == 0 && row_ < (a).N && nb_ < (a).batch) dst_[(int64_t)nb_ * nrows_] = v_;            \
+        }                                                                                                   \
     }
-}
+
+/* one chunk (index c) of R rows starting at row0 into registers; rows past the end re-read the last one */
+#define PSN_LOAD_ROWS(F, m, a, row0, c, w)                                                                  \
+    UNROLL for (int r_ = 0; r_ < R; ++r_) {                                                                 \
+        const int row_ = min((row0) + r_ * (m).S + (m).slot, (a).N - 1);                                    \
+        F::load(seg_row_ptr(row_) + (int64_t)(c) * F::BYTES, (w)[r_]);                                      \
+    }
 
 /* Quantized activations as the kernels see them: either the global three-field layout or a copy
  * staged in LDS.  In LDS every 256-byte chunk of qs is followed by 16 bytes of padding, so lanes
@@ -193,11 +220,12 @@ struct Stager {
     static constexpr int SLOTS = 8;
     uint4 t[SLOTS];
     uint4 td, ts;
-    int n_qs, n_d, n_s, C;
+    int n_qs, n_d, n_s, C, nthreads;
     bool in_regs;
 
     PSN_DEV void issue(const psn_matvec_args &a, int d_per_col, int s_per_col) {
         C = a.K >> 8;
+        nthreads = a.threads;
         n_qs = a.batch * C * 16;                                   /* 16-byte words of int8 */
         n_d = (a.batch * d_per_col * 4 + 15) / 16;                 /* the global fields are padded to 256 B */
         n_s = (a.batch * s_per_col * (int)sizeof(ST) + 15) / 16;
@@ -206,11 +234,11 @@ struct Stager {
         UNROLL for (int i = 0; i < SLOTS; ++i) t[i] = make_uint4(0, 0, 0, 0);
         td = ts = make_uint4(0, 0, 0, 0);
         if constexpr (XSRC == 1) {
-            in_regs = n_qs <= SLOTS * (int)blockDim.x && n_d <= (int)blockDim.x && n_s <= (int)blockDim.x;
+            in_regs = n_qs <= SLOTS * nthreads && n_d <= nthreads && n_s <= nthreads;
             if (in_regs) {
                 const uint4 *g_qs = reinterpret_cast<const uint4 *>(a.xqs);
                 UNROLL for (int i = 0; i < SLOTS; ++i) {
-                    const int idx = threadIdx.x + i * blockDim.x;
+                    const int idx = threadIdx.x + i * nthreads;
                     if (idx < n_qs) t[i] = g_qs[idx];
                 }
                 if ((int)threadIdx.x < n_d) td = reinterpret_cast<const uint4 *>(a.xd)[threadIdx.x];
@@ -220,15 +248,15 @@ struct Stager {
             const float4 *x4 = reinterpret_cast<const float4 *>(a.xf);
             if constexpr (sizeof(ST) == 4) {
                 const int total4 = a.batch * C * 64;               /* float4 words: whole waves, whole blocks */
-                in_regs = total4 <= SLOTS * (int)blockDim.x;
+                in_regs = total4 <= SLOTS * nthreads;
                 if (in_regs) {
                     UNROLL for (int i = 0; i < SLOTS; ++i) {
-                        const int idx = threadIdx.x + i * blockDim.x;
+                        const int idx = threadIdx.x + i * nthreads;
                         if (idx < total4) { const float4 v = x4[idx]; t[i] = make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)); }
                     }
                 }
             } else {
-                const int nsb = a.batch * C, wpb = blockDim.x >> 6, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+                const int nsb = a.batch * C, wpb = nthreads >> 6, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
                 in_regs = nsb <= SLOTS * wpb;
                 if (in_regs) {
                     UNROLL for (int i = 0; i < SLOTS; ++i) {
@@ -257,15 +285,15 @@ struct Stager {
                 const uint4 *g_s = reinterpret_cast<const uint4 *>(a.xs);
                 if (in_regs) {
                     UNROLL for (int i = 0; i < SLOTS; ++i) {
-                        const int idx = threadIdx.x + i * blockDim.x;
+                        const int idx = threadIdx.x + i * nthreads;
                         if (idx < n_qs) l_qs4[(idx >> 4) * 17 + (idx & 15)] = t[i];
                     }
                     if ((int)threadIdx.x < n_d) l_d4[threadIdx.x] = td;
                     if ((int)threadIdx.x < n_s) l_s4[threadIdx.x] = ts;
                 } else {
-                    for (int i = threadIdx.x; i < n_qs; i += blockDim.x) l_qs4[(i >> 4) * 17 + (i & 15)] = g_qs[i];
-                    for (int i = threadIdx.x; i < n_d; i += blockDim.x) l_d4[i] = g_d[i];
-                    for (int i = threadIdx.x; i < n_s; i += blockDim.x) l_s4[i] = g_s[i];
+                    for (int i = threadIdx.x; i < n_qs; i += nthreads) l_qs4[(i >> 4) * 17 + (i & 15)] = g_qs[i];
+                    for (int i = threadIdx.x; i < n_d; i += nthreads) l_d4[i] = g_d[i];
+                    for (int i = threadIdx.x; i < n_s; i += nthreads) l_s4[i] = g_s[i];
                 }
             } else {
                 u32 *l_qs = reinterpret_cast<u32 *>(l_qs4);
@@ -285,14 +313,14 @@ struct Stager {
                     };
                     if (in_regs) {
                         UNROLL for (int k = 0; k < SLOTS; ++k) {
-                            const int i = threadIdx.x + k * blockDim.x;
+                            const int i = threadIdx.x + k * nthreads;
                             if (i < total4) one(i, make_float4(__uint_as_float(t[k].x), __uint_as_float(t[k].y), __uint_as_float(t[k].z), __uint_as_float(t[k].w)));
                         }
                     } else {
-                        for (int i = threadIdx.x; i < total4; i += blockDim.x) one(i, x4[i]);
+                        for (int i = threadIdx.x; i < total4; i += nthreads) one(i, x4[i]);
                     }
                 } else {
-                    const int nsb = a.batch * C, wpb = blockDim.x >> 6, wid = threadIdx.x >> 6;
+                    const int nsb = a.batch * C, wpb = nthreads >> 6, wid = threadIdx.x >> 6;
                     auto one = [&](int sb, const float4 v) {
                         u32 packed;
                         float d;
@@ -593,14 +621,6 @@ struct FmtQ6_K {
 #define PSN_STAMP(a, m, slot) do { } while (0)
 #endif
 
-template <typename F, int G, int R>
-PSN_DEV void load_rows(const psn_matvec_args &a, const RowMap<G, R> &m, int row0, int c, u32 (&w)[R][F::DW]) {
-    UNROLL for (int r = 0; r < R; ++r) {
-        const int row = min(row0 + r * m.S + m.slot, a.N - 1);     /* rows past the end re-read the last one */
-        F::load(row_ptr(a, row) + (int64_t)c * F::BYTES, w[r]);
-    }
-}
-
 /* Scheme Q8.  A wave walks its work as (row set, chunk iteration) items.  Order of events: the
  * small activation loads are issued, then the first item's weight loads, then the activations are
  * staged (waiting only for their own loads) while the weights are still in flight.  With one row
@@ -611,14 +631,15 @@ template <typename F, int G, int R, int NB, int XSRC>
 PSN_DEV void mv_q8(const psn_matvec_args &a) {
     typedef typename F::ActSum ST;
     constexpr bool DB = PSN_DOUBLE_BUFFER && (R == 1 && NB == 1);
-    const RowMap<G, R> m;
+    const RowMap<G, R> m(a);
+    PSN_DECLARE_SEGMENTS(a);
     const int K = a.K, C = K >> 8, iters = (C + G - 1) / G, stride = m.nwaves * m.ROWS;
     int row0 = m.wave * m.ROWS, it = 0;
     PSN_STAMP(a, m, 0);
     Stager<ST, XSRC> st;
     st.issue(a, F::d_per_col(K), F::s_per_col(K));
     u32 wa[R][F::DW], wb[DB ? R : 1][DB ? F::DW : 1];
-    load_rows<F, G, R>(a, m, min(row0, a.N - 1), min(m.j, C - 1), wa);
+    PSN_LOAD_ROWS(F, m, a, min(row0, a.N - 1), min(m.j, C - 1), wa);
     PSN_STAMP(a, m, 1);
     const ActQ<ST> x = st.finish(a);
     PSN_STAMP(a, m, 2);
@@ -641,7 +662,7 @@ PSN_DEV void mv_q8(const psn_matvec_args &a) {
         }
         if (i == iters - 1) {
             PSN_STAMP(a, m, 3);
-            store_rows<G, R, NB>(m, acc, a, r0);
+            PSN_STORE_ROWS(m, acc, a, r0);
             UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
         }
     };
@@ -652,12 +673,12 @@ PSN_DEV void mv_q8(const psn_matvec_args &a) {
         while (row0 < a.N) {
             int r1 = row0, i1 = it;
             advance(r1, i1);
-            load_rows<F, G, R>(a, m, r1, min(m.j + i1 * G, C - 1), wb);
+            PSN_LOAD_ROWS(F, m, a, r1, min(m.j + i1 * G, C - 1), wb);
             consume(wa, row0, it);
             if (r1 >= a.N) break;
             int r2 = r1, i2 = i1;
             advance(r2, i2);
-            load_rows<F, G, R>(a, m, r2, min(m.j + i2 * G, C - 1), wa);
+            PSN_LOAD_ROWS(F, m, a, r2, min(m.j + i2 * G, C - 1), wa);
             consume(wb, r1, i1);
             row0 = r2;
             it = i2;
@@ -665,7 +686,7 @@ PSN_DEV void mv_q8(const psn_matvec_args &a) {
     } else {
         bool pre = true;
         while (row0 < a.N) {
-            if (!pre) load_rows<F, G, R>(a, m, row0, min(m.j + it * G, C - 1), wa);
+            if (!pre) { PSN_LOAD_ROWS(F, m, a, row0, min(m.j + it * G, C - 1), wa); }
             pre = false;
             consume(wa, row0, it);
             advance(row0, it);
@@ -688,14 +709,14 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
     constexpr int S = 64 / G;                                /* rows per pass; every matrix holds a multiple of S rows */
     extern __shared__ uint4 psn_smem[];
     const int lane = threadIdx.x & 63, slot = lane / G, j = lane % G;
-    const int wpb = blockDim.x >> 6;
+    const int wpb = a.threads >> 6;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   /* wave-uniform, and the compiler should know it */
     const int K = a.K, C = K >> 8, N = a.N;
     const int rb = (int)a.row_bytes;                         /* bytes per row; a multiple of 16 */
     const int span = S * rb, nloads = (span + 1023) >> 10;   /* bytes and 1 KB load instructions per pass */
     const int wbuf = nloads << 10;
     const int npass = N / S;
-    const int stride = gridDim.x * wpb;
+    const int stride = a.blocks * wpb;
     int p = blockIdx.x * wpb + wib;
 
     /* where the wave buffers start: right behind the staged activations (same arithmetic as the host) */
@@ -784,14 +805,15 @@ PSN_DEV void f32_step(const u32 (&w)[R][F::DW], const float *xf, int K, int k0, 
 
 template <typename F, int G, int R, int NB>
 PSN_DEV void mv_f32(const psn_matvec_args &a) {
-    const RowMap<G, R> m;
+    const RowMap<G, R> m(a);
+    PSN_DECLARE_SEGMENTS(a);
     const int K = a.K, C = K >> 8;
     for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
         float acc[R][NB];
         UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
         for (int c = m.j; c < C; c += G) {
             u32 w[R][F::DW];
-            load_rows<F, G, R>(a, m, row0, c, w);
+            PSN_LOAD_ROWS(F, m, a, row0, c, w);
             const int k0 = c * 256;
             f32_step<F, 0>(w, a.xf, K, k0, a.batch, acc);
             f32_step<F, 1>(w, a.xf, K, k0, a.batch, acc);
@@ -802,7 +824,7 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
             f32_step<F, 6>(w, a.xf, K, k0, a.batch, acc);
             f32_step<F, 7>(w, a.xf, K, k0, a.batch, acc);
         }
-        store_rows<G, R, NB>(m, acc, a, row0);
+        PSN_STORE_ROWS(m, acc, a, row0);
     }
 }
 
@@ -840,7 +862,7 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
 #define PSN_Q8_ALL_G(fmt, F, R, NB) \
     PSN_Q8_KERNEL(fmt, F, 8, R, NB) PSN_Q8_KERNEL(fmt, F, 16, R, NB) PSN_Q8_KERNEL(fmt, F, 32, R, NB) PSN_Q8_KERNEL(fmt, F, 64, R, NB)
 #define PSN_Q8_ALL(fmt, F)                                                                 \
-    PSN_Q8_ALL_G(fmt, F, 1, 1) PSN_Q8_ALL_G(fmt, F, 2, 1) PSN_Q8_ALL_G(fmt, F, 4, 1)       \
+    PSN_Q8_ALL_G(fmt, F, 1, 1) PSN_Q8_ALL_G(fmt, F, 2, 1)                                  \
     PSN_Q8_ALL_G(fmt, F, 1, 2) PSN_Q8_ALL_G(fmt, F, 1, 4) PSN_Q8_ALL_G(fmt, F, 1, 8)
 
 #define PSN_F32_ALL_G(fmt, F, R, NB) \

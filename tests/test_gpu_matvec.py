@@ -84,7 +84,7 @@ def test_quantize_q8_K_bit_exact(hip, orc, k, batch):
 def all_plans(scheme, batch):
     nb = 1 if batch <= 1 else 2 if batch <= 2 else 4 if batch <= 4 else 8
     if scheme == _ffi.ACT_Q8:
-        rs = (1, 2, 4) if nb == 1 else (1,)
+        rs = (1, 2) if nb == 1 else (1,)
     else:
         rs = (1, 2) if nb == 1 else (1,)
     for g in (8, 16, 32, 64):
