@@ -54,10 +54,10 @@ def actq_layout(act_type: int, k: int, batch: int) -> _ffi.ActqInfo:
 
 
 def prefill_plan(m: int, n: int, k: int, compute_units: int = 256):
-    """(tile_m, tile_n, ksplit) the library picks for a prefill shape."""
-    tm, tn, sp = C.c_int32(), C.c_int32(), C.c_int32()
-    _check(_ffi.load().psn_qmatmul_prefill_plan(m, n, k, compute_units, C.byref(tm), C.byref(tn), C.byref(sp)))
-    return int(tm.value), int(tn.value), int(sp.value)
+    """(tile_m, tile_n, ksplit, waves) the library picks for a prefill shape."""
+    tm, tn, sp, wv = C.c_int32(), C.c_int32(), C.c_int32(), C.c_int32()
+    _check(_ffi.load().psn_qmatmul_prefill_plan(m, n, k, compute_units, C.byref(tm), C.byref(tn), C.byref(sp), C.byref(wv)))
+    return int(tm.value), int(tn.value), int(sp.value), int(wv.value)
 
 
 def matvec_plan(qtype: int, scheme: int, n: int, k: int, batch: int, compute_units: int = 256, x_is_f32: bool = False) -> MatvecPlan:
@@ -269,12 +269,12 @@ class HipBackend:
         _check(self.lib.psn_graph_destroy(graph))
 
     def quantized_matmul(self, w: QuantizedTensor, x_f16: DeviceBuffer, y: DeviceBuffer, m: int, tile=None):
-        """Prefill: Y[m, n] = X[m, k] . deq(W)[n, k]^T, X fp16, Y fp32.  `tile` = (rows, cols[, ksplit]) overrides the library's choice."""
+        """Prefill: Y[m, n] = X[m, k] . deq(W)[n, k]^T, X fp16, Y fp32.  `tile` = (rows, cols[, ksplit[, waves]]) overrides the library's choice."""
         if tile is None:
             _check(self.lib.psn_qmatmul_prefill(self.module, self.stream, w.qtype, LAYOUT_GGUF, w.buf.handle, x_f16.handle, y.handle, m, w.n, w.k))
         else:
             _check(self.lib.psn_qmatmul_prefill_tiled(self.module, self.stream, w.qtype, w.buf.handle, x_f16.handle, y.handle, m, w.n, w.k,
-                                                      tile[0], tile[1], tile[2] if len(tile) > 2 else 1))
+                                                      tile[0], tile[1], tile[2] if len(tile) > 2 else 1, tile[3] if len(tile) > 3 else 4))
 
     def matmul_host(self, qtype: int, blocks: np.ndarray, x_f16: np.ndarray, n: int, k: int, tile=None) -> np.ndarray:
         x = np.ascontiguousarray(x_f16, dtype=np.float16)

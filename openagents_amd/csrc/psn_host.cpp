@@ -885,9 +885,13 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
  * many workgroups of that tile one compute unit holds (LDS and registers) */
 static const double k_prefill_step_us[] = {0.87, 1.10, 1.50, 2.00, 2.00, 2.44};
 static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
+/* eight-wave variants worth choosing: {tile index, step cost} (one workgroup per compute unit) */
+static const struct { int tile; double step_us; } k_prefill_w8[] = {{3, 1.45}, {5, 2.38}};
 
-extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit) {
-    if (!tile_m || !tile_n || !ksplit) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: out is null");
+extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
+                                            int32_t *waves) {
+    if (!tile_m || !tile_n || !ksplit || !waves) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: out is null");
+    *waves = 4;
     if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
     if (cus <= 0) cus = 256;
     /* estimated time = waves of workgroups over the chip's slots x K steps per workgroup x step cost,
@@ -905,7 +909,14 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
             const double steps = (double)(K / 64) / sp;
             double t = (double)rounds * steps * k_prefill_step_us[i] + 5.0;
             if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;   /* bytes / (3 TB/s) in us, + a launch */
-            if (t < best) { best = t; bi = i; bs = sp; }
+            if (t < best) { best = t; bi = i; bs = sp; *waves = 4; }
+            for (const auto &v : k_prefill_w8) {
+                if (v.tile != i) continue;
+                const int64_t r8 = (wgs + cus - 1) / cus;
+                double t8 = (double)r8 * steps * v.step_us + 5.0;
+                if (sp > 1) t8 += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;
+                if (t8 < best) { best = t8; bi = i; bs = sp; *waves = 8; }
+            }
         }
     }
     *tile_m = k_prefill_tiles[bi][0];
@@ -915,12 +926,14 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
 }
 
 extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X,
-                                             psn_buf *Y, int64_t M, int64_t N, int64_t K, int32_t bm, int32_t bn, int32_t ksplit) {
+                                             psn_buf *Y, int64_t M, int64_t N, int64_t K, int32_t bm, int32_t bn, int32_t ksplit,
+                                             int32_t waves) {
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
     bool known = false;
     for (int i = 0; i < 6; ++i) known = known || (k_prefill_tiles[i][0] == bm && k_prefill_tiles[i][1] == bn);
     if (!known) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel with a %dx%d tile", bm, bn);
+    if (waves != 4 && !(waves == 8 && bm >= 128 && bn >= 128)) return fail(PSN_E_UNSUPPORTED, "prefill: no %d-wave kernel for a %dx%d tile", waves, bm, bn);
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
     const int lds = 2 * (bm + bn) * 128;
@@ -946,8 +959,8 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
     const int64_t blocks = 8 * ((nt + 7) / 8) * mt * ksplit;      /* the kernel spreads N tiles over 8 XCDs */
     char name[96];
-    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d", fmt_name(qtype), bm, bn);
-    return launch(mod, s, name, (unsigned)blocks, 256, (unsigned)lds, &a);
+    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 8 ? "_w8" : "");
+    return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * waves), (unsigned)lds, &a);
 }
 
 extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
@@ -955,9 +968,9 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "prefill: layout %d", layout);
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
-    int32_t bm = 0, bn = 0, sp = 1;
-    if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp))) return rc;
-    return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp);
+    int32_t bm = 0, bn = 0, sp = 1, wv = 4;
+    if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv))) return rc;
+    return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }
 
 /* ------------------------------------------------------------------ decode-step glue */

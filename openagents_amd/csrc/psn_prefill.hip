@@ -137,10 +137,11 @@ PSN_DEV void stage_w_row(const u32 (&w)[WF::DW], char *tile, int row) {
 
 template <typename WF, int BM, int BN, int WM, int WN>
 PSN_DEV void prefill_body(const psn_prefill_args &a) {
-    static_assert(WM * WN == 4, "four waves");
+    static_assert(WM * WN == 4 || WM * WN == 8, "four or eight waves");
     static_assert(BN == 64 || BN == 128 || BN == 256, "BN");
+    constexpr int NT = 64 * WM * WN;                        /* threads per workgroup */
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;     /* 32x32 MFMA tiles per wave */
-    constexpr int KCH = 256 / BN;                           /* 256-wide K chunks held in registers per round */
+    constexpr int KCH = NT / BN;                            /* 256-wide K chunks held in registers per round */
     constexpr int XBYTES = BM * 128, WBYTES = BN * 128;
     extern __shared__ uint4 psn_smem[];
     char *smem = reinterpret_cast<char *>(psn_smem);
@@ -171,10 +172,10 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
 
     auto stage_x = [&](char *tile, int k0) {
         /* slot s = 16-byte word s of the tile in LDS order: row s/8, position s%8 holds chunk (s%8)^(row&7) */
-        UNROLL for (int i = 0; i < BM * 8 / 256; ++i) {
-            const int s = i * 256 + tid, row = s >> 3, chunk = (s & 7) ^ (row & 7);
+        UNROLL for (int i = 0; i < BM * 8 / NT; ++i) {
+            const int s = i * NT + tid, row = s >> 3, chunk = (s & 7) ^ (row & 7);
             const uint16_t *src = a.X + (int64_t)min(m0 + row, M - 1) * K + k0 + chunk * 8;
-            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + (i * 256 + wave * 64) * 16), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + (i * NT + wave * 64) * 16), 16, 0, 0);
         }
     };
     auto compute = [&](const char *xt, const char *wt) {
@@ -262,6 +263,11 @@ extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_a
     extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_m##BM##_n##BN(const psn_prefill_args a) { \
         prefill_body<WF, BM, BN, WM, WN>(a);                                                                 \
     }
+/* eight-wave variants (512 threads, two waves per SIMD: one can multiply while the other stages) */
+#define PSN_PREFILL_KERNEL8(fmt, WF, BM, BN, WM, WN)                                                         \
+    extern "C" __global__ void __launch_bounds__(512) psn_prefill_##fmt##_m##BM##_n##BN##_w8(const psn_prefill_args a) { \
+        prefill_body<WF, BM, BN, WM, WN>(a);                                                                 \
+    }
 
 #define PSN_PREFILL_ALL(fmt, WF)               \
     PSN_PREFILL_KERNEL(fmt, WF, 64, 64, 2, 2)    \
@@ -269,7 +275,11 @@ extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_a
     PSN_PREFILL_KERNEL(fmt, WF, 128, 128, 2, 2)  \
     PSN_PREFILL_KERNEL(fmt, WF, 128, 256, 2, 2)  \
     PSN_PREFILL_KERNEL(fmt, WF, 256, 128, 2, 2)  \
-    PSN_PREFILL_KERNEL(fmt, WF, 256, 256, 2, 2)
+    PSN_PREFILL_KERNEL(fmt, WF, 256, 256, 2, 2)  \
+    PSN_PREFILL_KERNEL8(fmt, WF, 128, 128, 2, 4) \
+    PSN_PREFILL_KERNEL8(fmt, WF, 256, 128, 4, 2) \
+    PSN_PREFILL_KERNEL8(fmt, WF, 128, 256, 2, 4) \
+    PSN_PREFILL_KERNEL8(fmt, WF, 256, 256, 2, 4)
 
 PSN_PREFILL_ALL(q4_0, PfQ4_0)
 PSN_PREFILL_ALL(q8_0, PfQ8_0)

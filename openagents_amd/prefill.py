@@ -1,0 +1,71 @@
+"""Quantized prefill matmul benchmark: Q4_0 / Q8_0 weights 4096->14336 and 14336->4096, fp16
+activations for M = 64, 512, 2048 tokens (seeded N(0,0.02) weights quantized on the host).
+
+    python -m openagents_amd.prefill [--iters 20] [--formats q4_0,q8_0] [--m 64,512,2048]
+
+Prints one JSON record per (format, shape, M): microseconds, TFLOP/s, GB/s and the fraction of the
+roofline that binds (fp16 MFMA 2.5 PFLOP/s, or HBM 8 TB/s when the arithmetic intensity is below
+the ridge of 312.5 FLOP/B).  Weight copies rotate so that the HBM-bound cases stream from memory.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+
+import numpy as np
+
+from . import quantize
+from ._ffi import Q4_0, Q8_0
+from .backend import HipBackend, prefill_plan, row_bytes
+
+MFMA_PEAK_TFLOPS = 2500.0
+HBM_PEAK_GBS = 8000.0
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--formats", default="q4_0,q8_0")
+    ap.add_argument("--m", default="64,512,2048")
+    ap.add_argument("--seed", type=int, default=7)
+    args = ap.parse_args(argv)
+    fmts = {"q4_0": (Q4_0, quantize.quantize_q4_0), "q8_0": (Q8_0, quantize.quantize_q8_0)}
+    be = HipBackend(0)
+    rng = np.random.default_rng(args.seed)
+    for fname in args.formats.split(","):
+        qt, quant = fmts[fname]
+        for n, k in ((14336, 4096), (4096, 14336)):
+            blocks = quant(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
+            copies = max(2, int(300e6 // blocks.nbytes) + 1)
+            ws = [be.upload_weight(qt, blocks, n, k) for _ in range(copies)]
+            for m in (int(v) for v in args.m.split(",")):
+                x = be.upload(rng.standard_normal((m, k), dtype=np.float32).astype(np.float16))
+                y = be.alloc(m * n * 4)
+                for i in range(3):
+                    be.quantized_matmul(ws[i % copies], x, y, m)
+                be.sync()
+                e0, e1 = be.event(), be.event()
+                be.record(e0)
+                for i in range(args.iters):
+                    be.quantized_matmul(ws[i % copies], x, y, m)
+                be.record(e1)
+                us = be.elapsed_us(e0, e1) / args.iters
+                be.destroy_event(e0)
+                be.destroy_event(e1)
+                flops = 2.0 * m * n * k
+                nbytes = n * row_bytes(qt, k) + m * k * 2 + m * n * 4
+                tflops, gbs = flops / us / 1e6, nbytes / us / 1e3
+                bound = "mfma" if flops / nbytes >= MFMA_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "hbm"
+                frac = tflops / MFMA_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS
+                tm, tn, sp, wv = prefill_plan(m, n, k, be.compute_units)
+                print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
+                                  "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
+                                  "kernel": f"psn_prefill_{fname}_m{tm}_n{tn}" + ("_w8" if wv == 8 else ""), "ksplit": sp, "iters": args.iters}), flush=True)
+            for w in ws:
+                w.buf.free()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

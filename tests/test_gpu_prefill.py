@@ -46,12 +46,13 @@ def test_every_tile_ragged_shapes(hip, orc, qname, tile):
         W = weights(orc, qname, 800, n, k)
         X = G.seeded_acts(801 + m, m, k).astype(np.float16)
         ref = orc.prefill(t, W, X, n, k)
-        for ksplit in (1, 2, 4):
-            if ksplit > 1 and (m * n) % 4:
-                continue
-            y = hip.matmul_host(t, W, X, n, k, tile + (ksplit,))
-            err = G.max_rel_err(y, ref)
-            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, m, n, k, err)
+        for waves in ((4, 8) if min(tile) >= 128 else (4,)):
+            for ksplit in (1, 2, 4):
+                if ksplit > 1 and (m * n) % 4:
+                    continue
+                y = hip.matmul_host(t, W, X, n, k, tile + (ksplit, waves))
+                err = G.max_rel_err(y, ref)
+                assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, waves, m, n, k, err)
 
 
 @pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
