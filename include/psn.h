@@ -206,8 +206,9 @@ int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32
 /* The launch shape the library picks for a prefill: the workgroup tile of Y (64x64, 64x128,
  * 128x128, 128x256, 256x128 or 256x256) and into how many ranges K is cut (1, 2, 4 or 8; with more
  * than one, Y is zeroed by a fill kernel and the partial sums are added atomically, so their order --
- * and the last bit of a sum -- can vary between runs), and the workgroup size in waves (4, or 8 for
- * the 128x128 .. 256x256 tiles).  Host arithmetic only ... */
+ * and the last bit of a sum -- can vary between runs), and the kernel family: 4 = four waves, 8 = eight
+ * waves (tiles of at least 128x128), -4 = four waves with X prefetched three K steps ahead and the
+ * weight decode interleaved with the MFMAs (64x128, 128x128, 128x256).  Host arithmetic only ... */
 int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m, int32_t *tile_n,
                                  int32_t *ksplit, int32_t *waves);
 /* ... and the same matmul with a caller-chosen shape (auto-tuners, benchmarks). */

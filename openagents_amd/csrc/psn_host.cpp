@@ -885,8 +885,10 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
  * many workgroups of that tile one compute unit holds (LDS and registers) */
 static const double k_prefill_step_us[] = {0.87, 1.10, 1.50, 2.00, 2.00, 2.44};
 static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
-/* eight-wave variants worth choosing: {tile index, step cost} (one workgroup per compute unit) */
-static const struct { int tile; double step_us; } k_prefill_w8[] = {{3, 1.45}, {5, 2.38}};
+/* other variants worth choosing: {tile index, waves (8, or -4 = interleaved four-wave schedule), step cost,
+ * workgroups per compute unit} */
+static const struct { int tile; int waves; double step_us; int per_cu; } k_prefill_alt[] = {
+    {3, 8, 1.45, 1}, {5, 8, 2.38, 1}, {3, -4, 1.33, 1}, {1, -4, 0.85, 2}};
 
 extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
                                             int32_t *waves) {
@@ -910,12 +912,13 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
             double t = (double)rounds * steps * k_prefill_step_us[i] + 5.0;
             if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;   /* bytes / (3 TB/s) in us, + a launch */
             if (t < best) { best = t; bi = i; bs = sp; *waves = 4; }
-            for (const auto &v : k_prefill_w8) {
+            for (const auto &v : k_prefill_alt) {
                 if (v.tile != i) continue;
-                const int64_t r8 = (wgs + cus - 1) / cus;
+                const int64_t sl = (int64_t)cus * v.per_cu;
+                const int64_t r8 = (wgs + sl - 1) / sl;
                 double t8 = (double)r8 * steps * v.step_us + 5.0;
                 if (sp > 1) t8 += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;
-                if (t8 < best) { best = t8; bi = i; bs = sp; *waves = 8; }
+                if (t8 < best) { best = t8; bi = i; bs = sp; *waves = v.waves; }
             }
         }
     }
@@ -933,10 +936,14 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     bool known = false;
     for (int i = 0; i < 6; ++i) known = known || (k_prefill_tiles[i][0] == bm && k_prefill_tiles[i][1] == bn);
     if (!known) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel with a %dx%d tile", bm, bn);
-    if (waves != 4 && !(waves == 8 && bm >= 128 && bn >= 128)) return fail(PSN_E_UNSUPPORTED, "prefill: no %d-wave kernel for a %dx%d tile", waves, bm, bn);
+    /* waves == -4 selects the four-wave kernel with the interleaved decode/MFMA schedule */
+    const bool has_il = (bm == 64 && bn == 128) || (bm == 128 && bn == 128) || (bm == 128 && bn == 256);
+    if (waves != 4 && !(waves == 8 && bm >= 128 && bn >= 128) && !(waves == -4 && has_il))
+        return fail(PSN_E_UNSUPPORTED, "prefill: no %d-wave kernel for a %dx%d tile", waves, bm, bn);
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
-    const int lds = 2 * (bm + bn) * 128;
+    /* the interleaved kernels carry their LDS as static arrays */
+    const int lds = waves == -4 ? 0 : 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);
     if ((rc = bind(mod->ctx))) return rc;
     if (ksplit > 1) {
@@ -959,8 +966,8 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
     const int64_t blocks = 8 * ((nt + 7) / 8) * mt * ksplit;      /* the kernel spreads N tiles over 8 XCDs */
     char name[96];
-    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 8 ? "_w8" : "");
-    return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * waves), (unsigned)lds, &a);
+    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 8 ? "_w8" : waves == -4 ? "_il" : "");
+    return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * (waves == 8 ? 8 : 4)), (unsigned)lds, &a);
 }
 
 extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
@@ -970,6 +977,7 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     if (rc) return rc;
     int32_t bm = 0, bn = 0, sp = 1, wv = 4;
     if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv))) return rc;
+    if (qtype == PSN_Q8_0 && wv == 8) wv = 4;     /* the eight-wave Q8_0 kernels spill registers (272-byte chunks) */
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }
 

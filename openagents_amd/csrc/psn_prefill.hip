@@ -252,6 +252,200 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
     }
 }
 
+/* ---- interleaved variant ------------------------------------------------------------------
+ * Same tiles and LDS layout, but arranged so that one basic block holds a whole K step:
+ *  - all 256 threads dequantize in every step (256/BN threads share a weight row, each turning
+ *    64*BN/256 weights of it into fp16), so there is no divergent branch around the dequantization;
+ *  - the operand fragments of k16 slice kk+1 are read while the MFMAs of slice kk are issued;
+ *  - scheduling barriers ask the compiler to issue, per MFMA, a share of the dequantization VALU
+ *    work and of the LDS traffic, so the matrix pipeline is fed while the vector ALUs decode. */
+
+/* raw quants and fp16 scale bits of GGUF block B of a chunk */
+template <int B> PSN_DEV void raw_block(const u32 (&w)[36], u32 (&q)[8], u32 &dbits) {       /* Q4_0: q[0..3] used */
+    constexpr int base = 9 * (B >> 1);
+    if constexpr ((B & 1) == 0) {
+        dbits = w[base] & 0xffffu;
+        UNROLL for (int i = 0; i < 4; ++i) q[i] = align2(w[base + i + 1], w[base + i]);
+    } else {
+        dbits = w[base + 4] >> 16;
+        UNROLL for (int i = 0; i < 4; ++i) q[i] = w[base + 5 + i];
+    }
+    UNROLL for (int i = 4; i < 8; ++i) q[i] = 0;
+}
+template <int B> PSN_DEV void raw_block(const u32 (&w)[68], u32 (&q)[8], u32 &dbits) {       /* Q8_0 */
+    constexpr int base = 17 * (B >> 1);
+    if constexpr ((B & 1) == 0) {
+        dbits = w[base] & 0xffffu;
+        UNROLL for (int i = 0; i < 8; ++i) q[i] = align2(w[base + i + 1], w[base + i]);
+    } else {
+        dbits = w[base + 8] >> 16;
+        UNROLL for (int i = 0; i < 8; ++i) q[i] = w[base + 9 + i];
+    }
+}
+/* 16 weights (half H of a block given raw) -> 8 dwords of fp16 */
+template <typename WF> PSN_DEV void deq16(const u32 (&q)[8], u32 dbits, int H, u32 (&o)[8]) {
+    const half2_t d2 = bits_h2(dbits | (dbits << 16));
+    if constexpr (WF::DW == 36) {
+        const half2_t bias = bits_h2(0x64086408u);
+        UNROLL for (int i = 0; i < 4; ++i) bytes_to_h4(q[i] >> (4 * H), 0x640f640fu, bias, d2, o[2 * i], o[2 * i + 1]);
+    } else {
+        const half2_t bias = bits_h2(0x64806480u);
+        UNROLL for (int i = 0; i < 4; ++i) bytes_to_h4((H ? q[4 + i] : q[i]) ^ 0x80808080u, 0x64ff64ffu, bias, d2, o[2 * i], o[2 * i + 1]);
+    }
+}
+/* the part of K step SUB (blocks 2*SUB, 2*SUB+1 of the chunk) that thread part `q` of P owns -> LDS */
+template <typename WF, int SUB, int P>
+PSN_DEV void stage_part(const u32 (&w)[WF::DW], char *tile, int row, int part) {
+    u32 qa[8], qb[8], da, db;
+    raw_block<2 * SUB>(w, qa, da);
+    raw_block<2 * SUB + 1>(w, qb, db);
+    if constexpr (P == 1) {
+        UNROLL for (int h = 0; h < 2; ++h) {
+            u32 o[8];
+            deq16<WF>(qa, da, h, o);
+            *reinterpret_cast<uint4 *>(tile + tile_off(row, 2 * h)) = make_uint4(o[0], o[1], o[2], o[3]);
+            *reinterpret_cast<uint4 *>(tile + tile_off(row, 2 * h + 1)) = make_uint4(o[4], o[5], o[6], o[7]);
+            deq16<WF>(qb, db, h, o);
+            *reinterpret_cast<uint4 *>(tile + tile_off(row, 4 + 2 * h)) = make_uint4(o[0], o[1], o[2], o[3]);
+            *reinterpret_cast<uint4 *>(tile + tile_off(row, 4 + 2 * h + 1)) = make_uint4(o[4], o[5], o[6], o[7]);
+        }
+    } else {
+        const bool second = P == 2 ? part == 1 : part >= 2;        /* which of the two blocks */
+        u32 q[8];
+        UNROLL for (int i = 0; i < 8; ++i) q[i] = second ? qb[i] : qa[i];
+        const u32 d = second ? db : da;
+        if constexpr (P == 2) {
+            UNROLL for (int h = 0; h < 2; ++h) {
+                u32 o[8];
+                deq16<WF>(q, d, h, o);
+                *reinterpret_cast<uint4 *>(tile + tile_off(row, 4 * part + 2 * h)) = make_uint4(o[0], o[1], o[2], o[3]);
+                *reinterpret_cast<uint4 *>(tile + tile_off(row, 4 * part + 2 * h + 1)) = make_uint4(o[4], o[5], o[6], o[7]);
+            }
+        } else {
+            u32 o[8];
+            deq16<WF>(q, d, part & 1, o);
+            *reinterpret_cast<uint4 *>(tile + tile_off(row, 2 * part)) = make_uint4(o[0], o[1], o[2], o[3]);
+            *reinterpret_cast<uint4 *>(tile + tile_off(row, 2 * part + 1)) = make_uint4(o[4], o[5], o[6], o[7]);
+        }
+    }
+}
+
+/* X tiles: four LDS stages filled three K steps ahead by direct-to-LDS loads; W tiles: two stages
+ * filled one step ahead from registers.  Every stage is its own __shared__ array so that alias
+ * analysis can tell the compiler that a W write or a fragment read never touches the stage a
+ * pending X load is landing in -- otherwise it waits for all outstanding loads in mid-step. */
+template <typename WF, int BM, int BN, int WM, int WN>
+PSN_DEV void prefill_body_il(const psn_prefill_args &a) {
+    static_assert(WM * WN == 4, "four waves");
+    constexpr int NT = 256;
+    constexpr int P = NT / BN;                              /* threads per weight row */
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int NX = BM * 8 / NT;                         /* direct-to-LDS instructions per X stage */
+    constexpr int NW = WF::DW / 4;                          /* global loads per weight chunk */
+    __shared__ uint4 xs0[BM * 8], xs1[BM * 8], xs2[BM * 8], xs3[BM * 8];
+    __shared__ uint4 ws0[BN * 8], ws1[BN * 8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
+    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+    const int S = a.ksplit;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_xcd_n = (nt + 7) >> 3;
+    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
+    const int tile_n = xcd + 8 * tn_local;
+    if (tn_local >= per_xcd_n || tile_n >= nt) return;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int per_split = (C + S - 1) / S;
+    const int c_begin = split * per_split, c_end = min(c_begin + per_split, C);
+    if (c_begin >= c_end) return;
+    const int k_last = c_end * 256 - 64;                    /* last K step of this range; later prefetches re-read it */
+
+    float16_t acc[TM][TN];
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    const int wrow = tid % BN, part = tid / BN;
+    const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
+    u32 w[WF::DW], wnext[WF::DW];
+
+    auto stage_x = [&](uint4 *tile, int k0) {
+        k0 = min(k0, k_last);
+        UNROLL for (int i = 0; i < NX; ++i) {
+            const int s = i * NT + tid, row = s >> 3, chunk = (s & 7) ^ (row & 7);
+            const uint16_t *src = a.X + (int64_t)min(m0 + row, M - 1) * K + k0 + chunk * 8;
+            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + i * NT + wave * 64), 16, 0, 0);
+        }
+    };
+    auto load_frags = [&](const uint4 *xt, const uint4 *wt, int kk, half8_t (&af)[TM], half8_t (&bf)[TN]) {
+        const int chunk = 2 * kk + (lane >> 5);
+        UNROLL for (int i = 0; i < TM; ++i)
+            af[i] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(xt) + tile_off(wm * (BM / WM) + 32 * i + (lane & 31), chunk));
+        UNROLL for (int j = 0; j < TN; ++j)
+            bf[j] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(wt) + tile_off(wn * (BN / WN) + 32 * j + (lane & 31), chunk));
+    };
+    auto mfmas = [&](const half8_t (&af)[TM], const half8_t (&bf)[TN]) {
+        UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    };
+
+    /* prologue: weight chunk, X stages for the first three steps, W stage for the first */
+    WF::load(wbase + (int64_t)c_begin * WF::BYTES, w);
+    const int k_begin = c_begin * 256;
+    stage_x(xs0, k_begin);
+    stage_x(xs1, k_begin + 64);
+    stage_x(xs2, k_begin + 128);
+    stage_part<WF, 0, P>(w, reinterpret_cast<char *>(ws0), wrow, part);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+
+    /* one K step: X stage `xc` and W stage `wc` are current; X for step +3 goes to `xp`, W for step +1
+     * to `wq` (from `wsrc`, blocks 2*NSUB and 2*NSUB+1).  KEEP = loads that may stay in flight past the
+     * barrier: the X stages of steps +2 and +3, plus the next weight chunk when it was requested after
+     * the X stage of step +1. */
+#define PSN_PF_STEP(SUB, NSUB, wsrc, xc, xp, wc, wq, KEEP)                                            \
+    {                                                                                                 \
+        stage_x(xp, (c * 4 + SUB + 3) * 64);                                                          \
+        half8_t af0[TM], bf0[TN], af1[TM], bf1[TN];                                                   \
+        load_frags(xc, wc, 0, af0, bf0);                                                              \
+        load_frags(xc, wc, 1, af1, bf1);                                                              \
+        mfmas(af0, bf0);                                                                              \
+        load_frags(xc, wc, 2, af0, bf0);                                                              \
+        mfmas(af1, bf1);                                                                              \
+        load_frags(xc, wc, 3, af1, bf1);                                                              \
+        mfmas(af0, bf0);                                                                              \
+        stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part);                      \
+        mfmas(af1, bf1);                                                                              \
+        UNROLL for (int i_ = 0; i_ < 4 * TM * TN; ++i_) {                                             \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                        \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                        \
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                        \
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                        \
+        }                                                                                             \
+        /* raw barrier: __syncthreads() would first drain every outstanding load, prefetches included */ \
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(KEEP) : "memory");            \
+    }
+
+    for (int c = c_begin; c < c_end; ++c) {
+        WF::load(wbase + (int64_t)min(c + 1, C - 1) * WF::BYTES, wnext);
+        PSN_PF_STEP(0, 1, w, xs0, xs3, ws0, ws1, 2 * NX + NW)
+        PSN_PF_STEP(1, 2, w, xs1, xs0, ws1, ws0, 2 * NX + NW)
+        PSN_PF_STEP(2, 3, w, xs2, xs1, ws0, ws1, 2 * NX)
+        PSN_PF_STEP(3, 0, wnext, xs3, xs2, ws1, ws0, 2 * NX)
+        UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = wnext[i];
+    }
+#undef PSN_PF_STEP
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
+        UNROLL for (int r = 0; r < 16; ++r) {
+            const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (row < M && col < N) {
+                if (S == 1) a.Y[(int64_t)row * N + col] = acc[i][j][r];
+                else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], acc[i][j][r]);
+            }
+        }
+    }
+}
+
 /* zero fill with plain vector stores (graph-safe stand-in for a memset node) */
 extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_args a) {
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -269,7 +463,15 @@ extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_a
         prefill_body<WF, BM, BN, WM, WN>(a);                                                                 \
     }
 
+#define PSN_PREFILL_KERNEL_IL(fmt, WF, BM, BN, WM, WN)                                                       \
+    extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_m##BM##_n##BN##_il(const psn_prefill_args a) { \
+        prefill_body_il<WF, BM, BN, WM, WN>(a);                                                              \
+    }
+
 #define PSN_PREFILL_ALL(fmt, WF)               \
+    PSN_PREFILL_KERNEL_IL(fmt, WF, 64, 128, 2, 2)  \
+    PSN_PREFILL_KERNEL_IL(fmt, WF, 128, 128, 2, 2) \
+    PSN_PREFILL_KERNEL_IL(fmt, WF, 128, 256, 2, 2) \
     PSN_PREFILL_KERNEL(fmt, WF, 64, 64, 2, 2)    \
     PSN_PREFILL_KERNEL(fmt, WF, 64, 128, 2, 2)   \
     PSN_PREFILL_KERNEL(fmt, WF, 128, 128, 2, 2)  \

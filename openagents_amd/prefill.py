@@ -25,7 +25,8 @@ HBM_PEAK_GBS = 8000.0
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("--iters", type=int, default=20)
+    ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--formats", default="q4_0,q8_0")
     ap.add_argument("--m", default="64,512,2048")
     ap.add_argument("--seed", type=int, default=7)
@@ -42,7 +43,7 @@ def main(argv=None):
             for m in (int(v) for v in args.m.split(",")):
                 x = be.upload(rng.standard_normal((m, k), dtype=np.float32).astype(np.float16))
                 y = be.alloc(m * n * 4)
-                for i in range(3):
+                for i in range(args.warmup):
                     be.quantized_matmul(ws[i % copies], x, y, m)
                 be.sync()
                 e0, e1 = be.event(), be.event()
@@ -59,9 +60,11 @@ def main(argv=None):
                 bound = "mfma" if flops / nbytes >= MFMA_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "hbm"
                 frac = tflops / MFMA_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS
                 tm, tn, sp, wv = prefill_plan(m, n, k, be.compute_units)
+                if fname == "q8_0" and wv == 8:
+                    wv = 4
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
-                                  "kernel": f"psn_prefill_{fname}_m{tm}_n{tn}" + ("_w8" if wv == 8 else ""), "ksplit": sp, "iters": args.iters}), flush=True)
+                                  "kernel": f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 8: "_w8", -4: "_il"}[wv], "ksplit": sp, "iters": args.iters}), flush=True)
             for w in ws:
                 w.buf.free()
     return 0
