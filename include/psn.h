@@ -102,6 +102,11 @@ int32_t psn_graph_begin_capture(psn_stream *s);
 int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out);
 int32_t psn_graph_launch(psn_graph *g, psn_stream *s);
 int32_t psn_graph_destroy(psn_graph *g);
+/* Makes `waiter` wait for everything enqueued on `signaler` so far (an event recorded on one stream
+ * and awaited on the other).  While `signaler` is being captured this joins `waiter` into the same
+ * capture, which is how a graph gets parallel branches: fork with (side, main), launch independent
+ * work on both, join with (main, side) before ending the capture. */
+int32_t psn_stream_wait_stream(psn_stream *waiter, psn_stream *signaler);
 /* Sizes the stream's activation workspace for psn_qmatvec / psn_qmatvec_multi with scheme Q8 up to
  * [batch][K], so later calls (and captures) never allocate. */
 int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch);

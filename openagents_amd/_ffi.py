@@ -58,6 +58,7 @@ SIGNATURES = {
     "psn_graph_launch": (_i32, [_vp, _vp]),
     "psn_graph_destroy": (_i32, [_vp]),
     "psn_stream_reserve": (_i32, [_vp, _i64, _i32]),
+    "psn_stream_wait_stream": (_i32, [_vp, _vp]),
     "psn_event_create": (_i32, [_vp, _pp]),
     "psn_event_destroy": (_i32, [_vp]),
     "psn_event_record": (_i32, [_vp, _vp]),

@@ -176,6 +176,33 @@ class HipBackend:
     def sync(self):
         _check(self.lib.psn_stream_sync(self.stream))
 
+    # -- additional streams -------------------------------------------------------------------
+    def new_stream(self) -> C.c_void_p:
+        st = C.c_void_p()
+        _check(self.lib.psn_stream_create(self.ctx, C.byref(st)))
+        return st
+
+    def destroy_stream(self, stream):
+        _check(self.lib.psn_stream_destroy(stream))
+
+    def stream_wait(self, waiter, signaler):
+        """`waiter` waits for what is enqueued on `signaler` so far; under capture this forks / joins graph branches."""
+        _check(self.lib.psn_stream_wait_stream(waiter, signaler))
+
+    def on_stream(self, stream):
+        """Context manager: route this backend's launches to `stream`."""
+        be = self
+
+        class _Swap:
+            def __enter__(self_inner):
+                self_inner.prev = be.stream
+                be.stream = stream
+
+            def __exit__(self_inner, *exc):
+                be.stream = self_inner.prev
+
+        return _Swap()
+
     # -- events -----------------------------------------------------------------------------
     def event(self) -> C.c_void_p:
         e = C.c_void_p()

@@ -139,6 +139,7 @@ struct psn_stream {
     hipStream_t s;
     void *ws;          /* activation workspace of psn_qmatvec (scheme Q8) */
     size_t ws_bytes;
+    hipEvent_t join_ev; /* created on first use by psn_stream_wait_stream */
 };
 struct psn_buf {
     psn_ctx *ctx;
@@ -286,6 +287,7 @@ extern "C" int32_t psn_stream_create(psn_ctx *c, psn_stream **out) {
     st->s = s;
     st->ws = nullptr;
     st->ws_bytes = 0;
+    st->join_ev = nullptr;
     *out = st;
     return PSN_OK;
 }
@@ -302,6 +304,7 @@ extern "C" int32_t psn_stream_destroy(psn_stream *s) {
     if (rc) return rc;
     (void)hipStreamSynchronize(s->s);
     if (s->ws) (void)hipFree(s->ws);
+    if (s->join_ev) (void)hipEventDestroy(s->join_ev);
     hipError_t e = hipStreamDestroy(s->s);
     delete s;
     if (e != hipSuccess) return hip_fail(e, "hipStreamDestroy");
@@ -340,6 +343,17 @@ extern "C" int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch) {
     if ((rc = psn_actq_layout(PSN_Q8_K, K, batch, &b))) return rc;
     if ((rc = bind(s->ctx))) return rc;
     return ensure_workspace(s, a.bytes > b.bytes ? a.bytes : b.bytes);
+}
+
+extern "C" int32_t psn_stream_wait_stream(psn_stream *waiter, psn_stream *signaler) {
+    if (!waiter || !signaler) return fail(PSN_E_INVALID_ARG, "stream is null");
+    if (waiter->ctx != signaler->ctx) return fail(PSN_E_INVALID_ARG, "streams belong to different contexts");
+    int32_t rc = bind(waiter->ctx);
+    if (rc) return rc;
+    if (!signaler->join_ev) HIP_TRY(hipEventCreateWithFlags(&signaler->join_ev, hipEventDisableTiming));
+    HIP_TRY(hipEventRecord(signaler->join_ev, signaler->s));
+    HIP_TRY(hipStreamWaitEvent(waiter->s, signaler->join_ev, 0));
+    return PSN_OK;
 }
 
 extern "C" int32_t psn_graph_begin_capture(psn_stream *s) {

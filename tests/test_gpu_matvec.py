@@ -392,3 +392,38 @@ def test_streaming_plan_is_refused_where_it_cannot_run(hip, orc):
         with pytest.raises(backend.PsnError) as e:
             hip.quantized_matvec_planned(w, x, y, 1, _ffi.ACT_Q8, p)
         assert e.value.code == _ffi.E_UNSUPPORTED
+
+
+def test_two_branch_graph_of_independent_launches(hip, orc):
+    """Fork a second stream inside a capture, run independent matvecs on both branches, join, replay:
+    every output equals the eager single-stream result bit for bit."""
+    t, k = orc.Q4_K, 2048
+    ns = [512, 768, 1024, 256]
+    ws = [hip.upload_weight(t, weights(orc, "Q4_K", 990 + i, n, k), n, k) for i, n in enumerate(ns)]
+    x = hip.upload(G.seeded_acts(991, 1, k))
+    ys = [hip.alloc(n * 4) for n in ns]
+    for w, y in zip(ws, ys):
+        hip.quantized_matvec(w, x, y)
+    want = [y.download(np.float32, (n,)) for y, n in zip(ys, ns)]
+    side = hip.new_stream()
+    main = hip.stream
+    hip.begin_capture()
+    hip.stream_wait(side, main)
+    for i, (w, y) in enumerate(zip(ws, ys)):
+        if i % 2:
+            with hip.on_stream(side):
+                hip.quantized_matvec(w, x, y)
+        else:
+            hip.quantized_matvec(w, x, y)
+    hip.stream_wait(main, side)
+    graph = hip.end_capture()
+    try:
+        for _ in range(3):
+            for y, n in zip(ys, ns):
+                y.upload(np.zeros(n, np.float32))
+            hip.launch_graph(graph)
+            for y, n, ref in zip(ys, ns, want):
+                assert np.array_equal(y.download(np.float32, (n,)), ref)
+    finally:
+        hip.destroy_graph(graph)
+        hip.destroy_stream(side)
