@@ -32,8 +32,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by
 # what the same counter reads for a 256 MiB device-to-device copy: x1.9998 and x1.0000; the copies
 # are what --calibrate-copy adds to a run).
-MEASURED_TRAFFIC_BYTES = {"qkv": 14.45e6 + 24.0 * 1024, "o": 9.74e6 + 16.0 * 1024,
-                          "gate_up": 66.38e6 + 114.2 * 1024, "down": 33.67e6 + 17.0 * 1024}
+MEASURED_TRAFFIC_BYTES = {"qkv": 14.465e6 + 24.0 * 1024, "o": 9.739e6 + 16.0 * 1024,
+                          "gate_up": 66.285e6 + 112.0 * 1024, "down": 33.684e6 + 17.0 * 1024}
 HIDDEN, KV, FFN, LAYERS = 4096, 1024, 14336, 32
 BPW_Q4_0 = 18.0 / 32.0
 
