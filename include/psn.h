@@ -213,7 +213,9 @@ int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32
  * than one, Y is zeroed by a fill kernel and the partial sums are added atomically, so their order --
  * and the last bit of a sum -- can vary between runs), and the kernel family: 4 = four waves, 8 = eight
  * waves (tiles of at least 128x128), -4 = four waves with X prefetched three K steps ahead and the
- * weight decode interleaved with the MFMAs (64x128, 128x128, 128x256).  Host arithmetic only ... */
+ * weight decode interleaved with the MFMAs (64x128, 128x128, 128x256), -5 = four waves with X prefetched
+ * through registers (tiles of at least 128x128), 16 = eight waves of which four only multiply and four
+ * only stage (128x128, 128x256).  Host arithmetic only ... */
 int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m, int32_t *tile_n,
                                  int32_t *ksplit, int32_t *waves);
 /* ... and the same matmul with a caller-chosen shape (auto-tuners, benchmarks). */

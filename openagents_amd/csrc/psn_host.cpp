@@ -899,10 +899,10 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
  * many workgroups of that tile one compute unit holds (LDS and registers) */
 static const double k_prefill_step_us[] = {0.87, 1.10, 1.50, 2.00, 2.00, 2.44};
 static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
-/* other variants worth choosing: {tile index, waves (8, or -4 = interleaved four-wave schedule), step cost,
- * workgroups per compute unit} */
+/* other variants worth choosing: {tile index, kernel family (8 = eight waves, -4 = interleaved four-wave
+ * schedule, 16 = four multiplying + four staging waves), step cost, workgroups per compute unit} */
 static const struct { int tile; int waves; double step_us; int per_cu; } k_prefill_alt[] = {
-    {3, 8, 1.45, 1}, {5, 8, 2.38, 1}, {3, -4, 1.33, 1}, {1, -4, 0.85, 2}};
+    {3, 8, 1.45, 1}, {5, 8, 2.38, 1}, {3, -4, 1.33, 1}, {1, -4, 0.85, 2}, {3, 16, 1.20, 1}, {2, 16, 0.76, 1}};
 
 extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
                                             int32_t *waves) {
@@ -952,12 +952,16 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     if (!known) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel with a %dx%d tile", bm, bn);
     /* waves == -4 selects the four-wave kernel with the interleaved decode/MFMA schedule */
     const bool has_il = (bm == 64 && bn == 128) || (bm == 128 && bn == 128) || (bm == 128 && bn == 256);
-    if (waves != 4 && !(waves == 8 && bm >= 128 && bn >= 128) && !(waves == -4 && has_il))
+    /* -5: four waves, X prefetched through registers */
+    /* 16: eight waves split into four multiplying and four staging ones */
+    const bool has_ws = bm == 128 && (bn == 128 || bn == 256);
+    if (waves != 4 && !(waves == 8 && bm >= 128 && bn >= 128) && !(waves == -4 && has_il) && !(waves == -5 && bm >= 128 && bn >= 128) &&
+        !(waves == 16 && has_ws))
         return fail(PSN_E_UNSUPPORTED, "prefill: no %d-wave kernel for a %dx%d tile", waves, bm, bn);
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
     /* the interleaved kernels carry their LDS as static arrays */
-    const int lds = waves == -4 ? 0 : 2 * (bm + bn) * 128;
+    const int lds = (waves < 0 || waves == 16) ? 0 : 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);
     if ((rc = bind(mod->ctx))) return rc;
     if (ksplit > 1) {
@@ -980,8 +984,8 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
     const int64_t blocks = 8 * ((nt + 7) / 8) * mt * ksplit;      /* the kernel spreads N tiles over 8 XCDs */
     char name[96];
-    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 8 ? "_w8" : waves == -4 ? "_il" : "");
-    return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * (waves == 8 ? 8 : 4)), (unsigned)lds, &a);
+    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 8 ? "_w8" : waves == -4 ? "_il" : waves == -5 ? "_rp" : waves == 16 ? "_ws" : "");
+    return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * ((waves == 8 || waves == 16) ? 8 : 4)), (unsigned)lds, &a);
 }
 
 extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,

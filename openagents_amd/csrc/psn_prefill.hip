@@ -22,6 +22,10 @@
 
 #define UNROLL _Pragma("unroll")
 
+#ifndef PSN_ABLATE
+#define PSN_ABLATE 0   /* development builds: 1 skips the weight decode, 2 the X loads, 4 the MFMAs of the K loop */
+#endif
+
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
@@ -402,17 +406,19 @@ PSN_DEV void prefill_body_il(const psn_prefill_args &a) {
      * the X stage of step +1. */
 #define PSN_PF_STEP(SUB, NSUB, wsrc, xc, xp, wc, wq, KEEP)                                            \
     {                                                                                                 \
-        stage_x(xp, (c * 4 + SUB + 3) * 64);                                                          \
+        if (!(PSN_ABLATE & 2)) stage_x(xp, (c * 4 + SUB + 3) * 64);                                   \
         half8_t af0[TM], bf0[TN], af1[TM], bf1[TN];                                                   \
-        load_frags(xc, wc, 0, af0, bf0);                                                              \
-        load_frags(xc, wc, 1, af1, bf1);                                                              \
-        mfmas(af0, bf0);                                                                              \
-        load_frags(xc, wc, 2, af0, bf0);                                                              \
-        mfmas(af1, bf1);                                                                              \
-        load_frags(xc, wc, 3, af1, bf1);                                                              \
-        mfmas(af0, bf0);                                                                              \
-        stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part);                      \
-        mfmas(af1, bf1);                                                                              \
+        if (!(PSN_ABLATE & 4)) {                                                                      \
+            load_frags(xc, wc, 0, af0, bf0);                                                          \
+            load_frags(xc, wc, 1, af1, bf1);                                                          \
+            mfmas(af0, bf0);                                                                          \
+            load_frags(xc, wc, 2, af0, bf0);                                                          \
+            mfmas(af1, bf1);                                                                          \
+            load_frags(xc, wc, 3, af1, bf1);                                                          \
+            mfmas(af0, bf0);                                                                          \
+        }                                                                                             \
+        if (!(PSN_ABLATE & 1)) stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part); \
+        if (!(PSN_ABLATE & 4)) mfmas(af1, bf1);                                                       \
         UNROLL for (int i_ = 0; i_ < 4 * TM * TN; ++i_) {                                             \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                        \
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                        \
@@ -433,6 +439,250 @@ PSN_DEV void prefill_body_il(const psn_prefill_args &a) {
     }
 #undef PSN_PF_STEP
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
+        UNROLL for (int r = 0; r < 16; ++r) {
+            const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (row < M && col < N) {
+                if (S == 1) a.Y[(int64_t)row * N + col] = acc[i][j][r];
+                else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], acc[i][j][r]);
+            }
+        }
+    }
+}
+
+/* ---- producer / consumer variant ----------------------------------------------------------------
+ * Measured on MI355X: a wave's own VALU work does not overlap its MFMAs (decode-only and MFMA-only
+ * runs of the kernels above add up to the full run), so the weight decode has to come from OTHER
+ * waves of the same SIMD.  512 threads: waves 0-3 only multiply (each a quarter of the BM x BN tile),
+ * waves 4-7 only stage -- X three K steps ahead by direct-to-LDS loads into four per-stage arrays,
+ * W one step ahead decoded from registers into two arrays.  One raw barrier per K step; producers
+ * wait only for the X stage that is due. */
+template <typename WF, int BM, int BN>
+PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
+    constexpr int NP = 256;                                 /* producer threads */
+    constexpr int P = NP / BN;                              /* producer threads per weight row */
+    constexpr int WM = 2, WN = 2;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int NX = BM * 8 / NP;
+    constexpr int NW = WF::DW / 4;
+    static_assert(P >= 1 && NX >= 1, "tile");
+    __shared__ uint4 xs0[BM * 8], xs1[BM * 8], xs2[BM * 8], xs3[BM * 8];
+    __shared__ uint4 ws0[BN * 8], ws1[BN * 8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool producer = wave >= 4;                        /* wave-uniform */
+    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
+    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+    const int S = a.ksplit;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_xcd_n = (nt + 7) >> 3;
+    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
+    const int tile_n = xcd + 8 * tn_local;
+    if (tn_local >= per_xcd_n || tile_n >= nt) return;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int per_split = (C + S - 1) / S;
+    const int c_begin = split * per_split, c_end = min(c_begin + per_split, C);
+    if (c_begin >= c_end) return;
+    const int k_last = c_end * 256 - 64;
+
+    if (producer) {
+        const int ptid = tid - 256, pwave = wave - 4;
+        const int wrow = ptid % BN, part = ptid / BN;
+        const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
+        u32 w[WF::DW], wnext[WF::DW];
+        auto stage_x = [&](uint4 *tile, int k0) {
+            k0 = min(k0, k_last);
+            UNROLL for (int i = 0; i < NX; ++i) {
+                const int s_ = i * NP + ptid, row = s_ >> 3, chunk = (s_ & 7) ^ (row & 7);
+                const uint16_t *src = a.X + (int64_t)min(m0 + row, M - 1) * K + k0 + chunk * 8;
+                __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + i * NP + pwave * 64), 16, 0, 0);
+            }
+        };
+        WF::load(wbase + (int64_t)c_begin * WF::BYTES, w);
+        const int k_begin = c_begin * 256;
+        stage_x(xs0, k_begin);
+        stage_x(xs1, k_begin + 64);
+        stage_x(xs2, k_begin + 128);
+        stage_part<WF, 0, P>(w, reinterpret_cast<char *>(ws0), wrow, part);
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#define PSN_WS_PRODUCE(SUB, NSUB, wsrc, xp, wq, KEEP)                                                 \
+        {                                                                                             \
+            if (!(PSN_ABLATE & 2)) stage_x(xp, (c * 4 + SUB + 3) * 64);                               \
+            if (!(PSN_ABLATE & 1)) stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part); \
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((PSN_ABLATE & 2) ? 0 : KEEP) : "memory"); \
+        }
+        for (int c = c_begin; c < c_end; ++c) {
+            WF::load(wbase + (int64_t)min(c + 1, C - 1) * WF::BYTES, wnext);
+            PSN_WS_PRODUCE(0, 1, w, xs3, ws1, 2 * NX + NW)
+            PSN_WS_PRODUCE(1, 2, w, xs0, ws0, 2 * NX + NW)
+            PSN_WS_PRODUCE(2, 3, w, xs1, ws1, 2 * NX)
+            PSN_WS_PRODUCE(3, 0, wnext, xs2, ws0, 2 * NX)
+            UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = wnext[i];
+        }
+#undef PSN_WS_PRODUCE
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        return;
+    }
+
+    /* consumers */
+    const int wm = wave / WN, wn = wave % WN;
+    float16_t acc[TM][TN];
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    auto load_frags = [&](const uint4 *xt, const uint4 *wt, int kk, half8_t (&af)[TM], half8_t (&bf)[TN]) {
+        const int chunk = 2 * kk + (lane >> 5);
+        UNROLL for (int i = 0; i < TM; ++i)
+            af[i] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(xt) + tile_off(wm * (BM / WM) + 32 * i + (lane & 31), chunk));
+        UNROLL for (int j = 0; j < TN; ++j)
+            bf[j] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(wt) + tile_off(wn * (BN / WN) + 32 * j + (lane & 31), chunk));
+    };
+    auto mfmas = [&](const half8_t (&af)[TM], const half8_t (&bf)[TN]) {
+        UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    };
+    asm volatile("s_barrier" ::: "memory");                  /* the prologue stages are in place */
+#define PSN_WS_CONSUME(xc, wc)                                                                        \
+    {                                                                                                 \
+        half8_t af0[TM], bf0[TN], af1[TM], bf1[TN];                                                   \
+        if (!(PSN_ABLATE & 4)) {                                                                      \
+            load_frags(xc, wc, 0, af0, bf0);                                                          \
+            load_frags(xc, wc, 1, af1, bf1);                                                          \
+            mfmas(af0, bf0);                                                                          \
+            load_frags(xc, wc, 2, af0, bf0);                                                          \
+            mfmas(af1, bf1);                                                                          \
+            load_frags(xc, wc, 3, af1, bf1);                                                          \
+            mfmas(af0, bf0);                                                                          \
+            mfmas(af1, bf1);                                                                          \
+        }                                                                                             \
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");                               \
+    }
+    for (int c = c_begin; c < c_end; ++c) {
+        PSN_WS_CONSUME(xs0, ws0)
+        PSN_WS_CONSUME(xs1, ws1)
+        PSN_WS_CONSUME(xs2, ws0)
+        PSN_WS_CONSUME(xs3, ws1)
+    }
+#undef PSN_WS_CONSUME
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
+        UNROLL for (int r = 0; r < 16; ++r) {
+            const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (row < M && col < N) {
+                if (S == 1) a.Y[(int64_t)row * N + col] = acc[i][j][r];
+                else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], acc[i][j][r]);
+            }
+        }
+    }
+}
+
+/* ---- register-prefetch variant ----------------------------------------------------------------
+ * As above, but the X tile travels global -> registers -> LDS: the loads of step s+3 are issued while
+ * step s multiplies (two register sets, each load has two full steps to land), and the tile of step
+ * s+1 is written to LDS from registers next to the decoded weights.  Ordinary register loads let the
+ * compiler count outstanding loads exactly, so nothing drains the queue in mid-loop; two LDS stages
+ * per operand suffice. */
+template <typename WF, int BM, int BN, int WM, int WN>
+PSN_DEV void prefill_body_rp(const psn_prefill_args &a) {
+    static_assert(WM * WN == 4, "four waves");
+    constexpr int NT = 256;
+    constexpr int P = NT / BN;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int NX = BM * 8 / NT;                         /* 16-byte words of X per thread and step */
+    __shared__ uint4 xs0[BM * 8], xs1[BM * 8];
+    __shared__ uint4 ws0[BN * 8], ws1[BN * 8];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
+    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+    const int S = a.ksplit;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_xcd_n = (nt + 7) >> 3;
+    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
+    const int tile_n = xcd + 8 * tn_local;
+    if (tn_local >= per_xcd_n || tile_n >= nt) return;
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int per_split = (C + S - 1) / S;
+    const int c_begin = split * per_split, c_end = min(c_begin + per_split, C);
+    if (c_begin >= c_end) return;
+    const int k_last = c_end * 256 - 64;
+
+    float16_t acc[TM][TN];
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    const int wrow = tid % BN, part = tid / BN;
+    const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
+    u32 w[WF::DW], wnext[WF::DW];
+
+    /* this thread's NX words of an X tile: word s = i*NT + tid -> row s/8, chunk (s%8)^(row&7) lands at s */
+    const uint16_t *xsrc[NX];
+    UNROLL for (int i = 0; i < NX; ++i) {
+        const int s_ = i * NT + tid, row = s_ >> 3, chunk = (s_ & 7) ^ (row & 7);
+        xsrc[i] = a.X + (int64_t)min(m0 + row, M - 1) * K + chunk * 8;
+    }
+    auto load_x = [&](uint4 (&r)[NX], int k0) {
+        k0 = min(k0, k_last);
+        UNROLL for (int i = 0; i < NX; ++i) r[i] = *reinterpret_cast<const uint4 *>(xsrc[i] + k0);
+    };
+    auto store_x = [&](uint4 *tile, const uint4 (&r)[NX]) {
+        UNROLL for (int i = 0; i < NX; ++i) tile[i * NT + tid] = r[i];
+    };
+    auto load_frags = [&](const uint4 *xt, const uint4 *wt, int kk, half8_t (&af)[TM], half8_t (&bf)[TN]) {
+        const int chunk = 2 * kk + (lane >> 5);
+        UNROLL for (int i = 0; i < TM; ++i)
+            af[i] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(xt) + tile_off(wm * (BM / WM) + 32 * i + (lane & 31), chunk));
+        UNROLL for (int j = 0; j < TN; ++j)
+            bf[j] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(wt) + tile_off(wn * (BN / WN) + 32 * j + (lane & 31), chunk));
+    };
+    auto mfmas = [&](const half8_t (&af)[TM], const half8_t (&bf)[TN]) {
+        UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+    };
+
+    /* prologue: step 0 into LDS, steps 1 and 2 into the two register sets */
+    uint4 xa[NX], xb[NX];
+    const int k_begin = c_begin * 256;
+    WF::load(wbase + (int64_t)c_begin * WF::BYTES, w);
+    load_x(xa, k_begin);
+    store_x(xs0, xa);
+    load_x(xb, k_begin + 64);                               /* X(1) */
+    load_x(xa, k_begin + 128);                              /* X(2) */
+    stage_part<WF, 0, P>(w, reinterpret_cast<char *>(ws0), wrow, part);
+    __syncthreads();
+
+    /* step SUB of chunk c: multiply from (xc, wc); X(step+1) goes from `xr` to LDS stage xq and `xr` is
+     * refilled with X(step+3); W(step+1) is decoded from `wsrc` (blocks 2*NSUB, 2*NSUB+1) into wq */
+#define PSN_RP_STEP(SUB, NSUB, wsrc, xc, xq, wc, wq, xr)                                               \
+    {                                                                                                 \
+        half8_t af0[TM], bf0[TN], af1[TM], bf1[TN];                                                   \
+        load_frags(xc, wc, 0, af0, bf0);                                                              \
+        load_frags(xc, wc, 1, af1, bf1);                                                              \
+        store_x(xq, xr);                                                                              \
+        load_x(xr, (c * 4 + SUB + 3) * 64);                                                           \
+        mfmas(af0, bf0);                                                                              \
+        load_frags(xc, wc, 2, af0, bf0);                                                              \
+        mfmas(af1, bf1);                                                                              \
+        load_frags(xc, wc, 3, af1, bf1);                                                              \
+        mfmas(af0, bf0);                                                                              \
+        stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part);                      \
+        mfmas(af1, bf1);                                                                              \
+        UNROLL for (int i_ = 0; i_ < 4 * TM * TN; ++i_) {                                             \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                        \
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                        \
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                        \
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                        \
+        }                                                                                             \
+        __builtin_amdgcn_s_waitcnt(0xC07F);                 /* lgkmcnt(0): this wave's LDS writes are done */ \
+        __builtin_amdgcn_s_barrier();                                                                 \
+    }
+
+    for (int c = c_begin; c < c_end; ++c) {
+        WF::load(wbase + (int64_t)min(c + 1, C - 1) * WF::BYTES, wnext);
+        PSN_RP_STEP(0, 1, w, xs0, xs1, ws0, ws1, xb)
+        PSN_RP_STEP(1, 2, w, xs1, xs0, ws1, ws0, xa)
+        PSN_RP_STEP(2, 3, w, xs0, xs1, ws0, ws1, xb)
+        PSN_RP_STEP(3, 0, wnext, xs1, xs0, ws1, ws0, xa)
+        UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = wnext[i];
+    }
+#undef PSN_RP_STEP
 
     UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
         const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
@@ -468,7 +718,23 @@ extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_a
         prefill_body_il<WF, BM, BN, WM, WN>(a);                                                              \
     }
 
+#define PSN_PREFILL_KERNEL_WS(fmt, WF, BM, BN)                                                               \
+    extern "C" __global__ void __launch_bounds__(512) psn_prefill_##fmt##_m##BM##_n##BN##_ws(const psn_prefill_args a) { \
+        prefill_body_ws<WF, BM, BN>(a);                                                                      \
+    }
+
+#define PSN_PREFILL_KERNEL_RP(fmt, WF, BM, BN, WM, WN)                                                       \
+    extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_m##BM##_n##BN##_rp(const psn_prefill_args a) { \
+        prefill_body_rp<WF, BM, BN, WM, WN>(a);                                                              \
+    }
+
 #define PSN_PREFILL_ALL(fmt, WF)               \
+    PSN_PREFILL_KERNEL_WS(fmt, WF, 128, 128)     \
+    PSN_PREFILL_KERNEL_WS(fmt, WF, 128, 256)     \
+    PSN_PREFILL_KERNEL_RP(fmt, WF, 128, 128, 2, 2) \
+    PSN_PREFILL_KERNEL_RP(fmt, WF, 128, 256, 2, 2) \
+    PSN_PREFILL_KERNEL_RP(fmt, WF, 256, 128, 2, 2) \
+    PSN_PREFILL_KERNEL_RP(fmt, WF, 256, 256, 2, 2) \
     PSN_PREFILL_KERNEL_IL(fmt, WF, 64, 128, 2, 2)  \
     PSN_PREFILL_KERNEL_IL(fmt, WF, 128, 128, 2, 2) \
     PSN_PREFILL_KERNEL_IL(fmt, WF, 128, 256, 2, 2) \

@@ -47,7 +47,8 @@ def test_every_tile_ragged_shapes(hip, orc, qname, tile):
         X = G.seeded_acts(801 + m, m, k).astype(np.float16)
         ref = orc.prefill(t, W, X, n, k)
         il = tile in ((64, 128), (128, 128), (128, 256))              # tiles with the interleaved (-4) kernel
-        for waves in (4,) + ((8,) if min(tile) >= 128 else ()) + ((-4,) if il else ()):
+        ws = tile in ((128, 128), (128, 256))                         # tiles with the producer/consumer (16) kernel
+        for waves in (4,) + ((8, -5) if min(tile) >= 128 else ()) + ((-4,) if il else ()) + ((16,) if ws else ()):
             for ksplit in (1, 2, 4):
                 if ksplit > 1 and (m * n) % 4:
                     continue
