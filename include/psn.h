@@ -244,6 +244,19 @@ int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const psn_buf *q, c
 /* out = silu(gate) * up; n % 4 == 0 */
 int32_t psn_swiglu(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, int64_t n);
 
+/* The same three producers with the activation quantization fused in: besides (or, with a NULL fp32
+ * output, instead of) the fp32 vector they write it as a one-row quantized activation tensor
+ * (psn_actq_layout(act_type, n, 1)) that psn_qmatvec_q8(_multi) consumes directly -- bit-identical to
+ * psn_act_quantize of the fp32 result.  n must be a multiple of 256 (psn_attention_decode_q8: an even
+ * number of heads). */
+int32_t psn_add_rmsnorm_q8(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
+                           psn_buf *y_q, int32_t act_type, int64_t n, float eps);
+int32_t psn_swiglu_q8(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, psn_buf *out_q,
+                      int32_t act_type, int64_t n);
+int32_t psn_attention_decode_q8(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
+                                psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
+                                int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx);
+
 #ifdef __cplusplus
 }
 #endif

@@ -87,6 +87,9 @@ SIGNATURES = {
     "psn_rope_kv_store": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, C.c_float]),
     "psn_attention_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32]),
     "psn_swiglu": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64]),
+    "psn_add_rmsnorm_q8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, C.c_float]),
+    "psn_swiglu_q8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64]),
+    "psn_attention_decode_q8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32]),
 }
 
 _lib = None

@@ -277,6 +277,21 @@ class HipBackend:
     def swiglu(self, gate, up, out, n: int):
         _check(self.lib.psn_swiglu(self.module, self.stream, gate.handle, up.handle, out.handle, n))
 
+    # the same producers with the activation quantization fused in (fp32 output optional)
+    @staticmethod
+    def _h(buf):
+        return buf.handle if buf is not None else None
+
+    def add_rmsnorm_q8(self, x, delta, weight, y, y_q, act_type: int, n: int, eps: float = 1e-5):
+        _check(self.lib.psn_add_rmsnorm_q8(self.module, self.stream, x.handle, self._h(delta), weight.handle, self._h(y), y_q.handle, act_type, n, eps))
+
+    def swiglu_q8(self, gate, up, out, out_q, act_type: int, n: int):
+        _check(self.lib.psn_swiglu_q8(self.module, self.stream, gate.handle, up.handle, self._h(out), out_q.handle, act_type, n))
+
+    def attention_decode_q8(self, q, k_cache, v_cache, workspace, out, out_q, act_type: int, n_heads: int, n_kv_heads: int, head_dim: int, n_ctx: int):
+        _check(self.lib.psn_attention_decode_q8(self.module, self.stream, q.handle, k_cache.handle, v_cache.handle, workspace.handle,
+                                                self._h(out), out_q.handle, act_type, n_heads, n_kv_heads, head_dim, n_ctx))
+
     # -- graphs -----------------------------------------------------------------------------
     def reserve(self, k: int, batch: int = 1):
         _check(self.lib.psn_stream_reserve(self.stream, k, batch))

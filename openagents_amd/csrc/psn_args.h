@@ -66,13 +66,22 @@ struct psn_fill_args {
 };
 
 /* decode-step glue kernels (psn_decode.hip) */
+/* optional quantized output of an elementwise kernel: the three fields of the activation layout for
+ * one row of n elements (qs null = not wanted); act_q8_K selects Q8_K (else Q8_0) */
+struct psn_actq_out {
+    int8_t *qs;
+    float *d;
+    void *s;
+    int32_t act_q8_K, pad;
+};
 struct psn_norm_args {
     float *x;             /* [n], updated in place when delta != null */
     const float *delta;   /* optional residual to add first */
     const float *weight;  /* [n] */
-    float *y;             /* [n] normalized output */
+    float *y;             /* [n] normalized output (may be null when only the quantized one is wanted) */
     int32_t n;
     float eps;
+    struct psn_actq_out qout;
 };
 struct psn_rope_args {
     float *q;             /* [n_heads][head_dim], rotated in place */
@@ -89,15 +98,17 @@ struct psn_attn_args {
     const void *k_cache;
     const void *v_cache;
     float *partial;       /* [n_heads][n_splits][130] */
-    float *out;           /* [n_heads][128] */
+    float *out;           /* [n_heads][128] (may be null when only the quantized one is wanted) */
     int32_t n_heads, n_kv_heads, n_ctx, n_splits;
     float scale;
     int32_t pad;
+    struct psn_actq_out qout;
 };
 struct psn_swiglu_args {
     const float *gate, *up;
-    float *out;
+    float *out;           /* may be null when only the quantized output is wanted */
     int32_t n, pad;
+    struct psn_actq_out qout;
 };
 
 #endif

@@ -10,6 +10,27 @@
 
 #define UNROLL _Pragma("unroll")
 
+/* Quantizes the four consecutive values a thread holds (element index 4*i4 of a row) into the row's
+ * activation fields.  Must be reached by whole waves: Q8_K needs the 64 lanes of a wave to hold one
+ * 256-element super-block (i4 = 64*sb + lane), Q8_0 needs 8 adjacent lanes per 32-element block. */
+PSN_DEV void quantize_out4(const psn_actq_out &q, int i4, float4 v) {
+    const int lane = threadIdx.x & 63;
+    u32 packed;
+    float d;
+    if (q.act_q8_K) {
+        int s16;
+        q8_K_quant_wave(v, lane, packed, d, s16);
+        reinterpret_cast<u32 *>(q.qs)[i4] = packed;
+        if ((lane & 3) == 0) reinterpret_cast<int16_t *>(q.s)[i4 >> 2] = (int16_t)s16;
+        if (lane == 0) q.d[i4 >> 6] = d;
+    } else {
+        int sum;
+        q8_0_quant4(v, packed, d, sum);
+        reinterpret_cast<u32 *>(q.qs)[i4] = packed;
+        if ((lane & 7) == 0) { q.d[i4 >> 3] = d; reinterpret_cast<int *>(q.s)[i4 >> 3] = sum; }
+    }
+}
+
 /* sum over a workgroup of up to 1024 threads; every thread gets the result */
 PSN_DEV float block_sum(float v, float *scratch) {
     v = group_sum<64>(v);
@@ -42,9 +63,12 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
     const float scale = 1.0f / sqrtf(ss / (float)a.n + a.eps);
     const float4 *w4 = reinterpret_cast<const float4 *>(a.weight);
     float4 *y4 = reinterpret_cast<float4 *>(a.y);
+    /* n is a multiple of 256 when a quantized output is asked for, so waves stay whole in this loop */
     for (int i = threadIdx.x; i < n4; i += blockDim.x) {
         const float4 v = x4[i], w = w4[i];
-        y4[i] = make_float4(v.x * scale * w.x, v.y * scale * w.y, v.z * scale * w.z, v.w * scale * w.w);
+        const float4 o = make_float4(v.x * scale * w.x, v.y * scale * w.y, v.z * scale * w.z, v.w * scale * w.w);
+        if (y4) y4[i] = o;
+        if (a.qout.qs) quantize_out4(a.qout, i, o);
     }
 }
 
@@ -135,11 +159,15 @@ extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_att
 /* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One workgroup of 128 threads per
  * head: the per-split (max, sum) pairs are fetched in parallel, the weights go through LDS, and the
  * partial outputs are summed eight loads at a time. */
-extern "C" __global__ void __launch_bounds__(128) psn_attn_combine(const psn_attn_args a) {
+template <bool PAIR>
+PSN_DEV void attn_combine_body(const psn_attn_args &a) {
     constexpr int D = 128;
-    __shared__ float wts[128];
-    __shared__ float red[4];
-    const int head = blockIdx.x, d = threadIdx.x;
+    __shared__ float wts_all[2][128];
+    __shared__ float red_all[2][4];
+    __shared__ float regroup[256];
+    const int hl = PAIR ? (threadIdx.x >> 7) : 0;             /* which of the workgroup's heads */
+    float *wts = wts_all[hl], *red = red_all[hl];
+    const int head = (PAIR ? 2 : 1) * blockIdx.x + hl, d = threadIdx.x & 127;
     const float *base = a.partial + (int64_t)head * a.n_splits * (D + 2);
     float num = 0.f, den = 0.f;
     /* global max first (splits are few: a strided pass per thread, then a block reduce) */
@@ -169,8 +197,23 @@ extern "C" __global__ void __launch_bounds__(128) psn_attn_combine(const psn_att
             UNROLL for (int u = 0; u < 8; ++u) if (i0 + u < cnt) num += o[u] * wts[i0 + u];
         }
     }
-    a.out[head * D + d] = num / den;
+    const float o = num / den;
+    if (a.out) a.out[head * D + d] = o;
+    if constexpr (PAIR) {
+        /* two heads = one 256-element super-block (or eight 32-element blocks): regroup through LDS so
+         * that wave 0 holds it four values per lane, the layout the quantizers work on */
+        regroup[threadIdx.x] = o;
+        __syncthreads();
+        if (threadIdx.x < 64) {
+            const float4 v = *reinterpret_cast<const float4 *>(&regroup[4 * threadIdx.x]);
+            quantize_out4(a.qout, blockIdx.x * 64 + threadIdx.x, v);
+        }
+    }
 }
+
+extern "C" __global__ void __launch_bounds__(128) psn_attn_combine(const psn_attn_args a) { attn_combine_body<false>(a); }
+/* two heads per workgroup, quantized output as well */
+extern "C" __global__ void __launch_bounds__(256) psn_attn_combine_q8(const psn_attn_args a) { attn_combine_body<true>(a); }
 
 /* out = silu(gate) * up */
 extern "C" __global__ void __launch_bounds__(256) psn_swiglu(const psn_swiglu_args a) {
@@ -182,5 +225,6 @@ extern "C" __global__ void __launch_bounds__(256) psn_swiglu(const psn_swiglu_ar
     o.y = g.y / (1.f + __expf(-g.y)) * u.y;
     o.z = g.z / (1.f + __expf(-g.z)) * u.z;
     o.w = g.w / (1.f + __expf(-g.w)) * u.w;
-    reinterpret_cast<float4 *>(a.out)[i] = o;
+    if (a.out) reinterpret_cast<float4 *>(a.out)[i] = o;
+    if (a.qout.qs) quantize_out4(a.qout, i, o);        /* n % 256 == 0 then: whole waves reach this point */
 }

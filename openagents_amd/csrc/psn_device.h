@@ -74,6 +74,54 @@ PSN_DEV int group_min_i(int v) {
     return v;
 }
 
+/* ---- activation quantizers (bit-exact restatements of the GGUF Q8_0 / Q8_K row quantizers); used by
+ *      the stand-alone quantize kernels, the matvec staging and the fused decode-step kernels ---- */
+
+/* Q8_0: the four elements a lane owns of a 32-element block shared by 8 adjacent lanes.
+ * d = amax/127, q = round-half-away(x/d); returns the packed int8x4, the fp16-rounded scale
+ * (widened) and the block's sum of q. */
+PSN_DEV void q8_0_quant4(const float4 v, u32 &packed, float &d_out, int &sum) {
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = group_max<8>(amax);
+    const float d = amax / 127.f;
+    const float id = d != 0.f ? 1.f / d : 0.f;
+    const int q0 = (int)roundf(v.x * id), q1 = (int)roundf(v.y * id);
+    const int q2 = (int)roundf(v.z * id), q3 = (int)roundf(v.w * id);
+    sum = group_sum_i<8>(q0 + q1 + q2 + q3);
+    packed = (u32)(q0 & 0xff) | ((u32)(q1 & 0xff) << 8) | ((u32)(q2 & 0xff) << 16) | ((u32)q3 << 24);
+    d_out = (float)(f16)d;            /* what a reader of the fp16 field would see */
+}
+
+/* Q8_K: one wave owns a 256-element super-block, four elements per lane.
+ * iscale = -127/(signed element of largest magnitude, first one on ties), q = min(127, rint(iscale*x)),
+ * d = 1/iscale; s16 = sum of q over the lane's 16-element group (valid in every lane of the quad). */
+PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out, int &s16) {
+    const float e[4] = {v.x, v.y, v.z, v.w};
+    float amax = 0.f;
+    int first = 4;
+    /* >= scanning downwards leaves the lowest index among equal magnitudes */
+    _Pragma("unroll") for (int i = 3; i >= 0; --i) if (fabsf(e[i]) >= amax) { amax = fabsf(e[i]); first = i; }
+    const float wmax = group_max<64>(amax);
+    const int cand = (amax == wmax) ? lane * 4 + first : 1 << 20;
+    const int idx = group_min_i<64>(cand);
+    const float mine = e[idx & 3];
+    const float vmax = __shfl(mine, idx >> 2, 64);
+    packed = 0;
+    int s4 = 0;
+    d_out = 0.f;
+    if (wmax != 0.f) {
+        const float iscale = -127.f / vmax;
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {
+            int q = (int)__builtin_rintf(iscale * e[i]);
+            q = q > 127 ? 127 : q;
+            s4 += q;
+            packed |= (u32)(q & 0xff) << (8 * i);
+        }
+        d_out = 1.f / iscale;
+    }
+    s16 = group_sum_i<4>(s4);
+}
+
 PSN_DEV void unpack4(const uint4 v, u32 *dst) { dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
 
 #endif

@@ -1007,24 +1007,48 @@ static int32_t need(const psn_buf *b, int64_t bytes, const char *what, const cha
     return PSN_OK;
 }
 
-extern "C" int32_t psn_add_rmsnorm(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
-                                   int64_t n, float eps) {
-    int32_t rc = check_same_ctx(mod, s, x, weight, y, "psn_add_rmsnorm");
+/* fills the optional quantized-output descriptor of an elementwise kernel (yq null: not wanted) */
+static int32_t set_actq_out(const char *what, psn_module *mod, psn_buf *yq, int32_t act_type, int64_t n, psn_actq_out *q) {
+    memset(q, 0, sizeof *q);
+    if (!yq) return PSN_OK;
+    if (yq->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "%s: handles belong to different contexts", what);
+    if (n % 256) return fail(PSN_E_SHAPE, "%s: a quantized output needs n to be a multiple of 256 (n=%lld)", what, (long long)n);
+    psn_actq_info li;
+    int32_t rc = psn_actq_layout(act_type, n, 1, &li);
     if (rc) return rc;
+    if ((int64_t)yq->bytes < li.bytes) return fail(PSN_E_INVALID_ARG, "%s: quantized output holds %zu bytes, need %lld", what, yq->bytes, (long long)li.bytes);
+    q->qs = (int8_t *)yq->p + li.off_qs;
+    q->d = (float *)((char *)yq->p + li.off_d);
+    q->s = (char *)yq->p + li.off_s;
+    q->act_q8_K = act_type == PSN_Q8_K;
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_add_rmsnorm_q8(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
+                                      psn_buf *yq, int32_t act_type, int64_t n, float eps) {
+    int32_t rc = check_same_ctx(mod, s, x, weight, x, "psn_add_rmsnorm");
+    if (rc) return rc;
+    if (!y && !yq) return fail(PSN_E_INVALID_ARG, "psn_add_rmsnorm: no output");
     if (n <= 0 || n % 4 || n > (1 << 24)) return fail(PSN_E_SHAPE, "psn_add_rmsnorm: n=%lld must be a positive multiple of 4", (long long)n);
     if ((rc = need(x, n * 4, "psn_add_rmsnorm", "x")) || (rc = need(weight, n * 4, "psn_add_rmsnorm", "weight")) ||
-        (rc = need(y, n * 4, "psn_add_rmsnorm", "y")) || (delta && (rc = need(delta, n * 4, "psn_add_rmsnorm", "delta"))))
+        (y && (rc = need(y, n * 4, "psn_add_rmsnorm", "y"))) || (delta && (rc = need(delta, n * 4, "psn_add_rmsnorm", "delta"))))
         return rc;
-    if ((rc = bind(mod->ctx))) return rc;
     psn_norm_args a;
+    if ((rc = set_actq_out("psn_add_rmsnorm", mod, yq, act_type, n, &a.qout))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
     a.x = (float *)x->p;
     a.delta = delta ? (const float *)delta->p : nullptr;
     a.weight = (const float *)weight->p;
-    a.y = (float *)y->p;
+    a.y = y ? (float *)y->p : nullptr;
     a.n = (int32_t)n;
     a.eps = eps;
     const unsigned threads = n >= 4096 ? 1024 : n >= 1024 ? 256 : 64;
     return launch(mod, s, "psn_add_rmsnorm", 1, threads, 0, &a);
+}
+extern "C" int32_t psn_add_rmsnorm(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
+                                   int64_t n, float eps) {
+    if (!y) return fail(PSN_E_INVALID_ARG, "psn_add_rmsnorm: y is null");
+    return psn_add_rmsnorm_q8(mod, s, x, delta, weight, y, nullptr, PSN_Q8_K, n, eps);
 }
 
 extern "C" int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q, psn_buf *k, const psn_buf *v, psn_buf *k_cache,
@@ -1054,49 +1078,66 @@ extern "C" int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q,
     return launch(mod, s, "psn_rope_kv_store", (unsigned)((pairs + 255) / 256), 256, 0, &a);
 }
 
-extern "C" int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
-                                        psn_buf *workspace, psn_buf *out, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx) {
+extern "C" int32_t psn_attention_decode_q8(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
+                                           psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
+                                           int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx) {
     int32_t rc = check_same_ctx(mod, s, q, k_cache, v_cache, "psn_attention_decode");
     if (rc) return rc;
+    if (!workspace || (!out && !out_q)) return fail(PSN_E_INVALID_ARG, "psn_attention_decode: null workspace or no output");
+    if (out_q && (n_heads & 1)) return fail(PSN_E_SHAPE, "psn_attention_decode: a quantized output needs an even number of heads");
     if (head_dim != 128) return fail(PSN_E_UNSUPPORTED, "psn_attention_decode: head_dim=%d (128 has a kernel)", head_dim);
     if (n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads || n_heads / n_kv_heads > 8)
         return fail(PSN_E_SHAPE, "psn_attention_decode: %d query heads over %d kv heads (need a multiple, at most 8 per group)", n_heads, n_kv_heads);
     if (n_ctx <= 0) return fail(PSN_E_SHAPE, "psn_attention_decode: n_ctx=%d", n_ctx);
     const int32_t splits = (n_ctx + 63) / 64;
     const int64_t row = (int64_t)n_kv_heads * head_dim * 2;
-    if ((rc = need(q, (int64_t)n_heads * 512, "psn_attention_decode", "q")) || (rc = need(out, (int64_t)n_heads * 512, "psn_attention_decode", "out")) ||
+    if ((rc = need(q, (int64_t)n_heads * 512, "psn_attention_decode", "q")) || (out && (rc = need(out, (int64_t)n_heads * 512, "psn_attention_decode", "out"))) ||
         (rc = need(k_cache, n_ctx * row, "psn_attention_decode", "k_cache")) || (rc = need(v_cache, n_ctx * row, "psn_attention_decode", "v_cache")) ||
         (rc = need(workspace, (int64_t)n_heads * splits * 130 * 4, "psn_attention_decode", "workspace")))
         return rc;
-    if (workspace->ctx != mod->ctx || out->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "psn_attention_decode: handles belong to different contexts");
-    if ((rc = bind(mod->ctx))) return rc;
+    if (workspace->ctx != mod->ctx || (out && out->ctx != mod->ctx)) return fail(PSN_E_INVALID_ARG, "psn_attention_decode: handles belong to different contexts");
     psn_attn_args a;
     memset(&a, 0, sizeof a);
+    if ((rc = set_actq_out("psn_attention_decode", mod, out_q, act_type, (int64_t)n_heads * 128, &a.qout))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
     a.q = (const float *)q->p;
     a.k_cache = k_cache->p;
     a.v_cache = v_cache->p;
     a.partial = (float *)workspace->p;
-    a.out = (float *)out->p;
+    a.out = out ? (float *)out->p : nullptr;
     a.n_heads = n_heads;
     a.n_kv_heads = n_kv_heads;
     a.n_ctx = n_ctx;
     a.n_splits = splits;
     a.scale = 0.08838834764831845f;                 /* 1/sqrt(128) */
     if ((rc = launch(mod, s, "psn_attn_partial", (unsigned)(n_kv_heads * splits), (unsigned)(64 * (n_heads / n_kv_heads)), 0, &a))) return rc;
+    if (out_q) return launch(mod, s, "psn_attn_combine_q8", (unsigned)(n_heads / 2), 256, 0, &a);
     return launch(mod, s, "psn_attn_combine", (unsigned)n_heads, 128, 0, &a);
 }
+extern "C" int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
+                                        psn_buf *workspace, psn_buf *out, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_attention_decode: out is null");
+    return psn_attention_decode_q8(mod, s, q, k_cache, v_cache, workspace, out, nullptr, PSN_Q8_K, n_heads, n_kv_heads, head_dim, n_ctx);
+}
 
-extern "C" int32_t psn_swiglu(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, int64_t n) {
-    int32_t rc = check_same_ctx(mod, s, gate, up, out, "psn_swiglu");
+extern "C" int32_t psn_swiglu_q8(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, psn_buf *out_q,
+                                 int32_t act_type, int64_t n) {
+    int32_t rc = check_same_ctx(mod, s, gate, up, gate, "psn_swiglu");
     if (rc) return rc;
+    if (!out && !out_q) return fail(PSN_E_INVALID_ARG, "psn_swiglu: no output");
     if (n <= 0 || n % 4 || n > (1 << 28)) return fail(PSN_E_SHAPE, "psn_swiglu: n=%lld must be a positive multiple of 4", (long long)n);
-    if ((rc = need(gate, n * 4, "psn_swiglu", "gate")) || (rc = need(up, n * 4, "psn_swiglu", "up")) || (rc = need(out, n * 4, "psn_swiglu", "out"))) return rc;
-    if ((rc = bind(mod->ctx))) return rc;
+    if ((rc = need(gate, n * 4, "psn_swiglu", "gate")) || (rc = need(up, n * 4, "psn_swiglu", "up")) || (out && (rc = need(out, n * 4, "psn_swiglu", "out")))) return rc;
     psn_swiglu_args a;
+    if ((rc = set_actq_out("psn_swiglu", mod, out_q, act_type, n, &a.qout))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
     a.gate = (const float *)gate->p;
     a.up = (const float *)up->p;
-    a.out = (float *)out->p;
+    a.out = out ? (float *)out->p : nullptr;
     a.n = (int32_t)n;
     a.pad = 0;
     return launch(mod, s, "psn_swiglu", (unsigned)((n / 4 + 255) / 256), 256, 0, &a);
+}
+extern "C" int32_t psn_swiglu(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, int64_t n) {
+    if (!out) return fail(PSN_E_INVALID_ARG, "psn_swiglu: out is null");
+    return psn_swiglu_q8(mod, s, gate, up, out, nullptr, PSN_Q8_K, n);
 }

@@ -22,7 +22,7 @@ from dataclasses import dataclass, field
 import numpy as np
 
 from ._ffi import ACT_Q8, Q4_K, Q6_K
-from .backend import DeviceBuffer, HipBackend, QuantizedTensor, row_bytes
+from .backend import DeviceBuffer, HipBackend, QuantizedTensor, act_type_for, actq_layout, row_bytes
 
 
 @dataclass
@@ -65,8 +65,13 @@ class ModelWeights:
 class DecodeStep:
     """Owns the activations, KV caches and scratch of one sequence and enqueues one token step."""
 
-    def __init__(self, be: HipBackend, shape: LlamaShape, weights: ModelWeights, max_ctx: int, scheme: int = ACT_Q8):
+    def __init__(self, be: HipBackend, shape: LlamaShape, weights: ModelWeights, max_ctx: int, scheme: int = ACT_Q8,
+                 fused_quant: bool = True):
+        """fused_quant (scheme Q8): the norm, attention and SwiGLU kernels emit their result already
+        quantized, and the matvecs read it with the pre-quantized entry points; otherwise every matvec
+        quantizes its fp32 input itself."""
         self.be, self.shape, self.w, self.max_ctx, self.scheme = be, shape, weights, max_ctx, scheme
+        self.fused = fused_quant and scheme == ACT_Q8
         s = shape
         if s.n_heads * s.head_dim != s.hidden:
             raise ValueError("n_heads * head_dim must equal hidden")
@@ -88,10 +93,43 @@ class DecodeStep:
         self.k_cache = [be.alloc(cache_bytes) for _ in range(s.n_layers)]
         self.v_cache = [be.alloc(cache_bytes) for _ in range(s.n_layers)]
         be.reserve(max(s.hidden, s.ffn), 1)
+        if self.fused:
+            l0 = weights.layers[0]
+            kinds = {act_type_for(t.qtype) for t in (l0.wq, l0.wo, l0.w_gate, l0.w_down, weights.lm_head)}
+            if len(kinds) != 1:
+                raise ValueError("fused quantization needs one activation type for all projections")
+            self.act_type = kinds.pop()
+            self.xq_h = be.alloc(int(actq_layout(self.act_type, s.hidden, 1).bytes))
+            self.xq_attn = be.alloc(int(actq_layout(self.act_type, s.hidden, 1).bytes))
+            self.xq_f = be.alloc(int(actq_layout(self.act_type, s.ffn, 1).bytes))
+
+    def _enqueue_fused(self, pos: int, matvecs_only: bool):
+        be, s, at = self.be, self.shape, self.act_type
+        glue = not matvecs_only
+        for li, lw in enumerate(self.w.layers):
+            if glue:
+                be.add_rmsnorm_q8(self.x, self.down if li > 0 else None, lw.attn_norm, None, self.xq_h, at, s.hidden, s.eps)
+            be.quantized_matvec_q8_multi([lw.wq, lw.wk, lw.wv], self.xq_h, [self.q, self.k, self.v], 1)
+            if glue:
+                be.rope_kv_store(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], s.n_heads, s.n_kv_heads, s.head_dim, pos, s.rope_theta)
+                be.attention_decode_q8(self.q, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn, at,
+                                       s.n_heads, s.n_kv_heads, s.head_dim, pos + 1)
+            be.quantized_matvec_q8(lw.wo, self.xq_attn, self.o, 1)
+            if glue:
+                be.add_rmsnorm_q8(self.x, self.o, lw.ffn_norm, None, self.xq_h, at, s.hidden, s.eps)
+            be.quantized_matvec_q8_multi([lw.w_gate, lw.w_up], self.xq_h, [self.gate, self.up], 1)
+            if glue:
+                be.swiglu_q8(self.gate, self.up, None, self.xq_f, at, s.ffn)
+            be.quantized_matvec_q8(lw.w_down, self.xq_f, self.down, 1)
+        if glue:
+            be.add_rmsnorm_q8(self.x, self.down, self.w.final_norm, None, self.xq_h, at, s.hidden, s.eps)
+        be.quantized_matvec_q8(self.w.lm_head, self.xq_h, self.logits, 1)
 
     def enqueue(self, pos: int, matvecs_only: bool = False):
         """All launches of one token at position `pos`; self.x holds the token's embedding on entry.
         With matvecs_only the glue ops are skipped (same matvec launches on whatever the buffers hold)."""
+        if self.fused:
+            return self._enqueue_fused(pos, matvecs_only)
         be, s, sch = self.be, self.shape, self.scheme
         glue = not matvecs_only
         for li, lw in enumerate(self.w.layers):
@@ -166,12 +204,13 @@ def main(argv=None):
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--unfused", action="store_true", help="every matvec quantizes its own fp32 input")
     args = ap.parse_args(argv)
     be = HipBackend(0)
     shape = LlamaShape(n_layers=args.layers)
     t0 = time.time()
     weights = synthetic_weights(be, shape, args.seed)
-    step = DecodeStep(be, shape, weights, args.ctx)
+    step = DecodeStep(be, shape, weights, args.ctx, fused_quant=not args.unfused)
     rng = np.random.default_rng(args.seed + 1)
     pos = args.ctx - 1
     kv = rng.standard_normal((pos, shape.kv_dim), dtype=np.float32).astype(np.float16)
@@ -209,7 +248,7 @@ def main(argv=None):
            "hbm_peak_GBps": 8000.0, "matvec_frac_of_hbm_peak": round(mbytes / t_mv / 1e3 / 8000.0, 4),
            "config": {"layers": shape.n_layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,
                       "ffn": shape.ffn, "vocab": shape.vocab, "context": args.ctx, "weights": "Q4_K projections, Q6_K LM head",
-                      "activation_scheme": "Q8 (Q8_K blocks, quantized inside the matvec launch)",
+                      "activation_scheme": "Q8 (Q8_K blocks, " + ("written by the producing kernel)" if step.fused else "quantized inside the matvec launch)"),
                       "launches_per_token": shape.n_layers * 10 + 2, "graph_replay": True},
            "data": "synthetic random-init weights (one unique layer copied to every layer's own allocation), fp16 N(0,1) KV cache",
            "logits_finite": bool(np.all(np.isfinite(logits))), "steps": args.steps, "setup_s": round(setup_s, 1),

@@ -112,6 +112,49 @@ def test_swiglu(hip):
     assert G.max_rel_err(out.download(np.float32, (n,)), ref) < 1e-5
 
 
+@pytest.mark.parametrize("act", ["Q8_0", "Q8_K"])
+def test_fused_quantized_outputs_match_separate_quantization(hip, act):
+    """RMSNorm, SwiGLU and attention with the activation quantization fused in must write exactly the
+    bytes psn_act_quantize produces from their fp32 result."""
+    from openagents_amd import backend
+    at = getattr(_ffi, act)
+    rng = np.random.default_rng(905)
+
+    def fields(buf, n):
+        li = backend.actq_layout(at, n, 1)
+        return buf.download(np.uint8, (int(li.bytes),))[: int(li.off_s) + (n // 32 * 4 if at == _ffi.Q8_0 else n // 16 * 2)]
+
+    def same(buf_q, y_f32, n):
+        ref = hip.quantize_activations(y_f32, n, 1, at)
+        li = backend.actq_layout(at, n, 1)
+        a, b = buf_q.download(np.uint8, (int(li.bytes),)), ref.download(np.uint8, (int(li.bytes),))
+        used = [(0, n), (int(li.off_d), n // (32 if at == _ffi.Q8_0 else 256) * 4), (int(li.off_s), n // 32 * 4 if at == _ffi.Q8_0 else n // 16 * 2)]
+        for off, ln in used:
+            assert np.array_equal(a[off:off + ln], b[off:off + ln])
+
+    for n in (256, 4096, 14336):
+        x = rng.standard_normal(n, dtype=np.float32) * 2
+        dl = rng.standard_normal(n, dtype=np.float32)
+        w = rng.standard_normal(n, dtype=np.float32)
+        y, yq = hip.alloc(n * 4), hip.alloc(int(backend.actq_layout(at, n, 1).bytes))
+        hip.add_rmsnorm_q8(hip.upload(x), hip.upload(dl), hip.upload(w), y, yq, at, n)
+        same(yq, y, n)
+        g, u = hip.upload(rng.standard_normal(n, dtype=np.float32) * 3), hip.upload(rng.standard_normal(n, dtype=np.float32))
+        hip.swiglu_q8(g, u, y, yq, at, n)
+        same(yq, y, n)
+    nh, nkv, d, n_ctx = 32, 8, 128, 300
+    q = hip.upload(rng.standard_normal(nh * d, dtype=np.float32))
+    kc = hip.upload(rng.standard_normal((n_ctx, nkv * d), dtype=np.float32).astype(np.float16))
+    vc = hip.upload(rng.standard_normal((n_ctx, nkv * d), dtype=np.float32).astype(np.float16))
+    ws = hip.alloc(nh * ((n_ctx + 63) // 64) * 130 * 4)
+    out, outq = hip.alloc(nh * d * 4), hip.alloc(int(backend.actq_layout(at, nh * d, 1).bytes))
+    ref_out = hip.alloc(nh * d * 4)
+    hip.attention_decode(q, kc, vc, ws, ref_out, nh, nkv, d, n_ctx)
+    hip.attention_decode_q8(q, kc, vc, ws, out, outq, at, nh, nkv, d, n_ctx)
+    assert np.array_equal(out.download(np.float32, (nh * d,)), ref_out.download(np.float32, (nh * d,)))
+    same(outq, out, nh * d)
+
+
 def test_whole_small_decode_step_eager_and_graph(hip, orc):
     s = LlamaShape(hidden=512, n_heads=4, n_kv_heads=2, head_dim=128, ffn=1024, vocab=768, n_layers=3)
     ctx, pos = 150, 149
@@ -135,6 +178,7 @@ def test_whole_small_decode_step_eager_and_graph(hip, orc):
     head = qmat(orc.Q6_K, s.vocab, s.hidden)
     weights = ModelWeights(dev_layers, hip.upload(final_norm), hip.upload_weight(orc.Q6_K, head, s.vocab, s.hidden))
     step = DecodeStep(hip, s, weights, ctx)
+    unfused = DecodeStep(hip, s, weights, ctx, fused_quant=False)
     kv0 = [(rng.standard_normal((ctx, s.kv_dim), dtype=np.float32).astype(np.float16), rng.standard_normal((ctx, s.kv_dim), dtype=np.float32).astype(np.float16))
            for _ in range(s.n_layers)]
     x0 = rng.standard_normal(s.hidden, dtype=np.float32)
@@ -172,6 +216,14 @@ def test_whole_small_decode_step_eager_and_graph(hip, orc):
     say(f"small decode step: logits max_rel_err={err:.3e}")
     assert err < 1e-3
     assert int(np.argmax(eager)) == int(np.argmax(ref_logits))
+
+    # the path where every matvec quantizes its own fp32 input gives the same logits bit for bit
+    for li in range(s.n_layers):
+        unfused.k_cache[li].upload(kv0[li][0])
+        unfused.v_cache[li].upload(kv0[li][1])
+    unfused.x.upload(x0)
+    unfused.enqueue(pos)
+    assert np.array_equal(unfused.logits.download(np.float32, (s.vocab,)), eager)
 
     graph = step.capture(pos)
     try:
