@@ -1,0 +1,85 @@
+"""GGUF container: writer -> reader round trip (CPU) and file -> device -> matvec parity (GPU).
+
+No .gguf file exists in the reference tree, so what is pinned here is the container layout as this
+module states it (header fields, typed metadata, alignment, tensor table) and that quantized tensor
+bytes reach the kernels unchanged; agreement with files written by other tools is not covered."""
+import struct
+
+import numpy as np
+import pytest
+
+import ggufref as G
+from openagents_amd import gguf
+
+
+def make_file(orc, path, alignment=32):
+    k = 1024
+    tensors, raw = [], {}
+    for name, t, n in (("blk.0.attn_q.weight", orc.Q4_0, 48), ("blk.0.ffn_down.weight", orc.Q4_K, 40),
+                       ("output.weight", orc.Q6_K, 72), ("blk.0.attn_k.weight", orc.Q8_0, 16)):
+        blocks = orc.quantize(t, G.seeded_weights(1000 + n, n, k))
+        raw[name] = (t, n, k, blocks)
+        tensors.append((name, (k, n), t, blocks))
+    norm = np.linspace(0.5, 1.5, 512, dtype=np.float32)
+    tensors.append(("output_norm.weight", (512,), 0, norm.view(np.uint8)))
+    md = {"general.architecture": (gguf.STRING, "llama"), "llama.block_count": (gguf.U32, 1),
+          "llama.rope.freq_base": (gguf.F32, 500000.0), "general.file_type": (gguf.I32, -7),
+          "tokenizer.ggml.tokens": (gguf.ARRAY, (gguf.STRING, ["<s>", "</s>", "héllo"])),
+          "some.u64": (gguf.U64, 2 ** 40 + 3), "some.bool": (gguf.BOOL, True), "some.f64": (gguf.F64, 0.1),
+          "some.i8s": (gguf.ARRAY, (gguf.I8, [-128, 0, 127]))}
+    gguf.write_gguf(str(path), md, tensors, alignment)
+    return raw, norm
+
+
+@pytest.mark.parametrize("alignment", [32, 64, 4096])
+def test_round_trip_header_metadata_and_tensor_bytes(orc, tmp_path, alignment):
+    path = tmp_path / "m.gguf"
+    raw, norm = make_file(orc, path, alignment)
+    f = gguf.GGUFFile(str(path))
+    assert f.version == 3 and f.alignment == alignment and f.data_start % alignment == 0
+    assert f.metadata["general.architecture"] == "llama" and f.metadata["llama.block_count"] == 1
+    assert f.metadata["llama.rope.freq_base"] == 500000.0 and f.metadata["general.file_type"] == -7
+    assert f.metadata["tokenizer.ggml.tokens"] == ["<s>", "</s>", "héllo"]
+    assert f.metadata["some.u64"] == 2 ** 40 + 3 and f.metadata["some.bool"] is True and f.metadata["some.i8s"] == [-128, 0, 127]
+    assert list(f.tensors) == list(raw) + ["output_norm.weight"]
+    for name, (t, n, k, blocks) in raw.items():
+        info = f.tensors[name]
+        assert (info.ggml_type, info.n, info.k, info.offset % alignment) == (t, n, k, 0)
+        assert np.array_equal(f.data(name), blocks.reshape(-1))
+    assert np.array_equal(f.data("output_norm.weight").view(np.float32), norm)
+    # the first bytes are exactly the documented header
+    head = open(path, "rb").read(24)
+    assert head[:4] == b"GGUF" and struct.unpack("<IQQ", head[4:]) == (3, 5, 9 + (alignment != 32))
+
+
+def test_malformed_files_are_rejected(orc, tmp_path):
+    path = tmp_path / "m.gguf"
+    make_file(orc, path)
+    good = open(path, "rb").read()
+    cases = {"magic": b"GGML" + good[4:], "version": good[:4] + struct.pack("<I", 9) + good[8:], "truncated": good[:-100],
+             "header cut": good[:40]}
+    for what, blob in cases.items():
+        p = tmp_path / f"bad_{what.replace(' ', '_')}.gguf"
+        p.write_bytes(blob)
+        with pytest.raises(gguf.GGUFError):
+            gguf.GGUFFile(str(p))
+    with pytest.raises(gguf.GGUFError):
+        gguf.write_gguf(str(tmp_path / "x.gguf"), {}, [("t", (100, 4), 2, np.zeros(10, np.uint8))])   # ragged row
+    with pytest.raises(gguf.GGUFError):
+        gguf.tensor_nbytes(13, (256, 4))                                                              # Q5_K: not supported
+
+
+@pytest.mark.gpu
+def test_tensors_from_a_file_reach_the_kernels_unchanged(hip, orc, tmp_path):
+    path = tmp_path / "m.gguf"
+    raw, _ = make_file(orc, path)
+    f = gguf.GGUFFile(str(path))
+    x = G.seeded_acts(1100, 1, 1024)
+    xb = hip.upload(x)
+    for name, (t, n, k, blocks) in raw.items():
+        w = f.upload(hip, name)
+        y = hip.alloc(n * 4)
+        hip.quantized_matvec(w, xb, y)
+        assert G.max_rel_err(y.download(np.float32, (1, n)), orc.matvec(t, orc.ACT_Q8, blocks, x, n, k)) < 2e-5
+    with pytest.raises(gguf.GGUFError):
+        f.upload(hip, "output_norm.weight")
