@@ -96,7 +96,12 @@ class DeviceBuffer:
 
     def free(self):
         if self.handle is not None and self._b.ctx is not None:
-            _check(self._b.lib.psn_buf_free(self.handle))
+            if self._b._capturing:
+                # freeing device memory while a stream of this thread is being captured would invalidate
+                # the capture (a buffer can die at any moment when the garbage collector runs)
+                self._b._deferred_free.append(self.handle)
+            else:
+                _check(self._b.lib.psn_buf_free(self.handle))
         self.handle = None
 
     def __del__(self):
@@ -123,6 +128,8 @@ class HipBackend:
     def __init__(self, device: int = 0):
         self.lib = _ffi.load()
         self.ctx = None
+        self._capturing = False
+        self._deferred_free = []
         ctx = C.c_void_p()
         _check(self.lib.psn_ctx_create(device, C.byref(ctx)))
         self.ctx = ctx
@@ -298,10 +305,17 @@ class HipBackend:
 
     def begin_capture(self):
         _check(self.lib.psn_graph_begin_capture(self.stream))
+        self._capturing = True
 
     def end_capture(self) -> C.c_void_p:
         g = C.c_void_p()
-        _check(self.lib.psn_graph_end_capture(self.stream, C.byref(g)))
+        try:
+            _check(self.lib.psn_graph_end_capture(self.stream, C.byref(g)))
+        finally:
+            self._capturing = False
+            pending, self._deferred_free = self._deferred_free, []
+            for h in pending:
+                self.lib.psn_buf_free(h)
         return g
 
     def launch_graph(self, graph):

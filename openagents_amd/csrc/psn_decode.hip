@@ -43,32 +43,66 @@ PSN_DEV float block_sum(float v, float *scratch) {
     return t;
 }
 
-/* x += delta (if delta != null);  y = x * rsqrt(mean(x^2) + eps) * weight.   One workgroup, n % 4 == 0. */
+/* x += delta (if delta != null);  y = x * rsqrt(mean(x^2) + eps) * weight.   One workgroup, n % 4 == 0.
+ * Up to four float4 per thread stay in registers between the two passes and the norm weights are
+ * requested before the reduction, so the kernel pays one memory round trip; longer vectors re-read x. */
 extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_norm_args a) {
     __shared__ float red[16];
-    const int n4 = a.n >> 2;
+    constexpr int KEEP = 4;
+    const int n4 = a.n >> 2, nt = blockDim.x;
     float4 *x4 = reinterpret_cast<float4 *>(a.x);
     const float4 *d4 = reinterpret_cast<const float4 *>(a.delta);
+    const float4 *w4 = reinterpret_cast<const float4 *>(a.weight);
+    float4 *y4 = reinterpret_cast<float4 *>(a.y);
+    const bool in_regs = n4 <= KEEP * nt;                          /* uniform */
+    float4 v[KEEP], w[KEEP];
     float ss = 0.f;
-    for (int i = threadIdx.x; i < n4; i += blockDim.x) {
-        float4 v = x4[i];
-        if (d4) {
-            const float4 d = d4[i];
-            v.x += d.x; v.y += d.y; v.z += d.z; v.w += d.w;
-            x4[i] = v;
+    if (in_regs) {
+        UNROLL for (int k = 0; k < KEEP; ++k) {
+            const int i = threadIdx.x + k * nt;
+            v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            w[k] = v[k];
+            if (i < n4) {
+                v[k] = x4[i];
+                w[k] = w4[i];
+                if (d4) {
+                    const float4 d = d4[i];
+                    v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
+                    x4[i] = v[k];
+                }
+            }
+            ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
         }
-        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    } else {
+        for (int i = threadIdx.x; i < n4; i += nt) {
+            float4 t = x4[i];
+            if (d4) {
+                const float4 d = d4[i];
+                t.x += d.x; t.y += d.y; t.z += d.z; t.w += d.w;
+                x4[i] = t;
+            }
+            ss += t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w;
+        }
     }
     ss = block_sum(ss, red);
     const float scale = 1.0f / sqrtf(ss / (float)a.n + a.eps);
-    const float4 *w4 = reinterpret_cast<const float4 *>(a.weight);
-    float4 *y4 = reinterpret_cast<float4 *>(a.y);
-    /* n is a multiple of 256 when a quantized output is asked for, so waves stay whole in this loop */
-    for (int i = threadIdx.x; i < n4; i += blockDim.x) {
-        const float4 v = x4[i], w = w4[i];
-        const float4 o = make_float4(v.x * scale * w.x, v.y * scale * w.y, v.z * scale * w.z, v.w * scale * w.w);
-        if (y4) y4[i] = o;
-        if (a.qout.qs) quantize_out4(a.qout, i, o);
+    /* n is a multiple of 256 when a quantized output is asked for, so waves stay whole in these loops */
+    if (in_regs) {
+        UNROLL for (int k = 0; k < KEEP; ++k) {
+            const int i = threadIdx.x + k * nt;
+            if (i < n4) {
+                const float4 o = make_float4(v[k].x * scale * w[k].x, v[k].y * scale * w[k].y, v[k].z * scale * w[k].z, v[k].w * scale * w[k].w);
+                if (y4) y4[i] = o;
+                if (a.qout.qs) quantize_out4(a.qout, i, o);
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < n4; i += nt) {
+            const float4 t = x4[i], ww = w4[i];
+            const float4 o = make_float4(t.x * scale * ww.x, t.y * scale * ww.y, t.z * scale * ww.z, t.w * scale * ww.w);
+            if (y4) y4[i] = o;
+            if (a.qout.qs) quantize_out4(a.qout, i, o);
+        }
     }
 }
 

@@ -658,7 +658,7 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
         /* small workgroups, one pass per wave where the chip can hold them */
         p.threads = 256;
         blocks = (waves + 3) / 4;
-        if (blocks > 4 * (int64_t)cus) blocks = 4 * (int64_t)cus;
+        if (blocks > 2 * (int64_t)cus) blocks = 2 * (int64_t)cus;     /* two workgroups per compute unit stream best (measured) */
         if (staged_lds_bytes(qtype, K, batch) > 40 * 1024) {
             /* a big staged copy limits how many workgroups fit a compute unit: fewer, larger ones */
             p.threads = 512;
