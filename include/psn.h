@@ -183,8 +183,8 @@ typedef struct psn_matvec_plan {
     int32_t lanes_per_row;  /* 8, 16, 32 or 64 lanes share one row */
     int32_t rows_in_flight; /* row sets per lane: 1 or 2 at batch_tile 1, else 1 */
     int32_t batch_tile;     /* compiled batch width: 1, 2, 4 or 8 (>= batch) */
-    int32_t stage_lds;      /* scheme Q8 only. 0: quantized x read from global memory; 1: staged in LDS;
-                               2: x is fp32 and every workgroup quantizes it while staging */
+    int32_t stage_lds;      /* 0: activations read from global memory; 1: staged in LDS; 2 (scheme Q8): x is
+                               fp32 and every workgroup quantizes it while staging */
     int32_t blocks;         /* workgroups */
     int32_t threads;        /* threads per workgroup: 256 or 512 (256, 512 or 768 with `stream`) */
     int32_t stream;         /* 1: weights land in per-wave LDS buffers by direct-to-LDS loads (scheme Q8,

@@ -627,8 +627,9 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
     /* the staged activations may take the whole 160 KB of a compute unit's LDS (batch 8 at K = 14336
      * needs 140 KB); re-quantizing inside the launch only pays up to batch 2 -- beyond that every
      * workgroup would redo batch x K of quantization, and one extra launch is cheaper (measured) */
-    const bool lds_fits = scheme == PSN_ACT_Q8 && staged_lds_bytes(qtype, K, batch) <= 160 * 1024;
-    p.stage_lds = lds_fits ? ((fuse_quantize && batch <= 2) ? 2 : 1) : 0;
+    const bool lds_fits = scheme == PSN_ACT_Q8 ? staged_lds_bytes(qtype, K, batch) <= 160 * 1024 : (int64_t)batch * C * 1040 <= 160 * 1024;
+    p.stage_lds = !lds_fits ? 0 : scheme == PSN_ACT_F32 ? 1 : ((fuse_quantize && batch <= 2) ? 2 : 1);
+
     /* lanes per row: the row's chunk count rounded up to a power of two, widened (idle lanes, more
      * waves) until the launch offers about four waves per compute unit */
     int g = C <= 8 ? 8 : C <= 16 ? 16 : C <= 32 ? 32 : 64;
@@ -658,7 +659,9 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
         /* small workgroups, one pass per wave where the chip can hold them */
         p.threads = 256;
         blocks = (waves + 3) / 4;
-        if (blocks > 2 * (int64_t)cus) blocks = 2 * (int64_t)cus;     /* two workgroups per compute unit stream best (measured) */
+        /* two workgroups per compute unit stream best for the int8 path, four for the fp32 path (measured) */
+        const int64_t cap = (scheme == PSN_ACT_F32 ? 4 : 2) * (int64_t)cus;
+        if (blocks > cap) blocks = cap;
         if (staged_lds_bytes(qtype, K, batch) > 40 * 1024) {
             /* a big staged copy limits how many workgroups fit a compute unit: fewer, larger ones */
             p.threads = 512;
@@ -690,8 +693,12 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
     int32_t lds = 0;
     if (p->stage_lds < 0 || p->stage_lds > 2) return fail(PSN_E_UNSUPPORTED, "plan: stage_lds=%d", p->stage_lds);
-    if (p->stage_lds) {
-        if (scheme != PSN_ACT_Q8) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging exists for scheme Q8 only");
+    if (p->stage_lds && scheme == PSN_ACT_F32) {
+        if (p->stage_lds != 1) return fail(PSN_E_UNSUPPORTED, "plan: scheme F32 stages fp32 activations (stage_lds 0 or 1)");
+        const int64_t total = (int64_t)batch * (K / 256) * 1040;
+        if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging needs %lld bytes, device offers %d", (long long)total, max_lds);
+        lds = (int32_t)total;
+    } else if (p->stage_lds) {
         const int64_t total = staged_lds_bytes(qtype, K, batch);
         if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: LDS staging needs %lld bytes, device offers %d", (long long)total, max_lds);
         lds = (int32_t)total;
@@ -774,7 +781,8 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
                  plan->batch_tile, plan->stage_lds ? "_lds" : "");
     } else {
         a.xf = (const float *)x;
-        snprintf(name, sizeof name, "psn_mv_%s_f32_g%d_r%d_b%d", fmt_name(qtype), plan->lanes_per_row, plan->rows_in_flight, plan->batch_tile);
+        snprintf(name, sizeof name, "psn_mv_%s_f32_g%d_r%d_b%d%s", fmt_name(qtype), plan->lanes_per_row, plan->rows_in_flight, plan->batch_tile,
+                 plan->stage_lds ? "_lds" : "");
     }
     return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)lds, &a);
 }

@@ -738,14 +738,17 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
     }
 }
 
-/* Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations. */
+/* Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations.
+ * XLDS: the activations are copied into LDS once per workgroup, every 1 KB chunk (256 floats) followed
+ * by 16 bytes of padding so that lanes on neighbouring chunks read disjoint banks; a lane then streams
+ * its chunk from LDS once per R rows instead of through the vector cache once per row. */
 template <typename F, int SB, int R, int NB>
-PSN_DEV void f32_step(const u32 (&w)[R][F::DW], const float *xf, int K, int k0, int batch, float (&acc)[R][NB]) {
+PSN_DEV void f32_step(const u32 (&w)[R][F::DW], const float *xbase, int col_stride, int chunk_off, int batch, float (&acc)[R][NB]) {
     float o[R][32];
     UNROLL for (int r = 0; r < R; ++r) F::template deq32<SB>(w[r], o[r]);
     UNROLL for (int nb = 0; nb < NB; ++nb) {
         const int col = nb < batch ? nb : batch - 1;
-        const float4 *xp = reinterpret_cast<const float4 *>(xf + (int64_t)col * K + k0 + SB * 32);
+        const float4 *xp = reinterpret_cast<const float4 *>(xbase + (int64_t)col * col_stride + chunk_off + SB * 32);
         UNROLL for (int i = 0; i < 8; ++i) {
             const float4 x = xp[i];
             UNROLL for (int r = 0; r < R; ++r) {
@@ -758,26 +761,44 @@ PSN_DEV void f32_step(const u32 (&w)[R][F::DW], const float *xf, int K, int k0, 
     }
 }
 
-template <typename F, int G, int R, int NB>
+template <typename F, int G, int R, int NB, bool XLDS>
 PSN_DEV void mv_f32(const psn_matvec_args &a) {
     const RowMap<G, R> m(a);
     PSN_DECLARE_SEGMENTS(a);
     const int K = a.K, C = K >> 8;
-    for (int row0 = m.wave * m.ROWS; row0 < a.N; row0 += m.nwaves * m.ROWS) {
+    const float *xbase = a.xf;
+    int col_stride = K, chunk_stride = 256;
+    u32 w[R][F::DW];
+    int row0 = m.wave * m.ROWS;
+    bool pre = false;
+    if constexpr (XLDS) {
+        extern __shared__ uint4 psn_smem[];
+        /* first chunk's weights on their way before the activations are staged */
+        pre = true;
+        PSN_LOAD_ROWS(F, m, a, min(row0, a.N - 1), min(m.j, C - 1), w);
+        const uint4 *g = reinterpret_cast<const uint4 *>(a.xf);
+        const int n16 = a.batch * C * 64;                             /* 16-byte words of fp32 activations */
+        for (int i = threadIdx.x; i < n16; i += a.threads) psn_smem[(i >> 6) * 65 + (i & 63)] = g[i];
+        __syncthreads();
+        xbase = reinterpret_cast<const float *>(psn_smem);
+        chunk_stride = 260;
+        col_stride = C * 260;
+    }
+    for (; row0 < a.N; row0 += m.nwaves * m.ROWS) {
         float acc[R][NB];
         UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
         for (int c = m.j; c < C; c += G) {
-            u32 w[R][F::DW];
-            PSN_LOAD_ROWS(F, m, a, row0, c, w);
-            const int k0 = c * 256;
-            f32_step<F, 0>(w, a.xf, K, k0, a.batch, acc);
-            f32_step<F, 1>(w, a.xf, K, k0, a.batch, acc);
-            f32_step<F, 2>(w, a.xf, K, k0, a.batch, acc);
-            f32_step<F, 3>(w, a.xf, K, k0, a.batch, acc);
-            f32_step<F, 4>(w, a.xf, K, k0, a.batch, acc);
-            f32_step<F, 5>(w, a.xf, K, k0, a.batch, acc);
-            f32_step<F, 6>(w, a.xf, K, k0, a.batch, acc);
-            f32_step<F, 7>(w, a.xf, K, k0, a.batch, acc);
+            if (!pre) { PSN_LOAD_ROWS(F, m, a, row0, c, w); }
+            pre = false;
+            const int off = c * chunk_stride;
+            f32_step<F, 0>(w, xbase, col_stride, off, a.batch, acc);
+            f32_step<F, 1>(w, xbase, col_stride, off, a.batch, acc);
+            f32_step<F, 2>(w, xbase, col_stride, off, a.batch, acc);
+            f32_step<F, 3>(w, xbase, col_stride, off, a.batch, acc);
+            f32_step<F, 4>(w, xbase, col_stride, off, a.batch, acc);
+            f32_step<F, 5>(w, xbase, col_stride, off, a.batch, acc);
+            f32_step<F, 6>(w, xbase, col_stride, off, a.batch, acc);
+            f32_step<F, 7>(w, xbase, col_stride, off, a.batch, acc);
         }
         PSN_STORE_ROWS(m, acc, a, row0);
     }
@@ -811,7 +832,10 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
 
 #define PSN_F32_KERNEL(fmt, F, G, R, NB)                                                                  \
     extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
-        mv_f32<F, G, R, NB>(a);                                                                           \
+        mv_f32<F, G, R, NB, false>(a);                                                                    \
+    }                                                                                                     \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
+        mv_f32<F, G, R, NB, true>(a);                                                                     \
     }
 
 #define PSN_Q8_ALL_G(fmt, F, R, NB) \

@@ -89,7 +89,7 @@ def all_plans(scheme, batch):
         rs = (1, 2) if nb == 1 else (1,)
     for g in (8, 16, 32, 64):
         for r in rs:
-            for lds in ((0, 1, 2) if scheme == _ffi.ACT_Q8 else (0,)):
+            for lds in ((0, 1, 2) if scheme == _ffi.ACT_Q8 else (0, 1)):
                 p = _ffi.MatvecPlan()
                 p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks = g, r, nb, lds, 3
                 p.threads = 512 if (g // 8 + r + lds) % 2 else 256
