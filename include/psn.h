@@ -256,6 +256,18 @@ int32_t psn_swiglu_q8(psn_module *mod, psn_stream *s, const psn_buf *gate, const
 int32_t psn_attention_decode_q8(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
                                 psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
                                 int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx);
+/* cos / sin of the head_dim/2 rotary pairs at position pos into `table` (head_dim floats); once per
+ * token, shared by all layers */
+int32_t psn_rope_table(psn_module *mod, psn_stream *s, psn_buf *table, int32_t head_dim, int32_t pos, float theta_base);
+/* psn_rope_kv_store + psn_attention_decode(_q8) in two launches instead of three: q, k, v are the raw
+ * projections of the token at position pos; the attention kernel rotates q and k itself with the
+ * coefficients of psn_rope_table (same arithmetic), appends k and v to the
+ * caches and attends over positions 0 .. pos.  q is left unrotated.  out and out_q as above (either
+ * may be NULL, not both). */
+int32_t psn_attention_decode_rope(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k, const psn_buf *v,
+                                  psn_buf *k_cache, psn_buf *v_cache, psn_buf *workspace, psn_buf *out, psn_buf *out_q,
+                                  int32_t act_type, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t pos,
+                                  const psn_buf *rope_table);
 
 #ifdef __cplusplus
 }

@@ -299,6 +299,16 @@ class HipBackend:
         _check(self.lib.psn_attention_decode_q8(self.module, self.stream, q.handle, k_cache.handle, v_cache.handle, workspace.handle,
                                                 self._h(out), out_q.handle, act_type, n_heads, n_kv_heads, head_dim, n_ctx))
 
+    def rope_table(self, table, head_dim: int, pos: int, theta_base: float):
+        _check(self.lib.psn_rope_table(self.module, self.stream, table.handle, head_dim, pos, theta_base))
+
+    def attention_decode_rope(self, q, k, v, k_cache, v_cache, workspace, out, out_q, act_type: int, n_heads: int, n_kv_heads: int,
+                              head_dim: int, pos: int, rope_table):
+        """Rotary embedding + KV append + attention over positions 0..pos (q, k, v are the raw projections)."""
+        _check(self.lib.psn_attention_decode_rope(self.module, self.stream, q.handle, k.handle, v.handle, k_cache.handle, v_cache.handle,
+                                                  workspace.handle, self._h(out), self._h(out_q), act_type, n_heads, n_kv_heads, head_dim, pos,
+                                                  rope_table.handle))
+
     # -- graphs -----------------------------------------------------------------------------
     def reserve(self, k: int, batch: int = 1):
         _check(self.lib.psn_stream_reserve(self.stream, k, batch))

@@ -103,6 +103,19 @@ struct psn_attn_args {
     float scale;
     int32_t pad;
     struct psn_actq_out qout;
+    /* fused rotary + cache append (psn_attn_partial_rope): q and k_new are the raw projections of the
+     * token at position n_ctx - 1; the kernel rotates them itself and stores k_new / v_new in the caches */
+    const float *k_new;   /* [n_kv_heads][128] */
+    const float *v_new;
+    void *k_cache_w;
+    void *v_cache_w;
+    const float *rope_table;   /* [head_dim/2][2]: cos, sin of pos * theta^(-2i/head_dim), from psn_rope_table */
+};
+struct psn_rope_table_args {
+    float *table;
+    int32_t head_dim, pos;
+    float theta_base;
+    int32_t pad;
 };
 struct psn_swiglu_args {
     const float *gate, *up;

@@ -106,6 +106,26 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
     }
 }
 
+/* one rotary pair; explicit roundings so that every kernel that rotates gives the same bits */
+PSN_DEV void rope_pair(float x0, float x1, float cs, float sn, float &r0, float &r1) {
+    r0 = __fsub_rn(__fmul_rn(x0, cs), __fmul_rn(x1, sn));
+    r1 = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, cs));
+}
+PSN_DEV void rope_coeff(float theta_base, int head_dim, int pos, int i, float &cs, float &sn) {
+    const float freq = powf(theta_base, -2.0f * (float)i / (float)head_dim);
+    sincosf((float)pos * freq, &sn, &cs);
+}
+
+/* cos / sin of every rotary pair at one position: computed once per token, read by every layer */
+extern "C" __global__ void __launch_bounds__(64) psn_rope_table(const psn_rope_table_args a) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= a.head_dim / 2) return;
+    float cs, sn;
+    rope_coeff(a.theta_base, a.head_dim, a.pos, i, cs, sn);
+    a.table[2 * i] = cs;
+    a.table[2 * i + 1] = sn;
+}
+
 /* Rotary embedding of q (in place) and k at position pos, pairs (2i, 2i+1), angle pos * base^(-2i/d);
  * k and v are appended to the fp16 cache row of that position.  One thread per pair. */
 extern "C" __global__ void __launch_bounds__(256) psn_rope_kv_store(const psn_rope_args a) {
@@ -116,12 +136,10 @@ extern "C" __global__ void __launch_bounds__(256) psn_rope_kv_store(const psn_ro
     const bool is_q = t < nq;
     const int idx = is_q ? t : t - nq;
     const int head = idx / half, i = idx % half;
-    const float freq = powf(a.theta_base, -2.0f * (float)i / (float)a.head_dim);
-    float sn, cs;
-    sincosf((float)a.pos * freq, &sn, &cs);
+    float sn, cs, r0, r1;
+    rope_coeff(a.theta_base, a.head_dim, a.pos, i, cs, sn);
     float *src = (is_q ? a.q : a.k) + head * a.head_dim + 2 * i;
-    const float x0 = src[0], x1 = src[1];
-    const float r0 = x0 * cs - x1 * sn, r1 = x0 * sn + x1 * cs;
+    rope_pair(src[0], src[1], cs, sn, r0, r1);
     if (is_q) {
         src[0] = r0;
         src[1] = r1;
@@ -143,9 +161,11 @@ extern "C" __global__ void __launch_bounds__(256) psn_rope_kv_store(const psn_ro
  * needs from the cache -- its K row and its two dims of all 64 V rows -- is requested up front,
  * so the kernel pays one memory round trip.  Rows past the context re-read the last valid one and
  * get weight 0.  Writes the unnormalized partial output plus (max, sum) per head and split. */
-extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_attn_args a) {
+template <bool ROPE>
+PSN_DEV void attn_partial_body(const psn_attn_args &a) {
     constexpr int D = 128;
     __shared__ float qs[8][D];
+    __shared__ uint4 knew_row[16];                            /* the new token's rotated key row, fp16 */
     const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
     const int kvh = blockIdx.x % a.n_kv_heads, split = blockIdx.x / a.n_kv_heads;
     const int group = a.n_heads / a.n_kv_heads;                  /* == blockDim.x / 64 */
@@ -164,9 +184,50 @@ extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_att
         const int64_t vstride = (int64_t)a.n_kv_heads * D / 2;   /* dwords between positions */
         UNROLL for (int i = 0; i < 64; ++i) vreg[i] = vbase[(int64_t)min(i, last) * vstride];
     }
-    qs[g][lane] = a.q[head * D + lane];
-    qs[g][lane + 64] = a.q[head * D + lane + 64];
+    if constexpr (ROPE) {
+        /* lane i rotates pair i of this wave's query head; wave 0 also leaves the coefficients in LDS
+         * for the lane that has to rotate the new key row */
+        const float2 tc = *reinterpret_cast<const float2 *>(a.rope_table + 2 * lane);
+        const float cs = tc.x, sn = tc.y;
+        float r0, r1;
+        const float2 qv = *reinterpret_cast<const float2 *>(a.q + head * D + 2 * lane);
+        rope_pair(qv.x, qv.y, cs, sn, r0, r1);
+        qs[g][2 * lane] = r0;
+        qs[g][2 * lane + 1] = r1;
+        if (g == 0 && split == ((a.n_ctx - 1) >> 6)) {
+            /* wave 0 of the split that owns the token's position rotates the new key row, one pair per
+             * lane, rounds it to fp16 like a cached row, leaves it in LDS and appends it to the cache */
+            const int pos = a.n_ctx - 1;
+            const float2 kv = *reinterpret_cast<const float2 *>(a.k_new + kvh * D + 2 * lane);
+            float k0, k1;
+            rope_pair(kv.x, kv.y, cs, sn, k0, k1);
+            const f16 h0 = (f16)k0, h1 = (f16)k1;
+            const u32 packed = (u32)__builtin_bit_cast(unsigned short, h0) | ((u32)__builtin_bit_cast(unsigned short, h1) << 16);
+            reinterpret_cast<u32 *>(knew_row)[lane] = packed;
+            reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.k_cache_w) + ((int64_t)pos * a.n_kv_heads + kvh) * D)[lane] = packed;
+        }
+    } else {
+        qs[g][lane] = a.q[head * D + lane];
+        qs[g][lane + 64] = a.q[head * D + lane + 64];
+    }
     __syncthreads();
+    if constexpr (ROPE) {
+        /* the token's own position is not in the cache yet: the split that owns it takes the key row from
+         * LDS (see above) and the value row from the fresh projection, rounded to fp16 like a cached row;
+         * wave 0 appends the value row to the cache */
+        const int pos = a.n_ctx - 1;
+        if (split == (pos >> 6)) {                               /* uniform */
+            const int pl = pos & 63;
+            if (lane == pl) {
+                UNROLL for (int c = 0; c < 16; ++c) kreg[c] = knew_row[c];
+            }
+            const float2 vn = *reinterpret_cast<const float2 *>(a.v_new + kvh * D + 2 * lane);
+            const f16 v0 = (f16)vn.x, v1 = (f16)vn.y;
+            const u32 vpacked = (u32)__builtin_bit_cast(unsigned short, v0) | ((u32)__builtin_bit_cast(unsigned short, v1) << 16);
+            UNROLL for (int i = 0; i < 64; ++i) if (i == pl) vreg[i] = vpacked;
+            if (g == 0) reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos * a.n_kv_heads + kvh) * D)[lane] = vpacked;
+        }
+    }
     float s = 0.f;
     UNROLL for (int c = 0; c < 16; ++c) {
         const u32 kw[4] = {kreg[c].x, kreg[c].y, kreg[c].z, kreg[c].w};
@@ -189,6 +250,10 @@ extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_att
     dst[2 * lane + 1] = o1;
     if (lane == 0) { dst[D] = m; dst[D + 1] = sum; }
 }
+
+extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_attn_args a) { attn_partial_body<false>(a); }
+/* the same with the rotary embedding of q and k and the KV-cache append of the new token folded in */
+extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_rope(const psn_attn_args a) { attn_partial_body<true>(a); }
 
 /* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One workgroup of 128 threads per
  * head: the per-split (max, sum) pairs are fetched in parallel, the weights go through LDS, and the

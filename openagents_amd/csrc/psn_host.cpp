@@ -1086,9 +1086,45 @@ extern "C" int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q,
     return launch(mod, s, "psn_rope_kv_store", (unsigned)((pairs + 255) / 256), 256, 0, &a);
 }
 
+struct rope_fusion {
+    const psn_buf *k_new, *v_new, *table;
+};
+extern "C" int32_t psn_rope_table(psn_module *mod, psn_stream *s, psn_buf *table, int32_t head_dim, int32_t pos, float theta_base) {
+    if (!mod || !s || !table) return fail(PSN_E_INVALID_ARG, "psn_rope_table: null handle");
+    if (s->ctx != mod->ctx || table->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "psn_rope_table: handles belong to different contexts");
+    if (head_dim <= 0 || head_dim % 2 || pos < 0) return fail(PSN_E_SHAPE, "psn_rope_table: head_dim=%d pos=%d", head_dim, pos);
+    int32_t rc = need(table, (int64_t)head_dim * 4, "psn_rope_table", "table");
+    if (rc) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    psn_rope_table_args a;
+    a.table = (float *)table->p;
+    a.head_dim = head_dim;
+    a.pos = pos;
+    a.theta_base = theta_base;
+    a.pad = 0;
+    return launch(mod, s, "psn_rope_table", (unsigned)((head_dim / 2 + 63) / 64), 64, 0, &a);
+}
+static int32_t attention_impl(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
+                              psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
+                              int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx, const rope_fusion *rope);
+
 extern "C" int32_t psn_attention_decode_q8(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
                                            psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
                                            int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx) {
+    return attention_impl(mod, s, q, k_cache, v_cache, workspace, out, out_q, act_type, n_heads, n_kv_heads, head_dim, n_ctx, nullptr);
+}
+extern "C" int32_t psn_attention_decode_rope(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k, const psn_buf *v,
+                                             psn_buf *k_cache, psn_buf *v_cache, psn_buf *workspace, psn_buf *out, psn_buf *out_q,
+                                             int32_t act_type, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t pos,
+                                             const psn_buf *rope_table) {
+    if (!k || !v || !rope_table) return fail(PSN_E_INVALID_ARG, "psn_attention_decode_rope: k, v or rope_table is null");
+    if (pos < 0) return fail(PSN_E_SHAPE, "psn_attention_decode_rope: pos=%d", pos);
+    rope_fusion rf = {k, v, rope_table};
+    return attention_impl(mod, s, q, k_cache, v_cache, workspace, out, out_q, act_type, n_heads, n_kv_heads, head_dim, pos + 1, &rf);
+}
+static int32_t attention_impl(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
+                              psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
+                              int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx, const rope_fusion *rope) {
     int32_t rc = check_same_ctx(mod, s, q, k_cache, v_cache, "psn_attention_decode");
     if (rc) return rc;
     if (!workspace || (!out && !out_q)) return fail(PSN_E_INVALID_ARG, "psn_attention_decode: null workspace or no output");
@@ -1118,7 +1154,21 @@ extern "C" int32_t psn_attention_decode_q8(psn_module *mod, psn_stream *s, const
     a.n_ctx = n_ctx;
     a.n_splits = splits;
     a.scale = 0.08838834764831845f;                 /* 1/sqrt(128) */
-    if ((rc = launch(mod, s, "psn_attn_partial", (unsigned)(n_kv_heads * splits), (unsigned)(64 * (n_heads / n_kv_heads)), 0, &a))) return rc;
+    if (rope) {
+        if (rope->k_new->ctx != mod->ctx || rope->v_new->ctx != mod->ctx || rope->table->ctx != mod->ctx)
+            return fail(PSN_E_INVALID_ARG, "psn_attention_decode_rope: handles belong to different contexts");
+        if ((rc = need(rope->k_new, row * 2, "psn_attention_decode_rope", "k")) || (rc = need(rope->v_new, row * 2, "psn_attention_decode_rope", "v")) ||
+            (rc = need(rope->table, 128 * 4, "psn_attention_decode_rope", "rope_table")))
+            return rc;
+        a.k_new = (const float *)rope->k_new->p;
+        a.v_new = (const float *)rope->v_new->p;
+        a.k_cache_w = k_cache->p;
+        a.v_cache_w = v_cache->p;
+        a.rope_table = (const float *)rope->table->p;
+    }
+    if ((rc = launch(mod, s, rope ? "psn_attn_partial_rope" : "psn_attn_partial", (unsigned)(n_kv_heads * splits),
+                     (unsigned)(64 * (n_heads / n_kv_heads)), 0, &a)))
+        return rc;
     if (out_q) return launch(mod, s, "psn_attn_combine_q8", (unsigned)(n_heads / 2), 256, 0, &a);
     return launch(mod, s, "psn_attn_combine", (unsigned)n_heads, 128, 0, &a);
 }

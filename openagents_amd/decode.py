@@ -102,18 +102,20 @@ class DecodeStep:
             self.xq_h = be.alloc(int(actq_layout(self.act_type, s.hidden, 1).bytes))
             self.xq_attn = be.alloc(int(actq_layout(self.act_type, s.hidden, 1).bytes))
             self.xq_f = be.alloc(int(actq_layout(self.act_type, s.ffn, 1).bytes))
+            self.rope_tab = be.alloc(s.head_dim * 4)
 
     def _enqueue_fused(self, pos: int, matvecs_only: bool):
         be, s, at = self.be, self.shape, self.act_type
         glue = not matvecs_only
+        if glue:
+            be.rope_table(self.rope_tab, s.head_dim, pos, s.rope_theta)      # once per token
         for li, lw in enumerate(self.w.layers):
             if glue:
                 be.add_rmsnorm_q8(self.x, self.down if li > 0 else None, lw.attn_norm, None, self.xq_h, at, s.hidden, s.eps)
             be.quantized_matvec_q8_multi([lw.wq, lw.wk, lw.wv], self.xq_h, [self.q, self.k, self.v], 1)
             if glue:
-                be.rope_kv_store(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], s.n_heads, s.n_kv_heads, s.head_dim, pos, s.rope_theta)
-                be.attention_decode_q8(self.q, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn, at,
-                                       s.n_heads, s.n_kv_heads, s.head_dim, pos + 1)
+                be.attention_decode_rope(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn, at,
+                                         s.n_heads, s.n_kv_heads, s.head_dim, pos, self.rope_tab)
             be.quantized_matvec_q8(lw.wo, self.xq_attn, self.o, 1)
             if glue:
                 be.add_rmsnorm_q8(self.x, self.o, lw.ffn_norm, None, self.xq_h, at, s.hidden, s.eps)
@@ -249,7 +251,7 @@ def main(argv=None):
            "config": {"layers": shape.n_layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,
                       "ffn": shape.ffn, "vocab": shape.vocab, "context": args.ctx, "weights": "Q4_K projections, Q6_K LM head",
                       "activation_scheme": "Q8 (Q8_K blocks, " + ("written by the producing kernel)" if step.fused else "quantized inside the matvec launch)"),
-                      "launches_per_token": shape.n_layers * 10 + 2, "graph_replay": True},
+                      "launches_per_token": shape.n_layers * (9 if step.fused else 10) + (3 if step.fused else 2), "graph_replay": True},
            "data": "synthetic random-init weights (one unique layer copied to every layer's own allocation), fp16 N(0,1) KV cache",
            "logits_finite": bool(np.all(np.isfinite(logits))), "steps": args.steps, "setup_s": round(setup_s, 1),
            "not_measured": ["sampling", "tokenizer", "host loop"]}

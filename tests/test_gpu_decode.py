@@ -101,6 +101,42 @@ def test_attention_decode(hip, nh, nkv):
         assert G.max_rel_err(got, attention_ref(q, kc, vc, nh, nkv, d, n_ctx)) < 2e-5
 
 
+@pytest.mark.parametrize("pos", [0, 63, 64, 149, 2047])
+def test_rope_fused_into_attention_matches_separate_launches(hip, pos):
+    """Two launches (attention that rotates and appends itself, combine) against three (rotary + append,
+    attention, combine): same cache rows and outputs up to the last bit of the rotary coefficients (the
+    table kernel and the stand-alone rotary kernel are compiled separately), untouched rows identical."""
+    rng = np.random.default_rng(906 + pos)
+    nh, nkv, d, ctx = 32, 8, 128, 2048
+    q = rng.standard_normal(nh * d, dtype=np.float32)
+    k = rng.standard_normal(nkv * d, dtype=np.float32)
+    v = rng.standard_normal(nkv * d, dtype=np.float32)
+    kc0 = rng.standard_normal((ctx, nkv * d), dtype=np.float32).astype(np.float16)
+    vc0 = rng.standard_normal((ctx, nkv * d), dtype=np.float32).astype(np.float16)
+    ws = hip.alloc(nh * ((ctx + 63) // 64) * 130 * 4)
+    # three launches
+    qb, kb, vb = hip.upload(q), hip.upload(k), hip.upload(v)
+    kc, vc = hip.upload(kc0), hip.upload(vc0)
+    ref = hip.alloc(nh * d * 4)
+    hip.rope_kv_store(qb, kb, vb, kc, vc, nh, nkv, d, pos, 500000.0)
+    hip.attention_decode(qb, kc, vc, ws, ref, nh, nkv, d, pos + 1)
+    # two launches
+    kc2, vc2 = hip.upload(kc0), hip.upload(vc0)
+    out = hip.alloc(nh * d * 4)
+    tab = hip.alloc(d * 4)
+    hip.rope_table(tab, d, pos, 500000.0)
+    hip.attention_decode_rope(hip.upload(q), hip.upload(k), hip.upload(v), kc2, vc2, ws, out, None, _ffi.Q8_K, nh, nkv, d, pos, tab)
+    assert G.max_rel_err(out.download(np.float32, (nh * d,)), ref.download(np.float32, (nh * d,))) < 2e-6
+    k_two, k_three = kc2.download(np.float16, (ctx, nkv * d)), kc.download(np.float16, (ctx, nkv * d))
+    assert np.array_equal(np.delete(k_two, pos, axis=0).view(np.uint16), np.delete(k_three, pos, axis=0).view(np.uint16))
+    assert np.max(np.abs(k_two[pos].astype(np.float32) - k_three[pos].astype(np.float32))) <= 2e-3        # one fp16 ulp at |k| < 4
+    assert np.array_equal(vc2.download(np.float16, (ctx, nkv * d)).view(np.uint16), vc.download(np.float16, (ctx, nkv * d)).view(np.uint16))
+    # against the fp64 restatement: the kernels form pos * theta^(-2i/d) in fp32, which at position 2047
+    # is an angle error of about 1e-4 rad in the fastest pair
+    assert G.max_rel_err(out.download(np.float32, (nh * d,)),
+                         attention_ref(rope_ref(q, nh, d, pos, 500000.0), kc2.download(np.float16, (ctx, nkv * d)), vc2.download(np.float16, (ctx, nkv * d)), nh, nkv, d, pos + 1)) < 1e-4
+
+
 def test_swiglu(hip):
     rng = np.random.default_rng(903)
     n = 14336
@@ -217,13 +253,14 @@ def test_whole_small_decode_step_eager_and_graph(hip, orc):
     assert err < 1e-3
     assert int(np.argmax(eager)) == int(np.argmax(ref_logits))
 
-    # the path where every matvec quantizes its own fp32 input gives the same logits bit for bit
+    # the path with separate rotary launches, where every matvec quantizes its own fp32 input, agrees up
+    # to int8 roundings flipped by last-bit differences of the rotary coefficients
     for li in range(s.n_layers):
         unfused.k_cache[li].upload(kv0[li][0])
         unfused.v_cache[li].upload(kv0[li][1])
     unfused.x.upload(x0)
     unfused.enqueue(pos)
-    assert np.array_equal(unfused.logits.download(np.float32, (s.vocab,)), eager)
+    assert G.max_rel_err(unfused.logits.download(np.float32, (s.vocab,)), eager) < 1e-3
 
     graph = step.capture(pos)
     try:
