@@ -108,7 +108,9 @@ int32_t psn_graph_destroy(psn_graph *g);
  * work on both, join with (main, side) before ending the capture. */
 int32_t psn_stream_wait_stream(psn_stream *waiter, psn_stream *signaler);
 /* Sizes the stream's activation workspace for psn_qmatvec / psn_qmatvec_multi with scheme Q8 up to
- * [batch][K], so later calls (and captures) never allocate. */
+ * [batch][K], so later calls (and captures) never allocate.  A graph captured from a call that uses the
+ * workspace holds its address: from then on the workspace cannot grow (calls that would need a larger
+ * one fail with PSN_E_INVALID_ARG), so reserve the largest K x batch before the first capture. */
 int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch);
 
 int32_t psn_event_create(psn_ctx *ctx, psn_event **out);
@@ -120,6 +122,8 @@ int32_t psn_event_elapsed_us(const psn_event *begin, const psn_event *end, doubl
 int32_t psn_buf_alloc(psn_ctx *ctx, size_t bytes, psn_buf **out);
 int32_t psn_buf_free(psn_buf *b);
 int64_t psn_buf_size(const psn_buf *b);
+/* upload, download and fill_zero are synchronous-ordered conveniences that are never recorded into a
+ * graph: on a stream that is being captured they fail with PSN_E_INVALID_ARG and leave the capture intact */
 int32_t psn_buf_upload(psn_buf *dst, size_t off, const void *src, size_t n, psn_stream *s);
 int32_t psn_buf_download(const psn_buf *src, size_t off, void *dst, size_t n, psn_stream *s);
 int32_t psn_buf_fill_zero(psn_buf *b, psn_stream *s);
@@ -181,7 +185,7 @@ int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t qtype, int3
  * caller-chosen one (auto-tuners, benchmarks). */
 typedef struct psn_matvec_plan {
     int32_t lanes_per_row;  /* 8, 16, 32 or 64 lanes share one row */
-    int32_t rows_in_flight; /* row sets per lane: 1 or 2 at batch_tile 1, else 1 */
+    int32_t rows_in_flight; /* row sets per lane: 1 */
     int32_t batch_tile;     /* compiled batch width: 1, 2, 4 or 8 (>= batch) */
     int32_t stage_lds;      /* 0: activations read from global memory; 1: staged in LDS; 2 (scheme Q8): x is
                                fp32 and every workgroup quantizes it while staging */

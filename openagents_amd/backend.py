@@ -94,6 +94,10 @@ class DeviceBuffer:
         _check(self._b.lib.psn_buf_download(self.handle, offset, C.c_void_p(out.ctypes.data), out.nbytes, self._b.stream))
         return out
 
+    def fill_zero(self) -> "DeviceBuffer":
+        _check(self._b.lib.psn_buf_fill_zero(self.handle, self._b.stream))
+        return self
+
     def free(self):
         if self.handle is not None and self._b.ctx is not None:
             if self._b._capturing:

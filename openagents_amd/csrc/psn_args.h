@@ -48,7 +48,6 @@ struct psn_matvec_args {
     int64_t row_bytes;
     int32_t threads;      /* launch geometry, passed in so that kernels never read the dispatch packet */
     int32_t blocks;
-    uint64_t *timeline;   /* development builds (-DPSN_TIMELINE): per-wave clock stamps; otherwise unused, null */
 };
 
 struct psn_prefill_args {

@@ -224,7 +224,9 @@ PSN_DEV void attn_partial_body(const psn_attn_args &a) {
             const float2 vn = *reinterpret_cast<const float2 *>(a.v_new + kvh * D + 2 * lane);
             const f16 v0 = (f16)vn.x, v1 = (f16)vn.y;
             const u32 vpacked = (u32)__builtin_bit_cast(unsigned short, v0) | ((u32)__builtin_bit_cast(unsigned short, v1) << 16);
-            UNROLL for (int i = 0; i < 64; ++i) if (i == pl) vreg[i] = vpacked;
+            /* rows behind the token's position were loaded from cache rows that nothing has written yet:
+             * they get weight 0, but 0 * (a stale Inf/NaN pattern) would still poison the sum */
+            UNROLL for (int i = 0; i < 64; ++i) if (i >= pl) vreg[i] = vpacked;
             if (g == 0) reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos * a.n_kv_heads + kvh) * D)[lane] = vpacked;
         }
     }

@@ -139,6 +139,7 @@ struct psn_stream {
     hipStream_t s;
     void *ws;          /* activation workspace of psn_qmatvec (scheme Q8) */
     size_t ws_bytes;
+    bool ws_in_graph;  /* a captured graph holds the address of ws: it must never move again */
     hipEvent_t join_ev; /* created on first use by psn_stream_wait_stream */
 };
 struct psn_buf {
@@ -287,6 +288,7 @@ extern "C" int32_t psn_stream_create(psn_ctx *c, psn_stream **out) {
     st->s = s;
     st->ws = nullptr;
     st->ws_bytes = 0;
+    st->ws_in_graph = false;
     st->join_ev = nullptr;
     *out = st;
     return PSN_OK;
@@ -317,12 +319,22 @@ static int32_t is_capturing(psn_stream *s, bool *out) {
     *out = st != hipStreamCaptureStatusNone;
     return PSN_OK;
 }
+static int32_t refuse_while_capturing(psn_stream *s, const char *what) {
+    bool cap = false;
+    int32_t rc = is_capturing(s, &cap);
+    if (rc) return rc;
+    if (cap) return fail(PSN_E_INVALID_ARG, "%s: the stream is being captured into a graph (uploads, downloads and memsets are not recorded)", what);
+    return PSN_OK;
+}
 static int32_t ensure_workspace(psn_stream *s, int64_t bytes) {
     if (s->ws_bytes >= (size_t)bytes) return PSN_OK;
     bool cap = false;
     int32_t rc = is_capturing(s, &cap);
     if (rc) return rc;
     if (cap) return fail(PSN_E_INVALID_ARG, "activation workspace must grow to %lld bytes during capture: call psn_stream_reserve first", (long long)bytes);
+    if (s->ws_in_graph)
+        return fail(PSN_E_INVALID_ARG, "activation workspace (%zu bytes) is referenced by a captured graph and cannot grow to %lld bytes: "
+                    "reserve the largest K x batch with psn_stream_reserve before the first capture", s->ws_bytes, (long long)bytes);
     /* earlier launches may still read the old workspace */
     HIP_TRY(hipStreamSynchronize(s->s));
     if (s->ws) HIP_TRY(hipFree(s->ws));
@@ -483,6 +495,7 @@ extern "C" int32_t psn_buf_upload(psn_buf *dst, size_t off, const void *src, siz
     if (!src || !s) return fail(PSN_E_INVALID_ARG, "psn_buf_upload: src or stream is null");
     if (s->ctx != dst->ctx) return fail(PSN_E_INVALID_ARG, "psn_buf_upload: stream and buffer belong to different contexts");
     if ((rc = bind(dst->ctx))) return rc;
+    if ((rc = refuse_while_capturing(s, "psn_buf_upload"))) return rc;
     if (n == 0) return PSN_OK;
     /* pageable source: the copy is staged, so the caller may reuse src on return */
     HIP_TRY(hipMemcpyAsync((char *)dst->p + off, src, n, hipMemcpyHostToDevice, s->s));
@@ -495,6 +508,7 @@ extern "C" int32_t psn_buf_download(const psn_buf *src, size_t off, void *dst, s
     if (!dst || !s) return fail(PSN_E_INVALID_ARG, "psn_buf_download: dst or stream is null");
     if (s->ctx != src->ctx) return fail(PSN_E_INVALID_ARG, "psn_buf_download: stream and buffer belong to different contexts");
     if ((rc = bind(src->ctx))) return rc;
+    if ((rc = refuse_while_capturing(s, "psn_buf_download"))) return rc;
     if (n == 0) return PSN_OK;
     HIP_TRY(hipMemcpyAsync(dst, (const char *)src->p + off, n, hipMemcpyDeviceToHost, s->s));
     HIP_TRY(hipStreamSynchronize(s->s));
@@ -502,8 +516,11 @@ extern "C" int32_t psn_buf_download(const psn_buf *src, size_t off, void *dst, s
 }
 extern "C" int32_t psn_buf_fill_zero(psn_buf *b, psn_stream *s) {
     if (!b || !s) return fail(PSN_E_INVALID_ARG, "buffer or stream is null");
+    if (s->ctx != b->ctx) return fail(PSN_E_INVALID_ARG, "psn_buf_fill_zero: stream and buffer belong to different contexts");
     int32_t rc = bind(b->ctx);
     if (rc) return rc;
+    /* a memset node must not end up in a graph (replays of such nodes have given wrong results) */
+    if ((rc = refuse_while_capturing(s, "psn_buf_fill_zero"))) return rc;
     HIP_TRY(hipMemsetAsync(b->p, 0, b->bytes, s->s));
     return PSN_OK;
 }
@@ -686,10 +703,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     if (!(g == 8 || g == 16 || g == 32 || g == 64)) return fail(PSN_E_UNSUPPORTED, "plan: lanes_per_row=%d", g);
     if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
     if (p->threads != 256 && p->threads != 512 && !(p->stream && p->threads == 768)) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
-    bool ok;
-    if (scheme == PSN_ACT_Q8) ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
-    else ok = (nb == 1 && (r == 1 || r == 2)) || (nb > 1 && r == 1);
-    if (!ok) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
+    if (r != 1) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
     int32_t lds = 0;
     if (p->stage_lds < 0 || p->stage_lds > 2) return fail(PSN_E_UNSUPPORTED, "plan: stage_lds=%d", p->stage_lds);
@@ -875,6 +889,9 @@ extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qty
     psn_actq_info li;
     if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;
     if ((rc = ensure_workspace(s, li.bytes))) return rc;
+    bool cap = false;
+    if ((rc = is_capturing(s, &cap))) return rc;
+    if (cap) s->ws_in_graph = true;      /* the graph being recorded bakes the workspace address into its nodes */
     if ((rc = quantize_into(mod, s, at, (const float *)x->p, s->ws, K, batch))) return rc;
     return run_matvec(mod, s, qtype, scheme, sg, s->ws, K, batch, &plan);
 }

@@ -22,14 +22,6 @@
 
 #define UNROLL _Pragma("unroll")
 
-/* build-time experiment switches */
-#ifndef PSN_DOUBLE_BUFFER
-#define PSN_DOUBLE_BUFFER 0
-#endif
-#ifndef PSN_KERNEL_ATTR
-#define PSN_KERNEL_ATTR
-#endif
-
 /* ------------------------------------------------------------------------------------------
  * Activation quantizers (bit-exact restatements of the Q8_0 / Q8_K row quantizers).  The same
  * math runs as stand-alone kernels and inside the matvec's staging step.
@@ -565,39 +557,22 @@ struct FmtQ6_K {
  * Drivers.
  * ------------------------------------------------------------------------------------------ */
 
-/* Development aid: with -DPSN_TIMELINE lane 0 of every wave records the 100 MHz steady clock at five
- * points of the kernel (8 slots per wave).  Compiled out of the shipped code objects. */
-#ifdef PSN_TIMELINE
-#define PSN_STAMP(a, m, slot)                                                                     \
-    do {                                                                                          \
-        if ((a).timeline && (m).lane == 0) (a).timeline[(int64_t)(m).wave * 8 + (slot)] = __builtin_readsteadycounter(); \
-    } while (0)
-#else
-#define PSN_STAMP(a, m, slot) do { } while (0)
-#endif
-
 /* Scheme Q8.  A wave walks its work as (row set, chunk iteration) items.  Order of events: the
  * small activation loads are issued, then the first item's weight loads, then the activations are
- * staged (waiting only for their own loads) while the weights are still in flight.  With one row
- * set and one batch column per lane (R = NB = 1) the weights are double-buffered: the next item's
- * loads are issued before the current item is consumed, and the lane's activation chunk stays in
- * registers for as long as the chunk index does not change. */
+ * staged (waiting only for their own loads) while the weights are still in flight.  At batch 1 the
+ * lane's activation chunk stays in registers for as long as the chunk index does not change. */
 template <typename F, int G, int R, int NB, int XSRC>
 PSN_DEV void mv_q8(const psn_matvec_args &a) {
     typedef typename F::ActSum ST;
-    constexpr bool DB = PSN_DOUBLE_BUFFER && (R == 1 && NB == 1);
     const RowMap<G, R> m(a);
     PSN_DECLARE_SEGMENTS(a);
     const int K = a.K, C = K >> 8, iters = (C + G - 1) / G, stride = m.nwaves * m.ROWS;
     int row0 = m.wave * m.ROWS, it = 0;
-    PSN_STAMP(a, m, 0);
     Stager<ST, XSRC> st;
     st.issue(a, F::d_per_col(K), F::s_per_col(K));
-    u32 wa[R][F::DW], wb[DB ? R : 1][DB ? F::DW : 1];
+    u32 wa[R][F::DW];
     PSN_LOAD_ROWS(F, m, a, min(row0, a.N - 1), min(m.j, C - 1), wa);
-    PSN_STAMP(a, m, 1);
     const ActQ<ST> x = st.finish(a);
-    PSN_STAMP(a, m, 2);
     u32 xr[F::XR];
     int xc = -1;
     float acc[R][NB];
@@ -616,38 +591,18 @@ PSN_DEV void mv_q8(const psn_matvec_args &a) {
             }
         }
         if (i == iters - 1) {
-            PSN_STAMP(a, m, 3);
             PSN_STORE_ROWS(m, acc, a, r0);
             UNROLL for (int r = 0; r < R; ++r) UNROLL for (int nb = 0; nb < NB; ++nb) acc[r][nb] = 0.f;
         }
     };
 
-    if constexpr (DB) {
-        /* Prefetches are unconditional (indices clamped into range) so that the loads sit in
-         * straight-line code and the compiler can wait for exactly the older buffer. */
-        while (row0 < a.N) {
-            int r1 = row0, i1 = it;
-            advance(r1, i1);
-            PSN_LOAD_ROWS(F, m, a, r1, min(m.j + i1 * G, C - 1), wb);
-            consume(wa, row0, it);
-            if (r1 >= a.N) break;
-            int r2 = r1, i2 = i1;
-            advance(r2, i2);
-            PSN_LOAD_ROWS(F, m, a, r2, min(m.j + i2 * G, C - 1), wa);
-            consume(wb, r1, i1);
-            row0 = r2;
-            it = i2;
-        }
-    } else {
-        bool pre = true;
-        while (row0 < a.N) {
-            if (!pre) { PSN_LOAD_ROWS(F, m, a, row0, min(m.j + it * G, C - 1), wa); }
-            pre = false;
-            consume(wa, row0, it);
-            advance(row0, it);
-        }
+    bool pre = true;
+    while (row0 < a.N) {
+        if (!pre) { PSN_LOAD_ROWS(F, m, a, row0, min(m.j + it * G, C - 1), wa); }
+        pre = false;
+        consume(wa, row0, it);
+        advance(row0, it);
     }
-    PSN_STAMP(a, m, 4);
 }
 
 /* Scheme Q8, streaming variant (batch 1, rows of at most G chunks).  The weights do not pass through
@@ -811,13 +766,13 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
  * ------------------------------------------------------------------------------------------ */
 
 #define PSN_Q8_KERNEL(fmt, F, G, R, NB)                                                                   \
-    extern "C" __global__ void PSN_KERNEL_ATTR __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
         mv_q8<F, G, R, NB, 0>(a);                                                                         \
     }                                                                                                     \
-    extern "C" __global__ void PSN_KERNEL_ATTR __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_lds(const psn_matvec_args a) { \
         mv_q8<F, G, R, NB, 1>(a);                                                                         \
     }                                                                                                     \
-    extern "C" __global__ void PSN_KERNEL_ATTR __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_xf(const psn_matvec_args a) { \
+    extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_q8_g##G##_r##R##_b##NB##_xf(const psn_matvec_args a) { \
         mv_q8<F, G, R, NB, 2>(a);                                                                         \
     }
 
@@ -841,13 +796,13 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
 #define PSN_Q8_ALL_G(fmt, F, R, NB) \
     PSN_Q8_KERNEL(fmt, F, 8, R, NB) PSN_Q8_KERNEL(fmt, F, 16, R, NB) PSN_Q8_KERNEL(fmt, F, 32, R, NB) PSN_Q8_KERNEL(fmt, F, 64, R, NB)
 #define PSN_Q8_ALL(fmt, F)                                                                 \
-    PSN_Q8_ALL_G(fmt, F, 1, 1) PSN_Q8_ALL_G(fmt, F, 2, 1)                                  \
+    PSN_Q8_ALL_G(fmt, F, 1, 1)                                                             \
     PSN_Q8_ALL_G(fmt, F, 1, 2) PSN_Q8_ALL_G(fmt, F, 1, 4) PSN_Q8_ALL_G(fmt, F, 1, 8)
 
 #define PSN_F32_ALL_G(fmt, F, R, NB) \
     PSN_F32_KERNEL(fmt, F, 8, R, NB) PSN_F32_KERNEL(fmt, F, 16, R, NB) PSN_F32_KERNEL(fmt, F, 32, R, NB) PSN_F32_KERNEL(fmt, F, 64, R, NB)
 #define PSN_F32_ALL(fmt, F)                                                               \
-    PSN_F32_ALL_G(fmt, F, 1, 1) PSN_F32_ALL_G(fmt, F, 2, 1)                                \
+    PSN_F32_ALL_G(fmt, F, 1, 1)                                                            \
     PSN_F32_ALL_G(fmt, F, 1, 2) PSN_F32_ALL_G(fmt, F, 1, 4) PSN_F32_ALL_G(fmt, F, 1, 8)
 
 /* The build compiles this file once per format (-DPSN_BUILD_ONLY -DPSN_BUILD_<FMT>) so the four

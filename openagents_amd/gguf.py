@@ -19,6 +19,7 @@ import numpy as np
 
 MAGIC = b"GGUF"
 DEFAULT_ALIGNMENT = 32
+MAX_DIMS = 4            # ggml tensors have at most four dimensions
 
 # ggml tensor types this module knows: id -> (elements per block, bytes per block, name)
 GGML_TYPES = {0: (1, 4, "F32"), 1: (1, 2, "F16"), 2: (32, 18, "Q4_0"), 8: (32, 34, "Q8_0"),
@@ -57,6 +58,8 @@ def tensor_nbytes(ggml_type: int, dims) -> int:
     if ggml_type not in GGML_TYPES:
         raise GGUFError(f"ggml type {ggml_type} is not supported")
     be, bb, name = GGML_TYPES[ggml_type]
+    if not 1 <= len(dims) <= MAX_DIMS or any(int(d) <= 0 for d in dims):
+        raise GGUFError(f"{name}: dims {tuple(dims)} (want 1..{MAX_DIMS} positive dimensions)")
     if dims[0] % be:
         raise GGUFError(f"{name}: row length {dims[0]} is not a whole number of {be}-element blocks")
     rows = 1
@@ -85,13 +88,28 @@ class _Cursor:
         self.pos += n
         return s
 
+    def remaining(self):
+        return len(self.buf) - self.pos
+
+    def count(self, min_bytes_each, what):
+        """A u64 element count, checked against what the rest of the file could possibly hold."""
+        n = self.take("<Q")
+        if n * min_bytes_each > self.remaining():
+            raise GGUFError(f"{what}: count {n} does not fit the remaining {self.remaining()} bytes")
+        return n
+
     def value(self, vtype):
         if vtype in _SCALAR:
             return self.take(_SCALAR[vtype])
         if vtype == STRING:
             return self.string()
         if vtype == ARRAY:
-            et, count = self.take("<I"), self.take("<Q")
+            et = self.take("<I")
+            if et == ARRAY:
+                raise GGUFError("nested metadata arrays are not supported")
+            if et != STRING and et not in _SCALAR:
+                raise GGUFError(f"unknown metadata array element type {et}")
+            count = self.count(8 if et == STRING else struct.calcsize(_SCALAR[et]), "metadata array")
             return [self.value(et) for _ in range(count)]
         raise GGUFError(f"unknown metadata value type {vtype}")
 
@@ -110,6 +128,9 @@ class GGUFFile:
         if self.version not in (2, 3):
             raise GGUFError(f"GGUF version {self.version} is not supported")
         n_tensors, n_kv = c.take("<Q"), c.take("<Q")
+        # a key/value pair takes at least 8 + 4 + 1 bytes, a tensor entry at least 8 + 4 + 8 + 4 + 8
+        if n_kv * 13 + n_tensors * 32 > c.remaining():
+            raise GGUFError(f"header counts ({n_tensors} tensors, {n_kv} metadata pairs) do not fit the file")
         self.metadata = {}
         for _ in range(n_kv):
             key = c.string()
@@ -121,7 +142,11 @@ class GGUFFile:
         for _ in range(n_tensors):
             name = c.string()
             nd = c.take("<I")
+            if not 1 <= nd <= MAX_DIMS:
+                raise GGUFError(f"tensor {name}: {nd} dimensions (want 1..{MAX_DIMS})")
             dims = tuple(c.take("<Q") for _ in range(nd))
+            if any(d <= 0 for d in dims):
+                raise GGUFError(f"tensor {name}: dims {dims} contain a zero")
             gtype, off = c.take("<I"), c.take("<Q")
             nbytes = tensor_nbytes(gtype, dims) if gtype in GGML_TYPES else -1
             self.tensors[name] = TensorInfo(name, dims, gtype, off, nbytes)

@@ -46,6 +46,8 @@ def lib() -> C.CDLL:
         L.orc_dequantize_row.argtypes = [i32, vp, vp, i64]; L.orc_dequantize_row.restype = i32
         L.orc_quantize_rows.argtypes = [i32, vp, vp, i64, i64, i32]; L.orc_quantize_rows.restype = i32
         L.orc_q4k_scale_min.argtypes = [vp, vp, vp]; L.orc_q4k_scale_min.restype = None
+        L.orc_q4k_fit_subblock.argtypes = [vp, vp, C.POINTER(C.c_float)]; L.orc_q4k_fit_subblock.restype = f32
+        L.orc_q6k_fit_subblock.argtypes = [vp, vp]; L.orc_q6k_fit_subblock.restype = f32
         L.orc_vec_dot_q.argtypes = [i32, vp, vp, i64]; L.orc_vec_dot_q.restype = f32
         L.orc_matvec.argtypes = [i32, i32, vp, vp, vp, i64, i64, i32, i32]; L.orc_matvec.restype = i32
         L.orc_matvec_f64.argtypes = [i32, vp, vp, vp, i64, i64, i32, i32]; L.orc_matvec_f64.restype = i32
@@ -124,6 +126,25 @@ def q4k_scale_min(scales12: np.ndarray):
     mn = np.zeros(8, dtype=np.uint8)
     lib().orc_q4k_scale_min(_p(s), _p(sc), _p(mn))
     return sc, mn
+
+
+def q4k_fit_subblock(x32: np.ndarray):
+    """(scale, min, L[32]) of one Q4_K sub-block: x ~ scale * L - min."""
+    x = np.ascontiguousarray(x32, dtype=np.float32)
+    assert x.size == 32
+    L = np.zeros(32, dtype=np.uint8)
+    mn = C.c_float()
+    sc = lib().orc_q4k_fit_subblock(_p(x), _p(L), C.byref(mn))
+    return float(sc), float(mn.value), L
+
+
+def q6k_fit_subblock(x16: np.ndarray):
+    """(scale, L[16]) of one Q6_K sub-block: x ~ scale * (L - 32)."""
+    x = np.ascontiguousarray(x16, dtype=np.float32)
+    assert x.size == 16
+    L = np.zeros(16, dtype=np.int8)
+    sc = lib().orc_q6k_fit_subblock(_p(x), _p(L))
+    return float(sc), L
 
 
 def vec_dot_q(wtype: int, w_row: np.ndarray, xq_row: np.ndarray, k: int) -> float:

@@ -246,18 +246,26 @@ void orc_q4k_scale_min(const uint8_t *q, uint8_t sc[8], uint8_t mn[8]) {
     }
 }
 
+/* One 32-element Q4_K sub-block: importance weights sqrt(mean x^2) + |x|, 16 levels, the
+ * 21-candidate search (rmin -1, step 0.1).  x ~ scale * L - min.  Exported so that tests can
+ * pin the search by what the mathematics fixes; quant_q4_K calls exactly this. */
+float orc_q4k_fit_subblock(const float *x, uint8_t *L, float *min_out) {
+    uint8_t Ltry[32];
+    float w[32], s2 = 0.f;
+    for (int l = 0; l < 32; l++) s2 += x[l] * x[l];
+    float av = sqrtf(s2 / 32.f);
+    for (int l = 0; l < 32; l++) w[l] = av + fabsf(x[l]);
+    return fit_scale_min(32, 15, x, w, L, min_out, Ltry, -1.f, 0.1f, 20);
+}
+
 static void quant_q4_K(const float *x, blk_q4_K *y, int64_t k) {
-    uint8_t L[QKK], Ltry[32];
-    float w[32], mins[8], scales[8];
+    uint8_t L[QKK];
+    float mins[8], scales[8];
     for (int64_t b = 0; b < k / QKK; b++) {
         const float *xb = x + b * QKK;
         float max_scale = 0.f, max_min = 0.f;
         for (int j = 0; j < 8; j++) {
-            float s2 = 0.f;
-            for (int l = 0; l < 32; l++) s2 += xb[32 * j + l] * xb[32 * j + l];
-            float av = sqrtf(s2 / 32.f);
-            for (int l = 0; l < 32; l++) w[l] = av + fabsf(xb[32 * j + l]);
-            scales[j] = fit_scale_min(32, 15, xb + 32 * j, w, L + 32 * j, &mins[j], Ltry, -1.f, 0.1f, 20);
+            scales[j] = orc_q4k_fit_subblock(xb + 32 * j, L + 32 * j, &mins[j]);
             if (scales[j] > max_scale) max_scale = scales[j];
             if (mins[j] > max_min) max_min = mins[j];
         }
@@ -330,6 +338,10 @@ static float fit_scale_sym(int n, int nmax, const float *x, int8_t *L) {
     return scale;
 }
 
+/* One 16-element Q6_K sub-block (64 levels, weights x^2): x ~ scale * (L - 32).  Exported for
+ * the tests that pin the search; quant_q6_K calls exactly this. */
+float orc_q6k_fit_subblock(const float *x, int8_t *L) { return fit_scale_sym(16, 32, x, L); }
+
 static void quant_q6_K(const float *x, blk_q6_K *y, int64_t k) {
     int8_t L[QKK];
     float scales[16];
@@ -337,7 +349,7 @@ static void quant_q6_K(const float *x, blk_q6_K *y, int64_t k) {
         const float *xb = x + b * QKK;
         float max_scale = 0.f, max_abs = 0.f;
         for (int g = 0; g < 16; g++) {
-            scales[g] = fit_scale_sym(16, 32, xb + 16 * g, L + 16 * g);
+            scales[g] = orc_q6k_fit_subblock(xb + 16 * g, L + 16 * g);
             float a = fabsf(scales[g]);
             if (a > max_abs) { max_abs = a; max_scale = scales[g]; }
         }

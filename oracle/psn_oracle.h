@@ -23,10 +23,16 @@
  *   Q8_K quantize ............ pinned: closed form + bsums invariant
  *   all dequantizers ......... pinned: independent bit-level packers (pack o unpack = id),
  *                              one-hot lane/nibble-order tests
- *   Q4_K / Q6_K quantize ..... PARITY UNPINNED for the scale search (only field-range
- *                              validity and reconstruction-error bounds are checkable
- *                              without Psionic's source); matvec parity does not depend
- *                              on it because oracle and kernel read the same bytes
+ *   Q4_K / Q6_K quantize ..... pinned by what the mathematics fixes (tests/test_oracle_kquant_search.py):
+ *                              sub-blocks and whole super-blocks that lie on the format's grid round-trip
+ *                              exactly (levels, 6-bit / int8 scales, fp16 d and dmin); the (scale, min)
+ *                              returned for a set of levels is the weighted least-squares fit
+ *                              (numpy.linalg.lstsq, weights sqrt(mean x^2)+|x| resp. x^2); the result is the
+ *                              outcome of the published candidate search restated independently in float64
+ *                              (both ends of the Q4_K step range, the coarse end of the Q6_K range), never
+ *                              worse than the plain min/max grid; min >= 0.  Bit-for-bit agreement with
+ *                              Psionic's own encoder on arbitrary data could only be shown with its source;
+ *                              matvec parity does not depend on it (oracle and kernel read the same bytes)
  *   matvec scheme F32 ........ pinned: one-hot activations return deq columns, fp64 truth
  *   matvec scheme Q8 ......... pinned: exact int64/fp64 re-evaluation from the same bytes
  *   prefill matmul ........... pinned: fp64 matmul of fp16-rounded deq(W) with fp16 X
@@ -66,6 +72,12 @@ int32_t orc_quantize_rows(int32_t qtype, const float *x, void *y, int64_t n, int
 
 /* unpack the eight 6-bit (scale, min) pairs of a Q4_K super-block's 12-byte field */
 void orc_q4k_scale_min(const uint8_t *scales12, uint8_t sc[8], uint8_t mn[8]);
+
+/* The per-sub-block searches of the K-quant quantizers (test hooks; the row quantizers call these):
+ * Q4_K: x[32] ~ scale * L - min, L in 0..15, returns scale, writes L and min;
+ * Q6_K: x[16] ~ scale * (L - 32), L in 0..63, returns scale, writes L. */
+float orc_q4k_fit_subblock(const float *x32, uint8_t *L, float *min_out);
+float orc_q6k_fit_subblock(const float *x16, int8_t *L);
 
 /* integer dot of one quantized weight row with one quantized activation row */
 float orc_vec_dot_q(int32_t wtype, const void *w, const void *xq, int64_t k);

@@ -63,6 +63,31 @@ def test_malformed_files_are_rejected(orc, tmp_path):
         p.write_bytes(blob)
         with pytest.raises(gguf.GGUFError):
             gguf.GGUFFile(str(p))
+    def header(n_tensors, n_kv, body=b""):
+        return b"GGUF" + struct.pack("<IQQ", 3, n_tensors, n_kv) + body
+
+    def s(text):
+        return struct.pack("<Q", len(text)) + text
+
+    hostile = {
+        "huge counts": header(2 ** 40, 2 ** 40),
+        "zero dims": header(1, 0, s(b"t") + struct.pack("<I", 0) + struct.pack("<IQ", 0, 0)),
+        "five dims": header(1, 0, s(b"t") + struct.pack("<I", 5) + struct.pack("<5Q", 32, 1, 1, 1, 1) + struct.pack("<IQ", 0, 0)),
+        "zero dim": header(1, 0, s(b"t") + struct.pack("<I", 2) + struct.pack("<2Q", 32, 0) + struct.pack("<IQ", 0, 0)),
+        "nested array": header(0, 1, s(b"k") + struct.pack("<I", gguf.ARRAY) + struct.pack("<IQ", gguf.ARRAY, 1) + struct.pack("<IQ", gguf.U8, 0)),
+        "deep nesting": header(0, 1, s(b"k") + struct.pack("<I", gguf.ARRAY) + struct.pack("<IQ", gguf.ARRAY, 1) * 5000),
+        "huge array": header(0, 1, s(b"k") + struct.pack("<I", gguf.ARRAY) + struct.pack("<IQ", gguf.U32, 2 ** 50)),
+        "bad array type": header(0, 1, s(b"k") + struct.pack("<I", gguf.ARRAY) + struct.pack("<IQ", 77, 1) + b"\0" * 64),
+        "huge string": header(0, 1, struct.pack("<Q", 2 ** 60) + b"abc"),
+    }
+    for what, blob in hostile.items():
+        p = tmp_path / f"hostile_{what.replace(' ', '_')}.gguf"
+        p.write_bytes(blob + b"\0" * 64)
+        with pytest.raises(gguf.GGUFError):
+            gguf.GGUFFile(str(p))
+    for dims in ((), (256, 0), (32, 1, 1, 1, 1)):
+        with pytest.raises(gguf.GGUFError):
+            gguf.tensor_nbytes(2, dims)
     with pytest.raises(gguf.GGUFError):
         gguf.write_gguf(str(tmp_path / "x.gguf"), {}, [("t", (100, 4), 2, np.zeros(10, np.uint8))])   # ragged row
     with pytest.raises(gguf.GGUFError):

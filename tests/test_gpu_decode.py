@@ -3,8 +3,9 @@ restatement of the textbook Llama layer, with the CPU oracle doing the quantized
 
 The reference here is plain numpy (fp64 where it matters): RMSNorm, rotary pairs (2i, 2i+1) with
 theta = 500000, grouped-query softmax attention over an fp16 cache, SwiGLU.  Sizes are reduced
-(hidden 512, 4 query / 2 kv heads of dim 128, FFN 1024, vocab 768, 3 layers, context 150); the
-8B-shaped step is exercised by `python -m openagents_amd.decode`, whose logits only have to be finite.
+(hidden 512, 4 query / 2 kv heads of dim 128, FFN 1024, vocab 768, 3 layers, context 150) for the
+comparison with numpy; the 32-layer 8B-shaped step is checked through properties that need no CPU
+restatement (graph replay = eager bit for bit, fused = unfused within the gate, same argmax).
 """
 import sys
 
@@ -12,7 +13,7 @@ import numpy as np
 import pytest
 
 import ggufref as G
-from openagents_amd import _ffi
+from openagents_amd import _ffi, backend
 from openagents_amd.decode import DecodeStep, LayerWeights, LlamaShape, ModelWeights
 
 pytestmark = pytest.mark.gpu
@@ -137,6 +138,38 @@ def test_rope_fused_into_attention_matches_separate_launches(hip, pos):
                          attention_ref(rope_ref(q, nh, d, pos, 500000.0), kc2.download(np.float16, (ctx, nkv * d)), vc2.download(np.float16, (ctx, nkv * d)), nh, nkv, d, pos + 1)) < 1e-4
 
 
+@pytest.mark.parametrize("pos", [0, 1, 63, 64, 149])
+def test_rope_fused_attention_ignores_rows_the_cache_does_not_hold_yet(hip, pos):
+    """Cache rows at and behind the token's position hold whatever the allocation held (here: fp16 NaN
+    and Inf patterns).  The kernel that appends the token itself must not let them reach the output."""
+    rng = np.random.default_rng(950 + pos)
+    nh, nkv, d, ctx = 32, 8, 128, 256
+    q, k, v = (rng.standard_normal(n * d, dtype=np.float32) for n in (nh, nkv, nkv))
+    good = rng.standard_normal((ctx, nkv * d), dtype=np.float32).astype(np.float16)
+    ws = hip.alloc(nh * ((ctx + 63) // 64) * 130 * 4)
+    tab = hip.alloc(d * 4)
+    hip.rope_table(tab, d, pos, 500000.0)
+    outs = []
+    for poison in (None, 0x7E00, 0x7C00, 0xFC00):
+        kc0, vc0 = good.copy(), good.copy()
+        if poison is not None:
+            kc0.view(np.uint16)[pos:] = poison
+            vc0.view(np.uint16)[pos:] = poison
+        kc, vc = hip.upload(kc0), hip.upload(vc0)
+        out = hip.alloc(nh * d * 4)
+        outq = hip.alloc(int(backend.actq_layout(_ffi.Q8_K, nh * d, 1).bytes))
+        hip.attention_decode_rope(hip.upload(q), hip.upload(k), hip.upload(v), kc, vc, ws, out, outq, _ffi.Q8_K, nh, nkv, d, pos, tab)
+        o = out.download(np.float32, (nh * d,))
+        assert np.all(np.isfinite(o)), (pos, poison)
+        outs.append((o, outq.download(np.int8, (nh * d,))))
+        # the appended rows are finite, rows behind the position are left alone
+        kr, vr = kc.download(np.float16, (ctx, nkv * d)), vc.download(np.float16, (ctx, nkv * d))
+        assert np.all(np.isfinite(kr[pos])) and np.all(np.isfinite(vr[pos]))
+        assert np.array_equal(kr[pos + 1:].view(np.uint16), kc0[pos + 1:].view(np.uint16))
+    for o, oq in outs[1:]:
+        assert np.array_equal(o, outs[0][0]) and np.array_equal(oq, outs[0][1])
+
+
 def test_swiglu(hip):
     rng = np.random.default_rng(903)
     n = 14336
@@ -152,7 +185,6 @@ def test_swiglu(hip):
 def test_fused_quantized_outputs_match_separate_quantization(hip, act):
     """RMSNorm, SwiGLU and attention with the activation quantization fused in must write exactly the
     bytes psn_act_quantize produces from their fp32 result."""
-    from openagents_amd import backend
     at = getattr(_ffi, act)
     rng = np.random.default_rng(905)
 
@@ -270,6 +302,58 @@ def test_whole_small_decode_step_eager_and_graph(hip, orc):
             replay = step.logits.download(np.float32, (s.vocab,))
             assert np.array_equal(replay, eager)
             hip.swiglu(step.gate, step.up, step.act, s.ffn)      # eager work between replays
+            hip.sync()
+    finally:
+        hip.destroy_graph(graph)
+
+
+def test_llama3_8b_shaped_step_properties(hip):
+    """Config 5 at its real shape (32 layers, hidden 4096, 32/8 heads, FFN 14336, context 2048, Q4_K
+    projections, Q6_K 128256-row LM head).  No CPU restatement at this size; instead: the captured graph
+    replays the eager result bit for bit (three replays with eager work in between), the path with fused
+    activation quantization agrees with the path where every matvec quantizes its own fp32 input to well
+    inside the 1e-3 gate with the same argmax, and the KV caches gain exactly one row per layer."""
+    from openagents_amd.decode import synthetic_weights
+    s = LlamaShape()
+    ctx, pos = 2048, 2047
+    say("8B-shaped step: building synthetic weights")
+    weights = synthetic_weights(hip, s, seed=5)
+    fused = DecodeStep(hip, s, weights, ctx)
+    unfused = DecodeStep(hip, s, weights, ctx, fused_quant=False)
+    rng = np.random.default_rng(960)
+    kv = rng.standard_normal((ctx, s.kv_dim), dtype=np.float32).astype(np.float16)
+    kv[pos] = 0
+    x0 = rng.standard_normal(s.hidden, dtype=np.float32)
+
+    def reset(step):
+        for li in range(s.n_layers):
+            step.k_cache[li].upload(kv)
+            step.v_cache[li].upload(kv)
+        step.x.upload(x0)
+
+    say("8B-shaped step: eager, fused")
+    reset(fused)
+    fused.enqueue(pos)
+    eager = fused.logits.download(np.float32, (s.vocab,))
+    assert np.all(np.isfinite(eager))
+    for li in (0, 17, 31):
+        kr = fused.k_cache[li].download(np.float16, (ctx, s.kv_dim))
+        assert np.array_equal(kr[:pos].view(np.uint16), kv[:pos].view(np.uint16)) and kr[pos].any()
+    say("8B-shaped step: eager, unfused")
+    reset(unfused)
+    unfused.enqueue(pos)
+    other = unfused.logits.download(np.float32, (s.vocab,))
+    err = G.max_rel_err(other, eager)
+    say(f"  fused vs unfused logits max_rel_err={err:.3e}")
+    assert err < 1e-3 and int(np.argmax(other)) == int(np.argmax(eager))
+    say("8B-shaped step: graph replays")
+    graph = fused.capture(pos)
+    try:
+        for _ in range(3):
+            reset(fused)
+            hip.launch_graph(graph)
+            assert np.array_equal(fused.logits.download(np.float32, (s.vocab,)), eager)
+            hip.swiglu(fused.gate, fused.up, fused.act, s.ffn)
             hip.sync()
     finally:
         hip.destroy_graph(graph)

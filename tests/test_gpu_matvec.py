@@ -83,10 +83,7 @@ def test_quantize_q8_K_bit_exact(hip, orc, k, batch):
 
 def all_plans(scheme, batch):
     nb = 1 if batch <= 1 else 2 if batch <= 2 else 4 if batch <= 4 else 8
-    if scheme == _ffi.ACT_Q8:
-        rs = (1, 2) if nb == 1 else (1,)
-    else:
-        rs = (1, 2) if nb == 1 else (1,)
+    rs = (1,)
     for g in (8, 16, 32, 64):
         for r in rs:
             for lds in ((0, 1, 2) if scheme == _ffi.ACT_Q8 else (0, 1)):
@@ -157,6 +154,68 @@ def test_q4_K_small_batch_shapes(hip, orc, n, k, batch):
         err = G.max_rel_err(hip.matvec_host(orc.Q4_K, W, x, n, k, scheme), orc.matvec(orc.Q4_K, scheme, W, x, n, k))
         say(f"  scheme={scheme} max_rel_err={err:.3e}")
         assert err < PARITY_TOL
+
+
+def test_config5_layer_full_shape_prequantized_path(hip, orc):
+    """One Llama-3-8B-shaped Q4_K layer exactly as the decode step launches it: the norm writes Q8_K
+    activations (hidden 4096), q|k|v go out as ONE launch of 4096 + 1024 + 1024 rows, o is 4096 x 4096,
+    gate|up one launch of 2 x 14336 rows, SwiGLU writes Q8_K activations (FFN 14336), down is
+    4096 x 14336.  Every quantized activation must equal the oracle's Q8_K bytes of the fp32 vector the
+    same kernel wrote, every projection the oracle's integer matvec of that vector."""
+    H, KV, F = 4096, 1024, 14336
+    t = orc.Q4_K
+    Wq, Wk, Wv, Wo = (weights(orc, "Q4_K", 440 + i, n, H) for i, n in enumerate((H, KV, KV, H)))
+    Wg = weights(orc, "Q4_K", 420, F, H)
+    Wu = np.ascontiguousarray(Wg[::-1])                         # a second, different 14336-row matrix
+    Wd = weights(orc, "Q4_K", 420, H, F)
+    dq, dk, dv, do_, dg, du, dd = (hip.upload_weight(t, W, n, k) for W, n, k in
+                                   ((Wq, H, H), (Wk, KV, H), (Wv, KV, H), (Wo, H, H), (Wg, F, H), (Wu, F, H), (Wd, H, F)))
+    rng = np.random.default_rng(445)
+
+    def check_q8k(buf, vec, n):
+        li = backend.actq_layout(_ffi.Q8_K, n, 1)
+        rd, rq, rbs = G.parse_q8_K(orc.quantize(orc.Q8_K, vec), n)
+        assert np.array_equal(buf.download(np.int8, (n,), li.off_qs), rq.reshape(-1).astype(np.int8))
+        assert np.array_equal(buf.download(np.float32, (n // 256,), li.off_d).astype(np.float64), rd)
+        assert np.array_equal(buf.download(np.int16, (n // 16,), li.off_s), rbs.reshape(-1).astype(np.int16))
+
+    def check(ybuf, W, vec, n, k, what):
+        err = G.max_rel_err(ybuf.download(np.float32, (n,)), orc.matvec(t, orc.ACT_Q8, W, vec, n, k))
+        say(f"  {what}: max_rel_err={err:.3e}")
+        assert err < PARITY_TOL
+
+    say("config-5 layer: norm -> q|k|v")
+    resid, delta, nw = (rng.standard_normal(H, dtype=np.float32) for _ in range(3))
+    xn, xq_h = hip.alloc(H * 4), hip.alloc(int(backend.actq_layout(_ffi.Q8_K, H, 1).bytes))
+    hip.add_rmsnorm_q8(hip.upload(resid), hip.upload(delta), hip.upload(nw), xn, xq_h, _ffi.Q8_K, H, 1e-5)
+    xn_h = xn.download(np.float32, (H,))
+    check_q8k(xq_h, xn_h, H)
+    yq, yk, yv = hip.alloc(H * 4), hip.alloc(KV * 4), hip.alloc(KV * 4)
+    hip.quantized_matvec_q8_multi([dq, dk, dv], xq_h, [yq, yk, yv], 1)
+    for y, W, n, what in ((yq, Wq, H, "q"), (yk, Wk, KV, "k"), (yv, Wv, KV, "v")):
+        check(y, W, xn_h, n, H, what)
+    say("config-5 layer: o")
+    att = rng.standard_normal(H, dtype=np.float32)
+    xq_a = hip.quantize_activations(hip.upload(att), H, 1, _ffi.Q8_K)
+    yo = hip.alloc(H * 4)
+    hip.quantized_matvec_q8(do_, xq_a, yo, 1)
+    check(yo, Wo, att, H, H, "o")
+    say("config-5 layer: gate|up -> SwiGLU -> down")
+    yg, yu = hip.alloc(F * 4), hip.alloc(F * 4)
+    hip.quantized_matvec_q8_multi([dg, du], xq_h, [yg, yu], 1)
+    check(yg, Wg, xn_h, F, H, "gate")
+    check(yu, Wu, xn_h, F, H, "up")
+    act, xq_f = hip.alloc(F * 4), hip.alloc(int(backend.actq_layout(_ffi.Q8_K, F, 1).bytes))
+    hip.swiglu_q8(yg, yu, act, xq_f, _ffi.Q8_K, F)
+    act_h = act.download(np.float32, (F,))
+    check_q8k(xq_f, act_h, F)
+    yd = hip.alloc(H * 4)
+    hip.quantized_matvec_q8(dd, xq_f, yd, 1)
+    check(yd, Wd, act_h, H, F, "down")
+    # the same launches from fp32 activations (quantization inside the matvec launch) agree bit for bit
+    y2 = hip.alloc(H * 4)
+    hip.quantized_matvec(dd, act, y2, 1, _ffi.ACT_Q8)
+    assert G.max_rel_err(y2.download(np.float32, (H,)), yd.download(np.float32, (H,))) < 2e-6
 
 
 def test_q6_K_lm_head_slice(hip, orc):

@@ -85,12 +85,13 @@ def test_prefill_baseline_shapes_m64(hip, orc, qname, n, k):
 
 @pytest.mark.parametrize("m", [512, 2048])
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
-def test_prefill_baseline_shapes_large_m_sampled(hip, orc, m, n, k):
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
+def test_prefill_baseline_shapes_large_m_sampled(hip, orc, qname, m, n, k):
     """The GPU computes the full [m, n] product; the oracle re-computes a sample of 96 activation rows x
     160 weight rows (tile corners, edges and random interior rows) that the full result must match."""
-    t = orc.Q4_0
-    say(f"prefill Q4_0 m={m} n={n} k={k} (sampled oracle)")
-    W = weights(orc, "Q4_0", 820, n, k)
+    t = getattr(orc, qname)
+    say(f"prefill {qname} m={m} n={n} k={k} (sampled oracle)")
+    W = weights(orc, qname, 820, n, k)
     X = G.seeded_acts(830 + m, m, k).astype(np.float16)
     y = hip.matmul_host(t, W, X, n, k)
     rng = np.random.default_rng(m + n)
