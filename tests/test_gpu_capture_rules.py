@@ -44,7 +44,7 @@ def test_workspace_cannot_grow_once_a_graph_refers_to_it(orc):
     been captured, a larger eager call on the same stream must fail instead of freeing memory the graph
     still points at; the graph keeps replaying correctly."""
     with backend.HipBackend(0) as be:
-        n, k_small, k_big, batch = 96, 1024, 4096, 4
+        n, k_small, k_big, batch = 8, 1024, 327680, 4        # the workspace grows in 1 MiB steps: 4 x 327680 int8 exceed one
         Ws, Wb = orc.quantize(orc.Q6_K, G.seeded_weights(970, n, k_small)), orc.quantize(orc.Q6_K, G.seeded_weights(971, n, k_big))
         xs, xb = G.seeded_acts(972, batch, k_small), G.seeded_acts(973, batch, k_big)
         ws, wb = be.upload_weight(orc.Q6_K, Ws, n, k_small), be.upload_weight(orc.Q6_K, Wb, n, k_big)
