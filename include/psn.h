@@ -179,6 +179,20 @@ int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t qtype, int3
                              const psn_buf *const *W, const psn_buf *x_q, psn_buf *const *y_f32, const int64_t *N, int64_t K,
                              int32_t batch);
 
+/* psn_qmatvec for callers that cannot allocate device memory (code under graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  This entry point has no counterpart in the reference: it exists
+ * for those callers only.  Same arguments and results as psn_qmatvec, but nothing is allocated or freed,
+ * on the device or through any allocating library routine: with scheme Q8 the quantized activations go
+ * into a static array in the library's device image (psn_noalloc_max_bytes() bytes per GPU, held until
+ * the process ends) instead of the stream's workspace.  Shapes whose quantized activations
+ * (psn_actq_layout(...).bytes) exceed that size fail with PSN_E_SHAPE.  Every call on a GPU shares that
+ * GPU's array: calls that overlap in time on one GPU (different streams, or graphs replayed
+ * concurrently) race on it -- serialize them.  Nothing has to be cleared between calls: each call
+ * overwrites every byte it later reads. */
+int32_t psn_qmatvec_noalloc(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, const psn_buf *W,
+                            const psn_buf *x_f32, psn_buf *y_f32, int64_t N, int64_t K, int32_t batch);
+int64_t psn_noalloc_max_bytes(void);
+
 /* Launch geometry of one matvec.  psn_qmatvec_plan fills in the library's choice for a shape
  * (pure host arithmetic, usable without a device; x_is_f32 != 0 asks for the plan psn_qmatvec uses
  * when it quantizes fp32 activations inside the matvec launch); psn_qmatvec_planned runs with a

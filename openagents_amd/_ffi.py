@@ -75,6 +75,8 @@ SIGNATURES = {
     "psn_act_type_for": (_i32, [_i32]),
     "psn_act_quantize": (_i32, [_vp, _vp, _i32, _vp, _vp, _i64, _i32]),
     "psn_qmatvec": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
+    "psn_qmatvec_noalloc": (_i32, [_vp, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
+    "psn_noalloc_max_bytes": (_i64, []),
     "psn_qmatvec_q8": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i32]),
     "psn_qmatvec_plan": (_i32, [_i32, _i32, _i64, _i64, _i32, _i32, _i32, C.POINTER(MatvecPlan)]),
     "psn_qmatvec_multi": (_i32, [_vp, _vp, _i32, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32]),

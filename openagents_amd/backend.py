@@ -241,6 +241,10 @@ class HipBackend:
     def quantized_matvec(self, w: QuantizedTensor, x: DeviceBuffer, y: DeviceBuffer, batch: int = 1, scheme: int = ACT_Q8):
         _check(self.lib.psn_qmatvec(self.module, self.stream, w.qtype, LAYOUT_GGUF, scheme, w.buf.handle, x.handle, y.handle, w.n, w.k, batch))
 
+    def quantized_matvec_noalloc(self, w: QuantizedTensor, x: DeviceBuffer, y: DeviceBuffer, batch: int = 1, scheme: int = ACT_Q8):
+        """quantized_matvec that allocates nothing (static device scratch; calls on one GPU must not overlap)."""
+        _check(self.lib.psn_qmatvec_noalloc(self.module, self.stream, w.qtype, LAYOUT_GGUF, scheme, w.buf.handle, x.handle, y.handle, w.n, w.k, batch))
+
     def quantized_matvec_q8(self, w: QuantizedTensor, xq: DeviceBuffer, y: DeviceBuffer, batch: int = 1):
         _check(self.lib.psn_qmatvec_q8(self.module, self.stream, w.qtype, LAYOUT_GGUF, w.buf.handle, xq.handle, y.handle, w.n, w.k, batch))
 

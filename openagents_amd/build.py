@@ -58,15 +58,21 @@ def code_object_paths():
             if os.path.exists(os.path.join(CSRC, src))]
 
 
-def build(jobs: int = 0, verbose: bool = True) -> str:
+def build(jobs: int = 0, verbose: bool = True, reuse_device: bool = False) -> str:
+    """Compiles everything; with reuse_device a code object newer than its source and the device headers is kept."""
     os.makedirs(LIB, exist_ok=True)
     hipcc = _hipcc()
     jobs = jobs or min(8, os.cpu_count() or 1)
     todo = [(stem, src, defs) for stem, src, defs in CODE_OBJECTS if os.path.exists(os.path.join(CSRC, src))]
 
+    device_headers = ["psn_args.h", "psn_device.h"]
+
     def compile_co(item):
         stem, src, defs = item
         out = os.path.join(LIB, f"{stem}.{ARCH}.hsaco")
+        newest_src = max(os.path.getmtime(os.path.join(CSRC, f)) for f in [src, *device_headers])
+        if reuse_device and os.path.exists(out) and os.path.getmtime(out) > newest_src:
+            return out
         _run([hipcc, *DEVICE_FLAGS, *defs, "-I", CSRC, "-o", out, os.path.join(CSRC, src)])
         return out
 
@@ -91,13 +97,18 @@ def build(jobs: int = 0, verbose: bool = True) -> str:
     blob_o = os.path.join(LIB, "psn_blobs.o")
     _run(["gcc", "-c", "-fPIC", "-o", blob_o, asm])
 
+    # the translation unit that owns the static device scratch: host + gfx950 device code in one object
+    noalloc_o = os.path.join(LIB, "psn_noalloc.o")
+    _run([hipcc, "-O2", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          "-I", CSRC, "-c", "-o", noalloc_o, os.path.join(CSRC, "psn_noalloc.hip")])
+
     host_o = os.path.join(LIB, "psn_host.o")
     rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__",
           "-I", INCLUDE, "-I", CSRC, "-isystem", os.path.join(rocm, "include"),
           "-c", "-o", host_o, os.path.join(CSRC, "psn_host.cpp")])
     out = lib_path()
-    _run(["g++", "-shared", "-fPIC", "-o", out, host_o, blob_o, "-Wl,--no-undefined",
+    _run(["g++", "-shared", "-fPIC", "-o", out, host_o, noalloc_o, blob_o, "-Wl,--no-undefined",
           "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib")])
     if verbose:
         print("built", os.path.relpath(out, os.path.dirname(HERE)), os.path.getsize(out), "bytes")
@@ -107,8 +118,9 @@ def build(jobs: int = 0, verbose: bool = True) -> str:
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=0)
+    ap.add_argument("--reuse-device", action="store_true", help="keep code objects that are newer than every source file")
     args = ap.parse_args(argv)
-    build(args.jobs)
+    build(args.jobs, reuse_device=args.reuse_device)
 
 
 if __name__ == "__main__":

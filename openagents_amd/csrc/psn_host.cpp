@@ -7,6 +7,7 @@
  */
 #include "../../include/psn.h"
 #include "psn_args.h"
+#include "psn_noalloc.h"
 
 #include <hip/hip_runtime_api.h>
 
@@ -216,6 +217,14 @@ static int32_t load_images(psn_ctx *c, const psn_blob *blobs, int n, psn_module 
     }
     int32_t rc = bind(c);
     if (rc) return rc;
+    /* set-up of the no-allocation entry point: look up this GPU's copy of the static scratch now, so
+     * that psn_qmatvec_noalloc itself never has to */
+    {
+        void *sp = nullptr;
+        int herr = 0;
+        if (psn_noalloc_scratch(c->device, &sp, nullptr, &herr) != 0)
+            return fail(PSN_E_HIP, "static scratch of device %d could not be located: hipError %d (%s)", c->device, herr, hipGetErrorString((hipError_t)herr));
+    }
     psn_module *mod = new (std::nothrow) psn_module();
     if (!mod) return fail(PSN_E_OOM, "host allocation failed");
     mod->ctx = c;
@@ -899,6 +908,41 @@ extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qty
 extern "C" int32_t psn_qmatvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, const psn_buf *W,
                                const psn_buf *x, psn_buf *y, int64_t N, int64_t K, int32_t batch) {
     return psn_qmatvec_multi(mod, s, qtype, layout, scheme, 1, &W, x, &y, &N, K, batch);
+}
+
+extern "C" int64_t psn_noalloc_max_bytes(void) { return (int64_t)PSN_NOALLOC_SCRATCH_BYTES; }
+
+/* psn_qmatvec without any allocation: scheme Q8 quantizes x into the library's static device scratch
+ * (one array per GPU, shared by every call on that GPU) and runs the pre-quantized kernel from there;
+ * scheme F32 needs no scratch at all.  Only launches are issued, so the call is legal under capture. */
+extern "C" int32_t psn_qmatvec_noalloc(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, const psn_buf *W,
+                                       const psn_buf *x, psn_buf *y, int64_t N, int64_t K, int32_t batch) {
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
+    seg_list sg;
+    int32_t rc = gather_segments("psn_qmatvec_noalloc", mod, s, qtype, scheme, 1, &W, x, &y, &N, K, batch, &sg);
+    if (rc) return rc;
+    if ((rc = check_x_f32("psn_qmatvec_noalloc", x, K, batch))) return rc;
+    psn_matvec_plan plan;
+    if ((rc = make_plan(qtype, scheme, sg.total, K, batch, mod->ctx->compute_units, false, sg.N, sg.count, &plan))) return rc;
+    if (scheme == PSN_ACT_F32) {
+        if ((rc = bind(mod->ctx))) return rc;
+        return run_matvec(mod, s, qtype, scheme, sg, x->p, K, batch, &plan);
+    }
+    const int32_t at = psn_act_type_for(qtype);
+    psn_actq_info li;
+    if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;
+    if (li.bytes > (int64_t)PSN_NOALLOC_SCRATCH_BYTES)
+        return fail(PSN_E_SHAPE, "psn_qmatvec_noalloc: quantized activations of K=%lld x batch %d take %lld bytes, the static scratch holds %u "
+                    "(use psn_qmatvec, which sizes a workspace)", (long long)K, batch, (long long)li.bytes, PSN_NOALLOC_SCRATCH_BYTES);
+    void *scratch_ptr = nullptr;
+    int herr = 0;
+    if (psn_noalloc_scratch(mod->ctx->device, &scratch_ptr, nullptr, &herr) != 0)
+        return fail(PSN_E_HIP, "psn_qmatvec_noalloc: static scratch of device %d is not available: hipError %d", mod->ctx->device, herr);
+    if ((rc = bind(mod->ctx))) return rc;
+    /* the quantize launch overwrites every byte the matvec reads (qs, scales, sums of batch x K), so
+     * nothing left behind by an earlier, larger call can be seen: no clearing is needed */
+    if ((rc = quantize_into(mod, s, at, (const float *)x->p, scratch_ptr, K, batch))) return rc;
+    return run_matvec(mod, s, qtype, scheme, sg, scratch_ptr, K, batch, &plan);
 }
 
 /* ------------------------------------------------------------------ prefill */

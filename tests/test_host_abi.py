@@ -117,3 +117,24 @@ def test_integration_doc_binding_lists_every_entry_point():
     doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     rust = set(re.findall(r"pub fn (psn_[a-z0-9_]+)\(", doc))
     assert rust == set(header_functions())
+
+
+def test_static_scratch_is_exported_by_the_device_image():
+    """The no-allocation entry point finds its scratch with hipGetSymbolAddress, which looks the
+    registered name up among the symbols the gfx950 image EXPORTS; a file-local symbol there makes the
+    runtime abort.  Checked on the built object, no GPU needed."""
+    import shutil
+    import subprocess
+    import tempfile
+    obj = os.path.join(ROOT, "openagents_amd", "lib", "psn_noalloc.o")
+    bundler, readelf = "/opt/rocm/llvm/bin/clang-offload-bundler", "/opt/rocm/llvm/bin/llvm-readelf"
+    if not (os.path.exists(obj) and os.path.exists(bundler) and os.path.exists(readelf) and shutil.which("objcopy")):
+        pytest.skip("built object or LLVM binutils not present")
+    with tempfile.TemporaryDirectory() as d:
+        fat, elf = os.path.join(d, "fat.bin"), os.path.join(d, "dev.elf")
+        subprocess.check_call(["objcopy", "-O", "binary", "--only-section=.hip_fatbin", obj, fat])
+        subprocess.check_call([bundler, "--unbundle", "--type=o", f"--input={fat}", "--targets=hipv4-amdgcn-amd-amdhsa--gfx950", f"--output={elf}"])
+        syms = subprocess.check_output([readelf, "--dyn-syms", elf], text=True)
+    rows = [ln.split() for ln in syms.splitlines() if ln.strip().endswith("scratch")]
+    assert rows, syms
+    assert all(r[3] == "OBJECT" and r[4] == "GLOBAL" and int(r[2]) == 1 << 20 for r in rows), rows
