@@ -204,10 +204,11 @@ typedef struct psn_matvec_plan {
     int32_t stage_lds;      /* 0: activations read from global memory; 1: staged in LDS; 2 (scheme Q8): x is
                                fp32 and every workgroup quantizes it while staging */
     int32_t blocks;         /* workgroups */
-    int32_t threads;        /* threads per workgroup: 256 or 512 (256, 512 or 768 with `stream`) */
-    int32_t stream;         /* 1: weights land in per-wave LDS buffers by direct-to-LDS loads (scheme Q8,
-                               batch 1, Q4_0/Q8_0/Q4_K, rows of at most lanes_per_row chunks, every matrix a
-                               multiple of 64/lanes_per_row rows, stage_lds 1 or 2); 0: register kernels */
+    int32_t threads;        /* threads per workgroup: 256 or 512 */
+    int32_t stream;         /* 0: register kernels; 1..8: streaming kernel -- weights land in per-wave rings of that
+                               many LDS buffers by direct-to-LDS loads (scheme Q8, batch 1, rows of whole 16-byte
+                               words and at most lanes_per_row chunks, every matrix a multiple of 64/lanes_per_row
+                               rows, stage_lds 1 or 2, 256 or 512 threads) */
     int32_t reserved;
 } psn_matvec_plan;
 int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t compute_units,
@@ -217,6 +218,14 @@ int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
 int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, int32_t count,
                             const psn_buf *const *W, const psn_buf *x, psn_buf *const *y_f32, const int64_t *N, int64_t K,
                             int32_t batch, const psn_matvec_plan *plan);
+
+/* ---- calibration -----------------------------------------------------------------------------
+ * A launch that only reads `bytes` of `src` (whole 4 KB slabs; lds_depth 0: vector loads into registers,
+ * 1..64: direct-to-LDS loads cycling through that many 1 KB slots per wave) and stores one dword per wave
+ * to `out` (may be NULL).  Benchmarks time it beside a matvec of the same size to separate what the
+ * machine allows a dependent launch from what the kernel adds.  No counterpart in the reference. */
+int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, int64_t bytes, int32_t blocks, int32_t threads,
+                           int32_t lds_depth, psn_buf *out);
 
 /* ---- prefill matmul ----------------------------------------------------------------------- */
 

@@ -32,6 +32,7 @@ CODE_OBJECTS = [
     ("psn_mv_q6_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q6_K"]),
     ("psn_prefill", "psn_prefill.hip", []),
     ("psn_decode", "psn_decode.hip", []),
+    ("psn_calib", "psn_calib.hip", []),
 ]
 
 

@@ -48,6 +48,8 @@ struct psn_matvec_args {
     int64_t row_bytes;
     int32_t threads;      /* launch geometry, passed in so that kernels never read the dispatch packet */
     int32_t blocks;
+    int32_t ring;         /* streaming kernels: LDS buffers (passes in flight) per wave */
+    int32_t pad;
 };
 
 struct psn_prefill_args {
@@ -62,6 +64,14 @@ struct psn_prefill_args {
 struct psn_fill_args {
     uint32_t *p;          /* 16-byte aligned */
     int64_t n16;          /* number of 16-byte words to zero */
+};
+
+struct psn_calib_args {
+    const uint8_t *src;   /* 16-byte aligned */
+    uint32_t *out;        /* one dword per wave (may be null) */
+    int64_t bytes;
+    int32_t depth;        /* psn_calib_read_lds: 1 KB LDS slots per wave */
+    int32_t pad;
 };
 
 /* decode-step glue kernels (psn_decode.hip) */

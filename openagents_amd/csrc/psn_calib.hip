@@ -1,0 +1,53 @@
+/*
+ * psn_calib.hip -- calibration kernels: what a launch that ONLY reads a byte range achieves on this
+ * machine.  The matvec kernels are judged against the 8 TB/s HBM peak; these kernels tell how much of
+ * that a dependent launch of the same size can reach at all (launch ramp, drain and the memory fabric
+ * included), which is the number a kernel's own overhead has to be compared with.
+ *
+ *   psn_calib_read      16-byte vector loads into registers, xor-folded, one dword stored per wave;
+ *   psn_calib_read_lds  16-byte direct-to-LDS loads (the path the streaming matvec uses), each wave
+ *                       cycling through `depth` 1 KB slots of its own LDS region.
+ */
+#include "psn_args.h"
+#include "psn_device.h"
+
+extern "C" __global__ void __launch_bounds__(1024) psn_calib_read(const psn_calib_args a) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    const int64_t slab = 64 * 16 * 4;                       /* 4 KB per wave and iteration */
+    const int64_t nslabs = a.bytes / slab;
+    uint4 acc = make_uint4(0, 0, 0, 0);
+    for (int64_t s = wave; s < nslabs; s += nwaves) {
+        const uint4 *p = reinterpret_cast<const uint4 *>(a.src + s * slab) + lane;
+        const uint4 v0 = p[0], v1 = p[64], v2 = p[128], v3 = p[192];
+        acc.x ^= v0.x ^ v1.x ^ v2.x ^ v3.x;
+        acc.y ^= v0.y ^ v1.y ^ v2.y ^ v3.y;
+        acc.z ^= v0.z ^ v1.z ^ v2.z ^ v3.z;
+        acc.w ^= v0.w ^ v1.w ^ v2.w ^ v3.w;
+    }
+    u32 r = acc.x ^ acc.y ^ acc.z ^ acc.w;
+    r ^= (u32)__shfl_xor((int)r, 32, 64);
+    if (lane == 0 && a.out) a.out[wave] = r;
+}
+
+extern "C" __global__ void __launch_bounds__(1024) psn_calib_read_lds(const psn_calib_args a) {
+    extern __shared__ uint4 psn_smem[];
+    const int lane = threadIdx.x & 63, wib = threadIdx.x >> 6;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + wib;
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    const int depth = a.depth;                              /* 1 KB slots per wave */
+    const int64_t slab = (int64_t)depth << 10;
+    const int64_t nslabs = a.bytes / slab;
+    char *buf = reinterpret_cast<char *>(psn_smem) + (int64_t)wib * slab;
+    u32 r = 0;
+    for (int64_t s = wave; s < nslabs; s += nwaves) {
+        const uint8_t *src = a.src + s * slab + lane * 16;
+        for (int i = 0; i < depth; ++i)
+            __builtin_amdgcn_global_load_lds((const void *)(src + i * 1024), (__attribute__((address_space(3))) void *)(buf + i * 1024), 16, 0, 0);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        r ^= reinterpret_cast<const u32 *>(buf)[lane];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    if (lane == 0 && a.out) a.out[wave] = r;
+}

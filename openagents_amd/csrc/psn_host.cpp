@@ -638,6 +638,40 @@ static int64_t staged_lds_bytes(int32_t qtype, int64_t K, int32_t batch) {
     return qs + d + align_up(sb, 16);
 }
 
+/* Can the streaming kernel run this plan?  Fills in the dynamic LDS it needs.  n_rows may be null
+ * (row counts unknown: only the shape-independent conditions are checked). */
+static int32_t stream_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32_t batch, const psn_matvec_plan *plan, const int64_t *n_rows,
+                                 int32_t count, int max_lds, int64_t *lds_out) {
+    const int g = plan->lanes_per_row, rows = 64 / g, ring = plan->stream;
+    const int64_t C = K / 256;
+    if (scheme != PSN_ACT_Q8 || batch != 1 || plan->batch_tile != 1 || plan->rows_in_flight != 1)
+        return fail(PSN_E_UNSUPPORTED, "plan: the streaming kernels serve scheme Q8 at batch 1");
+    if (psn_row_bytes(qtype, K) % 16) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs rows of whole 16-byte words (Q6_K: K a multiple of 2048)");
+    if (C > g) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs rows of at most lanes_per_row chunks (K <= %d)", g * 256);
+    if (plan->stage_lds != 1 && plan->stage_lds != 2) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs stage_lds 1 or 2");
+    if (plan->threads != 256 && plan->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", plan->threads);
+    if (ring < 1 || ring > 8) return fail(PSN_E_UNSUPPORTED, "plan: stream=%d (passes in flight per wave, 1..8)", ring);
+    for (int i = 0; n_rows && i < count; ++i)
+        if (n_rows[i] % rows) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs every matrix to hold a multiple of %d rows", rows);
+    const int32_t at = psn_act_type_for(qtype);
+    const int64_t be = psn_block_elems(at);
+    const int64_t rb = psn_row_bytes(qtype, K);
+    const int64_t nloads = (rows * rb + 1023) / 1024;
+    if ((ring - 1) * nloads > 63) return fail(PSN_E_UNSUPPORTED, "plan: %d passes of %lld loads exceed the load counter", ring, (long long)nloads);
+    /* the activations pass through at most eight 16-byte registers per thread on their way into LDS */
+    const int64_t slots = 8 * (int64_t)plan->threads;
+    const bool fits = plan->stage_lds == 1 ? (C * 16 <= slots && (K / be) * 4 <= 16 * (int64_t)plan->threads)
+                      : at == PSN_Q8_0   ? C * 64 <= slots
+                                         : C <= 8 * (int64_t)(plan->threads / 64);
+    if (!fits) return fail(PSN_E_UNSUPPORTED, "plan: K=%lld is too long for %d threads to stage in one round", (long long)K, plan->threads);
+    const int64_t n_d = ((K / be) * 4 + 15) / 16, n_s = ((at == PSN_Q8_0 ? (K / 32) * 4 : (K / 16) * 2) + 15) / 16;
+    const int64_t stage = (C * 272 + (n_d + n_s) * 16 + 1023) / 1024 * 1024;
+    const int64_t total = stage + (int64_t)(plan->threads / 64) * ring * nloads * 1024;
+    if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs %lld bytes of LDS, device offers %d", (long long)total, max_lds);
+    *lds_out = total;
+    return PSN_OK;
+}
+
 /* n_rows: the row counts of the matrices sharing the launch (count of them), or null when unknown */
 static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, bool fuse_quantize,
                          const int64_t *n_rows, int32_t count, psn_matvec_plan *out) {
@@ -662,6 +696,35 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
     while (g < 64 && (N + (64 / g) - 1) / (64 / g) < (int64_t)cus * 4) g *= 2;
     int64_t waves = (N + (64 / g) - 1) / (64 / g);
     int64_t blocks;
+    /* Batch 1, int8 path, rows of at most 64 chunks, whole passes in every matrix: the streaming kernel
+     * (weights by direct-to-LDS loads).  One pass per wave where the chip holds that many waves, else as
+     * many workgroups as stay resident (LDS) and the waves loop; measured on MI355X. */
+    if (scheme == PSN_ACT_Q8 && batch == 1 && C <= 64 && n_rows != nullptr && p.stage_lds != 0) {
+        int gs = 8;
+        while (gs < C) gs *= 2;
+        const int rows = 64 / gs;
+        bool whole = true;
+        for (int i = 0; i < count; ++i) whole = whole && n_rows[i] % rows == 0;
+        psn_matvec_plan q = p;
+        q.lanes_per_row = gs;
+        q.stream = 1;
+        /* fp32 activations pass through registers on their way into LDS: 256 threads hold K <= 8192 */
+        q.threads = (p.stage_lds == 2 && K > 8192) ? 512 : 256;
+        int64_t lds = 0;
+        q.blocks = 1;
+        if (whole && stream_plan_check(qtype, scheme, K, batch, &q, n_rows, count, 160 * 1024, &lds) == PSN_OK) {
+            const int64_t npass = N / rows, wpb = q.threads / 64;
+            int64_t resident = (160 * 1024) / lds;
+            if (resident > 3) resident = 3;
+            if (resident < 1) resident = 1;
+            int64_t b = (npass + wpb - 1) / wpb;
+            if (b > resident * cus) b = resident * cus;
+            q.blocks = (int32_t)b;
+            *out = q;
+            return PSN_OK;
+        }
+        g_err[0] = 0;                                   /* not streamable after all: the register kernels take it */
+    }
     if (p.stage_lds == 2) {
         /* Every workgroup re-quantizes x while staging it, a cost proportional to K: keep to about
          * eight waves per compute unit in as few workgroups as stream well (measured on MI355X). */
@@ -672,15 +735,6 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
         blocks = (waves + wpb - 1) / wpb;
         const int64_t cap = small_groups ? 2 * (int64_t)cus : (int64_t)cus;
         if (blocks > cap) blocks = cap;
-        /* tall matrices with short rows: the direct-to-LDS streaming kernel wins once every wave has
-         * several passes to pipeline (measured: 2 x 14336 x 4096 Q4_0, 15.3 us against 16.4 us) */
-        bool can_stream = small_groups && batch == 1 && qtype != PSN_Q6_K && C <= g && n_rows != nullptr;
-        for (int i = 0; can_stream && i < count; ++i) can_stream = n_rows[i] % (64 / g) == 0;
-        if (can_stream) {
-            p.stream = 1;
-            p.threads = 512;
-            blocks = 2 * (int64_t)cus;
-        }
     } else {
         /* small workgroups, one pass per wave where the chip can hold them */
         p.threads = 256;
@@ -711,7 +765,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     const int g = p->lanes_per_row, r = p->rows_in_flight, nb = p->batch_tile;
     if (!(g == 8 || g == 16 || g == 32 || g == 64)) return fail(PSN_E_UNSUPPORTED, "plan: lanes_per_row=%d", g);
     if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
-    if (p->threads != 256 && p->threads != 512 && !(p->stream && p->threads == 768)) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
+    if (p->threads != 256 && p->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
     if (r != 1) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
     int32_t lds = 0;
@@ -762,23 +816,10 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
     a.blocks = plan->blocks;
     char name[96];
     if (plan->stream) {
-        const int g = plan->lanes_per_row, rows = 64 / g;
-        const int64_t C = K / 256;
-        if (scheme != PSN_ACT_Q8 || batch != 1 || plan->batch_tile != 1 || plan->rows_in_flight != 1)
-            return fail(PSN_E_UNSUPPORTED, "plan: the streaming kernels serve scheme Q8 at batch 1");
-        if (qtype == PSN_Q6_K) return fail(PSN_E_UNSUPPORTED, "plan: no streaming kernel for Q6_K (rows are not 16-byte multiples)");
-        if (C > g) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs rows of at most lanes_per_row chunks (K <= %d)", g * 256);
-        if (plan->stage_lds != 1 && plan->stage_lds != 2) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs stage_lds 1 or 2");
-        if (plan->threads != 256 && plan->threads != 512 && plan->threads != 768) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d", plan->threads);
-        for (int i = 0; i < sg.count; ++i)
-            if (sg.N[i] % rows) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs every matrix to hold a multiple of %d rows", rows);
+        const int g = plan->lanes_per_row, rows = 64 / g, ring = plan->stream;
+        int64_t total = 0;
+        if ((rc = stream_plan_check(qtype, scheme, K, batch, plan, sg.N, sg.count, mod->ctx->max_lds, &total))) return rc;
         const int32_t at = psn_act_type_for(qtype);
-        const int64_t be = psn_block_elems(at);
-        const int64_t n_d = ((K / be) * 4 + 15) / 16, n_s = ((at == PSN_Q8_0 ? (K / 32) * 4 : (K / 16) * 2) + 15) / 16;
-        const int64_t stage = (C * 272 + (n_d + n_s) * 16 + 1023) / 1024 * 1024;
-        const int64_t wbuf = (rows * a.row_bytes + 1023) / 1024 * 1024;
-        const int64_t total = stage + (plan->threads / 64) * wbuf;
-        if (total > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs %lld bytes of LDS, device offers %d", (long long)total, mod->ctx->max_lds);
         if (plan->stage_lds == 2) {
             a.xf = (const float *)x;
         } else {
@@ -788,6 +829,8 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
             a.xd = (const float *)((const char *)x + li.off_d);
             a.xs = (const char *)x + li.off_s;
         }
+        a.ring = ring;
+        (void)rows;
         snprintf(name, sizeof name, "psn_mvs_%s_q8_g%d_%s", fmt_name(qtype), g, plan->stage_lds == 2 ? "xf" : "lds");
         return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)total, &a);
     }
@@ -943,6 +986,30 @@ extern "C" int32_t psn_qmatvec_noalloc(psn_module *mod, psn_stream *s, int32_t q
      * nothing left behind by an earlier, larger call can be seen: no clearing is needed */
     if ((rc = quantize_into(mod, s, at, (const float *)x->p, scratch_ptr, K, batch))) return rc;
     return run_matvec(mod, s, qtype, scheme, sg, scratch_ptr, K, batch, &plan);
+}
+
+/* ------------------------------------------------------------------ calibration */
+
+extern "C" int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, int64_t bytes, int32_t blocks, int32_t threads,
+                                      int32_t lds_depth, psn_buf *out) {
+    if (!mod || !s || !src) return fail(PSN_E_INVALID_ARG, "psn_calibrate_read: null handle");
+    if (s->ctx != mod->ctx || src->ctx != mod->ctx || (out && out->ctx != mod->ctx)) return fail(PSN_E_INVALID_ARG, "psn_calibrate_read: handles belong to different contexts");
+    if (bytes <= 0 || (int64_t)src->bytes < bytes) return fail(PSN_E_INVALID_ARG, "psn_calibrate_read: %lld bytes asked of a buffer of %zu", (long long)bytes, src->bytes);
+    if (blocks < 1 || blocks > (1 << 20) || threads < 64 || threads > 1024 || threads % 64) return fail(PSN_E_SHAPE, "psn_calibrate_read: blocks=%d threads=%d", blocks, threads);
+    if (lds_depth < 0 || lds_depth > 64) return fail(PSN_E_SHAPE, "psn_calibrate_read: lds_depth=%d outside 0..64", lds_depth);
+    const int64_t waves = (int64_t)blocks * (threads / 64);
+    if (out && (int64_t)out->bytes < waves * 4) return fail(PSN_E_INVALID_ARG, "psn_calibrate_read: out holds %zu bytes, need %lld", out->bytes, (long long)(waves * 4));
+    const int64_t lds = (int64_t)lds_depth * 1024 * (threads / 64);
+    if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "psn_calibrate_read: %lld bytes of LDS asked, device offers %d", (long long)lds, mod->ctx->max_lds);
+    int32_t rc = bind(mod->ctx);
+    if (rc) return rc;
+    psn_calib_args a;
+    a.src = (const uint8_t *)src->p;
+    a.out = out ? (uint32_t *)out->p : nullptr;
+    a.bytes = bytes;
+    a.depth = lds_depth;
+    a.pad = 0;
+    return launch(mod, s, lds_depth ? "psn_calib_read_lds" : "psn_calib_read", (unsigned)blocks, (unsigned)threads, (unsigned)lds, &a);
 }
 
 /* ------------------------------------------------------------------ prefill */

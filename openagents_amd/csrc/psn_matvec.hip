@@ -605,19 +605,223 @@ PSN_DEV void mv_q8(const psn_matvec_args &a) {
     }
 }
 
-/* Scheme Q8, streaming variant (batch 1, rows of at most G chunks).  The weights do not pass through
- * registers on their way in: each wave owns an LDS buffer that holds the 64/G rows of one pass and
- * fills it with 16-byte direct-to-LDS loads (lanes fetch consecutive 16-byte words, so every load
- * instruction covers 1 KB of contiguous row bytes).  Per pass: wait for the buffer, copy the lane's
- * chunk into registers, immediately start the next pass's loads into the same buffer, then do the
- * dot products -- the memory latency of pass p+1 runs under the arithmetic of pass p without a
- * second register set.  The lane's activation chunk is read from the staged copy once and kept.
- * One workgroup per compute unit (LDS-limited); waves stride over the passes. */
+/* ------------------------------------------------------------------------------------------
+ * Scheme Q8, streaming variant (batch 1, rows of at most G chunks).
+ *
+ * The weights do not pass through registers on their way in: every wave owns a ring of LDS buffers,
+ * one pass (the 64/G rows a wave retires together, a contiguous byte range of the matrix) per
+ * buffer, filled by 16-byte direct-to-LDS loads (lanes fetch consecutive 16-byte words, so one load
+ * instruction covers 1 KB of contiguous row bytes).  A wave first puts all the passes its ring holds
+ * in flight, then the workgroup stages the activations (their loads were issued even earlier, and
+ * loads return in order), and from then on: wait for the oldest pass only, copy the lane's chunk
+ * LDS -> registers, refill that buffer with the pass `ring` steps ahead, multiply.  The memory
+ * system therefore always has ring x waves passes queued, independent of the arithmetic.
+ *
+ * Every wait in this kernel is written by hand.  The compiler's own wait insertion cannot tell the
+ * ring buffers (dynamic LDS, run-time offsets) apart and would wait for ALL outstanding loads before
+ * any LDS read; so LDS and the activation loads are accessed through inline assembly it does not
+ * model, and the vmcnt / lgkmcnt waits are placed explicitly (loads complete in issue order, hence
+ * "at most n younger loads outstanding" identifies the pass that has landed).
+ * ------------------------------------------------------------------------------------------ */
+
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+
+/* wave-uniform n: wait until at most n vector-memory loads are outstanding */
+PSN_DEV void wait_vmcnt(int n) {
+#define PSN_W(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;
+    switch (n) {
+        PSN_W(1) PSN_W(2) PSN_W(3) PSN_W(4) PSN_W(5) PSN_W(6) PSN_W(7) PSN_W(8) PSN_W(9) PSN_W(10) PSN_W(11) PSN_W(12)
+        PSN_W(13) PSN_W(14) PSN_W(15) PSN_W(16) PSN_W(17) PSN_W(18) PSN_W(19) PSN_W(20) PSN_W(21) PSN_W(22) PSN_W(23)
+        PSN_W(24) PSN_W(25) PSN_W(26) PSN_W(27) PSN_W(28) PSN_W(29) PSN_W(30) PSN_W(31) PSN_W(32) PSN_W(33) PSN_W(34)
+        PSN_W(35) PSN_W(36) PSN_W(37) PSN_W(38) PSN_W(39) PSN_W(40) PSN_W(41) PSN_W(42) PSN_W(43) PSN_W(44) PSN_W(45)
+        PSN_W(46) PSN_W(47) PSN_W(48) PSN_W(49) PSN_W(50) PSN_W(51) PSN_W(52) PSN_W(53) PSN_W(54) PSN_W(55) PSN_W(56)
+        PSN_W(57) PSN_W(58) PSN_W(59) PSN_W(60) PSN_W(61) PSN_W(62) PSN_W(63)
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;      /* 0, or more than the counter holds */
+    }
+#undef PSN_W
+}
+/* LDS and global accesses the compiler does not see as memory operations (no automatic waits) */
+template <int OFF> PSN_DEV u32x4 lds_read128(u32 addr) {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+PSN_DEV u32 lds_read32(u32 addr) {
+    u32 v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+PSN_DEV u32 lds_read_u16(u32 addr) {
+    u32 v;
+    asm volatile("ds_read_u16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+PSN_DEV void lds_write128(u32 addr, u32x4 v) { asm volatile("ds_write_b128 %0, %1" ::"v"(addr), "v"(v) : "memory"); }
+PSN_DEV void lds_write32(u32 addr, u32 v) { asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(v) : "memory"); }
+PSN_DEV void lds_write16(u32 addr, u32 v) { asm volatile("ds_write_b16 %0, %1" ::"v"(addr), "v"(v) : "memory"); }
+PSN_DEV u32x4 global_read128(const void *p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+/* the values written by the reads above may be used after this (volatile asm statements stay in order) */
+PSN_DEV void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+template <int N> PSN_DEV void tie(u32x4 (&v)[N]) { UNROLL for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i])); }
+PSN_DEV void tie1(u32 &v) { asm volatile("" : "+v"(v)); }
+/* workgroup barrier that waits for this wave's LDS traffic only, not for loads still in flight */
+PSN_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+/* a lane's chunk, LDS -> registers */
+template <typename F> PSN_DEV void stream_load_chunk(u32 addr, u32 (&w)[F::DW]);
+template <int NW, int I = 0> PSN_DEV void lds_read_seq(u32 addr, u32x4 (&v)[NW]) {
+    if constexpr (I < NW) {
+        v[I] = lds_read128<16 * I>(addr);                   /* offsets are instruction immediates */
+        lds_read_seq<NW, I + 1>(addr, v);
+    }
+}
+template <int NW> PSN_DEV void stream_read_words(u32 addr, u32 *w) {
+    u32x4 v[NW];
+    lds_read_seq<NW>(addr, v);
+    lds_wait();
+    tie(v);
+    UNROLL for (int i = 0; i < NW; ++i) { w[4 * i] = v[i].x; w[4 * i + 1] = v[i].y; w[4 * i + 2] = v[i].z; w[4 * i + 3] = v[i].w; }
+}
+
+/* The staged activations of one chunk, LDS -> registers: 64 dwords of int8 and, for Q8_0 activations, 8
+ * scales + 8 block sums, for Q8_K one scale + 16 int16 group sums (same register layout as load_x_*). */
+template <typename ST, int XR> PSN_DEV void stream_load_x(u32 qs_addr, u32 d_addr, u32 s_addr, int j, u32 (&xr)[XR]) {
+    u32x4 q[16], e[4];
+    const u32 qa = qs_addr + (u32)j * 272u;
+    lds_read_seq<16>(qa, q);
+    u32 dk = 0;
+    if constexpr (sizeof(ST) == 4) {
+        e[0] = lds_read128<0>(d_addr + (u32)j * 32u);
+        e[1] = lds_read128<16>(d_addr + (u32)j * 32u);
+        e[2] = lds_read128<0>(s_addr + (u32)j * 32u);
+        e[3] = lds_read128<16>(s_addr + (u32)j * 32u);
+    } else {
+        dk = lds_read32(d_addr + (u32)j * 4u);
+        e[0] = lds_read128<0>(s_addr + (u32)j * 32u);
+        e[1] = lds_read128<16>(s_addr + (u32)j * 32u);
+        e[2] = e[3] = e[0];
+    }
+    lds_wait();
+    tie(q);
+    tie(e);
+    tie1(dk);
+    UNROLL for (int i = 0; i < 16; ++i) { xr[4 * i] = q[i].x; xr[4 * i + 1] = q[i].y; xr[4 * i + 2] = q[i].z; xr[4 * i + 3] = q[i].w; }
+    if constexpr (sizeof(ST) == 4) {
+        UNROLL for (int i = 0; i < 4; ++i) { xr[64 + 4 * i] = e[i].x; xr[65 + 4 * i] = e[i].y; xr[66 + 4 * i] = e[i].z; xr[67 + 4 * i] = e[i].w; }
+    } else {
+        xr[64] = dk;
+        UNROLL for (int i = 0; i < 2; ++i) { xr[65 + 4 * i] = e[i].x; xr[66 + 4 * i] = e[i].y; xr[67 + 4 * i] = e[i].z; xr[68 + 4 * i] = e[i].w; }
+    }
+}
+
+/* Activations into LDS for the streaming kernel (layout as in Stager: every 256-byte chunk of int8
+ * followed by 16 bytes of padding, then the scales, then the sums).  issue() starts the global loads
+ * (at most SLOTS 16-byte words per thread -- the host only picks this kernel when that suffices),
+ * finish(pending) waits until at most `pending` younger loads are outstanding, quantizes if the input
+ * was fp32 and writes LDS; the caller crosses the workgroup barrier. */
+template <typename ST, int XSRC>
+struct StreamStager {
+    static constexpr int SLOTS = 8;
+    u32x4 t[SLOTS];
+    u32x4 td, ts;
+    int C, nthreads, n_qs, n_d, n_s;
+
+    PSN_DEV void issue(const psn_matvec_args &a, int d_per_col, int s_per_col) {
+        C = a.K >> 8;
+        nthreads = a.threads;
+        n_qs = C * 16;
+        n_d = (d_per_col * 4 + 15) / 16;
+        n_s = (s_per_col * (int)sizeof(ST) + 15) / 16;
+        UNROLL for (int i = 0; i < SLOTS; ++i) t[i] = (u32x4)(0u);
+        td = ts = (u32x4)(0u);
+        if constexpr (XSRC == 1) {
+            const uint4 *g_qs = reinterpret_cast<const uint4 *>(a.xqs);
+            UNROLL for (int i = 0; i < SLOTS; ++i) {
+                const int idx = threadIdx.x + i * nthreads;
+                if (idx < n_qs) t[i] = global_read128(g_qs + idx);
+            }
+            if ((int)threadIdx.x < n_d) td = global_read128(reinterpret_cast<const uint4 *>(a.xd) + threadIdx.x);
+            if ((int)threadIdx.x < n_s) ts = global_read128(reinterpret_cast<const uint4 *>(a.xs) + threadIdx.x);
+        } else {
+            const float4 *x4 = reinterpret_cast<const float4 *>(a.xf);
+            if constexpr (sizeof(ST) == 4) {
+                const int total4 = C * 64;
+                UNROLL for (int i = 0; i < SLOTS; ++i) {
+                    const int idx = threadIdx.x + i * nthreads;
+                    if (idx < total4) t[i] = global_read128(x4 + idx);
+                }
+            } else {
+                const int wpb = nthreads >> 6, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+                UNROLL for (int i = 0; i < SLOTS; ++i) {
+                    const int sb = wid + i * wpb;
+                    if (sb < C) t[i] = global_read128(x4 + sb * 64 + lane);
+                }
+            }
+        }
+    }
+
+    /* base: LDS byte address of the staging area; returns the addresses of the three fields */
+    PSN_DEV void finish(int pending, u32 base, u32 &qs_addr, u32 &d_addr, u32 &s_addr) {
+        qs_addr = base;
+        d_addr = base + (u32)C * 272u;
+        s_addr = d_addr + (u32)n_d * 16u;
+        wait_vmcnt(pending);
+        tie(t);
+        asm volatile("" : "+v"(td), "+v"(ts));
+        const int lane = threadIdx.x & 63;
+        if constexpr (XSRC == 1) {
+            UNROLL for (int i = 0; i < SLOTS; ++i) {
+                const int idx = threadIdx.x + i * nthreads;
+                if (idx < n_qs) lds_write128(qs_addr + (u32)((idx >> 4) * 272 + (idx & 15) * 16), t[i]);
+            }
+            if ((int)threadIdx.x < n_d) lds_write128(d_addr + threadIdx.x * 16u, td);
+            if ((int)threadIdx.x < n_s) lds_write128(s_addr + threadIdx.x * 16u, ts);
+        } else if constexpr (sizeof(ST) == 4) {
+            const int total4 = C * 64;
+            UNROLL for (int k = 0; k < SLOTS; ++k) {
+                const int i = threadIdx.x + k * nthreads;
+                if (i < total4) {                                  /* whole 8-lane groups: K is a multiple of 256 */
+                    u32 packed;
+                    float d;
+                    int sum;
+                    q8_0_quant4(make_float4(__uint_as_float(t[k].x), __uint_as_float(t[k].y), __uint_as_float(t[k].z), __uint_as_float(t[k].w)), packed, d, sum);
+                    lds_write32(qs_addr + (u32)((i >> 6) * 272 + (i & 63) * 4), packed);
+                    if ((lane & 7) == 0) {
+                        lds_write32(d_addr + (u32)(i >> 3) * 4u, __float_as_uint(d));
+                        lds_write32(s_addr + (u32)(i >> 3) * 4u, (u32)sum);
+                    }
+                }
+            }
+        } else {
+            const int wpb = nthreads >> 6, wid = threadIdx.x >> 6;
+            UNROLL for (int k = 0; k < SLOTS; ++k) {
+                const int sb = wid + k * wpb;
+                if (sb < C) {                                      /* wave-uniform */
+                    u32 packed;
+                    float d;
+                    int s16;
+                    q8_K_quant_wave(make_float4(__uint_as_float(t[k].x), __uint_as_float(t[k].y), __uint_as_float(t[k].z), __uint_as_float(t[k].w)), lane, packed, d, s16);
+                    lds_write32(qs_addr + (u32)(sb * 272 + lane * 4), packed);
+                    if ((lane & 3) == 0) lds_write16(s_addr + (u32)(sb * 16 + (lane >> 2)) * 2u, (u32)s16 & 0xffffu);
+                    if (lane == 0) lds_write32(d_addr + (u32)sb * 4u, __float_as_uint(d));
+                }
+            }
+        }
+    }
+};
+
 template <typename F, int G, int XSRC>
 PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
     typedef typename F::ActSum ST;
     constexpr int S = 64 / G;                                /* rows per pass; every matrix holds a multiple of S rows */
     extern __shared__ uint4 psn_smem[];
+    typedef __attribute__((address_space(3))) char lds_char;
+    lds_char *const lds_ptr = (lds_char *)psn_smem;
+    const u32 lds0 = (u32)(uintptr_t)lds_ptr;
     const int lane = threadIdx.x & 63, slot = lane / G, j = lane % G;
     const int wpb = a.threads >> 6;
     const int wib = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   /* wave-uniform, and the compiler should know it */
@@ -625,19 +829,24 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
     const int rb = (int)a.row_bytes;                         /* bytes per row; a multiple of 16 */
     const int span = S * rb, nloads = (span + 1023) >> 10;   /* bytes and 1 KB load instructions per pass */
     const int wbuf = nloads << 10;
+    const int ring = a.ring;                                 /* passes a wave keeps in flight (LDS buffers per wave) */
     const int npass = N / S;
     const int stride = a.blocks * wpb;
-    int p = blockIdx.x * wpb + wib;
+    const int p0 = blockIdx.x * wpb + wib;                   /* this wave's passes: p0, p0 + stride, ... */
+
+    /* The activation loads go out before anything else is computed: they are small, and every load
+     * issued later (the weights) completes after them. */
+    StreamStager<ST, XSRC> st;
+    st.issue(a, F::d_per_col(K), F::s_per_col(K));
 
     /* where the wave buffers start: right behind the staged activations (same arithmetic as the host) */
     const int n_d = (F::d_per_col(K) * 4 + 15) / 16, n_s = (F::s_per_col(K) * (int)sizeof(ST) + 15) / 16;
     const int stage_bytes = ((C * 272 + (n_d + n_s) * 16 + 1023) >> 10) << 10;
-    char *buf = reinterpret_cast<char *>(psn_smem) + stage_bytes + wib * wbuf;
+    const u32 ring_base = lds0 + (u32)stage_bytes + (u32)(wib * ring) * (u32)wbuf;
 
-    /* a pass never straddles two matrices, so its rows are one contiguous range of one of them;
-     * all of this is scalar arithmetic on kernel arguments */
-    /* The four base pointers are pinned in scalar registers (the empty asm keeps the compiler from
-     * turning the selects below back into an indexed load from a private copy of the arguments). */
+    /* a pass never straddles two matrices, so its rows are one contiguous range of one of them; the
+     * four base pointers are pinned in scalar registers (the empty asm keeps the compiler from turning
+     * the selects below back into an indexed load from a private copy of the arguments) */
     const uint8_t *W0 = a.W[0], *W1 = a.W[1], *W2 = a.W[2], *W3 = a.W[3];
     float *Y0 = a.y[0], *Y1 = a.y[1], *Y2 = a.y[2], *Y3 = a.y[3];
     int E0 = a.row_end[0], E1 = a.row_end[1], E2 = a.row_end[2];
@@ -654,43 +863,64 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
         w = wb + (int64_t)(row0 - first) * rb;
         y = yb + (row0 - first);
     };
-    /* straight-line issue: up to F::DW / 4 (+1 when G > chunks leaves a ragged tail) predicated loads */
-    auto issue = [&](const uint8_t *w) {
-        const uint8_t *src = w + lane * 16;
-        UNROLL for (int i = 0; i < F::DW / 4 + 1; ++i)
-            if (i * 1024 + lane * 16 < span)
-                __builtin_amdgcn_global_load_lds((const void *)(src + i * 1024), (__attribute__((address_space(3))) void *)(buf + i * 1024), 16, 0, 0);
+    /* one pass into ring buffer `b`: exactly `nloads` load instructions of 1 KB each.  Lanes past the end
+     * of the pass re-read its last 16 bytes (into the unused tail of the buffer) instead of being
+     * masked off: a masked load costs a branch around every instruction. */
+    auto issue = [&](int pass, int b) {
+        const uint8_t *w;
+        float *y;
+        pass_base(pass, w, y);
+        lds_char *dst = lds_ptr + (ring_base - lds0) + b * wbuf;
+        int off = lane * 16;
+        for (int l = 0; l < nloads; ++l) {
+            __builtin_amdgcn_global_load_lds((const void *)(w + min(off, span - 16)), (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+            off += 1024;
+            dst += 1024;
+        }
     };
 
-    Stager<ST, XSRC, false> st;                                  /* staged after the first loads are on their way */
-    st.issue(a, F::d_per_col(K), F::s_per_col(K));
-    const uint8_t *wsrc = nullptr;
-    float *ydst = nullptr;
-    if (p < npass) {
-        pass_base(p, wsrc, ydst);
-        issue(wsrc);
-    }
-    const ActQ<ST> x = st.finish(a);
+    /* everything the ring holds goes in flight at once */
+    int issued = 0;                                          /* passes issued so far */
+    for (; issued < ring && p0 + issued * stride < npass; ++issued) issue(p0 + issued * stride, issued);
+    u32 qs_addr, d_addr, s_addr;
+    st.finish(issued * nloads, lds0, qs_addr, d_addr, s_addr);   /* waits for the activation loads only */
+    lds_barrier();
     u32 xr[F::XR];
     UNROLL for (int i = 0; i < F::XR; ++i) xr[i] = 0;
-    if (j < C) F::load_x(x, K, 0, j, xr);
-    while (p < npass) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                 /* this pass's rows are in the buffer */
+    if (j < C) stream_load_x<ST, F::XR>(qs_addr, d_addr, s_addr, j, xr);
+    int b = 0;                                               /* ring buffer of the current pass */
+    for (int p = p0, done = 0; p < npass; p += stride, ++done) {
+        /* the passes issued after this one (at most ring - 1) may stay in flight */
+        wait_vmcnt((issued - done - 1) * nloads);
         u32 w[F::DW];
-        UNROLL for (int i = 0; i < F::DW; ++i) w[i] = 0;
-        if (j < C) F::load(reinterpret_cast<const uint8_t *>(buf) + slot * rb + j * F::BYTES, w);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");               /* ... and in registers: the buffer is free */
-        float *ycur = ydst;
-        const int pn = p + stride;
-        if (pn < npass) {
-            pass_base(pn, wsrc, ydst);
-            issue(wsrc);
+        UNROLL for (int q = 0; q < F::DW; ++q) w[q] = 0;
+        if (j < C) stream_load_chunk<F>(ring_base + (u32)(b * wbuf + slot * rb + j * F::BYTES), w);
+        else lds_wait();
+        const uint8_t *wsrc;
+        float *ydst;
+        pass_base(p, wsrc, ydst);
+        const int pn = p0 + issued * stride;
+        if (pn < npass) {                                    /* this buffer is free again: refill it */
+            issue(pn, b);
+            ++issued;
         }
+        b = b + 1 == ring ? 0 : b + 1;
         float acc = (j < C) ? F::dot(w, xr) : 0.f;
         acc = group_sum<G>(acc);
-        if (j == 0) ycur[slot] = acc;
-        p = pn;
+        if (j == 0) ydst[slot] = acc;
     }
+}
+
+template <> PSN_DEV void stream_load_chunk<FmtQ4_0>(u32 addr, u32 (&w)[FmtQ4_0::DW]) { stream_read_words<9>(addr, w); }
+template <> PSN_DEV void stream_load_chunk<FmtQ4_K>(u32 addr, u32 (&w)[FmtQ4_K::DW]) { stream_read_words<9>(addr, w); }
+template <> PSN_DEV void stream_load_chunk<FmtQ8_0>(u32 addr, u32 (&w)[FmtQ8_0::DW]) { stream_read_words<17>(addr, w); }
+/* Q6_K super-blocks are 210 bytes: a chunk starts on an even byte, not on a 16-byte word (gfx950 reads
+ * LDS at any alignment); 13 words cover bytes 0..207, the fp16 d sits in the last two */
+template <> PSN_DEV void stream_load_chunk<FmtQ6_K>(u32 addr, u32 (&w)[FmtQ6_K::DW]) {
+    u32 d = lds_read_u16(addr + 208u);
+    stream_read_words<13>(addr, w);
+    tie1(d);
+    w[52] = d;
 }
 
 /* Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations.
@@ -777,10 +1007,10 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
     }
 
 #define PSN_STREAM_KERNEL(fmt, F, G)                                                                      \
-    extern "C" __global__ void __launch_bounds__(768) psn_mvs_##fmt##_q8_g##G##_lds(const psn_matvec_args a) { \
+    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_lds(const psn_matvec_args a) { \
         mv_q8_stream<F, G, 1>(a);                                                                         \
     }                                                                                                     \
-    extern "C" __global__ void __launch_bounds__(768) psn_mvs_##fmt##_q8_g##G##_xf(const psn_matvec_args a) {  \
+    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_xf(const psn_matvec_args a) {  \
         mv_q8_stream<F, G, 2>(a);                                                                         \
     }
 #define PSN_STREAM_ALL(fmt, F) PSN_STREAM_KERNEL(fmt, F, 8) PSN_STREAM_KERNEL(fmt, F, 16) PSN_STREAM_KERNEL(fmt, F, 32) PSN_STREAM_KERNEL(fmt, F, 64)
@@ -825,4 +1055,5 @@ PSN_STREAM_ALL(q4_K, FmtQ4_K)
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q6_K)
 PSN_Q8_ALL(q6_K, FmtQ6_K)
 PSN_F32_ALL(q6_K, FmtQ6_K)
+PSN_STREAM_ALL(q6_K, FmtQ6_K)
 #endif

@@ -406,13 +406,17 @@ def test_graph_replay_matches_eager(hip, orc):
 
 # ------------------------------------------------------------------ streaming (direct-to-LDS) kernels
 
-@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K"])
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
 def test_streaming_kernels_every_variant(hip, orc, qname):
-    """Weights land in per-wave LDS buffers; rows per pass = 64 / lanes_per_row, so the matrices hold
-    multiples of 8 rows.  k = 2048 fills 8-lane groups exactly, k = 2560 (10 chunks) leaves idle lanes
-    and a ragged last 1 KB load; few workgroups force several passes per wave."""
+    """Weights land in per-wave rings of LDS buffers (1 to 4 passes in flight); rows per pass =
+    64 / lanes_per_row, so the matrices hold multiples of 8 rows.  k = 2048 fills 8-lane groups exactly,
+    k = 2560 (10 chunks) leaves idle lanes and a ragged last 1 KB load; few workgroups force many passes
+    per wave, so every ring slot is refilled several times."""
     t = getattr(orc, qname)
+    ran = refused = 0
     for k, ns in ((2048, [80]), (2560, [80, 8, 136, 16]), (4096, [1024, 256, 256]), (14336, [64])):
+        if qname == "Q6_K" and k % 2048:
+            continue                                         # 210-byte super-blocks: rows of whole 16-byte words need K % 2048 == 0
         Ws = [weights(orc, qname, 900 + i, n, k) for i, n in enumerate(ns)]
         x = G.seeded_acts(901, 1, k)
         refs = [orc.matvec(t, orc.ACT_Q8, W, x, n, k) for W, n in zip(Ws, ns)]
@@ -423,34 +427,43 @@ def test_streaming_kernels_every_variant(hip, orc, qname):
             if k // 256 > g:
                 continue
             for stage in (1, 2):
-                for threads, blocks in ((256, 2), (512, 1), (768, 3)):
+                for threads, blocks, ring in ((256, 2, 1), (512, 1, 2), (512, 3, 3), (256, 5, 4)):
                     p = _ffi.MatvecPlan()
-                    p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream = g, 1, 1, stage, blocks, threads, 1
+                    p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream = g, 1, 1, stage, blocks, threads, ring
                     say(f"stream {qname} k={k} ns={ns} {p.as_dict()}")
                     ys = [hip.upload(np.full((1, n), np.nan, np.float32)) for n in ns]
                     try:
                         hip.quantized_matvec_planned(ws, xb if stage == 2 else xq, ys, 1, _ffi.ACT_Q8, p)
-                    except backend.PsnError as e:              # 12 waves x 17 KB of Q8_0 rows do not fit 160 KB
-                        assert e.code == _ffi.E_UNSUPPORTED and "LDS" in str(e) and qname == "Q8_0" and threads == 768
+                    except backend.PsnError as e:
+                        # refused before anything is launched: the ring does not fit 160 KB of LDS, its loads
+                        # exceed the hardware's load counter, or K is too long for the workgroup to stage
+                        assert e.code == _ffi.E_UNSUPPORTED and any(w in str(e) for w in ("LDS", "load counter", "too long")), str(e)
+                        refused += 1
                         continue
+                    ran += 1
                     for y, ref, n in zip(ys, refs, ns):
                         err = G.max_rel_err(y.download(np.float32, (1, n)), ref)
                         assert err < PARITY_TOL, (p.as_dict(), k, n, err)
+    say(f"stream {qname}: {ran} variants ran, {refused} refused")
+    assert ran >= (20 if qname == "Q6_K" else 40)
 
 
 def test_streaming_plan_is_refused_where_it_cannot_run(hip, orc):
-    k = 2048
-    W = weights(orc, "Q6_K", 910, 80, k)
-    w6 = hip.upload_weight(orc.Q6_K, W, 80, k)
-    w4 = hip.upload_weight(orc.Q4_0, weights(orc, "Q4_0", 911, 84, k), 84, k)
+    k = 2560
+    w6 = hip.upload_weight(orc.Q6_K, weights(orc, "Q6_K", 910, 80, k), 80, k)
+    w4 = hip.upload_weight(orc.Q4_0, weights(orc, "Q4_0", 911, 82, k), 82, k)
     x = hip.upload(np.zeros(k, np.float32))
     y = hip.alloc(84 * 4)
     p = _ffi.MatvecPlan()
-    p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream = 8, 1, 1, 2, 4, 256, 1
-    for w in (w6, w4):                                   # Q6_K has no streaming kernel; 84 rows is not a multiple of 8
+    p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream = 16, 1, 1, 2, 4, 256, 1
+    for w in (w6, w4):                 # Q6_K rows of 2100 bytes are not whole 16-byte words; 82 rows is not a multiple of 4
         with pytest.raises(backend.PsnError) as e:
             hip.quantized_matvec_planned(w, x, y, 1, _ffi.ACT_Q8, p)
         assert e.value.code == _ffi.E_UNSUPPORTED
+    p.stream = 9
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_planned(w4, x, y, 1, _ffi.ACT_Q8, p)
+    assert e.value.code == _ffi.E_UNSUPPORTED
 
 
 def test_two_branch_graph_of_independent_launches(hip, orc):
