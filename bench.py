@@ -170,7 +170,7 @@ def main(argv=None):
     def kernel_of(ns, k):
         p = matvec_plan(_ffi.Q4_0, _ffi.ACT_Q8, sum(ns), k, 1, be.compute_units, True)
         if p.stream:
-            return f"psn_mvs_q4_0_q8_g{p.lanes_per_row}" + {1: "_lds", 2: "_xf"}[p.stage_lds]
+            return f"psn_mvs_q4_0_q8_g{p.lanes_per_row}" + {1: "_lds", 2: "_xf"}[p.stage_lds] + f"_s{len(ns)}"
         return f"psn_mv_q4_0_q8_g{p.lanes_per_row}_r{p.rows_in_flight}_b{p.batch_tile}" + {0: "", 1: "_lds", 2: "_xf"}[p.stage_lds]
     groups = {}
     for name, ns, k in LAUNCHES:

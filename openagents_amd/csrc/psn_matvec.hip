@@ -814,7 +814,7 @@ struct StreamStager {
     }
 };
 
-template <typename F, int G, int XSRC>
+template <typename F, int G, int XSRC, int NSEG>
 PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
     typedef typename F::ActSum ST;
     constexpr int S = 64 / G;                                /* rows per pass; every matrix holds a multiple of S rows */
@@ -857,9 +857,11 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
         const uint8_t *wb = W0;
         float *yb = Y0;
         int first = 0;
-        if (nseg > 1 && row0 >= E0) { wb = W1; yb = Y1; first = E0; }
-        if (nseg > 2 && row0 >= E1) { wb = W2; yb = Y2; first = E1; }
-        if (nseg > 3 && row0 >= E2) { wb = W3; yb = Y3; first = E2; }
+        /* with three or four matrices the count is compared at run time: the compiler turns a chain of
+         * selects whose length it knows into an indexed load from a private (scratch) copy of the arguments */
+        if (NSEG > 1 && row0 >= E0) { wb = W1; yb = Y1; first = E0; }
+        if (NSEG > 2 && nseg > 2 && row0 >= E1) { wb = W2; yb = Y2; first = E1; }
+        if (NSEG > 2 && nseg > 3 && row0 >= E2) { wb = W3; yb = Y3; first = E2; }
         w = wb + (int64_t)(row0 - first) * rb;
         y = yb + (row0 - first);
     };
@@ -1006,14 +1008,16 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
         mv_q8<F, G, R, NB, 2>(a);                                                                         \
     }
 
-#define PSN_STREAM_KERNEL(fmt, F, G)                                                                      \
-    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_lds(const psn_matvec_args a) { \
-        mv_q8_stream<F, G, 1>(a);                                                                         \
+/* streaming kernels: psn_mvs_<fmt>_q8_g<G>_{lds|xf}_s<matrices sharing the launch> */
+#define PSN_STREAM_KERNEL(fmt, F, G, NSEG)                                                                \
+    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_lds_s##NSEG(const psn_matvec_args a) { \
+        mv_q8_stream<F, G, 1, NSEG>(a);                                                                   \
     }                                                                                                     \
-    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_xf(const psn_matvec_args a) {  \
-        mv_q8_stream<F, G, 2>(a);                                                                         \
+    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_xf_s##NSEG(const psn_matvec_args a) {  \
+        mv_q8_stream<F, G, 2, NSEG>(a);                                                                   \
     }
-#define PSN_STREAM_ALL(fmt, F) PSN_STREAM_KERNEL(fmt, F, 8) PSN_STREAM_KERNEL(fmt, F, 16) PSN_STREAM_KERNEL(fmt, F, 32) PSN_STREAM_KERNEL(fmt, F, 64)
+#define PSN_STREAM_G(fmt, F, G) PSN_STREAM_KERNEL(fmt, F, G, 1) PSN_STREAM_KERNEL(fmt, F, G, 2) PSN_STREAM_KERNEL(fmt, F, G, 3) PSN_STREAM_KERNEL(fmt, F, G, 4)
+#define PSN_STREAM_ALL(fmt, F) PSN_STREAM_G(fmt, F, 8) PSN_STREAM_G(fmt, F, 16) PSN_STREAM_G(fmt, F, 32) PSN_STREAM_G(fmt, F, 64)
 
 #define PSN_F32_KERNEL(fmt, F, G, R, NB)                                                                  \
     extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB(const psn_matvec_args a) { \
