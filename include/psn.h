@@ -222,10 +222,11 @@ int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32
 /* ---- calibration -----------------------------------------------------------------------------
  * A launch that only reads `bytes` of `src` (whole 4 KB slabs; lds_depth 0: vector loads into registers,
  * 1..64: direct-to-LDS loads cycling through that many 1 KB slots per wave) and stores one dword per wave
- * to `out` (may be NULL).  Benchmarks time it beside a matvec of the same size to separate what the
+ * to `out` (may be NULL).  With every_workgroup != 0 each workgroup reads the whole range instead of the
+ * workgroups sharing it (the pattern of an operand all workgroups need, served from L2).  Benchmarks time it beside a matvec of the same size to separate what the
  * machine allows a dependent launch from what the kernel adds.  No counterpart in the reference. */
 int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, int64_t bytes, int32_t blocks, int32_t threads,
-                           int32_t lds_depth, psn_buf *out);
+                           int32_t lds_depth, int32_t every_workgroup, psn_buf *out);
 
 /* ---- prefill matmul ----------------------------------------------------------------------- */
 
@@ -235,14 +236,16 @@ int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, i
  * matmul op. */
 int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
                             const psn_buf *X_f16, psn_buf *Y_f32, int64_t M, int64_t N, int64_t K);
-/* The launch shape the library picks for a prefill: the workgroup tile of Y (64x64, 64x128,
- * 128x128, 128x256, 256x128 or 256x256) and into how many ranges K is cut (1, 2, 4 or 8; with more
- * than one, Y is zeroed by a fill kernel and the partial sums are added atomically, so their order --
- * and the last bit of a sum -- can vary between runs), and the kernel family: 4 = four waves, 8 = eight
- * waves (tiles of at least 128x128), -4 = four waves with X prefetched three K steps ahead and the
- * weight decode interleaved with the MFMAs (64x128, 128x128, 128x256), -5 = four waves with X prefetched
- * through registers (tiles of at least 128x128), 16 = eight waves of which four only multiply and four
- * only stage (128x128, 128x256).  Host arithmetic only ... */
+/* The launch shape the library picks for a prefill: the workgroup tile of Y (64x64, 64x128, 128x128,
+ * 128x256, 256x128 or 256x256), into how many ranges K is cut (1, 2, 4 or 8; with more than one, Y is
+ * zeroed by a fill kernel and the partial sums are added atomically, so their order -- and the last bit
+ * of a sum -- can vary between runs), and the kernel family:
+ *    4  four waves, every wave stages and multiplies (any tile);
+ *   16  eight waves of which four only multiply and four only stage: X by direct-to-LDS loads three K
+ *       steps ahead, weights decoded from registers one step ahead (64x64, 64x128, 128x128, 128x256);
+ *   64  the weight-streaming kernel for M <= 64 (64x64 tiles): X and the raw GGUF bytes arrive in LDS
+ *       rings by direct-to-LDS loads, every wave decodes its own MFMA operand, one barrier per 256 of K.
+ * Host arithmetic only ... */
 int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m, int32_t *tile_n,
                                  int32_t *ksplit, int32_t *waves);
 /* ... and the same matmul with a caller-chosen shape (auto-tuners, benchmarks). */

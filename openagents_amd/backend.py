@@ -276,9 +276,10 @@ class HipBackend:
         w0, n, W, Y, N = self._pack(ws, ys)
         _check(self.lib.psn_qmatvec_planned(self.module, self.stream, w0.qtype, scheme, n, W, x.handle, Y, N, w0.k, batch, C.byref(plan)))
 
-    def calibrate_read(self, src: DeviceBuffer, nbytes: int, blocks: int, threads: int = 256, lds_depth: int = 0, out: DeviceBuffer | None = None):
+    def calibrate_read(self, src: DeviceBuffer, nbytes: int, blocks: int, threads: int = 256, lds_depth: int = 0, out: DeviceBuffer | None = None,
+                       every_workgroup: bool = False):
         """A launch that only reads nbytes of src (see psn_calibrate_read)."""
-        _check(self.lib.psn_calibrate_read(self.module, self.stream, src.handle, nbytes, blocks, threads, lds_depth, self._h(out)))
+        _check(self.lib.psn_calibrate_read(self.module, self.stream, src.handle, nbytes, blocks, threads, lds_depth, int(every_workgroup), self._h(out)))
 
     # -- decode-step glue --------------------------------------------------------------------
     def add_rmsnorm(self, x: DeviceBuffer, delta, weight: DeviceBuffer, y: DeviceBuffer, n: int, eps: float = 1e-5):

@@ -30,7 +30,9 @@ CODE_OBJECTS = [
     ("psn_mv_q8_0", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q8_0"]),
     ("psn_mv_q4_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q4_K"]),
     ("psn_mv_q6_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q6_K"]),
-    ("psn_prefill", "psn_prefill.hip", []),
+    ("psn_pf_skinny", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=0"]),
+    *[(f"psn_pf_{fmt}_{fam}", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", f"-DPSN_BUILD_PF={num}", f"-DPSN_BUILD_PF_{fmt.upper()}"])
+      for fmt in ("q4_0", "q8_0") for num, fam in ((1, "ws"), (4, "base"))],
     ("psn_decode", "psn_decode.hip", []),
     ("psn_calib", "psn_calib.hip", []),
 ]

@@ -71,7 +71,7 @@ struct psn_calib_args {
     uint32_t *out;        /* one dword per wave (may be null) */
     int64_t bytes;
     int32_t depth;        /* psn_calib_read_lds: 1 KB LDS slots per wave */
-    int32_t pad;
+    int32_t every_wg;     /* 1: every workgroup reads the whole range; 0: the workgroups share it */
 };
 
 /* decode-step glue kernels (psn_decode.hip) */

@@ -13,8 +13,9 @@
 
 extern "C" __global__ void __launch_bounds__(1024) psn_calib_read(const psn_calib_args a) {
     const int lane = threadIdx.x & 63;
-    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    /* every_wg: each workgroup reads the whole range (the access pattern of an operand all workgroups share) */
+    const int64_t wave = a.every_wg ? (threadIdx.x >> 6) : (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = a.every_wg ? (blockDim.x >> 6) : (int64_t)gridDim.x * (blockDim.x >> 6);
     const int64_t slab = 64 * 16 * 4;                       /* 4 KB per wave and iteration */
     const int64_t nslabs = a.bytes / slab;
     uint4 acc = make_uint4(0, 0, 0, 0);
@@ -28,14 +29,14 @@ extern "C" __global__ void __launch_bounds__(1024) psn_calib_read(const psn_cali
     }
     u32 r = acc.x ^ acc.y ^ acc.z ^ acc.w;
     r ^= (u32)__shfl_xor((int)r, 32, 64);
-    if (lane == 0 && a.out) a.out[wave] = r;
+    if (lane == 0 && a.out) a.out[(int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)] = r;
 }
 
 extern "C" __global__ void __launch_bounds__(1024) psn_calib_read_lds(const psn_calib_args a) {
     extern __shared__ uint4 psn_smem[];
     const int lane = threadIdx.x & 63, wib = threadIdx.x >> 6;
-    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + wib;
-    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    const int64_t wave = a.every_wg ? wib : (int64_t)blockIdx.x * (blockDim.x >> 6) + wib;
+    const int64_t nwaves = a.every_wg ? (blockDim.x >> 6) : (int64_t)gridDim.x * (blockDim.x >> 6);
     const int depth = a.depth;                              /* 1 KB slots per wave */
     const int64_t slab = (int64_t)depth << 10;
     const int64_t nslabs = a.bytes / slab;
@@ -49,5 +50,5 @@ extern "C" __global__ void __launch_bounds__(1024) psn_calib_read_lds(const psn_
         r ^= reinterpret_cast<const u32 *>(buf)[lane];
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
-    if (lane == 0 && a.out) a.out[wave] = r;
+    if (lane == 0 && a.out) a.out[(int64_t)blockIdx.x * (blockDim.x >> 6) + wib] = r;
 }

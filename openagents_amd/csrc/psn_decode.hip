@@ -216,17 +216,21 @@ PSN_DEV void attn_partial_body(const psn_attn_args &a) {
          * LDS (see above) and the value row from the fresh projection, rounded to fp16 like a cached row;
          * wave 0 appends the value row to the cache */
         const int pos = a.n_ctx - 1;
-        if (split == (pos >> 6)) {                               /* uniform */
-            const int pl = pos & 63;
-            if (lane == pl) {
+        const bool own = split == (pos >> 6);                    /* uniform */
+        const float2 vn = *reinterpret_cast<const float2 *>(a.v_new + kvh * D + 2 * lane);
+        const f16 v0 = (f16)vn.x, v1 = (f16)vn.y;
+        const u32 vpacked = (u32)__builtin_bit_cast(unsigned short, v0) | ((u32)__builtin_bit_cast(unsigned short, v1) << 16);
+        /* rows behind the token's position were loaded from cache rows that nothing has written yet:
+         * they get weight 0, but 0 * (a stale Inf/NaN pattern) would still poison the sum.  The first
+         * row to replace sits in a vector register (64 = none, for the other splits), so that each row
+         * is one compare and one select with no scalar masks to hold. */
+        int pl_v = own ? (pos & 63) : 64;
+        asm volatile("" : "+v"(pl_v));
+        UNROLL for (int i = 0; i < 64; ++i) vreg[i] = i >= pl_v ? vpacked : vreg[i];
+        if (own) {
+            if (lane == (pos & 63)) {
                 UNROLL for (int c = 0; c < 16; ++c) kreg[c] = knew_row[c];
             }
-            const float2 vn = *reinterpret_cast<const float2 *>(a.v_new + kvh * D + 2 * lane);
-            const f16 v0 = (f16)vn.x, v1 = (f16)vn.y;
-            const u32 vpacked = (u32)__builtin_bit_cast(unsigned short, v0) | ((u32)__builtin_bit_cast(unsigned short, v1) << 16);
-            /* rows behind the token's position were loaded from cache rows that nothing has written yet:
-             * they get weight 0, but 0 * (a stale Inf/NaN pattern) would still poison the sum */
-            UNROLL for (int i = 0; i < 64; ++i) if (i >= pl) vreg[i] = vpacked;
             if (g == 0) reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos * a.n_kv_heads + kvh) * D)[lane] = vpacked;
         }
     }

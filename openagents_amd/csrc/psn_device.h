@@ -122,6 +122,63 @@ PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out
     s16 = group_sum_i<4>(s4);
 }
 
+/* ---- hand-scheduled memory access ------------------------------------------------------------
+ * Kernels that keep several direct-to-LDS loads in flight place every wait themselves: the compiler's
+ * wait insertion cannot tell ring buffers in dynamic LDS apart and would drain ALL outstanding loads
+ * before any LDS read.  LDS is therefore accessed through inline assembly the compiler does not model
+ * as memory traffic, and vmcnt / lgkmcnt waits are explicit (loads complete in issue order, so "at
+ * most n younger loads outstanding" identifies what has landed). */
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+
+/* wave-uniform n: wait until at most n vector-memory loads are outstanding */
+PSN_DEV void wait_vmcnt(int n) {
+#define PSN_W(k) case k: asm volatile("s_waitcnt vmcnt(" #k ")" ::: "memory"); break;
+    switch (n) {
+        PSN_W(1) PSN_W(2) PSN_W(3) PSN_W(4) PSN_W(5) PSN_W(6) PSN_W(7) PSN_W(8) PSN_W(9) PSN_W(10) PSN_W(11) PSN_W(12)
+        PSN_W(13) PSN_W(14) PSN_W(15) PSN_W(16) PSN_W(17) PSN_W(18) PSN_W(19) PSN_W(20) PSN_W(21) PSN_W(22) PSN_W(23)
+        PSN_W(24) PSN_W(25) PSN_W(26) PSN_W(27) PSN_W(28) PSN_W(29) PSN_W(30) PSN_W(31) PSN_W(32) PSN_W(33) PSN_W(34)
+        PSN_W(35) PSN_W(36) PSN_W(37) PSN_W(38) PSN_W(39) PSN_W(40) PSN_W(41) PSN_W(42) PSN_W(43) PSN_W(44) PSN_W(45)
+        PSN_W(46) PSN_W(47) PSN_W(48) PSN_W(49) PSN_W(50) PSN_W(51) PSN_W(52) PSN_W(53) PSN_W(54) PSN_W(55) PSN_W(56)
+        PSN_W(57) PSN_W(58) PSN_W(59) PSN_W(60) PSN_W(61) PSN_W(62) PSN_W(63)
+        default:
+            /* more than the 6-bit counter can hold: never more than 63 are outstanding, nothing to wait for */
+            if (n <= 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            break;
+    }
+#undef PSN_W
+}
+/* LDS and global accesses the compiler does not see as memory operations (no automatic waits) */
+template <int OFF> PSN_DEV u32x4 lds_read128(u32 addr) {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+PSN_DEV u32 lds_read32(u32 addr) {
+    u32 v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+PSN_DEV u32 lds_read_u16(u32 addr) {
+    u32 v;
+    asm volatile("ds_read_u16 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+    return v;
+}
+PSN_DEV void lds_write128(u32 addr, u32x4 v) { asm volatile("ds_write_b128 %0, %1" ::"v"(addr), "v"(v) : "memory"); }
+PSN_DEV void lds_write32(u32 addr, u32 v) { asm volatile("ds_write_b32 %0, %1" ::"v"(addr), "v"(v) : "memory"); }
+PSN_DEV void lds_write16(u32 addr, u32 v) { asm volatile("ds_write_b16 %0, %1" ::"v"(addr), "v"(v) : "memory"); }
+PSN_DEV u32x4 global_read128(const void *p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+/* the values written by the reads above may be used after this (volatile asm statements stay in order) */
+PSN_DEV void lds_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+template <int N> PSN_DEV void tie(u32x4 (&v)[N]) { _Pragma("unroll") for (int i = 0; i < N; ++i) asm volatile("" : "+v"(v[i])); }
+PSN_DEV void tie1(u32 &v) { asm volatile("" : "+v"(v)); }
+/* workgroup barrier that waits for this wave's LDS traffic only, not for loads still in flight */
+PSN_DEV void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+
 PSN_DEV void unpack4(const uint4 v, u32 *dst) { dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w; }
 
 #endif

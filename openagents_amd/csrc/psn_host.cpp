@@ -996,7 +996,7 @@ extern "C" int32_t psn_qmatvec_noalloc(psn_module *mod, psn_stream *s, int32_t q
 /* ------------------------------------------------------------------ calibration */
 
 extern "C" int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, int64_t bytes, int32_t blocks, int32_t threads,
-                                      int32_t lds_depth, psn_buf *out) {
+                                      int32_t lds_depth, int32_t every_workgroup, psn_buf *out) {
     if (!mod || !s || !src) return fail(PSN_E_INVALID_ARG, "psn_calibrate_read: null handle");
     if (s->ctx != mod->ctx || src->ctx != mod->ctx || (out && out->ctx != mod->ctx)) return fail(PSN_E_INVALID_ARG, "psn_calibrate_read: handles belong to different contexts");
     if (bytes <= 0 || (int64_t)src->bytes < bytes) return fail(PSN_E_INVALID_ARG, "psn_calibrate_read: %lld bytes asked of a buffer of %zu", (long long)bytes, src->bytes);
@@ -1013,7 +1013,7 @@ extern "C" int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_
     a.out = out ? (uint32_t *)out->p : nullptr;
     a.bytes = bytes;
     a.depth = lds_depth;
-    a.pad = 0;
+    a.every_wg = every_workgroup != 0;
     return launch(mod, s, lds_depth ? "psn_calib_read_lds" : "psn_calib_read", (unsigned)blocks, (unsigned)threads, (unsigned)lds, &a);
 }
 
@@ -1040,10 +1040,9 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
  * many workgroups of that tile one compute unit holds (LDS and registers) */
 static const double k_prefill_step_us[] = {0.87, 1.10, 1.50, 2.00, 2.00, 2.44};
 static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
-/* other variants worth choosing: {tile index, kernel family (8 = eight waves, -4 = interleaved four-wave
- * schedule, 16 = four multiplying + four staging waves), step cost, workgroups per compute unit} */
-static const struct { int tile; int waves; double step_us; int per_cu; } k_prefill_alt[] = {
-    {3, 8, 1.45, 1}, {5, 8, 2.38, 1}, {3, -4, 1.33, 1}, {1, -4, 0.85, 2}, {3, 16, 1.20, 1}, {2, 16, 0.76, 1}};
+/* the producer / consumer kernels (16 = four multiplying + four staging waves):
+ * {tile index, kernel family, step cost, workgroups per compute unit} */
+static const struct { int tile; int waves; double step_us; int per_cu; } k_prefill_alt[] = {{3, 16, 1.20, 1}, {2, 16, 0.76, 1}};
 
 extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
                                             int32_t *waves) {
@@ -1051,6 +1050,18 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
     *waves = 4;
     if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
     if (cus <= 0) cus = 256;
+    if (M <= 64) {
+        /* at most 64 rows: the weight-streaming kernel on 64 x 64 tiles; K is cut (atomic adds) only when
+         * the weight rows alone leave most compute units without a workgroup */
+        const int64_t nt = (N + 63) / 64, C = K / 256;
+        int sp = 1;
+        while (nt * sp * 2 <= cus && C / (sp * 2) >= 4 && (M * N) % 4 == 0) sp *= 2;
+        *tile_m = 64;
+        *tile_n = 64;
+        *ksplit = sp;
+        *waves = 64;
+        return PSN_OK;
+    }
     /* estimated time = waves of workgroups over the chip's slots x K steps per workgroup x step cost,
      * plus, when K is split, zeroing Y and the atomic adds of the partial sums */
     double best = 1e300;
@@ -1088,21 +1099,21 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
                                              int32_t waves) {
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
+    /* waves == 64 selects the skinny kernel (M <= 64, 64 x 64 tiles, deep LDS rings) */
+    const bool skinny = waves == 64;
+    if (skinny && (bm != 64 || bn != 64 || M > 64)) return fail(PSN_E_UNSUPPORTED, "prefill: the skinny kernel serves M <= 64 with a 64x64 tile");
     bool known = false;
     for (int i = 0; i < 6; ++i) known = known || (k_prefill_tiles[i][0] == bm && k_prefill_tiles[i][1] == bn);
     if (!known) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel with a %dx%d tile", bm, bn);
-    /* waves == -4 selects the four-wave kernel with the interleaved decode/MFMA schedule */
-    const bool has_il = (bm == 64 && bn == 128) || (bm == 128 && bn == 128) || (bm == 128 && bn == 256);
-    /* -5: four waves, X prefetched through registers */
     /* 16: eight waves split into four multiplying and four staging ones */
-    const bool has_ws = bm == 128 && (bn == 128 || bn == 256);
-    if (waves != 4 && !(waves == 8 && bm >= 128 && bn >= 128) && !(waves == -4 && has_il) && !(waves == -5 && bm >= 128 && bn >= 128) &&
-        !(waves == 16 && has_ws))
-        return fail(PSN_E_UNSUPPORTED, "prefill: no %d-wave kernel for a %dx%d tile", waves, bm, bn);
+    const bool has_ws = (bm == 64 && (bn == 64 || bn == 128)) || (bm == 128 && (bn == 128 || bn == 256));
+    if (!skinny && waves != 4 && !(waves == 16 && has_ws)) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel family %d for a %dx%d tile", waves, bm, bn);
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
-    /* the interleaved kernels carry their LDS as static arrays */
-    const int lds = (waves < 0 || waves == 16) ? 0 : 2 * (bm + bn) * 128;
+    /* the interleaved kernels carry their LDS as static arrays; the skinny kernel: rings of three X chunks
+     * (64 rows x 256 k fp16) and three raw weight chunks (64 rows), reused for the final 8 x 16 KB reduction */
+    const int skinny_rings = 3 * 32768 + 3 * 64 * (qtype == PSN_Q4_0 ? 144 : 272);
+    const int lds = skinny ? (skinny_rings > 8 * 16384 ? skinny_rings : 8 * 16384) : waves == 16 ? 0 : 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);
     if ((rc = bind(mod->ctx))) return rc;
     if (ksplit > 1) {
@@ -1123,10 +1134,14 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     a.ksplit = ksplit;
     a.row_bytes = psn_row_bytes(qtype, K);
     const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
-    const int64_t blocks = 8 * ((nt + 7) / 8) * mt * ksplit;      /* the kernel spreads N tiles over 8 XCDs */
     char name[96];
-    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 8 ? "_w8" : waves == -4 ? "_il" : waves == -5 ? "_rp" : waves == 16 ? "_ws" : "");
-    return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * ((waves == 8 || waves == 16) ? 8 : 4)), (unsigned)lds, &a);
+    if (skinny) {
+        snprintf(name, sizeof name, "psn_prefill_%s_skinny", fmt_name(qtype));
+        return launch(mod, s, name, (unsigned)(nt * ksplit), 512, (unsigned)lds, &a);
+    }
+    const int64_t blocks = 8 * ((nt + 7) / 8) * mt * ksplit;      /* the kernel spreads N tiles over 8 XCDs */
+    snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 16 ? "_ws" : "");
+    return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * (waves == 16 ? 8 : 4)), (unsigned)lds, &a);
 }
 
 extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
@@ -1136,7 +1151,6 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     if (rc) return rc;
     int32_t bm = 0, bn = 0, sp = 1, wv = 4;
     if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv))) return rc;
-    if (qtype == PSN_Q8_0 && wv == 8) wv = 4;     /* the eight-wave Q8_0 kernels spill registers (272-byte chunks) */
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }
 

@@ -22,10 +22,6 @@
 
 #define UNROLL _Pragma("unroll")
 
-#ifndef PSN_ABLATE
-#define PSN_ABLATE 0   /* development builds: 1 skips the weight decode, 2 the X loads, 4 the MFMAs of the K loop */
-#endif
-
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
 typedef float float16_t __attribute__((ext_vector_type(16)));
@@ -130,18 +126,18 @@ struct PfQ8_0 {
 /* 64 dequantized fp16 (blocks 2P and 2P+1 of the chunk) into one swizzled tile row */
 template <typename WF, int P>
 PSN_DEV void stage_w_row(const u32 (&w)[WF::DW], char *tile, int row) {
-    u32 o[32];
-    u32 (&o0)[16] = *reinterpret_cast<u32 (*)[16]>(&o[0]);
-    u32 (&o1)[16] = *reinterpret_cast<u32 (*)[16]>(&o[16]);
-    WF::template deq_block<2 * P>(w, o0);
-    WF::template deq_block<2 * P + 1>(w, o1);
-    UNROLL for (int c = 0; c < 8; ++c)
+    u32 o[16];
+    WF::template deq_block<2 * P>(w, o);
+    UNROLL for (int c = 0; c < 4; ++c)
         *reinterpret_cast<uint4 *>(tile + tile_off(row, c)) = make_uint4(o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]);
+    WF::template deq_block<2 * P + 1>(w, o);
+    UNROLL for (int c = 0; c < 4; ++c)
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 4 + c)) = make_uint4(o[4 * c], o[4 * c + 1], o[4 * c + 2], o[4 * c + 3]);
 }
 
 template <typename WF, int BM, int BN, int WM, int WN>
 PSN_DEV void prefill_body(const psn_prefill_args &a) {
-    static_assert(WM * WN == 4 || WM * WN == 8, "four or eight waves");
+    static_assert(WM * WN == 4, "four waves");
     static_assert(BN == 64 || BN == 128 || BN == 256, "BN");
     constexpr int NT = 64 * WM * WN;                        /* threads per workgroup */
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;     /* 32x32 MFMA tiles per wave */
@@ -179,7 +175,7 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
         UNROLL for (int i = 0; i < BM * 8 / NT; ++i) {
             const int s = i * NT + tid, row = s >> 3, chunk = (s & 7) ^ (row & 7);
             const uint16_t *src = a.X + (int64_t)min(m0 + row, M - 1) * K + k0 + chunk * 8;
-            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + (i * NT + wave * 64) * 16), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + (i * NT + __builtin_amdgcn_readfirstlane(wave) * 64) * 16), 16, 0, 0);
         }
     };
     auto compute = [&](const char *xt, const char *wt) {
@@ -243,11 +239,16 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
         UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = wnext[i];
     }
 
-    /* 32x32 accumulator: lane holds column (lane & 31); register r is row 8*(r/4) + 4*(lane/32) + r%4 */
+    /* 32x32 accumulator: lane holds column (lane & 31); register r is row 8*(r/4) + 4*(lane/32) + r%4.
+     * The wave's tile position is worked out again from the thread index (opaque to the compiler), so
+     * that nothing of it has to stay in a register through the K loop. */
+    int tid_out = threadIdx.x;
+    asm volatile("" : "+v"(tid_out));
+    const int wm_out = (tid_out >> 6) / WN, wn_out = (tid_out >> 6) % WN, lane_out = tid_out & 63;
     UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
+        const int col = n0 + wn_out * (BN / WN) + 32 * j + (lane_out & 31);
         UNROLL for (int r = 0; r < 16; ++r) {
-            const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            const int row = m0 + wm_out * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane_out >> 5) + (r & 3);
             if (row < M && col < N) {
                 if (S == 1) a.Y[(int64_t)row * N + col] = acc[i][j][r];
                 else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], acc[i][j][r]);
@@ -256,13 +257,8 @@ PSN_DEV void prefill_body(const psn_prefill_args &a) {
     }
 }
 
-/* ---- interleaved variant ------------------------------------------------------------------
- * Same tiles and LDS layout, but arranged so that one basic block holds a whole K step:
- *  - all 256 threads dequantize in every step (256/BN threads share a weight row, each turning
- *    64*BN/256 weights of it into fp16), so there is no divergent branch around the dequantization;
- *  - the operand fragments of k16 slice kk+1 are read while the MFMAs of slice kk are issued;
- *  - scheduling barriers ask the compiler to issue, per MFMA, a share of the dequantization VALU
- *    work and of the LDS traffic, so the matrix pipeline is fed while the vector ALUs decode. */
+/* ---- decode helpers of the producer / consumer variant: 256/BN threads share a weight row, each
+ *      turning 64*BN/256 weights of a K step into fp16 ---- */
 
 /* raw quants and fp16 scale bits of GGUF block B of a chunk */
 template <int B> PSN_DEV void raw_block(const u32 (&w)[36], u32 (&q)[8], u32 &dbits) {       /* Q4_0: q[0..3] used */
@@ -334,124 +330,6 @@ PSN_DEV void stage_part(const u32 (&w)[WF::DW], char *tile, int row, int part) {
     }
 }
 
-/* X tiles: four LDS stages filled three K steps ahead by direct-to-LDS loads; W tiles: two stages
- * filled one step ahead from registers.  Every stage is its own __shared__ array so that alias
- * analysis can tell the compiler that a W write or a fragment read never touches the stage a
- * pending X load is landing in -- otherwise it waits for all outstanding loads in mid-step. */
-template <typename WF, int BM, int BN, int WM, int WN>
-PSN_DEV void prefill_body_il(const psn_prefill_args &a) {
-    static_assert(WM * WN == 4, "four waves");
-    constexpr int NT = 256;
-    constexpr int P = NT / BN;                              /* threads per weight row */
-    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int NX = BM * 8 / NT;                         /* direct-to-LDS instructions per X stage */
-    constexpr int NW = WF::DW / 4;                          /* global loads per weight chunk */
-    __shared__ uint4 xs0[BM * 8], xs1[BM * 8], xs2[BM * 8], xs3[BM * 8];
-    __shared__ uint4 ws0[BN * 8], ws1[BN * 8];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
-    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
-    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
-    const int S = a.ksplit;
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int per_xcd_n = (nt + 7) >> 3;
-    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
-    const int tile_n = xcd + 8 * tn_local;
-    if (tn_local >= per_xcd_n || tile_n >= nt) return;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int per_split = (C + S - 1) / S;
-    const int c_begin = split * per_split, c_end = min(c_begin + per_split, C);
-    if (c_begin >= c_end) return;
-    const int k_last = c_end * 256 - 64;                    /* last K step of this range; later prefetches re-read it */
-
-    float16_t acc[TM][TN];
-    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    const int wrow = tid % BN, part = tid / BN;
-    const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
-    u32 w[WF::DW], wnext[WF::DW];
-
-    auto stage_x = [&](uint4 *tile, int k0) {
-        k0 = min(k0, k_last);
-        UNROLL for (int i = 0; i < NX; ++i) {
-            const int s = i * NT + tid, row = s >> 3, chunk = (s & 7) ^ (row & 7);
-            const uint16_t *src = a.X + (int64_t)min(m0 + row, M - 1) * K + k0 + chunk * 8;
-            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(tile + i * NT + wave * 64), 16, 0, 0);
-        }
-    };
-    auto load_frags = [&](const uint4 *xt, const uint4 *wt, int kk, half8_t (&af)[TM], half8_t (&bf)[TN]) {
-        const int chunk = 2 * kk + (lane >> 5);
-        UNROLL for (int i = 0; i < TM; ++i)
-            af[i] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(xt) + tile_off(wm * (BM / WM) + 32 * i + (lane & 31), chunk));
-        UNROLL for (int j = 0; j < TN; ++j)
-            bf[j] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(wt) + tile_off(wn * (BN / WN) + 32 * j + (lane & 31), chunk));
-    };
-    auto mfmas = [&](const half8_t (&af)[TM], const half8_t (&bf)[TN]) {
-        UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    };
-
-    /* prologue: weight chunk, X stages for the first three steps, W stage for the first */
-    WF::load(wbase + (int64_t)c_begin * WF::BYTES, w);
-    const int k_begin = c_begin * 256;
-    stage_x(xs0, k_begin);
-    stage_x(xs1, k_begin + 64);
-    stage_x(xs2, k_begin + 128);
-    stage_part<WF, 0, P>(w, reinterpret_cast<char *>(ws0), wrow, part);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-
-    /* one K step: X stage `xc` and W stage `wc` are current; X for step +3 goes to `xp`, W for step +1
-     * to `wq` (from `wsrc`, blocks 2*NSUB and 2*NSUB+1).  KEEP = loads that may stay in flight past the
-     * barrier: the X stages of steps +2 and +3, plus the next weight chunk when it was requested after
-     * the X stage of step +1. */
-#define PSN_PF_STEP(SUB, NSUB, wsrc, xc, xp, wc, wq, KEEP)                                            \
-    {                                                                                                 \
-        if (!(PSN_ABLATE & 2)) stage_x(xp, (c * 4 + SUB + 3) * 64);                                   \
-        half8_t af0[TM], bf0[TN], af1[TM], bf1[TN];                                                   \
-        if (!(PSN_ABLATE & 4)) {                                                                      \
-            load_frags(xc, wc, 0, af0, bf0);                                                          \
-            load_frags(xc, wc, 1, af1, bf1);                                                          \
-            mfmas(af0, bf0);                                                                          \
-            load_frags(xc, wc, 2, af0, bf0);                                                          \
-            mfmas(af1, bf1);                                                                          \
-            load_frags(xc, wc, 3, af1, bf1);                                                          \
-            mfmas(af0, bf0);                                                                          \
-        }                                                                                             \
-        if (!(PSN_ABLATE & 1)) stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part); \
-        if (!(PSN_ABLATE & 4)) mfmas(af1, bf1);                                                       \
-        UNROLL for (int i_ = 0; i_ < 4 * TM * TN; ++i_) {                                             \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                        \
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                        \
-            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                        \
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                        \
-        }                                                                                             \
-        /* raw barrier: __syncthreads() would first drain every outstanding load, prefetches included */ \
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(KEEP) : "memory");            \
-    }
-
-    for (int c = c_begin; c < c_end; ++c) {
-        WF::load(wbase + (int64_t)min(c + 1, C - 1) * WF::BYTES, wnext);
-        PSN_PF_STEP(0, 1, w, xs0, xs3, ws0, ws1, 2 * NX + NW)
-        PSN_PF_STEP(1, 2, w, xs1, xs0, ws1, ws0, 2 * NX + NW)
-        PSN_PF_STEP(2, 3, w, xs2, xs1, ws0, ws1, 2 * NX)
-        PSN_PF_STEP(3, 0, wnext, xs3, xs2, ws1, ws0, 2 * NX)
-        UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = wnext[i];
-    }
-#undef PSN_PF_STEP
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-
-    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
-        UNROLL for (int r = 0; r < 16; ++r) {
-            const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (row < M && col < N) {
-                if (S == 1) a.Y[(int64_t)row * N + col] = acc[i][j][r];
-                else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], acc[i][j][r]);
-            }
-        }
-    }
-}
-
 /* ---- producer / consumer variant ----------------------------------------------------------------
  * Measured on MI355X: a wave's own VALU work does not overlap its MFMAs (decode-only and MFMA-only
  * runs of the kernels above add up to the full run), so the weight decode has to come from OTHER
@@ -487,7 +365,8 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
     const int k_last = c_end * 256 - 64;
 
     if (producer) {
-        const int ptid = tid - 256, pwave = wave - 4;
+        const int ptid = tid - 256;
+        const int pwave = __builtin_amdgcn_readfirstlane(wave) - 4;   /* scalar: it addresses the LDS side of the DMA */
         const int wrow = ptid % BN, part = ptid / BN;
         const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
         u32 w[WF::DW], wnext[WF::DW];
@@ -508,9 +387,9 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #define PSN_WS_PRODUCE(SUB, NSUB, wsrc, xp, wq, KEEP)                                                 \
         {                                                                                             \
-            if (!(PSN_ABLATE & 2)) stage_x(xp, (c * 4 + SUB + 3) * 64);                               \
-            if (!(PSN_ABLATE & 1)) stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part); \
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"((PSN_ABLATE & 2) ? 0 : KEEP) : "memory"); \
+            stage_x(xp, (c * 4 + SUB + 3) * 64);                                               \
+            stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part);                  \
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(KEEP) : "memory");            \
         }
         for (int c = c_begin; c < c_end; ++c) {
             WF::load(wbase + (int64_t)min(c + 1, C - 1) * WF::BYTES, wnext);
@@ -544,16 +423,14 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
 #define PSN_WS_CONSUME(xc, wc)                                                                        \
     {                                                                                                 \
         half8_t af0[TM], bf0[TN], af1[TM], bf1[TN];                                                   \
-        if (!(PSN_ABLATE & 4)) {                                                                      \
-            load_frags(xc, wc, 0, af0, bf0);                                                          \
-            load_frags(xc, wc, 1, af1, bf1);                                                          \
-            mfmas(af0, bf0);                                                                          \
-            load_frags(xc, wc, 2, af0, bf0);                                                          \
-            mfmas(af1, bf1);                                                                          \
-            load_frags(xc, wc, 3, af1, bf1);                                                          \
-            mfmas(af0, bf0);                                                                          \
-            mfmas(af1, bf1);                                                                          \
-        }                                                                                             \
+        load_frags(xc, wc, 0, af0, bf0);                                                              \
+        load_frags(xc, wc, 1, af1, bf1);                                                              \
+        mfmas(af0, bf0);                                                                              \
+        load_frags(xc, wc, 2, af0, bf0);                                                              \
+        mfmas(af1, bf1);                                                                              \
+        load_frags(xc, wc, 3, af1, bf1);                                                              \
+        mfmas(af0, bf0);                                                                              \
+        mfmas(af1, bf1);                                                                              \
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");                               \
     }
     for (int c = c_begin; c < c_end; ++c) {
@@ -575,179 +452,250 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
     }
 }
 
-/* ---- register-prefetch variant ----------------------------------------------------------------
- * As above, but the X tile travels global -> registers -> LDS: the loads of step s+3 are issued while
- * step s multiplies (two register sets, each load has two full steps to land), and the tile of step
- * s+1 is written to LDS from registers next to the decoded weights.  Ordinary register loads let the
- * compiler count outstanding loads exactly, so nothing drains the queue in mid-loop; two LDS stages
- * per operand suffice. */
-template <typename WF, int BM, int BN, int WM, int WN>
-PSN_DEV void prefill_body_rp(const psn_prefill_args &a) {
-    static_assert(WM * WN == 4, "four waves");
-    constexpr int NT = 256;
-    constexpr int P = NT / BN;
-    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
-    constexpr int NX = BM * 8 / NT;                         /* 16-byte words of X per thread and step */
-    __shared__ uint4 xs0[BM * 8], xs1[BM * 8];
-    __shared__ uint4 ws0[BN * 8], ws1[BN * 8];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave / WN, wn = wave % WN;
-    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
-    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
-    const int S = a.ksplit;
-    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int per_xcd_n = (nt + 7) >> 3;
-    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
-    const int tile_n = xcd + 8 * tn_local;
-    if (tn_local >= per_xcd_n || tile_n >= nt) return;
-    const int m0 = tile_m * BM, n0 = tile_n * BN;
+/* ---- skinny variant (M <= 64) ---------------------------------------------------------------------
+ * With at most 64 activation rows the matmul is a weight stream (HBM-bound), and a workgroup's 64-wide K
+ * step carries so little arithmetic (a 64 x 64 tile: 16 MFMAs) that the step time of the kernels above
+ * is their per-step chain of barrier, decode and memory latency.  This kernel has no per-step
+ * synchronization at all:
+ *   - everything arrives by direct-to-LDS loads into rings of dynamic LDS, a whole 256-wide chunk of K
+ *     at a time: X (64 rows x 256 k, four swizzled 64-k tiles) and the raw GGUF bytes of 64 weight rows
+ *     exactly as they sit in memory; chunks are requested XR-1 / RS-1 iterations ahead;
+ *   - eight waves multiply; a chunk is 16 k16-slices and wave w owns two of them in two of the four
+ *     steps, for the whole 64 x 64 tile.  A wave decodes the eight weights per lane its own MFMA operand
+ *     needs straight from the raw ring (8 bytes + the fp16 scale), so there is no fp16 weight tile, no
+ *     decode stage and no producer wave; two waves per SIMD let one wave's decode run under the
+ *     other's MFMAs;
+ *   - one workgroup barrier per CHUNK (every wave waits for its own share of the next chunk's loads
+ *     first -- loads complete in issue order, so a constant "at most n outstanding" identifies them);
+ *   - the eight partial tiles are summed through LDS at the end, in a fixed order.
+ * Loads past the end of the K range re-read its last chunk into ring slots nothing reads any more, so
+ * every iteration issues the same number of loads and the outstanding-load count is a constant. */
+template <typename WF, bool WAVE0>
+PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, int n0, int c_begin, int nq, int rot,
+                                 u32 xs_base, u32 raw_base, __attribute__((address_space(3))) char *lds_ptr, u32 lds0, float16_t (&acc)[2][2]) {
+    constexpr int BN = 64, XR = 3, RS = 3;
+    constexpr int XBYTES = 4 * 64 * 128, RBYTES = BN * WF::BYTES;
+    constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9 or 17 */
+    constexpr int CX = 4;                                   /* X loads per wave and chunk (32 KB over 8 waves) */
+    constexpr int CR = (RINSTR + (WAVE0 ? 7 : 0)) / 8;      /* raw loads per wave and chunk: wave 0 takes the odd one */
+    const int M = a.M, N = a.N, K = a.K;
+    auto chunk_of = [&](int q) { const int r = min(q, nq - 1) + rot; return c_begin + (r >= nq ? r - nq : r); };
+    auto issue_raw = [&](int q) {
+        const int c = chunk_of(q);
+        __attribute__((address_space(3))) char *dst = lds_ptr + (raw_base - lds0) + (q % RS) * RBYTES;
+        UNROLL for (int u = 0; u < CR; ++u) {
+            const int i = wave + 8 * u;                     /* instruction index; with WAVE0 the last one is index 8 or 16 */
+            const int word = i * 64 + lane, row = word / (WF::BYTES / 16), wd = word % (WF::BYTES / 16);
+            const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + (int64_t)c * WF::BYTES + wd * 16;
+            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
+        }
+    };
+    auto issue_x = [&](int q) {
+        const int k0 = chunk_of(q) * 256;
+        __attribute__((address_space(3))) char *dst = lds_ptr + (xs_base - lds0) + (q % XR) * XBYTES;
+        UNROLL for (int u = 0; u < CX; ++u) {
+            /* 16-byte word s_ of the stage in LDS order: step s_/512, row (s_%512)/8, position s_%8 holds chunk pos^(row&7) */
+            const int i = wave * CX + u, s_ = i * 64 + lane, step = s_ >> 9, row = (s_ >> 3) & 63, chunk = (s_ & 7) ^ (row & 7);
+            const uint16_t *src = a.X + (int64_t)min(row, M - 1) * K + k0 + step * 64 + chunk * 8;
+            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
+        }
+    };
+    const int kk = wave & 3, sp = wave >> 2, h = lane >> 5;  /* this wave: k16 slice kk of steps sp and sp + 2 */
+    u32 xoff[2], roff[2];
+    UNROLL for (int i = 0; i < 2; ++i) {
+        xoff[i] = (u32)tile_off(32 * i + (lane & 31), 2 * kk + h);
+        /* GGUF block (2*step + kk/2) of the row; the 8 weights are plane kk%2, bytes 8h.. (Q4_0: nibble plane
+         * of bytes 8h..8h+7; Q8_0: the 8 int8 at 16*(kk%2) + 8h) */
+        roff[i] = (u32)((32 * i + (lane & 31)) * WF::BYTES + (kk >> 1) * (WF::BYTES / 8));
+    }
+    constexpr int BB = WF::BYTES / 8;                       /* bytes of a GGUF block: 18 or 34 */
+    const u32 qoff = WF::DW == 36 ? 2u + 8u * (u32)h : 2u + 16u * (u32)(kk & 1) + 8u * (u32)h;
+
+    for (int q = 0; q < RS - 1; ++q) issue_raw(q);
+    for (int q = 0; q < XR - 1; ++q) issue_x(q);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((XR - 2) * CX) : "memory");   /* my share of chunk 0 has landed */
+    lds_barrier();
+    for (int q = 0; q < nq; ++q) {
+        issue_raw(q + RS - 1);
+        issue_x(q + XR - 1);
+        const u32 xst = xs_base + (u32)((q % XR) * XBYTES), rst = raw_base + (u32)((q % RS) * RBYTES);
+        UNROLL for (int s2 = 0; s2 < 2; ++s2) {
+            const int step = sp + 2 * s2;
+            u32x4 xf[2];
+            u32 wq[2][2], wd[2];
+            UNROLL for (int i = 0; i < 2; ++i) xf[i] = lds_read128<0>(xst + (u32)(step * 8192) + xoff[i]);
+            /* GGUF blocks start on even bytes, not on dwords, and LDS reads that straddle dwords are very slow:
+             * read the aligned dwords around the eight quant bytes and shift them into place.  Block index
+             * 2*step + kk/2 is even or odd for the whole wave: an even block starts on a dword (scale in the
+             * low half, quants shifted by two bytes), an odd one two bytes later (scale in the high half of the
+             * dword before, quants aligned). */
+            u32 raw[2][3];
+            UNROLL for (int j = 0; j < 2; ++j) {
+                const u32 baddr = rst + roff[j] + (u32)(2 * step * BB);      /* block start */
+                if ((kk & 2) == 0) {
+                    wd[j] = lds_read32(baddr);                               /* scale | first two quant bytes */
+                    raw[j][0] = lds_read32(baddr + qoff - 2u);
+                    raw[j][1] = lds_read32(baddr + qoff + 2u);
+                    raw[j][2] = lds_read32(baddr + qoff + 6u);
+                } else {
+                    wd[j] = lds_read32(baddr - 2u);                          /* last two bytes of the block before | scale */
+                    raw[j][0] = lds_read32(baddr + qoff);
+                    raw[j][1] = lds_read32(baddr + qoff + 4u);
+                    raw[j][2] = 0;
+                }
+            }
+            lds_wait();
+            tie(xf);
+            UNROLL for (int j = 0; j < 2; ++j) {
+                tie1(wd[j]); tie1(raw[j][0]); tie1(raw[j][1]); tie1(raw[j][2]);
+                if ((kk & 2) == 0) {
+                    wq[j][0] = align2(raw[j][1], raw[j][0]);
+                    wq[j][1] = align2(raw[j][2], raw[j][1]);
+                    wd[j] &= 0xffffu;
+                } else {
+                    wq[j][0] = raw[j][0];
+                    wq[j][1] = raw[j][1];
+                    wd[j] >>= 16;
+                }
+            }
+            u32x4 wf[2];
+            UNROLL for (int j = 0; j < 2; ++j) {
+                const half2_t d2 = bits_h2(wd[j] | (wd[j] << 16));
+                u32 o[4];
+                if constexpr (WF::DW == 36) {
+                    const int sh = 4 * (kk & 1);
+                    bytes_to_h4(wq[j][0] >> sh, 0x640f640fu, bits_h2(0x64086408u), d2, o[0], o[1]);
+                    bytes_to_h4(wq[j][1] >> sh, 0x640f640fu, bits_h2(0x64086408u), d2, o[2], o[3]);
+                } else {
+                    bytes_to_h4(wq[j][0] ^ 0x80808080u, 0x64ff64ffu, bits_h2(0x64806480u), d2, o[0], o[1]);
+                    bytes_to_h4(wq[j][1] ^ 0x80808080u, 0x64ff64ffu, bits_h2(0x64806480u), d2, o[2], o[3]);
+                }
+                wf[j] = (u32x4){o[0], o[1], o[2], o[3]};
+            }
+            UNROLL for (int i = 0; i < 2; ++i) UNROLL for (int j = 0; j < 2; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, xf[i]), __builtin_bit_cast(half8_t, wf[j]), acc[i][j], 0, 0, 0);
+        }
+        /* my share of chunk q+1: everything but this iteration's own loads */
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((XR - 2) * (CX + CR)) : "memory");
+        lds_barrier();
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        /* nothing lands in the rings any more ... */
+    lds_barrier();                                          /* ... for any wave: they can hold the partial tiles */
+}
+
+template <typename WF>
+PSN_DEV void prefill_skinny_body(const psn_prefill_args &a) {
+    constexpr int BN = 64, XR = 3;
+    constexpr int XBYTES = 4 * 64 * 128;
+    extern __shared__ uint4 psn_smem[];
+    typedef __attribute__((address_space(3))) char lds_char;
+    lds_char *const lds_ptr = (lds_char *)psn_smem;
+    const u32 lds0 = (u32)(uintptr_t)lds_ptr;
+    const u32 xs_base = lds0, raw_base = xs_base + XR * XBYTES;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = a.M, N = a.N, C = a.K >> 8;
+    const int nt = (N + BN - 1) / BN, S = a.ksplit;
+    const int tile_n = blockIdx.x % nt, split = blockIdx.x / nt;
     const int per_split = (C + S - 1) / S;
     const int c_begin = split * per_split, c_end = min(c_begin + per_split, C);
-    if (c_begin >= c_end) return;
-    const int k_last = c_end * 256 - 64;
+    if (c_begin >= c_end) return;                           /* whole workgroup leaves together */
+    const int n0 = tile_n * BN, nq = c_end - c_begin;
+    /* Every workgroup walks the same X, so workgroups that started together would ask the same cache
+     * lines of the same L2 channel at the same moment: each one starts its (cyclic) walk over the K
+     * range at a different chunk.  The summation order of an output element depends only on its tile. */
+    const int rot = (int)((blockIdx.x * 5u) % (unsigned)nq);
 
-    float16_t acc[TM][TN];
-    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    const int wrow = tid % BN, part = tid / BN;
-    const uint8_t *wbase = a.W + (int64_t)min(n0 + wrow, N - 1) * a.row_bytes;
-    u32 w[WF::DW], wnext[WF::DW];
+    float16_t acc[2][2];
+    UNROLL for (int i = 0; i < 2; ++i) UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    if (wave == 0) prefill_skinny_loop<WF, true>(a, wave, lane, n0, c_begin, nq, rot, xs_base, raw_base, lds_ptr, lds0, acc);
+    else prefill_skinny_loop<WF, false>(a, wave, lane, n0, c_begin, nq, rot, xs_base, raw_base, lds_ptr, lds0, acc);
 
-    /* this thread's NX words of an X tile: word s = i*NT + tid -> row s/8, chunk (s%8)^(row&7) lands at s */
-    const uint16_t *xsrc[NX];
-    UNROLL for (int i = 0; i < NX; ++i) {
-        const int s_ = i * NT + tid, row = s_ >> 3, chunk = (s_ & 7) ^ (row & 7);
-        xsrc[i] = a.X + (int64_t)min(m0 + row, M - 1) * K + chunk * 8;
+    /* partial tiles of the eight waves -> LDS (16 KB each, lane-contiguous); then wave w sums registers
+     * 8*(w/4) .. +8 of tile w%4 over the eight waves, always in the order 0 .. 7 */
+    {
+        const u32 base = lds0 + (u32)(wave * 16384 + lane * 4);
+        UNROLL for (int i = 0; i < 2; ++i) UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int r = 0; r < 16; ++r)
+            lds_write32(base + (u32)(((i * 2 + j) * 16 + r) * 256), __float_as_uint(acc[i][j][r]));
     }
-    auto load_x = [&](uint4 (&r)[NX], int k0) {
-        k0 = min(k0, k_last);
-        UNROLL for (int i = 0; i < NX; ++i) r[i] = *reinterpret_cast<const uint4 *>(xsrc[i] + k0);
-    };
-    auto store_x = [&](uint4 *tile, const uint4 (&r)[NX]) {
-        UNROLL for (int i = 0; i < NX; ++i) tile[i * NT + tid] = r[i];
-    };
-    auto load_frags = [&](const uint4 *xt, const uint4 *wt, int kk, half8_t (&af)[TM], half8_t (&bf)[TN]) {
-        const int chunk = 2 * kk + (lane >> 5);
-        UNROLL for (int i = 0; i < TM; ++i)
-            af[i] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(xt) + tile_off(wm * (BM / WM) + 32 * i + (lane & 31), chunk));
-        UNROLL for (int j = 0; j < TN; ++j)
-            bf[j] = *reinterpret_cast<const half8_t *>(reinterpret_cast<const char *>(wt) + tile_off(wn * (BN / WN) + 32 * j + (lane & 31), chunk));
-    };
-    auto mfmas = [&](const half8_t (&af)[TM], const half8_t (&bf)[TN]) {
-        UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
-    };
-
-    /* prologue: step 0 into LDS, steps 1 and 2 into the two register sets */
-    uint4 xa[NX], xb[NX];
-    const int k_begin = c_begin * 256;
-    WF::load(wbase + (int64_t)c_begin * WF::BYTES, w);
-    load_x(xa, k_begin);
-    store_x(xs0, xa);
-    load_x(xb, k_begin + 64);                               /* X(1) */
-    load_x(xa, k_begin + 128);                              /* X(2) */
-    stage_part<WF, 0, P>(w, reinterpret_cast<char *>(ws0), wrow, part);
-    __syncthreads();
-
-    /* step SUB of chunk c: multiply from (xc, wc); X(step+1) goes from `xr` to LDS stage xq and `xr` is
-     * refilled with X(step+3); W(step+1) is decoded from `wsrc` (blocks 2*NSUB, 2*NSUB+1) into wq */
-#define PSN_RP_STEP(SUB, NSUB, wsrc, xc, xq, wc, wq, xr)                                               \
-    {                                                                                                 \
-        half8_t af0[TM], bf0[TN], af1[TM], bf1[TN];                                                   \
-        load_frags(xc, wc, 0, af0, bf0);                                                              \
-        load_frags(xc, wc, 1, af1, bf1);                                                              \
-        store_x(xq, xr);                                                                              \
-        load_x(xr, (c * 4 + SUB + 3) * 64);                                                           \
-        mfmas(af0, bf0);                                                                              \
-        load_frags(xc, wc, 2, af0, bf0);                                                              \
-        mfmas(af1, bf1);                                                                              \
-        load_frags(xc, wc, 3, af1, bf1);                                                              \
-        mfmas(af0, bf0);                                                                              \
-        stage_part<WF, NSUB, P>(wsrc, reinterpret_cast<char *>(wq), wrow, part);                      \
-        mfmas(af1, bf1);                                                                              \
-        UNROLL for (int i_ = 0; i_ < 4 * TM * TN; ++i_) {                                             \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                        \
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                                        \
-            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);                                        \
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);                                        \
-        }                                                                                             \
-        __builtin_amdgcn_s_waitcnt(0xC07F);                 /* lgkmcnt(0): this wave's LDS writes are done */ \
-        __builtin_amdgcn_s_barrier();                                                                 \
-    }
-
-    for (int c = c_begin; c < c_end; ++c) {
-        WF::load(wbase + (int64_t)min(c + 1, C - 1) * WF::BYTES, wnext);
-        PSN_RP_STEP(0, 1, w, xs0, xs1, ws0, ws1, xb)
-        PSN_RP_STEP(1, 2, w, xs1, xs0, ws1, ws0, xa)
-        PSN_RP_STEP(2, 3, w, xs0, xs1, ws0, ws1, xb)
-        PSN_RP_STEP(3, 0, wnext, xs1, xs0, ws1, ws0, xa)
-        UNROLL for (int i = 0; i < WF::DW; ++i) w[i] = wnext[i];
-    }
-#undef PSN_RP_STEP
-
-    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wn * (BN / WN) + 32 * j + (lane & 31);
-        UNROLL for (int r = 0; r < 16; ++r) {
-            const int row = m0 + wm * (BM / WM) + 32 * i + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+    lds_barrier();
+    {
+        const int t = wave & 3, i = t >> 1, j = t & 1, r0 = 8 * (wave >> 2);
+        u32 v[8][8];
+        UNROLL for (int w = 0; w < 8; ++w) UNROLL for (int r = 0; r < 8; ++r)
+            v[w][r] = lds_read32(lds0 + (u32)(w * 16384 + (t * 16 + r0 + r) * 256 + lane * 4));
+        lds_wait();
+        UNROLL for (int w = 0; w < 8; ++w) UNROLL for (int r = 0; r < 8; ++r) tie1(v[w][r]);
+        const int col = n0 + 32 * j + (lane & 31);
+        UNROLL for (int r = 0; r < 8; ++r) {
+            float sum = __uint_as_float(v[0][r]);
+            UNROLL for (int w = 1; w < 8; ++w) sum += __uint_as_float(v[w][r]);
+            const int rr = r0 + r, row = 32 * i + 8 * (rr >> 2) + 4 * (lane >> 5) + (rr & 3);
             if (row < M && col < N) {
-                if (S == 1) a.Y[(int64_t)row * N + col] = acc[i][j][r];
-                else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], acc[i][j][r]);
+                if (S == 1) a.Y[(int64_t)row * N + col] = sum;
+                else unsafeAtomicAdd(&a.Y[(int64_t)row * N + col], sum);
             }
         }
     }
 }
 
-/* zero fill with plain vector stores (graph-safe stand-in for a memset node) */
-extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_args a) {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    uint4 *p = reinterpret_cast<uint4 *>(a.p);
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
-}
+#define PSN_PREFILL_KERNEL_SKINNY(fmt, WF)                                                                   \
+    extern "C" __global__ void __launch_bounds__(512) psn_prefill_##fmt##_skinny(const psn_prefill_args a) { \
+        prefill_skinny_body<WF>(a);                                                                          \
+    }
 
 #define PSN_PREFILL_KERNEL(fmt, WF, BM, BN, WM, WN)                                                          \
     extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_m##BM##_n##BN(const psn_prefill_args a) { \
         prefill_body<WF, BM, BN, WM, WN>(a);                                                                 \
     }
-/* eight-wave variants (512 threads, two waves per SIMD: one can multiply while the other stages) */
-#define PSN_PREFILL_KERNEL8(fmt, WF, BM, BN, WM, WN)                                                         \
-    extern "C" __global__ void __launch_bounds__(512) psn_prefill_##fmt##_m##BM##_n##BN##_w8(const psn_prefill_args a) { \
-        prefill_body<WF, BM, BN, WM, WN>(a);                                                                 \
-    }
 
-#define PSN_PREFILL_KERNEL_IL(fmt, WF, BM, BN, WM, WN)                                                       \
-    extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_m##BM##_n##BN##_il(const psn_prefill_args a) { \
-        prefill_body_il<WF, BM, BN, WM, WN>(a);                                                              \
-    }
 
 #define PSN_PREFILL_KERNEL_WS(fmt, WF, BM, BN)                                                               \
     extern "C" __global__ void __launch_bounds__(512) psn_prefill_##fmt##_m##BM##_n##BN##_ws(const psn_prefill_args a) { \
         prefill_body_ws<WF, BM, BN>(a);                                                                      \
     }
 
-#define PSN_PREFILL_KERNEL_RP(fmt, WF, BM, BN, WM, WN)                                                       \
-    extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_m##BM##_n##BN##_rp(const psn_prefill_args a) { \
-        prefill_body_rp<WF, BM, BN, WM, WN>(a);                                                              \
-    }
 
-#define PSN_PREFILL_ALL(fmt, WF)               \
+#define PSN_PREFILL_FAMILY_WS(fmt, WF)           \
+    PSN_PREFILL_KERNEL_WS(fmt, WF, 64, 64)       \
+    PSN_PREFILL_KERNEL_WS(fmt, WF, 64, 128)      \
     PSN_PREFILL_KERNEL_WS(fmt, WF, 128, 128)     \
-    PSN_PREFILL_KERNEL_WS(fmt, WF, 128, 256)     \
-    PSN_PREFILL_KERNEL_RP(fmt, WF, 128, 128, 2, 2) \
-    PSN_PREFILL_KERNEL_RP(fmt, WF, 128, 256, 2, 2) \
-    PSN_PREFILL_KERNEL_RP(fmt, WF, 256, 128, 2, 2) \
-    PSN_PREFILL_KERNEL_RP(fmt, WF, 256, 256, 2, 2) \
-    PSN_PREFILL_KERNEL_IL(fmt, WF, 64, 128, 2, 2)  \
-    PSN_PREFILL_KERNEL_IL(fmt, WF, 128, 128, 2, 2) \
-    PSN_PREFILL_KERNEL_IL(fmt, WF, 128, 256, 2, 2) \
+    PSN_PREFILL_KERNEL_WS(fmt, WF, 128, 256)
+#define PSN_PREFILL_FAMILY_BASE(fmt, WF)         \
     PSN_PREFILL_KERNEL(fmt, WF, 64, 64, 2, 2)    \
     PSN_PREFILL_KERNEL(fmt, WF, 64, 128, 2, 2)   \
     PSN_PREFILL_KERNEL(fmt, WF, 128, 128, 2, 2)  \
     PSN_PREFILL_KERNEL(fmt, WF, 128, 256, 2, 2)  \
     PSN_PREFILL_KERNEL(fmt, WF, 256, 128, 2, 2)  \
-    PSN_PREFILL_KERNEL(fmt, WF, 256, 256, 2, 2)  \
-    PSN_PREFILL_KERNEL8(fmt, WF, 128, 128, 2, 4) \
-    PSN_PREFILL_KERNEL8(fmt, WF, 256, 128, 4, 2) \
-    PSN_PREFILL_KERNEL8(fmt, WF, 128, 256, 2, 4) \
-    PSN_PREFILL_KERNEL8(fmt, WF, 256, 256, 2, 4)
+    PSN_PREFILL_KERNEL(fmt, WF, 256, 256, 2, 2)
 
-PSN_PREFILL_ALL(q4_0, PfQ4_0)
-PSN_PREFILL_ALL(q8_0, PfQ8_0)
+/* The build compiles this file once per (format, kernel family) -- -DPSN_BUILD_ONLY -DPSN_BUILD_PF=<n>
+ * -DPSN_BUILD_PF_Q4_0 or _Q8_0 -- so that the code objects build in parallel; without PSN_BUILD_ONLY
+ * everything lands in one.  Family numbers: 0 skinny + fill, 1 ws (producer / consumer), 4 base (four waves). */
+
+#if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 0
+/* zero fill with plain vector stores (graph-safe stand-in for a memset node) */
+extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_args a) {
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    uint4 *p = reinterpret_cast<uint4 *>(a.p);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n16; i += stride) p[i] = make_uint4(0, 0, 0, 0);
+}
+PSN_PREFILL_KERNEL_SKINNY(q4_0, PfQ4_0)
+PSN_PREFILL_KERNEL_SKINNY(q8_0, PfQ8_0)
+#endif
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_PF_Q4_0)
+#if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 1
+PSN_PREFILL_FAMILY_WS(q4_0, PfQ4_0)
+#endif
+#if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 4
+PSN_PREFILL_FAMILY_BASE(q4_0, PfQ4_0)
+#endif
+#endif
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_PF_Q8_0)
+#if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 1
+PSN_PREFILL_FAMILY_WS(q8_0, PfQ8_0)
+#endif
+#if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 4
+PSN_PREFILL_FAMILY_BASE(q8_0, PfQ8_0)
+#endif
+#endif

@@ -60,11 +60,10 @@ def main(argv=None):
                 bound = "mfma" if flops / nbytes >= MFMA_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "hbm"
                 frac = tflops / MFMA_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS
                 tm, tn, sp, wv = prefill_plan(m, n, k, be.compute_units)
-                if fname == "q8_0" and wv == 8:
-                    wv = 4
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
-                                  "kernel": f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 8: "_w8", -4: "_il", -5: "_rp", 16: "_ws"}[wv], "ksplit": sp, "iters": args.iters}), flush=True)
+                                  "kernel": f"psn_prefill_{fname}_skinny" if wv == 64 else f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}[wv],
+                                  "ksplit": sp, "iters": args.iters}), flush=True)
             for w in ws:
                 w.buf.free()
     return 0

@@ -46,15 +46,40 @@ def test_every_tile_ragged_shapes(hip, orc, qname, tile):
         W = weights(orc, qname, 800, n, k)
         X = G.seeded_acts(801 + m, m, k).astype(np.float16)
         ref = orc.prefill(t, W, X, n, k)
-        il = tile in ((64, 128), (128, 128), (128, 256))              # tiles with the interleaved (-4) kernel
-        ws = tile in ((128, 128), (128, 256))                         # tiles with the producer/consumer (16) kernel
-        for waves in (4,) + ((8, -5) if min(tile) >= 128 else ()) + ((-4,) if il else ()) + ((16,) if ws else ()):
+        ws = tile in ((64, 64), (64, 128), (128, 128), (128, 256))   # tiles with the producer/consumer (16) kernel
+        for waves in (4,) + ((16,) if ws else ()):
             for ksplit in (1, 2, 4):
                 if ksplit > 1 and (m * n) % 4:
                     continue
                 y = hip.matmul_host(t, W, X, n, k, tile + (ksplit, waves))
                 err = G.max_rel_err(y, ref)
                 assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, waves, m, n, k, err)
+
+
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
+def test_skinny_kernel_ragged_shapes(hip, orc, qname):
+    """The M <= 64 kernel (waves code 64): every combination of ragged m and n, K ranges of one to many
+    256-wide chunks (one chunk: the load rings are deeper than the whole range), with and without K split."""
+    t = getattr(orc, qname)
+    for m, n, k in ((1, 70, 256), (37, 300, 768), (64, 130, 1280), (50, 516, 4096), (64, 64, 14336)):
+        say(f"skinny {qname} m={m} n={n} k={k}")
+        W = weights(orc, qname, 860, n, k)
+        X = G.seeded_acts(861 + m, m, k).astype(np.float16)
+        ref = orc.prefill(t, W, X, n, k)
+        for ksplit in (1, 2, 4, 8):
+            if ksplit > 1 and (m * n) % 4:
+                continue
+            y = hip.matmul_host(t, W, X, n, k, (64, 64, ksplit, 64))
+            err = G.max_rel_err(y, ref)
+            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (ksplit, m, n, k, err)
+    # the result without K split does not depend on the run (fixed summation order)
+    W = weights(orc, qname, 860, 516, 4096)
+    X = G.seeded_acts(861 + 50, 50, 4096).astype(np.float16)
+    ys = [hip.matmul_host(t, W, X, 516, 4096, (64, 64, 1, 64)) for _ in range(3)]
+    assert np.array_equal(ys[0], ys[1]) and np.array_equal(ys[0], ys[2])
+    with pytest.raises(backend.PsnError) as e:
+        hip.matmul_host(t, W, G.seeded_acts(1, 65, 4096).astype(np.float16), 516, 4096, (64, 64, 1, 64))
+    assert e.value.code == _ffi.E_UNSUPPORTED
 
 
 @pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])

@@ -138,3 +138,38 @@ def test_static_scratch_is_exported_by_the_device_image():
     rows = [ln.split() for ln in syms.splitlines() if ln.strip().endswith("scratch")]
     assert rows, syms
     assert all(r[3] == "OBJECT" and r[4] == "GLOBAL" and int(r[2]) == 1 << 20 for r in rows), rows
+
+
+def _kernel_resources():
+    """name -> (vgpr spills, sgpr spills, scratch bytes per lane) for every kernel of every built code object,
+    read from the code objects' own metadata notes."""
+    import glob
+    import subprocess
+    import tempfile
+    bundler, readelf = "/opt/rocm/llvm/bin/clang-offload-bundler", "/opt/rocm/llvm/bin/llvm-readelf"
+    objs = sorted(glob.glob(os.path.join(ROOT, "openagents_amd", "lib", "*.gfx950.hsaco")))
+    if not objs or not (os.path.exists(bundler) and os.path.exists(readelf)):
+        pytest.skip("built code objects or LLVM binutils not present")
+    out = {}
+    with tempfile.TemporaryDirectory() as d:
+        for path in objs:
+            elf = os.path.join(d, os.path.basename(path) + ".elf")
+            subprocess.check_call([bundler, "--unbundle", "--type=o", f"--input={path}", "--targets=hipv4-amdgcn-amd-amdhsa--gfx950", f"--output={elf}"])
+            notes = subprocess.check_output([readelf, "--notes", elf], text=True)
+            for blk in notes.split("- .agpr_count:")[1:]:
+                get = lambda key: re.search(r"\." + key + r":\s+(\S+)", blk).group(1)
+                out[get("name")] = (int(get("vgpr_spill_count")), int(get("sgpr_spill_count")), int(get("private_segment_fixed_size")))
+    return out
+
+
+def test_no_kernel_spills_registers_or_uses_scratch():
+    """Every kernel a planner can return (and every other kernel of the library) keeps its working set in
+    registers: a spilled register or a scratch copy of the kernel arguments costs memory round trips in the
+    middle of a stream and has gone unnoticed before."""
+    res = _kernel_resources()
+    assert len(res) > 300
+    for family in ("psn_mvs_q4_0_q8_g16_xf_s2", "psn_mvs_q6_K_q8_g16_lds_s1", "psn_prefill_q4_0_skinny", "psn_prefill_q8_0_m128_n256_ws",
+                   "psn_prefill_q4_0_m256_n256", "psn_attn_partial_rope", "psn_mv_q4_K_q8_g16_r1_b8_lds"):
+        assert family in res, family
+    bad = {k: v for k, v in res.items() if v != (0, 0, 0)}
+    assert not bad, bad
