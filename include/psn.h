@@ -45,7 +45,7 @@ typedef struct psn_event psn_event;
 typedef struct psn_graph psn_graph;
 
 /* GGUF tensor type ids */
-typedef enum { PSN_Q4_0 = 2, PSN_Q8_0 = 8, PSN_Q4_K = 12, PSN_Q6_K = 14, PSN_Q8_K = 15 } psn_qtype;
+typedef enum { PSN_Q4_0 = 2, PSN_Q8_0 = 8, PSN_Q4_K = 12, PSN_Q5_K = 13, PSN_Q6_K = 14, PSN_Q8_K = 15 } psn_qtype;
 /* how activations enter the dot product */
 typedef enum {
     PSN_ACT_F32 = 0, /* weights dequantized to fp32, fp32 FMA */
@@ -74,6 +74,15 @@ const char *psn_error_name(int32_t code);
 int32_t psn_block_elems(int32_t qtype);
 int32_t psn_block_bytes(int32_t qtype);
 int64_t psn_row_bytes(int32_t qtype, int64_t k);
+
+/* Host-side weight quantizer: fp32 rows x[n][k] -> n * psn_row_bytes(qtype, k) bytes of GGUF blocks
+ * (Q4_0, Q8_0, Q4_K, Q5_K, Q6_K), byte-identical to the published ggml reference quantizers
+ * (quantize_row_*_ref: closed forms for Q4_0/Q8_0, the weighted least-squares scale searches for the
+ * K-quants).  Runs on `threads` host threads (rows are independent; < 1 means 1); touches no device.
+ * This is the "reference quantizer" step that produces the weights of every benchmark configuration
+ * (/root/reference/docs/muse/muse-glimmer.md:112 names the served formats); it replaces the CPU
+ * quantize pass a loader runs when a checkpoint arrives as fp32/fp16. */
+int32_t psn_quantize_rows(int32_t qtype, const float *x, int64_t n, int64_t k, void *out, size_t out_bytes, int32_t threads);
 
 /* ---- context, module, stream, event, buffer  (the "module load, buffer alloc, launch and
  *      stream sync" surface; replaces the CUDA backend's context/module/stream/buffer wrappers) -- */

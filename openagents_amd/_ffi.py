@@ -12,7 +12,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpsn_hip.so")
 
-Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 2, 8, 12, 14, 15
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K = 2, 8, 12, 13, 14, 15
 ACT_F32, ACT_Q8 = 0, 1
 LAYOUT_GGUF = 0
 
@@ -43,6 +43,7 @@ SIGNATURES = {
     "psn_block_elems": (_i32, [_i32]),
     "psn_block_bytes": (_i32, [_i32]),
     "psn_row_bytes": (_i64, [_i32, _i64]),
+    "psn_quantize_rows": (_i32, [_i32, _vp, _i64, _i64, _vp, _sz, _i32]),
     "psn_ctx_create": (_i32, [_i32, _pp]),
     "psn_ctx_destroy": (_i32, [_vp]),
     "psn_ctx_info": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_i64), C.c_char_p, _sz]),

@@ -110,8 +110,12 @@ def build(jobs: int = 0, verbose: bool = True, reuse_device: bool = False) -> st
     _run(["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__",
           "-I", INCLUDE, "-I", CSRC, "-isystem", os.path.join(rocm, "include"),
           "-c", "-o", host_o, os.path.join(CSRC, "psn_host.cpp")])
+    # the host quantizer keeps a*b+c as two roundings, like the reference quantizers it restates
+    quant_o = os.path.join(LIB, "psn_quantize.o")
+    _run(["g++", "-O3", "-march=x86-64-v3", "-std=c++17", "-fPIC", "-Wall", "-Wextra", "-ffp-contract=off", "-I", INCLUDE,
+          "-c", "-o", quant_o, os.path.join(CSRC, "psn_quantize.cpp")])
     out = lib_path()
-    _run(["g++", "-shared", "-fPIC", "-o", out, host_o, noalloc_o, blob_o, "-Wl,--no-undefined",
+    _run(["g++", "-shared", "-fPIC", "-pthread", "-o", out, host_o, quant_o, noalloc_o, blob_o, "-Wl,--no-undefined",
           "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-Wl,-rpath," + os.path.join(rocm, "lib")])
     if verbose:
         print("built", os.path.relpath(out, os.path.dirname(HERE)), os.path.getsize(out), "bytes")

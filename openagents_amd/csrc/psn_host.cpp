@@ -73,7 +73,7 @@ extern "C" const char *psn_error_name(int32_t code) {
 extern "C" int32_t psn_block_elems(int32_t t) {
     switch (t) {
         case PSN_Q4_0: case PSN_Q8_0: return 32;
-        case PSN_Q4_K: case PSN_Q6_K: case PSN_Q8_K: return 256;
+        case PSN_Q4_K: case PSN_Q5_K: case PSN_Q6_K: case PSN_Q8_K: return 256;
         default: return 0;
     }
 }
@@ -82,6 +82,7 @@ extern "C" int32_t psn_block_bytes(int32_t t) {
         case PSN_Q4_0: return 18;
         case PSN_Q8_0: return 34;
         case PSN_Q4_K: return 144;
+        case PSN_Q5_K: return 176;
         case PSN_Q6_K: return 210;
         case PSN_Q8_K: return 292;
         default: return 0;
@@ -93,6 +94,23 @@ extern "C" int64_t psn_row_bytes(int32_t t, int64_t k) {
     if (k <= 0 || k % be) return fail(PSN_E_SHAPE, "K=%lld is not a positive multiple of the block size %lld", (long long)k, (long long)be);
     return k / be * psn_block_bytes(t);
 }
+/* psn_quantize.cpp */
+int psn_quantize_rows_impl(int32_t qtype, const float *x, int64_t n, int64_t k, uint8_t *out, int64_t row_bytes, int32_t threads);
+
+extern "C" int32_t psn_quantize_rows(int32_t qtype, const float *x, int64_t n, int64_t k, void *out, size_t out_bytes, int32_t threads) {
+    if (!x || !out) return fail(PSN_E_INVALID_ARG, "psn_quantize_rows: null pointer");
+    if (qtype == PSN_Q8_K) return fail(PSN_E_UNSUPPORTED, "psn_quantize_rows: Q8_K is an activation format (psn_quantize_activations)");
+    const int64_t rb = psn_row_bytes(qtype, k);
+    if (rb < 0) return (int32_t)rb;
+    if (n <= 0) return fail(PSN_E_SHAPE, "psn_quantize_rows: n=%lld", (long long)n);
+    if ((uint64_t)n * (uint64_t)rb > out_bytes)
+        return fail(PSN_E_INVALID_ARG, "psn_quantize_rows: output holds %zu bytes, %lld rows of %lld bytes need %lld", out_bytes,
+                    (long long)n, (long long)rb, (long long)(n * rb));
+    if (psn_quantize_rows_impl(qtype, x, n, k, static_cast<uint8_t *>(out), rb, threads < 1 ? 1 : threads) != 0)
+        return fail(PSN_E_UNSUPPORTED, "psn_quantize_rows: type %d has no quantizer", qtype);
+    return PSN_OK;
+}
+
 static bool is_weight_type(int32_t t) { return t == PSN_Q4_0 || t == PSN_Q8_0 || t == PSN_Q4_K || t == PSN_Q6_K; }
 static const char *fmt_name(int32_t t) {
     switch (t) {

@@ -1,42 +1,64 @@
-"""The numpy quantizers that feed benchmarks must produce exactly the oracle's bytes."""
+"""The library's native host quantizer (psn_quantize_rows) must produce exactly the oracle's bytes:
+it is a second, separately written statement of the same published quantizers."""
+import ctypes as C
+
 import numpy as np
+import pytest
 
 import ggufref as G
-from openagents_amd import quantize
+from openagents_amd import _ffi, quantize
 
 
-def test_numpy_q4_0_and_q8_0_match_oracle_bit_for_bit(orc):
-    w = G.seeded_weights(700, 64, 2048)
-    w[0, :32] = 0
+def special_rows(k):
+    """Rows that exercise the branches of the quantizers: zero blocks, exact grids, sign ties, one-sided
+    sub-blocks, scales that land in fp16 subnormals and near the fp16 maximum."""
+    w = G.seeded_weights(700, 24, k)
+    w[0, :256] = 0
     w[1, :32] = np.float32(0.5) * (np.arange(32) % 16 - 8)
     w[2, :4] = [8, -7, -8, 0]
     w[3, 5] = 1.0
     w[3, 9] = -1.0                     # equal magnitudes: the first one sets the sign of d
-    assert np.array_equal(quantize.quantize_q4_0(w), orc.quantize(orc.Q4_0, w))
-    assert np.array_equal(quantize.quantize_q8_0(w), orc.quantize(orc.Q8_0, w))
-    x = G.seeded_acts(701, 4, 4096)
-    assert np.array_equal(quantize.quantize_q8_0(x), orc.quantize(orc.Q8_0, x))
-    assert np.array_equal(quantize.quantize_q4_0(x), orc.quantize(orc.Q4_0, x))
+    w[4, :32] = np.abs(w[4, :32])      # a one-sided sub-block
+    w[5, :32] = -np.abs(w[5, :32])
+    w[6] *= np.float32(1e-6)           # block scales in the fp16 subnormal range
+    w[7] *= np.float32(3e-8)           # scales that round to zero in fp16
+    w[8] *= np.float32(2e5)            # scales in the thousands
+    w[9, :256] = np.float32(0.25)      # a constant super-block
+    w[10, :16] = np.linspace(-1, 1, 16, dtype=np.float32)
+    w[11] = np.round(w[11] * 200) / 200
+    return w
 
 
-def test_numpy_k_quant_producers_are_valid_and_close(orc):
-    """The simple Q4_K / Q6_K producers (no scale search) must emit blocks the oracle's dequantizer
-    reads back close to the input: the element-index parsers pin the byte layout, the error bounds
-    pin the scale/min arithmetic."""
-    w = G.seeded_weights(710, 16, 1024)
-    w[0, :256] = 0
-    w[1, :32] = np.abs(w[1, :32])                       # an all-positive sub-block: min stays 0
-    r4 = quantize.quantize_q4_K(w)
-    d, dmin, sc, mn, q = G.parse_q4_K(r4, 1024)
-    assert sc.max() <= 63 and mn.max() <= 63 and q.max() <= 15 and np.all(d >= 0) and np.all(dmin >= 0)
-    y4 = orc.dequantize(orc.Q4_K, r4, 1024)
-    assert np.sqrt(np.mean((y4 - w) ** 2)) / np.sqrt(np.mean(w ** 2)) < 0.10
-    step = (d[:, :, None] * sc).repeat(32, axis=2).reshape(16, 1024)
-    assert np.all(np.abs(y4 - w) <= step + 1e-6)
-    assert not y4[0, :256].any()
-    r6 = quantize.quantize_q6_K(w)
-    d6, s6, q6 = G.parse_q6_K(r6, 1024)
-    assert q6.min() >= -32 and q6.max() <= 31
-    y6 = orc.dequantize(orc.Q6_K, r6, 1024)
-    assert np.sqrt(np.mean((y6 - w) ** 2)) / np.sqrt(np.mean(w ** 2)) < 0.03
-    assert not y6[0, :256].any()
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+def test_native_quantizer_matches_oracle_bit_for_bit(orc, name):
+    qt = getattr(_ffi, name)
+    for k in (256, 2048):
+        w = special_rows(k)
+        assert np.array_equal(quantize.quantize(qt, w), orc.quantize(getattr(orc, name), w)), (name, k)
+    x = G.seeded_acts(701, 6, 4096)                     # N(0,1) rows, the activation range
+    assert np.array_equal(quantize.quantize(qt, x), orc.quantize(getattr(orc, name), x))
+
+
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+def test_native_quantizer_is_the_same_on_any_number_of_threads(name):
+    qt = getattr(_ffi, name)
+    w = G.seeded_weights(702, 37, 512)                  # rows do not divide evenly over the threads
+    one = quantize.quantize(qt, w, threads=1)
+    for t in (2, 5, 64):
+        assert np.array_equal(quantize.quantize(qt, w, threads=t), one)
+
+
+def test_native_quantizer_argument_errors():
+    lib = _ffi.load()
+    x = np.zeros((2, 256), np.float32)
+    out = np.zeros(2 * 144, np.uint8)
+    call = lambda qt, n, k, nbytes: lib.psn_quantize_rows(qt, C.c_void_p(x.ctypes.data), n, k, C.c_void_p(out.ctypes.data), nbytes, 1)
+    assert call(_ffi.Q4_K, 2, 256, out.nbytes) == 0
+    assert lib.psn_error_name(call(_ffi.Q4_K, 2, 256, out.nbytes - 1)) == b"PSN_E_INVALID_ARG"      # output too small
+    assert lib.psn_error_name(call(_ffi.Q4_K, 2, 250, out.nbytes)) == b"PSN_E_SHAPE"                # ragged K
+    assert lib.psn_error_name(call(_ffi.Q4_K, 0, 256, out.nbytes)) == b"PSN_E_SHAPE"
+    assert lib.psn_error_name(call(_ffi.Q8_K, 2, 256, 4096)) == b"PSN_E_UNSUPPORTED"                # activation format
+    assert lib.psn_error_name(call(7, 2, 256, out.nbytes)) == b"PSN_E_UNSUPPORTED"                  # unknown type id
+    assert lib.psn_error_name(lib.psn_quantize_rows(_ffi.Q4_K, None, 2, 256, C.c_void_p(out.ctypes.data), out.nbytes, 1)) == b"PSN_E_INVALID_ARG"
+    with pytest.raises(ValueError):
+        quantize.quantize(_ffi.Q4_0, np.zeros((2, 48), np.float32))
