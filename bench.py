@@ -12,7 +12,10 @@ buffers (3.93 GB per step), which defeats the 256 MB Infinity Cache.
 Prints ONE JSON line.  `value` is whole-step algorithmic GB/s with everything resident in HBM
 before the timed region; `roofline` is the dominant kernel's achieved HBM bandwidth measured with
 HIP events on the launch stream; `cpu_baseline` is the CPU oracle timed on this host's cores on a
-bounded sample of the same workload (a reported baseline, not the target).
+bounded sample of the same workload (a reported baseline, not the target).  `records` carries the
+other configurations of the metric -- Q8_0 4096x4096, Q4_K at batch 1/2/4/8, the twelve prefill
+cells, the 8B-shaped decode step -- one throughput record each (openagents_amd/records.py), and
+`read_calibration` what a kernel that only reads reaches at the four launch sizes.
 """
 from __future__ import annotations
 
@@ -48,6 +51,17 @@ LAUNCHES = [("qkv", [HIDDEN, KV, KV], HIDDEN), ("o", [HIDDEN], HIDDEN),
             ("gate_up", [FFN, FFN], HIDDEN), ("down", [HIDDEN], FFN)]
 
 
+def cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def make_layer(seed):
     """One layer's seeded N(0, 0.02) weights, quantized to Q4_0 by the host quantizer."""
     from openagents_amd import quantize
@@ -67,6 +81,8 @@ def main(argv=None):
     ap.add_argument("--cpu-seconds", type=float, default=10.0, help="budget of the CPU baseline leg (0 skips it)")
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--calibrate-copy", action="store_true", help="also run four 256 MiB device-to-device copies (counter calibration)")
+    ap.add_argument("--no-records", action="store_true", help="headline only: skip the records of the other configurations")
+    ap.add_argument("--record-samples", type=int, default=7)
     args = ap.parse_args(argv)
     if args.gpus != 1:
         print("bench.py: this build drives one GPU; --gpus N with N > 1 is not supported "
@@ -215,21 +231,42 @@ def main(argv=None):
                 got = y.download(np.float32, (n,))
                 worst = max(worst, float(np.max(np.abs(got - ref)) / np.max(np.abs(ref))))
         parity = {"metric": "max|y-ref|/max|ref| over all 7 projections vs CPU oracle, scheme Q8", "value": worst, "gate": 1e-3}
-        threads = oracle.max_threads()
         layer_bytes = sum(algo_bytes([n], k) for _, ns, k in LAUNCHES for n in ns)
-        done, t_cpu0 = 0, time.perf_counter()
-        while True:
-            for name, ns, k in LAUNCHES:
-                for blk, n in zip(layer[name], ns):
-                    oracle.matvec(oracle.Q4_0, oracle.ACT_Q8, blk, x_host[name], n, k, nthreads=threads)
-            done += 1
-            if time.perf_counter() - t_cpu0 >= args.cpu_seconds:
-                break
-        cpu_s = time.perf_counter() - t_cpu0
-        cpu = {"value": round(done * layer_bytes / cpu_s / 1e9, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+
+        def cpu_leg(threads, seconds):
+            done, t_cpu0 = 0, time.perf_counter()
+            while True:
+                for name, ns, k in LAUNCHES:
+                    for blk, n in zip(layer[name], ns):
+                        oracle.matvec(oracle.Q4_0, oracle.ACT_Q8, blk, x_host[name], n, k, nthreads=threads)
+                done += 1
+                if time.perf_counter() - t_cpu0 >= seconds:
+                    break
+            cpu_s = time.perf_counter() - t_cpu0
+            return done, cpu_s, round(done * layer_bytes / cpu_s / 1e9, 2)
+
+        threads = oracle.max_threads()
+        done1, s1, gbs1 = cpu_leg(1, args.cpu_seconds * 0.4)
+        done, cpu_s, gbs = cpu_leg(threads, args.cpu_seconds * 0.6)
+        cpu = {"value": gbs, "unit": "GB/s", "cores": threads, "kind": "port",
                "sample": f"{done} x one layer's 7 Q4_0 projections (same bytes and activations as the GPU run), "
                          f"{cpu_s:.1f} s, OpenMP over rows",
+               "single_thread": {"value": gbs1, "unit": "GB/s", "cores": 1, "sample": f"{done1} x the same layer, {s1:.1f} s"},
+               "host": {"nproc": os.cpu_count(), "usable_threads": threads, "cpu_model": cpu_model()},
                "provenance": "this build's C restatement of the CPU quantized path (oracle/), not Psionic's binary"}
+
+    records, calibration = None, None
+    if not args.no_records:
+        from openagents_amd import records as R
+        for lw in weights:                                   # the headline's 3.9 GB of copies are no longer needed
+            for ts in lw.values():
+                for t in ts:
+                    t.buf.free()
+        weights.clear()
+        calibration = R.read_calibration(be, args.record_samples)
+        shared = {(_ffi.Q4_0, FFN, HIDDEN): layer["gate_up"][0], (_ffi.Q4_0, HIDDEN, FFN): layer["down"][0]}
+        records = (R.config1(be, args.record_samples, cpu=args.cpu_seconds > 0) + R.config3(be, args.record_samples)
+                   + R.config4(be, args.record_samples, weights=shared) + R.config5(be, args.record_samples))
 
     out = {
         "metric": "quant matvec GB/s", "value": round(value, 1), "unit": "GB/s", "n_gpus": 1,
@@ -249,6 +286,8 @@ def main(argv=None):
         "roofline": roofline,
         "cpu_baseline": cpu,
         "parity": parity,
+        "read_calibration": calibration,
+        "records": records,
         "device": {"arch": be.arch, "compute_units": be.compute_units}, "setup_s": round(setup_s, 1),
     }
     print(json.dumps(out))

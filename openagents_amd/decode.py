@@ -104,6 +104,14 @@ class DecodeStep:
             self.xq_f = be.alloc(int(actq_layout(self.act_type, s.ffn, 1).bytes))
             self.rope_tab = be.alloc(s.head_dim * 4)
 
+    @property
+    def launches_per_layer(self) -> int:
+        return 9 if self.fused else 10
+
+    @property
+    def launches_outside_layers(self) -> int:
+        return 3 if self.fused else 2
+
     def _enqueue_fused(self, pos: int, matvecs_only: bool):
         be, s, at = self.be, self.shape, self.act_type
         glue = not matvecs_only
@@ -168,10 +176,12 @@ class DecodeStep:
         return total + t.n * row_bytes(t.qtype, t.k) + 4 * (t.n + t.k)
 
 
-def synthetic_weights(be: HipBackend, shape: LlamaShape, seed: int = 0, unique_layers: int = 1, head_rows_unique: int = 16032) -> ModelWeights:
-    """Random-init weights of the given architecture: fp32 N(0, 0.02) quantized on the host (Q4_K
-    projections, Q6_K LM head).  `unique_layers` layers are generated and uploaded round-robin into
-    n_layers distinct device allocations; the LM head is `head_rows_unique` unique rows tiled."""
+def synthetic_weights(be: HipBackend, shape: LlamaShape, seed: int = 0, unique_layers: int = 1, head_rows_unique: int = 16032,
+                      keep_host: dict | None = None) -> ModelWeights:
+    """Random-init weights of the given architecture: fp32 N(0, 0.02) quantized on the host by the
+    library's reference quantizers (Q4_K projections, Q6_K LM head).  `unique_layers` layers are generated
+    and uploaded round-robin into n_layers distinct device allocations; the LM head is `head_rows_unique`
+    unique rows tiled.  With `keep_host` the unique host blocks are left in that dict (name -> uint8 array)."""
     from . import quantize
     rng = np.random.default_rng(seed)
     s = shape
@@ -196,6 +206,10 @@ def synthetic_weights(be: HipBackend, shape: LlamaShape, seed: int = 0, unique_l
     head = qmat(uniq, s.hidden, Q6_K)
     reps = -(-s.vocab // uniq)
     head_full = np.tile(head, (reps, 1))[:s.vocab]
+    if keep_host is not None:
+        for i, p in enumerate(protos):
+            keep_host.update({f"layer{i}.{name}": blk for name, blk in p.items()})
+        keep_host["lm_head"] = head
     return ModelWeights(layers, be.upload(np.ones(s.hidden, np.float32)), be.upload_weight(Q6_K, head_full, s.vocab, s.hidden))
 
 
@@ -251,7 +265,7 @@ def main(argv=None):
            "config": {"layers": shape.n_layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,
                       "ffn": shape.ffn, "vocab": shape.vocab, "context": args.ctx, "weights": "Q4_K projections, Q6_K LM head",
                       "activation_scheme": "Q8 (Q8_K blocks, " + ("written by the producing kernel)" if step.fused else "quantized inside the matvec launch)"),
-                      "launches_per_token": shape.n_layers * (9 if step.fused else 10) + (3 if step.fused else 2), "graph_replay": True},
+                      "launches_per_token": shape.n_layers * step.launches_per_layer + step.launches_outside_layers, "graph_replay": True},
            "data": "synthetic random-init weights (one unique layer copied to every layer's own allocation), fp16 N(0,1) KV cache",
            "logits_finite": bool(np.all(np.isfinite(logits))), "steps": args.steps, "setup_s": round(setup_s, 1),
            "not_measured": ["sampling", "tokenizer", "host loop"]}
