@@ -292,6 +292,18 @@ int32_t psn_add_rmsnorm_q8(psn_module *mod, psn_stream *s, psn_buf *x, const psn
                            psn_buf *y_q, int32_t act_type, int64_t n, float eps);
 int32_t psn_swiglu_q8(psn_module *mod, psn_stream *s, const psn_buf *gate, const psn_buf *up, psn_buf *out, psn_buf *out_q,
                       int32_t act_type, int64_t n);
+/* psn_add_rmsnorm_q8 folded into the projection that consumes it (batch 1, scheme Q8):
+ *     h = x + delta (delta may be NULL);  y_i = W_i . q8(h * rsqrt(mean(h^2) + eps) * norm_weight)
+ * Every workgroup of the streaming matvec adds, normalizes and quantizes the K fp32 values while it
+ * stages them (its weight loads are already in flight), so the norm costs no launch of its own;
+ * workgroup 0 also stores h to h_out (may be NULL), which must not alias x or delta -- a decoder
+ * alternates two residual buffers.  Shapes the fused kernels do not serve (rows longer than 8192, more
+ * than three matrices, row counts that are not whole passes) run the norm kernel and the pre-quantized
+ * matvec as two launches with the same result.  No counterpart in the reference's CPU path, which
+ * normalizes, quantizes and multiplies as separate steps; the arithmetic per element is the same. */
+int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t count,
+                               const psn_buf *const *W, const psn_buf *x, const psn_buf *delta, const psn_buf *norm_weight,
+                               psn_buf *h_out, psn_buf *const *y_f32, const int64_t *N, int64_t K, float eps);
 int32_t psn_attention_decode_q8(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
                                 psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
                                 int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx);

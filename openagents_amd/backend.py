@@ -272,6 +272,12 @@ class HipBackend:
         w0, n, W, Y, N = self._pack(ws, ys)
         _check(self.lib.psn_qmatvec_q8_multi(self.module, self.stream, w0.qtype, LAYOUT_GGUF, n, W, xq.handle, Y, N, w0.k, batch))
 
+    def quantized_matvec_norm_multi(self, ws, x: DeviceBuffer, delta, norm_weight: DeviceBuffer, h_out, ys, eps: float = 1e-5):
+        """ys[i] = ws[i] . q8(rmsnorm(x + delta) * norm_weight); h_out (optional, not x or delta) receives x + delta."""
+        w0, n, W, Y, N = self._pack(ws, ys)
+        _check(self.lib.psn_qmatvec_norm_multi(self.module, self.stream, w0.qtype, LAYOUT_GGUF, n, W, x.handle, self._h(delta), norm_weight.handle,
+                                               self._h(h_out), Y, N, w0.k, eps))
+
     def quantized_matvec_planned(self, ws, x: DeviceBuffer, ys, batch: int, scheme: int, plan: MatvecPlan):
         w0, n, W, Y, N = self._pack(ws, ys)
         _check(self.lib.psn_qmatvec_planned(self.module, self.stream, w0.qtype, scheme, n, W, x.handle, Y, N, w0.k, batch, C.byref(plan)))

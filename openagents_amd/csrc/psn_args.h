@@ -49,7 +49,10 @@ struct psn_matvec_args {
     int32_t threads;      /* launch geometry, passed in so that kernels never read the dispatch packet */
     int32_t blocks;
     int32_t ring;         /* streaming kernels: LDS buffers (passes in flight) per wave */
-    int32_t pad;
+    float eps;            /* the fields below: streaming kernels that normalize while staging (_xn) */
+    const float *x_delta; /* [K] added to xf before the norm (may be null) */
+    const float *norm_w;  /* [K] RMSNorm weights */
+    float *h_out;         /* [K] receives xf + x_delta, written by workgroup 0 (may be null; must not alias xf or x_delta) */
 };
 
 struct psn_prefill_args {
@@ -91,6 +94,7 @@ struct psn_norm_args {
     int32_t n;
     float eps;
     struct psn_actq_out qout;
+    float *x_out;         /* when set, x + delta goes here and x is left alone */
 };
 struct psn_rope_args {
     float *q;             /* [n_heads][head_dim], rotated in place */

@@ -50,7 +50,9 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
     __shared__ float red[16];
     constexpr int KEEP = 4;
     const int n4 = a.n >> 2, nt = blockDim.x;
-    float4 *x4 = reinterpret_cast<float4 *>(a.x);
+    const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
+    float4 *xo4 = reinterpret_cast<float4 *>(a.x_out ? a.x_out : a.x);      /* where x + delta goes */
+    const bool store_sum = a.delta != nullptr || a.x_out != nullptr;
     const float4 *d4 = reinterpret_cast<const float4 *>(a.delta);
     const float4 *w4 = reinterpret_cast<const float4 *>(a.weight);
     float4 *y4 = reinterpret_cast<float4 *>(a.y);
@@ -68,8 +70,8 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
                 if (d4) {
                     const float4 d = d4[i];
                     v[k].x += d.x; v[k].y += d.y; v[k].z += d.z; v[k].w += d.w;
-                    x4[i] = v[k];
                 }
+                if (store_sum) xo4[i] = v[k];
             }
             ss += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
         }
@@ -79,8 +81,8 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
             if (d4) {
                 const float4 d = d4[i];
                 t.x += d.x; t.y += d.y; t.z += d.z; t.w += d.w;
-                x4[i] = t;
             }
+            if (store_sum) xo4[i] = t;
             ss += t.x * t.x + t.y * t.y + t.z * t.z + t.w * t.w;
         }
     }
@@ -98,7 +100,7 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
         }
     } else {
         for (int i = threadIdx.x; i < n4; i += nt) {
-            const float4 t = x4[i], ww = w4[i];
+            const float4 t = store_sum ? xo4[i] : x4[i], ww = w4[i];
             const float4 o = make_float4(t.x * scale * ww.x, t.y * scale * ww.y, t.z * scale * ww.z, t.w * scale * ww.w);
             if (y4) y4[i] = o;
             if (a.qout.qs) quantize_out4(a.qout, i, o);

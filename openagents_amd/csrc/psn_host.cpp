@@ -666,7 +666,8 @@ static int32_t stream_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32
         return fail(PSN_E_UNSUPPORTED, "plan: the streaming kernels serve scheme Q8 at batch 1");
     if (psn_row_bytes(qtype, K) % 16) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs rows of whole 16-byte words (Q6_K: K a multiple of 2048)");
     if (C > g) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs rows of at most lanes_per_row chunks (K <= %d)", g * 256);
-    if (plan->stage_lds != 1 && plan->stage_lds != 2) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs stage_lds 1 or 2");
+    if (plan->stage_lds < 1 || plan->stage_lds > 3) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs stage_lds 1, 2 or 3");
+    if (plan->stage_lds == 3 && (g > 32 || count > 3)) return fail(PSN_E_UNSUPPORTED, "plan: the norm-fused kernels exist for rows of at most 32 chunks and three matrices");
     if (plan->threads != 256 && plan->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", plan->threads);
     if (ring < 1 || ring > 8) return fail(PSN_E_UNSUPPORTED, "plan: stream=%d (passes in flight per wave, 1..8)", ring);
     for (int i = 0; n_rows && i < count; ++i)
@@ -678,12 +679,14 @@ static int32_t stream_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32
     if ((ring - 1) * nloads > 63) return fail(PSN_E_UNSUPPORTED, "plan: %d passes of %lld loads exceed the load counter", ring, (long long)nloads);
     /* the activations pass through at most eight 16-byte registers per thread on their way into LDS */
     const int64_t slots = 8 * (int64_t)plan->threads;
+    /* (four, when x, the residual delta and the norm weights travel together) */
+    const int64_t f32_regs = plan->stage_lds == 3 ? 4 : 8;
     const bool fits = plan->stage_lds == 1 ? (C * 16 <= slots && (K / be) * 4 <= 16 * (int64_t)plan->threads)
-                      : at == PSN_Q8_0   ? C * 64 <= slots
-                                         : C <= 8 * (int64_t)(plan->threads / 64);
+                      : at == PSN_Q8_0   ? C * 64 <= f32_regs * (int64_t)plan->threads
+                                         : C <= f32_regs * (int64_t)(plan->threads / 64);
     if (!fits) return fail(PSN_E_UNSUPPORTED, "plan: K=%lld is too long for %d threads to stage in one round", (long long)K, plan->threads);
     const int64_t n_d = ((K / be) * 4 + 15) / 16, n_s = ((at == PSN_Q8_0 ? (K / 32) * 4 : (K / 16) * 2) + 15) / 16;
-    const int64_t stage = (C * 272 + (n_d + n_s) * 16 + 1023) / 1024 * 1024;
+    const int64_t stage = (C * 272 + (n_d + n_s) * 16 + (plan->stage_lds == 3 ? 64 : 0) + 1023) / 1024 * 1024;
     const int64_t total = stage + (int64_t)(plan->threads / 64) * ring * nloads * 1024;
     if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs %lld bytes of LDS, device offers %d", (long long)total, max_lds);
     *lds_out = total;
@@ -792,7 +795,7 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     if (r != 1) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
     int32_t lds = 0;
-    if (p->stage_lds < 0 || p->stage_lds > 2) return fail(PSN_E_UNSUPPORTED, "plan: stage_lds=%d", p->stage_lds);
+    if (p->stage_lds < 0 || p->stage_lds > 3 || (p->stage_lds == 3 && !p->stream)) return fail(PSN_E_UNSUPPORTED, "plan: stage_lds=%d", p->stage_lds);
     if (p->stage_lds && scheme == PSN_ACT_F32) {
         if (p->stage_lds != 1) return fail(PSN_E_UNSUPPORTED, "plan: scheme F32 stages fp32 activations (stage_lds 0 or 1)");
         const int64_t total = (int64_t)batch * (K / 256) * 1040;
@@ -815,8 +818,15 @@ struct seg_list {
     int64_t total;
 };
 
+/* the extra operands of a launch that adds a residual and normalizes while it stages x (stage_lds 3) */
+struct norm_fusion {
+    const float *delta, *weight;
+    float *h_out;
+    float eps;
+};
+
 static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const seg_list &sg, const void *x,
-                          int64_t K, int32_t batch, const psn_matvec_plan *plan) {
+                          int64_t K, int32_t batch, const psn_matvec_plan *plan, const norm_fusion *norm = nullptr) {
     int32_t lds = 0;
     int32_t rc = plan_is_valid(plan, qtype, scheme, K, batch, mod->ctx->max_lds, &lds);
     if (rc) return rc;
@@ -843,7 +853,14 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
         int64_t total = 0;
         if ((rc = stream_plan_check(qtype, scheme, K, batch, plan, sg.N, sg.count, mod->ctx->max_lds, &total))) return rc;
         const int32_t at = psn_act_type_for(qtype);
-        if (plan->stage_lds == 2) {
+        if (plan->stage_lds == 3) {
+            if (!norm) return fail(PSN_E_INVALID_ARG, "plan: stage_lds 3 is the norm-fused launch (psn_qmatvec_norm_multi)");
+            a.xf = (const float *)x;
+            a.x_delta = norm->delta;
+            a.norm_w = norm->weight;
+            a.h_out = norm->h_out;
+            a.eps = norm->eps;
+        } else if (plan->stage_lds == 2) {
             a.xf = (const float *)x;
         } else {
             psn_actq_info li;
@@ -854,7 +871,8 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
         }
         a.ring = ring;
         (void)rows;
-        snprintf(name, sizeof name, "psn_mvs_%s_q8_g%d_%s_s%d", fmt_name(qtype), g, plan->stage_lds == 2 ? "xf" : "lds", sg.count);
+        snprintf(name, sizeof name, "psn_mvs_%s_q8_g%d_%s_s%d", fmt_name(qtype), g,
+                 plan->stage_lds == 3 ? "xn" : plan->stage_lds == 2 ? "xf" : "lds", sg.count);
         return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)total, &a);
     }
     if (scheme == PSN_ACT_Q8 && plan->stage_lds == 2) {
@@ -1197,6 +1215,21 @@ static int32_t set_actq_out(const char *what, psn_module *mod, psn_buf *yq, int3
     return PSN_OK;
 }
 
+static int32_t launch_add_rmsnorm(psn_module *mod, psn_stream *s, float *x, const float *delta, const float *weight, float *y, float *x_out,
+                                  const psn_actq_out &qout, int64_t n, float eps) {
+    psn_norm_args a;
+    a.x = x;
+    a.delta = delta;
+    a.weight = weight;
+    a.y = y;
+    a.n = (int32_t)n;
+    a.eps = eps;
+    a.qout = qout;
+    a.x_out = x_out;
+    const unsigned threads = n >= 4096 ? 1024 : n >= 1024 ? 256 : 64;
+    return launch(mod, s, "psn_add_rmsnorm", 1, threads, 0, &a);
+}
+
 extern "C" int32_t psn_add_rmsnorm_q8(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
                                       psn_buf *yq, int32_t act_type, int64_t n, float eps) {
     int32_t rc = check_same_ctx(mod, s, x, weight, x, "psn_add_rmsnorm");
@@ -1206,22 +1239,74 @@ extern "C" int32_t psn_add_rmsnorm_q8(psn_module *mod, psn_stream *s, psn_buf *x
     if ((rc = need(x, n * 4, "psn_add_rmsnorm", "x")) || (rc = need(weight, n * 4, "psn_add_rmsnorm", "weight")) ||
         (y && (rc = need(y, n * 4, "psn_add_rmsnorm", "y"))) || (delta && (rc = need(delta, n * 4, "psn_add_rmsnorm", "delta"))))
         return rc;
-    psn_norm_args a;
-    if ((rc = set_actq_out("psn_add_rmsnorm", mod, yq, act_type, n, &a.qout))) return rc;
+    psn_actq_out qo;
+    if ((rc = set_actq_out("psn_add_rmsnorm", mod, yq, act_type, n, &qo))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
-    a.x = (float *)x->p;
-    a.delta = delta ? (const float *)delta->p : nullptr;
-    a.weight = (const float *)weight->p;
-    a.y = y ? (float *)y->p : nullptr;
-    a.n = (int32_t)n;
-    a.eps = eps;
-    const unsigned threads = n >= 4096 ? 1024 : n >= 1024 ? 256 : 64;
-    return launch(mod, s, "psn_add_rmsnorm", 1, threads, 0, &a);
+    return launch_add_rmsnorm(mod, s, (float *)x->p, delta ? (const float *)delta->p : nullptr, (const float *)weight->p,
+                              y ? (float *)y->p : nullptr, nullptr, qo, n, eps);
 }
 extern "C" int32_t psn_add_rmsnorm(psn_module *mod, psn_stream *s, psn_buf *x, const psn_buf *delta, const psn_buf *weight, psn_buf *y,
                                    int64_t n, float eps) {
     if (!y) return fail(PSN_E_INVALID_ARG, "psn_add_rmsnorm: y is null");
     return psn_add_rmsnorm_q8(mod, s, x, delta, weight, y, nullptr, PSN_Q8_K, n, eps);
+}
+
+/* y_i = W_i . q8(rmsnorm(x + delta) * weight), batch 1, scheme Q8: the residual add, the RMSNorm and the
+ * activation quantization happen while every workgroup stages the fp32 vector (one launch); shapes the
+ * norm-fused kernels do not serve take the norm kernel plus the pre-quantized matvec (two launches). */
+extern "C" int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t count,
+                                          const psn_buf *const *W, const psn_buf *x, const psn_buf *delta, const psn_buf *norm_weight,
+                                          psn_buf *h_out, psn_buf *const *y, const int64_t *N, int64_t K, float eps) {
+    const char *what = "psn_qmatvec_norm_multi";
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
+    if (!norm_weight) return fail(PSN_E_INVALID_ARG, "%s: norm_weight is null", what);
+    seg_list sg;
+    int32_t rc = gather_segments(what, mod, s, qtype, PSN_ACT_Q8, count, W, x, y, N, K, 1, &sg);
+    if (rc) return rc;
+    if ((rc = check_x_f32(what, x, K, 1)) || (rc = need(norm_weight, K * 4, what, "norm_weight")) ||
+        (delta && (rc = need(delta, K * 4, what, "delta"))) || (h_out && (rc = need(h_out, K * 4, what, "h_out"))))
+        return rc;
+    if (norm_weight->ctx != mod->ctx || (delta && delta->ctx != mod->ctx) || (h_out && h_out->ctx != mod->ctx))
+        return fail(PSN_E_INVALID_ARG, "%s: handles belong to different contexts", what);
+    if (h_out && (h_out->p == x->p || (delta && h_out->p == delta->p)))
+        return fail(PSN_E_INVALID_ARG, "%s: h_out must not alias x or delta (every workgroup reads them while one writes h_out)", what);
+    psn_matvec_plan plan;
+    if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, 1, mod->ctx->compute_units, true, sg.N, sg.count, &plan))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    norm_fusion nf = {delta ? (const float *)delta->p : nullptr, (const float *)norm_weight->p, h_out ? (float *)h_out->p : nullptr, eps};
+    if (plan.stream && plan.stage_lds == 2) {
+        psn_matvec_plan q = plan;
+        q.stage_lds = 3;
+        int64_t lds = 0;
+        if (K > 4096 && q.threads == 256) q.threads = 512;       /* x, delta and the weights: four 16-byte registers each per thread */
+        if (stream_plan_check(qtype, PSN_ACT_Q8, K, 1, &q, sg.N, sg.count, mod->ctx->max_lds, &lds) == PSN_OK) {
+            if (q.threads != plan.threads) {
+                const int64_t rows = 64 / q.lanes_per_row, npass = sg.total / rows, wpb = q.threads / 64;
+                int64_t resident = (160 * 1024) / lds;
+                resident = resident > 3 ? 3 : resident < 1 ? 1 : resident;
+                int64_t b = (npass + wpb - 1) / wpb;
+                q.blocks = (int32_t)(b > resident * mod->ctx->compute_units ? resident * mod->ctx->compute_units : b);
+            }
+            return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, x->p, K, 1, &q, &nf);
+        }
+        g_err[0] = 0;
+    }
+    /* two launches: norm (+ quantize) into the stream's workspace, then the pre-quantized matvec */
+    const int32_t at = psn_act_type_for(qtype);
+    psn_actq_info li;
+    if ((rc = psn_actq_layout(at, K, 1, &li))) return rc;
+    if ((rc = ensure_workspace(s, li.bytes))) return rc;
+    bool cap = false;
+    if ((rc = is_capturing(s, &cap))) return rc;
+    if (cap) s->ws_in_graph = true;
+    psn_actq_out qo;
+    qo.qs = (int8_t *)s->ws + li.off_qs;
+    qo.d = (float *)((char *)s->ws + li.off_d);
+    qo.s = (char *)s->ws + li.off_s;
+    qo.act_q8_K = at == PSN_Q8_K;
+    if ((rc = launch_add_rmsnorm(mod, s, (float *)x->p, nf.delta, nf.weight, nullptr, nf.h_out, qo, K, eps))) return rc;
+    if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, 1, mod->ctx->compute_units, false, sg.N, sg.count, &plan))) return rc;
+    return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, s->ws, K, 1, &plan);
 }
 
 extern "C" int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q, psn_buf *k, const psn_buf *v, psn_buf *k_cache,
@@ -1331,8 +1416,9 @@ static int32_t attention_impl(psn_module *mod, psn_stream *s, const psn_buf *q, 
         a.v_cache_w = v_cache->p;
         a.rope_table = (const float *)rope->table->p;
     }
+    const int32_t group = n_heads / n_kv_heads;
     if ((rc = launch(mod, s, rope ? "psn_attn_partial_rope" : "psn_attn_partial", (unsigned)(n_kv_heads * splits),
-                     (unsigned)(64 * (n_heads / n_kv_heads)), 0, &a)))
+                     (unsigned)(64 * group), 0, &a)))
         return rc;
     if (out_q) return launch(mod, s, "psn_attn_combine_q8", (unsigned)(n_heads / 2), 256, 0, &a);
     return launch(mod, s, "psn_attn_combine", (unsigned)n_heads, 128, 0, &a);

@@ -679,9 +679,22 @@ template <typename ST, int XR> PSN_DEV void stream_load_x(u32 qs_addr, u32 d_add
 template <typename ST, int XSRC>
 struct StreamStager {
     static constexpr int SLOTS = 8;
+    static constexpr int NORM_SLOTS = 4;                     /* XSRC 3 holds x, the delta and the norm weights: half the reach */
     u32x4 t[SLOTS];
     u32x4 td, ts;
+    u32x4 tdl[XSRC == 3 ? NORM_SLOTS : 1], tw[XSRC == 3 ? NORM_SLOTS : 1];
     int C, nthreads, n_qs, n_d, n_s;
+
+    /* 16-byte word of the fp32 vector that slot i of this thread holds, or -1 */
+    PSN_DEV int f32_word(int i) const {
+        if constexpr (sizeof(ST) == 4) {
+            const int idx = threadIdx.x + i * nthreads;
+            return idx < C * 64 ? idx : -1;
+        } else {
+            const int sb = (threadIdx.x >> 6) + i * (nthreads >> 6);
+            return sb < C ? sb * 64 + (int)(threadIdx.x & 63) : -1;
+        }
+    }
 
     PSN_DEV void issue(const psn_matvec_args &a, int d_per_col, int s_per_col) {
         C = a.K >> 8;
@@ -699,6 +712,18 @@ struct StreamStager {
             }
             if ((int)threadIdx.x < n_d) td = global_read128(reinterpret_cast<const uint4 *>(a.xd) + threadIdx.x);
             if ((int)threadIdx.x < n_s) ts = global_read128(reinterpret_cast<const uint4 *>(a.xs) + threadIdx.x);
+        } else if constexpr (XSRC == 3) {
+            const uint4 *x4 = reinterpret_cast<const uint4 *>(a.xf), *d4 = reinterpret_cast<const uint4 *>(a.x_delta);
+            const uint4 *w4 = reinterpret_cast<const uint4 *>(a.norm_w);
+            UNROLL for (int i = 0; i < NORM_SLOTS; ++i) {
+                tdl[i] = tw[i] = (u32x4)(0u);
+                const int idx = f32_word(i);
+                if (idx >= 0) {
+                    t[i] = global_read128(x4 + idx);
+                    if (d4) tdl[i] = global_read128(d4 + idx);
+                    tw[i] = global_read128(w4 + idx);
+                }
+            }
         } else {
             const float4 *x4 = reinterpret_cast<const float4 *>(a.xf);
             if constexpr (sizeof(ST) == 4) {
@@ -717,14 +742,47 @@ struct StreamStager {
         }
     }
 
+    /* XSRC 3: t <- (x + delta) * rsqrt(mean((x + delta)^2) + eps) * weight, in place; workgroup 0 also
+     * stores x + delta.  `red` is the LDS address of one float per wave; crosses a workgroup barrier. */
+    PSN_DEV void normalize(const psn_matvec_args &a, u32 red) {
+        tie(tdl);
+        tie(tw);
+        float ss = 0.f;
+        UNROLL for (int i = 0; i < NORM_SLOTS; ++i) {
+            float h[4];
+            UNROLL for (int e = 0; e < 4; ++e) {
+                h[e] = __uint_as_float(t[i][e]) + __uint_as_float(tdl[i][e]);
+                ss += h[e] * h[e];
+                t[i][e] = __float_as_uint(h[e]);
+            }
+            const int idx = f32_word(i);
+            if (blockIdx.x == 0 && a.h_out && idx >= 0) reinterpret_cast<float4 *>(a.h_out)[idx] = make_float4(h[0], h[1], h[2], h[3]);
+        }
+        ss = group_sum<64>(ss);
+        const int wpb = nthreads >> 6;
+        if ((threadIdx.x & 63) == 0) lds_write32(red + (threadIdx.x >> 6) * 4u, __float_as_uint(ss));
+        lds_barrier();
+        float total = 0.f;
+        for (int w = 0; w < wpb; ++w) {
+            u32 v = lds_read32(red + (u32)w * 4u);
+            lds_wait();
+            tie1(v);
+            total += __uint_as_float(v);
+        }
+        const float scale = 1.0f / sqrtf(total / (float)a.K + a.eps);
+        UNROLL for (int i = 0; i < NORM_SLOTS; ++i)
+            UNROLL for (int e = 0; e < 4; ++e) t[i][e] = __float_as_uint(__uint_as_float(t[i][e]) * scale * __uint_as_float(tw[i][e]));
+    }
+
     /* base: LDS byte address of the staging area; returns the addresses of the three fields */
-    PSN_DEV void finish(int pending, u32 base, u32 &qs_addr, u32 &d_addr, u32 &s_addr) {
+    PSN_DEV void finish(const psn_matvec_args &a, int pending, u32 base, u32 &qs_addr, u32 &d_addr, u32 &s_addr) {
         qs_addr = base;
         d_addr = base + (u32)C * 272u;
         s_addr = d_addr + (u32)n_d * 16u;
         wait_vmcnt(pending);
         tie(t);
         asm volatile("" : "+v"(td), "+v"(ts));
+        if constexpr (XSRC == 3) normalize(a, s_addr + (u32)n_s * 16u);
         const int lane = threadIdx.x & 63;
         if constexpr (XSRC == 1) {
             UNROLL for (int i = 0; i < SLOTS; ++i) {
@@ -794,7 +852,7 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
 
     /* where the wave buffers start: right behind the staged activations (same arithmetic as the host) */
     const int n_d = (F::d_per_col(K) * 4 + 15) / 16, n_s = (F::s_per_col(K) * (int)sizeof(ST) + 15) / 16;
-    const int stage_bytes = ((C * 272 + (n_d + n_s) * 16 + 1023) >> 10) << 10;
+    const int stage_bytes = ((C * 272 + (n_d + n_s) * 16 + (XSRC == 3 ? 64 : 0) + 1023) >> 10) << 10;   /* XSRC 3: one float per wave behind the fields */
     const u32 ring_base = lds0 + (u32)stage_bytes + (u32)(wib * ring) * (u32)wbuf;
 
     /* a pass never straddles two matrices, so its rows are one contiguous range of one of them; the
@@ -838,7 +896,7 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
     int issued = 0;                                          /* passes issued so far */
     for (; issued < ring && p0 + issued * stride < npass; ++issued) issue(p0 + issued * stride, issued);
     u32 qs_addr, d_addr, s_addr;
-    st.finish(issued * nloads, lds0, qs_addr, d_addr, s_addr);   /* waits for the activation loads only */
+    st.finish(a, issued * nloads, lds0, qs_addr, d_addr, s_addr);   /* waits for the activation loads only */
     lds_barrier();
     u32 xr[F::XR];
     UNROLL for (int i = 0; i < F::XR; ++i) xr[i] = 0;
@@ -969,8 +1027,15 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
     extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_xf_s##NSEG(const psn_matvec_args a) {  \
         mv_q8_stream<F, G, 2, NSEG>(a);                                                                   \
     }
+/* ... and with the residual add + RMSNorm folded into the staging of fp32 activations (_xn) */
+#define PSN_STREAM_NORM_KERNEL(fmt, F, G, NSEG)                                                           \
+    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_xn_s##NSEG(const psn_matvec_args a) {  \
+        mv_q8_stream<F, G, 3, NSEG>(a);                                                                   \
+    }
+#define PSN_STREAM_NORM_G(fmt, F, G) PSN_STREAM_NORM_KERNEL(fmt, F, G, 1) PSN_STREAM_NORM_KERNEL(fmt, F, G, 2) PSN_STREAM_NORM_KERNEL(fmt, F, G, 3)
 #define PSN_STREAM_G(fmt, F, G) PSN_STREAM_KERNEL(fmt, F, G, 1) PSN_STREAM_KERNEL(fmt, F, G, 2) PSN_STREAM_KERNEL(fmt, F, G, 3) PSN_STREAM_KERNEL(fmt, F, G, 4)
-#define PSN_STREAM_ALL(fmt, F) PSN_STREAM_G(fmt, F, 8) PSN_STREAM_G(fmt, F, 16) PSN_STREAM_G(fmt, F, 32) PSN_STREAM_G(fmt, F, 64)
+#define PSN_STREAM_ALL(fmt, F) PSN_STREAM_G(fmt, F, 8) PSN_STREAM_G(fmt, F, 16) PSN_STREAM_G(fmt, F, 32) PSN_STREAM_G(fmt, F, 64) \
+    PSN_STREAM_NORM_G(fmt, F, 8) PSN_STREAM_NORM_G(fmt, F, 16) PSN_STREAM_NORM_G(fmt, F, 32)
 
 #define PSN_F32_KERNEL(fmt, F, G, R, NB)                                                                  \
     extern "C" __global__ void __launch_bounds__(512) psn_mv_##fmt##_f32_g##G##_r##R##_b##NB(const psn_matvec_args a) { \

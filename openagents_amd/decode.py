@@ -66,18 +66,22 @@ class DecodeStep:
     """Owns the activations, KV caches and scratch of one sequence and enqueues one token step."""
 
     def __init__(self, be: HipBackend, shape: LlamaShape, weights: ModelWeights, max_ctx: int, scheme: int = ACT_Q8,
-                 fused_quant: bool = True):
+                 fused_quant: bool = True, fused_norm: bool = True):
         """fused_quant (scheme Q8): the norm, attention and SwiGLU kernels emit their result already
         quantized, and the matvecs read it with the pre-quantized entry points; otherwise every matvec
-        quantizes its fp32 input itself."""
+        quantizes its fp32 input itself.  fused_norm (with fused_quant): the residual add and the RMSNorm
+        run inside the projection that consumes them (psn_qmatvec_norm_multi), the residual stream
+        alternating between two buffers."""
         self.be, self.shape, self.w, self.max_ctx, self.scheme = be, shape, weights, max_ctx, scheme
         self.fused = fused_quant and scheme == ACT_Q8
+        self.fused_norm = self.fused and fused_norm
         s = shape
         if s.n_heads * s.head_dim != s.hidden:
             raise ValueError("n_heads * head_dim must equal hidden")
         f32 = 4
         self.x = be.alloc(s.hidden * f32)            # residual stream
         self.xn = be.alloc(s.hidden * f32)           # normalized copy fed to the matvecs
+        self.x2 = be.alloc(s.hidden * f32)           # second residual buffer (norm-fused path)
         self.q = be.alloc(s.hidden * f32)
         self.k = be.alloc(s.kv_dim * f32)
         self.v = be.alloc(s.kv_dim * f32)
@@ -106,15 +110,33 @@ class DecodeStep:
 
     @property
     def launches_per_layer(self) -> int:
-        return 9 if self.fused else 10
+        return 7 if self.fused_norm else 9 if self.fused else 10
 
     @property
     def launches_outside_layers(self) -> int:
-        return 3 if self.fused else 2
+        return 2 if self.fused_norm else 3 if self.fused else 2
+
+    def _enqueue_norm_fused(self, pos: int):
+        """Seven launches per layer: q|k|v (with add + norm), attention partial, combine, o, gate|up (with
+        add + norm), SwiGLU, down.  The residual stream moves self.x -> self.x2 -> self.x within a layer."""
+        be, s, at = self.be, self.shape, self.act_type
+        be.rope_table(self.rope_tab, s.head_dim, pos, s.rope_theta)
+        for li, lw in enumerate(self.w.layers):
+            be.quantized_matvec_norm_multi([lw.wq, lw.wk, lw.wv], self.x, self.down if li > 0 else None, lw.attn_norm, self.x2,
+                                           [self.q, self.k, self.v], s.eps)
+            be.attention_decode_rope(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn, at,
+                                     s.n_heads, s.n_kv_heads, s.head_dim, pos, self.rope_tab)
+            be.quantized_matvec_q8(lw.wo, self.xq_attn, self.o, 1)
+            be.quantized_matvec_norm_multi([lw.w_gate, lw.w_up], self.x2, self.o, lw.ffn_norm, self.x, [self.gate, self.up], s.eps)
+            be.swiglu_q8(self.gate, self.up, None, self.xq_f, at, s.ffn)
+            be.quantized_matvec_q8(lw.w_down, self.xq_f, self.down, 1)
+        be.quantized_matvec_norm_multi([self.w.lm_head], self.x, self.down, self.w.final_norm, None, [self.logits], s.eps)
 
     def _enqueue_fused(self, pos: int, matvecs_only: bool):
         be, s, at = self.be, self.shape, self.act_type
         glue = not matvecs_only
+        if glue and self.fused_norm:
+            return self._enqueue_norm_fused(pos)
         if glue:
             be.rope_table(self.rope_tab, s.head_dim, pos, s.rope_theta)      # once per token
         for li, lw in enumerate(self.w.layers):
@@ -221,12 +243,13 @@ def main(argv=None):
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--unfused", action="store_true", help="every matvec quantizes its own fp32 input")
+    ap.add_argument("--separate-norm", action="store_true", help="RMSNorm as its own launch instead of inside the consuming projection")
     args = ap.parse_args(argv)
     be = HipBackend(0)
     shape = LlamaShape(n_layers=args.layers)
     t0 = time.time()
     weights = synthetic_weights(be, shape, args.seed)
-    step = DecodeStep(be, shape, weights, args.ctx, fused_quant=not args.unfused)
+    step = DecodeStep(be, shape, weights, args.ctx, fused_quant=not args.unfused, fused_norm=not args.separate_norm)
     rng = np.random.default_rng(args.seed + 1)
     pos = args.ctx - 1
     kv = rng.standard_normal((pos, shape.kv_dim), dtype=np.float32).astype(np.float16)

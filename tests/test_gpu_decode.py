@@ -246,6 +246,8 @@ def test_whole_small_decode_step_eager_and_graph(hip, orc):
     head = qmat(orc.Q6_K, s.vocab, s.hidden)
     weights = ModelWeights(dev_layers, hip.upload(final_norm), hip.upload_weight(orc.Q6_K, head, s.vocab, s.hidden))
     step = DecodeStep(hip, s, weights, ctx)
+    assert step.fused_norm and step.launches_per_layer == 7
+    separate = DecodeStep(hip, s, weights, ctx, fused_norm=False)
     unfused = DecodeStep(hip, s, weights, ctx, fused_quant=False)
     kv0 = [(rng.standard_normal((ctx, s.kv_dim), dtype=np.float32).astype(np.float16), rng.standard_normal((ctx, s.kv_dim), dtype=np.float32).astype(np.float16))
            for _ in range(s.n_layers)]
@@ -293,6 +295,13 @@ def test_whole_small_decode_step_eager_and_graph(hip, orc):
     unfused.x.upload(x0)
     unfused.enqueue(pos)
     assert G.max_rel_err(unfused.logits.download(np.float32, (s.vocab,)), eager) < 1e-3
+    # ... and so does the path whose norms are launches of their own
+    for li in range(s.n_layers):
+        separate.k_cache[li].upload(kv0[li][0])
+        separate.v_cache[li].upload(kv0[li][1])
+    separate.x.upload(x0)
+    separate.enqueue(pos)
+    assert G.max_rel_err(separate.logits.download(np.float32, (s.vocab,)), eager) < 1e-3
 
     graph = step.capture(pos)
     try:

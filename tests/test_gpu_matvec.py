@@ -499,3 +499,84 @@ def test_two_branch_graph_of_independent_launches(hip, orc):
     finally:
         hip.destroy_graph(graph)
         hip.destroy_stream(side)
+
+
+# ------------------------------------------------------------------ residual add + RMSNorm folded into the projection
+
+def norm_ref(x, delta, w, eps):
+    """fp32 restatement of the fused staging: h = x + delta; xn = h * (1 / sqrt(mean(h^2) + eps)) * w."""
+    h = (x + delta).astype(np.float32) if delta is not None else x.copy()
+    ms = np.float32(np.mean(h.astype(np.float64) ** 2))
+    scale = np.float32(1.0) / np.sqrt(ms + np.float32(eps), dtype=np.float32)
+    return h, (h * scale * w).astype(np.float32)
+
+
+@pytest.mark.parametrize("qname,ns,k", [
+    ("Q4_K", [4096, 1024, 1024], 4096),      # q | k | v
+    ("Q4_K", [14336, 14336], 4096),          # gate | up
+    ("Q4_0", [4096, 1024, 1024], 4096),      # Q8_0 activations
+    ("Q8_0", [1024, 1024], 2048),
+    ("Q6_K", [4096], 4096),                  # an LM-head slice
+    ("Q4_K", [2048, 512], 8192),             # 512-thread staging
+    ("Q4_K", [512, 256, 256], 512),          # two chunks per row
+    ("Q4_K", [4096], 14336),                 # rows too long for the fused kernels: two launches
+    ("Q4_0", [256, 256, 256, 256], 4096),    # four matrices: two launches
+    ("Q4_K", [1026], 4096),                  # not whole passes: two launches
+])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_norm_fused_projection_matches_oracle(hip, orc, qname, ns, k, with_delta):
+    qt = getattr(orc, qname)
+    rng = np.random.default_rng(4200 + k + len(ns))
+    x = rng.standard_normal(k, dtype=np.float32) * 2
+    delta = rng.standard_normal(k, dtype=np.float32) if with_delta else None
+    wn = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    eps = 1e-5
+    blocks = [weights(orc, qname, 4300 + i, n, k) for i, n in enumerate(ns)]
+    ws = [hip.upload_weight(qt, b, n, k) for b, n in zip(blocks, ns)]
+    ys = [hip.alloc(n * 4) for n in ns]
+    xb, wb = hip.upload(x), hip.upload(wn)
+    db = hip.upload(delta) if with_delta else None
+    hb = hip.alloc(k * 4)
+    say(f"norm-fused {qname} ns={ns} k={k} delta={with_delta}")
+    hip.quantized_matvec_norm_multi(ws, xb, db, wb, hb, ys, eps)
+    h_ref, xn_ref = norm_ref(x, delta, wn, eps)
+    assert np.array_equal(hb.download(np.float32, (k,)), h_ref)
+    assert np.array_equal(xb.download(np.float32, (k,)), x)                      # x is left alone
+    for b, n, y in zip(blocks, ns, ys):
+        ref = orc.matvec(qt, orc.ACT_Q8, b, xn_ref, n, k)
+        got = y.download(np.float32, (n,))
+        # the sum of squares is added up in another order than numpy's, so a rounding of the int8
+        # activations can flip now and then; far inside the gate
+        assert G.max_rel_err(got, ref) < 2e-4, (qname, n, k)
+    # the same through the separate launches: norm kernel with quantized output, then the pre-quantized matvec
+    at = backend.act_type_for(qt)
+    xq = hip.alloc(int(backend.actq_layout(at, k, 1).bytes))
+    x2 = hip.upload(x)
+    hip.add_rmsnorm_q8(x2, db, wb, None, xq, at, k, eps)
+    y2 = [hip.alloc(n * 4) for n in ns]
+    hip.quantized_matvec_q8_multi(ws, xq, y2, 1)
+    for n, y, yy in zip(ns, ys, y2):
+        assert G.max_rel_err(y.download(np.float32, (n,)), yy.download(np.float32, (n,))) < 2e-4
+    # without h_out
+    y3 = [hip.alloc(n * 4) for n in ns]
+    hip.quantized_matvec_norm_multi(ws, xb, db, wb, None, y3, eps)
+    for n, y, yy in zip(ns, ys, y3):
+        assert np.array_equal(y.download(np.float32, (n,)), yy.download(np.float32, (n,)))
+
+
+def test_norm_fused_projection_argument_errors(hip, orc):
+    k, n = 4096, 256
+    w = hip.upload_weight(orc.Q4_K, weights(orc, "Q4_K", 4400, n, k), n, k)
+    x, wn, y = hip.alloc(k * 4), hip.alloc(k * 4), hip.alloc(n * 4)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_norm_multi([w], x, None, wn, x, [y])                 # h_out aliases x
+    assert e.value.name == "PSN_E_INVALID_ARG"
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_norm_multi([w], x, x, wn, x, [y])
+    assert e.value.name == "PSN_E_INVALID_ARG"
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_norm_multi([w], x, None, hip.alloc(k * 2), None, [y])   # norm weights too short
+    assert e.value.name == "PSN_E_INVALID_ARG"
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_norm_multi([w], hip.alloc(k * 2), None, wn, None, [y])
+    assert e.value.name == "PSN_E_INVALID_ARG"
