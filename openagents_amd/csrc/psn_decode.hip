@@ -263,64 +263,48 @@ extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_att
 /* the same with the rotary embedding of q and k and the KV-cache append of the new token folded in */
 extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_rope(const psn_attn_args a) { attn_partial_body<true>(a); }
 
-/* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One workgroup of 128 threads per
- * head: the per-split (max, sum) pairs are fetched in parallel, the weights go through LDS, and the
- * partial outputs are summed eight loads at a time. */
-template <bool PAIR>
-PSN_DEV void attn_combine_body(const psn_attn_args &a) {
+/* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One wave per head, two heads per
+ * workgroup; a lane owns two output dims.  The splits are taken 32 at a time and everything a wave needs
+ * of them -- the (max, sum) pairs and its two dims of every partial output -- is requested before
+ * anything is used, so 32 splits cost one trip to memory; the running sums are rescaled when the maximum
+ * moves.  With a quantized output the two heads (256 consecutive values, one Q8_K super-block or eight
+ * Q8_0 blocks) are regrouped through LDS into the four-values-per-lane layout the quantizers work on. */
+extern "C" __global__ void __launch_bounds__(128) psn_attn_combine(const psn_attn_args a) {
     constexpr int D = 128;
-    __shared__ float wts_all[2][128];
-    __shared__ float red_all[2][4];
-    __shared__ float regroup[256];
-    const int hl = PAIR ? (threadIdx.x >> 7) : 0;             /* which of the workgroup's heads */
-    float *wts = wts_all[hl], *red = red_all[hl];
-    const int head = (PAIR ? 2 : 1) * blockIdx.x + hl, d = threadIdx.x & 127;
+    __shared__ float regroup[2 * D];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int head = min(2 * (int)blockIdx.x + w, a.n_heads - 1);      /* an odd head count: the spare wave repeats the last head */
     const float *base = a.partial + (int64_t)head * a.n_splits * (D + 2);
-    float num = 0.f, den = 0.f;
-    /* global max first (splits are few: a strided pass per thread, then a block reduce) */
-    float m = -INFINITY;
-    for (int s = d; s < a.n_splits; s += 128) m = fmaxf(m, base[(int64_t)s * (D + 2) + D]);
-    m = group_max<64>(m);
-    if ((d & 63) == 0) red[d >> 6] = m;
-    __syncthreads();
-    const float M = fmaxf(red[0], red[1]);
-    for (int s0 = 0; s0 < a.n_splits; s0 += 128) {
-        const int s = s0 + d;
-        float w = 0.f, l = 0.f;
-        if (s < a.n_splits) {
-            w = __expf(base[(int64_t)s * (D + 2) + D] - M);
-            l = base[(int64_t)s * (D + 2) + D + 1] * w;
+    float M = -INFINITY, n0 = 0.f, n1 = 0.f, den = 0.f;
+    for (int c0 = 0; c0 < a.n_splits; c0 += 32) {
+        const int cnt = min(32, a.n_splits - c0);
+        const float2 ml = *reinterpret_cast<const float2 *>(base + (int64_t)(c0 + min(lane, cnt - 1)) * (D + 2) + D);
+        float2 o[32];
+        UNROLL for (int u = 0; u < 32; ++u)
+            o[u] = *reinterpret_cast<const float2 *>(base + (int64_t)(c0 + min(u, cnt - 1)) * (D + 2) + 2 * lane);
+        const float Mn = fmaxf(M, group_max<64>(lane < cnt ? ml.x : -INFINITY));
+        const float keep = __expf(M - Mn);                            /* 0 on the first round (M = -inf) */
+        const float wt = lane < cnt ? __expf(ml.x - Mn) : 0.f;
+        n0 *= keep;
+        n1 *= keep;
+        den = den * keep + group_sum<64>(ml.y * wt);
+        UNROLL for (int u = 0; u < 32; ++u) {
+            const float wi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wt), u));   /* 0 past cnt */
+            n0 += wi * o[u].x;
+            n1 += wi * o[u].y;
         }
-        __syncthreads();                                          /* wts from the previous round is consumed */
-        wts[d] = w;
-        l = group_sum<64>(l);
-        if ((d & 63) == 0) red[2 + (d >> 6)] = l;
-        __syncthreads();
-        den += red[2] + red[3];
-        const int cnt = min(128, a.n_splits - s0);
-        for (int i0 = 0; i0 < cnt; i0 += 8) {
-            float o[8];
-            UNROLL for (int u = 0; u < 8; ++u) o[u] = base[(int64_t)(s0 + min(i0 + u, cnt - 1)) * (D + 2) + d];
-            UNROLL for (int u = 0; u < 8; ++u) if (i0 + u < cnt) num += o[u] * wts[i0 + u];
-        }
+        M = Mn;
     }
-    const float o = num / den;
-    if (a.out) a.out[head * D + d] = o;
-    if constexpr (PAIR) {
-        /* two heads = one 256-element super-block (or eight 32-element blocks): regroup through LDS so
-         * that wave 0 holds it four values per lane, the layout the quantizers work on */
-        regroup[threadIdx.x] = o;
+    const float r0 = n0 / den, r1 = n1 / den;
+    const bool mine = 2 * (int)blockIdx.x + w < a.n_heads;
+    if (a.out && mine) *reinterpret_cast<float2 *>(a.out + head * D + 2 * lane) = make_float2(r0, r1);
+    if (a.qout.qs) {                                                     /* the host asks for this with an even head count only */
+        regroup[w * D + 2 * lane] = r0;
+        regroup[w * D + 2 * lane + 1] = r1;
         __syncthreads();
-        if (threadIdx.x < 64) {
-            const float4 v = *reinterpret_cast<const float4 *>(&regroup[4 * threadIdx.x]);
-            quantize_out4(a.qout, blockIdx.x * 64 + threadIdx.x, v);
-        }
+        if (w == 0) quantize_out4(a.qout, blockIdx.x * 64 + lane, *reinterpret_cast<const float4 *>(&regroup[4 * lane]));
     }
 }
-
-extern "C" __global__ void __launch_bounds__(128) psn_attn_combine(const psn_attn_args a) { attn_combine_body<false>(a); }
-/* two heads per workgroup, quantized output as well */
-extern "C" __global__ void __launch_bounds__(256) psn_attn_combine_q8(const psn_attn_args a) { attn_combine_body<true>(a); }
 
 /* out = silu(gate) * up */
 extern "C" __global__ void __launch_bounds__(256) psn_swiglu(const psn_swiglu_args a) {

@@ -1420,8 +1420,7 @@ static int32_t attention_impl(psn_module *mod, psn_stream *s, const psn_buf *q, 
     if ((rc = launch(mod, s, rope ? "psn_attn_partial_rope" : "psn_attn_partial", (unsigned)(n_kv_heads * splits),
                      (unsigned)(64 * group), 0, &a)))
         return rc;
-    if (out_q) return launch(mod, s, "psn_attn_combine_q8", (unsigned)(n_heads / 2), 256, 0, &a);
-    return launch(mod, s, "psn_attn_combine", (unsigned)n_heads, 128, 0, &a);
+    return launch(mod, s, "psn_attn_combine", (unsigned)((n_heads + 1) / 2), 128, 0, &a);
 }
 extern "C" int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
                                         psn_buf *workspace, psn_buf *out, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx) {

@@ -241,8 +241,8 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
     digest = graph_digest(f"decode-step:l{layers}:ctx{ctx}:h{shape.hidden}:ffn{shape.ffn}:v{shape.vocab}",
                           *[protos[name] for name in sorted(protos)])
     launches = shape.n_layers * step.launches_per_layer + step.launches_outside_layers
-    rec = record(be, "decode.step.q4_K.b1", f"psn decode-step graph ({launches} launches: psn_mvs_q4_K_q8_*, psn_mvs_q6_K_q8_*, "
-                 "psn_add_rmsnorm_q8, psn_attn_partial_rope, psn_attn_combine_q8, psn_swiglu_q8, psn_rope_table)",
+    rec = record(be, "decode.step.q4_K.b1", f"psn decode-step graph ({launches} launches: psn_mvs_q4_K_q8_g*_xn_s*, psn_mvs_q4_K_q8_g*_lds_s1, "
+                 "psn_mvs_q6_K_q8_g16_xn_s1, psn_attn_partial_rope, psn_attn_combine, psn_swiglu, psn_rope_table)",
                  digest, 1e6 / t_full, shape={"layers": layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,
                                               "head_dim": shape.head_dim, "ffn": shape.ffn, "vocab": shape.vocab, "context": ctx,
                                               "weights": "Q4_K projections, Q6_K LM head"},
