@@ -49,7 +49,7 @@ typedef enum { PSN_Q4_0 = 2, PSN_Q8_0 = 8, PSN_Q4_K = 12, PSN_Q5_K = 13, PSN_Q6_
 /* how activations enter the dot product */
 typedef enum {
     PSN_ACT_F32 = 0, /* weights dequantized to fp32, fp32 FMA */
-    PSN_ACT_Q8 = 1   /* x quantized to Q8_0 (Q4_0/Q8_0 weights) or Q8_K (Q4_K/Q6_K), int8 dot */
+    PSN_ACT_Q8 = 1   /* x quantized to Q8_0 (Q4_0/Q8_0 weights) or Q8_K (Q4_K/Q5_K/Q6_K), int8 dot */
 } psn_act_scheme;
 typedef enum { PSN_LAYOUT_GGUF = 0 /* raw GGUF blocks, row-major [N][K/block] */ } psn_layout;
 

@@ -18,9 +18,9 @@ from dataclasses import dataclass
 import numpy as np
 
 from . import _ffi
-from ._ffi import (ACT_F32, ACT_Q8, LAYOUT_GGUF, Q4_0, Q4_K, Q6_K, Q8_0, Q8_K, MatvecPlan)  # noqa: F401
+from ._ffi import (ACT_F32, ACT_Q8, LAYOUT_GGUF, Q4_0, Q4_K, Q5_K, Q6_K, Q8_0, Q8_K, MatvecPlan)  # noqa: F401
 
-TYPE_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", Q8_K: "Q8_K"}
+TYPE_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", Q8_K: "Q8_K"}
 
 
 class PsnError(RuntimeError):

@@ -29,6 +29,7 @@ CODE_OBJECTS = [
     ("psn_mv_q4_0", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q4_0"]),
     ("psn_mv_q8_0", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q8_0"]),
     ("psn_mv_q4_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q4_K"]),
+    ("psn_mv_q5_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q5_K"]),
     ("psn_mv_q6_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q6_K"]),
     ("psn_pf_skinny", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=0"]),
     *[(f"psn_pf_{fmt}_{fam}", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", f"-DPSN_BUILD_PF={num}", f"-DPSN_BUILD_PF_{fmt.upper()}"])

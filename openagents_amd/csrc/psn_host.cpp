@@ -111,19 +111,20 @@ extern "C" int32_t psn_quantize_rows(int32_t qtype, const float *x, int64_t n, i
     return PSN_OK;
 }
 
-static bool is_weight_type(int32_t t) { return t == PSN_Q4_0 || t == PSN_Q8_0 || t == PSN_Q4_K || t == PSN_Q6_K; }
+static bool is_weight_type(int32_t t) { return t == PSN_Q4_0 || t == PSN_Q8_0 || t == PSN_Q4_K || t == PSN_Q5_K || t == PSN_Q6_K; }
 static const char *fmt_name(int32_t t) {
     switch (t) {
         case PSN_Q4_0: return "q4_0";
         case PSN_Q8_0: return "q8_0";
         case PSN_Q4_K: return "q4_K";
+        case PSN_Q5_K: return "q5_K";
         case PSN_Q6_K: return "q6_K";
         default: return "?";
     }
 }
 extern "C" int32_t psn_act_type_for(int32_t wt) {
     if (wt == PSN_Q4_0 || wt == PSN_Q8_0) return PSN_Q8_0;
-    if (wt == PSN_Q4_K || wt == PSN_Q6_K) return PSN_Q8_K;
+    if (wt == PSN_Q4_K || wt == PSN_Q5_K || wt == PSN_Q6_K) return PSN_Q8_K;
     return fail(PSN_E_UNSUPPORTED, "type %d is not a weight type", wt);
 }
 
@@ -569,7 +570,7 @@ extern "C" int32_t psn_weight_upload(psn_ctx *c, int32_t qtype, int64_t N, int64
     if (!out) return fail(PSN_E_INVALID_ARG, "psn_weight_upload: out is null");
     *out = nullptr;
     if (!c || !blocks || !s) return fail(PSN_E_INVALID_ARG, "psn_weight_upload: null argument");
-    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "psn_weight_upload: type %d is not Q4_0/Q8_0/Q4_K/Q6_K", qtype);
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "psn_weight_upload: type %d is not Q4_0/Q8_0/Q4_K/Q5_K/Q6_K", qtype);
     if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "psn_weight_upload: layout %d", layout);
     if (N <= 0) return fail(PSN_E_SHAPE, "N=%lld must be positive", (long long)N);
     const int64_t rb = psn_row_bytes(qtype, K);
@@ -635,7 +636,7 @@ extern "C" int32_t psn_act_quantize(psn_module *mod, psn_stream *s, int32_t act_
 }
 
 static int32_t check_matvec_shape(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch) {
-    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "matvec: type %d is not Q4_0/Q8_0/Q4_K/Q6_K", qtype);
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "matvec: type %d is not Q4_0/Q8_0/Q4_K/Q5_K/Q6_K", qtype);
     if (scheme != PSN_ACT_F32 && scheme != PSN_ACT_Q8) return fail(PSN_E_UNSUPPORTED, "matvec: activation scheme %d", scheme);
     if (N <= 0 || N > INT32_MAX / 2) return fail(PSN_E_SHAPE, "N=%lld must be in 1..2^30", (long long)N);
     if (batch < 1 || batch > 8) return fail(PSN_E_SHAPE, "batch=%d outside 1..8", batch);

@@ -490,6 +490,58 @@ struct FmtQ4_K {
     }
 };
 
+/* Q5_K: chunk = one 176-byte super-block (11 dwordx4): dword 0 = fp16 d | fp16 dmin, dwords 1..3 =
+ * Q4_K's scale/min field, dwords 4..11 = qh (bit j of byte l: fifth bit of element l of sub-block j),
+ * dwords 12..43 = the nibble bytes laid out as Q4_K's.  Values 0..31 stay unsigned for the int8 dot. */
+struct FmtQ5_K {
+    static constexpr int DW = 44, BYTES = 176, XR = 73;
+    typedef int16_t ActSum;
+    static PSN_DEV int d_per_col(int K) { return K >> 8; }
+    static PSN_DEV int s_per_col(int K) { return K >> 4; }
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 11; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    static PSN_DEV void load_x(const ActQ<int16_t> &x, int K, int col, int c, u32 (&xr)[XR]) { load_x_q8_K(x, K, col, c, xr); }
+    static PSN_DEV float dot(const u32 (&w)[DW], const u32 (&xr)[XR]) {
+        u32 sc[2], mn[2];
+        q4_K_scales(w[1], w[2], w[3], sc, mn);
+        int isum = 0, msum = 0;
+        UNROLL for (int i = 0; i < 8; ++i) {
+            const u32 b = xr[65 + i];
+            msum += byte_of(mn, i) * ((int)(int16_t)(b & 0xffffu) + ((int)b >> 16));
+        }
+        UNROLL for (int ch = 0; ch < 4; ++ch) {
+            int sl = 0, sh = 0;
+            UNROLL for (int i = 0; i < 8; ++i) {
+                const u32 q = w[12 + 8 * ch + i], h = w[4 + i];
+                /* bit 2ch (2ch + 1) of every qh byte moves to bit 4 of the same byte; what a shift drags
+                 * in from the neighbouring byte lands on other bits and is masked away */
+                const u32 lo = (q & 0x0f0f0f0fu) | (((h >> (2 * ch)) << 4) & 0x10101010u);
+                const u32 hi = ((q >> 4) & 0x0f0f0f0fu) | (((h >> (2 * ch + 1)) << 4) & 0x10101010u);
+                sl = dot4(lo, xr[16 * ch + i], sl);
+                sh = dot4(hi, xr[16 * ch + 8 + i], sh);
+            }
+            isum += byte_of(sc, 2 * ch) * sl + byte_of(sc, 2 * ch + 1) * sh;
+        }
+        const float dx = __uint_as_float(xr[64]);
+        const float d = h2f_lo(w[0]) * dx, dm = h2f_hi(w[0]) * dx;
+        return d * (float)isum - dm * (float)msum;
+    }
+    template <int SB>
+    static PSN_DEV void deq32(const u32 (&w)[DW], float (&o)[32]) {
+        u32 sc[2], mn[2];
+        q4_K_scales(w[1], w[2], w[3], sc, mn);
+        const float d = h2f_lo(w[0]) * (float)byte_of(sc, SB);
+        const float mv = h2f_hi(w[0]) * (float)byte_of(mn, SB);
+        constexpr int ch = SB >> 1, sh = (SB & 1) * 4;
+        UNROLL for (int i = 0; i < 8; ++i) UNROLL for (int b = 0; b < 4; ++b) {
+            const u32 v = ((w[12 + 8 * ch + i] >> (8 * b + sh)) & 0xfu) | (((w[4 + i] >> (8 * b + SB)) & 1u) << 4);
+            o[4 * i + b] = d * (float)v - mv;
+        }
+    }
+};
+
 /* Q6_K: chunk = one 210-byte super-block at a 2-byte-aligned address: ql[128] | qh[64] |
  * int8 scales[16] | fp16 d.  13 dwordx4 loads cover bytes 0..207.  sum (q-32)*x =
  * sum q*x - 32*bsum per 16-element group keeps the 6-bit values unsigned. */
@@ -926,6 +978,7 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
 
 template <> PSN_DEV void stream_load_chunk<FmtQ4_0>(u32 addr, u32 (&w)[FmtQ4_0::DW]) { stream_read_words<9>(addr, w); }
 template <> PSN_DEV void stream_load_chunk<FmtQ4_K>(u32 addr, u32 (&w)[FmtQ4_K::DW]) { stream_read_words<9>(addr, w); }
+template <> PSN_DEV void stream_load_chunk<FmtQ5_K>(u32 addr, u32 (&w)[FmtQ5_K::DW]) { stream_read_words<11>(addr, w); }
 template <> PSN_DEV void stream_load_chunk<FmtQ8_0>(u32 addr, u32 (&w)[FmtQ8_0::DW]) { stream_read_words<17>(addr, w); }
 /* Q6_K super-blocks are 210 bytes: a chunk starts on an even byte, not on a 16-byte word (gfx950 reads
  * LDS at any alignment); 13 words cover bytes 0..207, the fp16 d sits in the last two */
@@ -1073,6 +1126,11 @@ PSN_STREAM_ALL(q8_0, FmtQ8_0)
 PSN_Q8_ALL(q4_K, FmtQ4_K)
 PSN_F32_ALL(q4_K, FmtQ4_K)
 PSN_STREAM_ALL(q4_K, FmtQ4_K)
+#endif
+#if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q5_K)
+PSN_Q8_ALL(q5_K, FmtQ5_K)
+PSN_F32_ALL(q5_K, FmtQ5_K)
+PSN_STREAM_ALL(q5_K, FmtQ5_K)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_Q6_K)
 PSN_Q8_ALL(q6_K, FmtQ6_K)

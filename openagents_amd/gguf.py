@@ -23,7 +23,7 @@ MAX_DIMS = 4            # ggml tensors have at most four dimensions
 
 # ggml tensor types this module knows: id -> (elements per block, bytes per block, name)
 GGML_TYPES = {0: (1, 4, "F32"), 1: (1, 2, "F16"), 2: (32, 18, "Q4_0"), 8: (32, 34, "Q8_0"),
-              12: (256, 144, "Q4_K"), 14: (256, 210, "Q6_K")}
+              12: (256, 144, "Q4_K"), 13: (256, 176, "Q5_K"), 14: (256, 210, "Q6_K")}
 
 # metadata value types
 U8, I8, U16, I16, U32, I32, F32, BOOL, STRING, ARRAY, U64, I64, F64 = range(13)
@@ -166,7 +166,7 @@ class GGUFFile:
     def upload(self, backend, name: str):
         """Upload a quantized 2-D tensor [n, k]; returns backend.QuantizedTensor."""
         t = self.tensors[name]
-        if t.ggml_type not in (2, 8, 12, 14):
+        if t.ggml_type not in (2, 8, 12, 13, 14):
             raise GGUFError(f"tensor {name}: type {GGML_TYPES.get(t.ggml_type, (0, 0, t.ggml_type))[2]} is not a quantized weight format of this backend")
         return backend.upload_weight(t.ggml_type, self.data(name), t.n, t.k)
 

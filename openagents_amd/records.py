@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 TARGET_MODEL = "llama-3-8b-shaped-synthetic"
 DEVICE_CLASS = "hip"
-FMT_NAME = {Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", Q6_K: "q6_K"}
+FMT_NAME = {Q4_0: "q4_0", Q8_0: "q8_0", Q4_K: "q4_K", _ffi.Q5_K: "q5_K", Q6_K: "q6_K"}
 
 
 def hardware_ref(be: HipBackend) -> str:

@@ -14,10 +14,10 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libpsn_oracle.so")
 
-Q4_0, Q8_0, Q4_K, Q6_K, Q8_K = 2, 8, 12, 14, 15
+Q4_0, Q8_0, Q4_K, Q5_K, Q6_K, Q8_K = 2, 8, 12, 13, 14, 15
 ACT_F32, ACT_Q8 = 0, 1
-WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q6_K)
-TYPE_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q6_K: "Q6_K", Q8_K: "Q8_K"}
+WEIGHT_TYPES = (Q4_0, Q8_0, Q4_K, Q5_K, Q6_K)
+TYPE_NAMES = {Q4_0: "Q4_0", Q8_0: "Q8_0", Q4_K: "Q4_K", Q5_K: "Q5_K", Q6_K: "Q6_K", Q8_K: "Q8_K"}
 
 
 def build(force: bool = False) -> str:
@@ -48,6 +48,7 @@ def lib() -> C.CDLL:
         L.orc_q4k_scale_min.argtypes = [vp, vp, vp]; L.orc_q4k_scale_min.restype = None
         L.orc_q4k_fit_subblock.argtypes = [vp, vp, C.POINTER(C.c_float)]; L.orc_q4k_fit_subblock.restype = f32
         L.orc_q6k_fit_subblock.argtypes = [vp, vp]; L.orc_q6k_fit_subblock.restype = f32
+        L.orc_q5k_fit_subblock.argtypes = [vp, vp, C.POINTER(C.c_float)]; L.orc_q5k_fit_subblock.restype = f32
         L.orc_vec_dot_q.argtypes = [i32, vp, vp, i64]; L.orc_vec_dot_q.restype = f32
         L.orc_matvec.argtypes = [i32, i32, vp, vp, vp, i64, i64, i32, i32]; L.orc_matvec.restype = i32
         L.orc_matvec_f64.argtypes = [i32, vp, vp, vp, i64, i64, i32, i32]; L.orc_matvec_f64.restype = i32
@@ -135,6 +136,16 @@ def q4k_fit_subblock(x32: np.ndarray):
     L = np.zeros(32, dtype=np.uint8)
     mn = C.c_float()
     sc = lib().orc_q4k_fit_subblock(_p(x), _p(L), C.byref(mn))
+    return float(sc), float(mn.value), L
+
+
+def q5k_fit_subblock(x32: np.ndarray):
+    """(scale, min, L[32]) of one Q5_K sub-block: x ~ scale * L - min, L in 0..31."""
+    x = np.ascontiguousarray(x32, dtype=np.float32)
+    assert x.size == 32
+    L = np.zeros(32, dtype=np.uint8)
+    mn = C.c_float()
+    sc = lib().orc_q5k_fit_subblock(_p(x), _p(L), C.byref(mn))
     return float(sc), float(mn.value), L
 
 

@@ -26,6 +26,7 @@
 typedef struct { uint16_t d; int8_t qs[QK]; } blk_q8_0;
 typedef struct { uint16_t d; uint8_t qs[QK / 2]; } blk_q4_0;
 typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qs[QKK / 2]; } blk_q4_K;
+typedef struct { uint16_t d; uint16_t dmin; uint8_t scales[12]; uint8_t qh[QKK / 8]; uint8_t qs[QKK / 2]; } blk_q5_K;
 typedef struct { uint8_t ql[QKK / 2]; uint8_t qh[QKK / 4]; int8_t scales[QKK / 16]; uint16_t d; } blk_q6_K;
 typedef struct { float d; int8_t qs[QKK]; int16_t bsums[QKK / 16]; } blk_q8_K;
 #pragma pack(pop)
@@ -33,6 +34,7 @@ typedef struct { float d; int8_t qs[QKK]; int16_t bsums[QKK / 16]; } blk_q8_K;
 _Static_assert(sizeof(blk_q8_0) == 34, "q8_0");
 _Static_assert(sizeof(blk_q4_0) == 18, "q4_0");
 _Static_assert(sizeof(blk_q4_K) == 144, "q4_K");
+_Static_assert(sizeof(blk_q5_K) == 176, "q5_K");
 _Static_assert(sizeof(blk_q6_K) == 210, "q6_K");
 _Static_assert(sizeof(blk_q8_K) == 292, "q8_K");
 
@@ -98,7 +100,7 @@ static inline int imax(int a, int b) { return a > b ? a : b; }
 int64_t orc_block_elems(int32_t t) {
     switch (t) {
         case ORC_Q4_0: case ORC_Q8_0: return QK;
-        case ORC_Q4_K: case ORC_Q6_K: case ORC_Q8_K: return QKK;
+        case ORC_Q4_K: case ORC_Q5_K: case ORC_Q6_K: case ORC_Q8_K: return QKK;
         default: return 0;
     }
 }
@@ -107,6 +109,7 @@ int64_t orc_block_bytes(int32_t t) {
         case ORC_Q4_0: return sizeof(blk_q4_0);
         case ORC_Q8_0: return sizeof(blk_q8_0);
         case ORC_Q4_K: return sizeof(blk_q4_K);
+        case ORC_Q5_K: return sizeof(blk_q5_K);
         case ORC_Q6_K: return sizeof(blk_q6_K);
         case ORC_Q8_K: return sizeof(blk_q8_K);
         default: return 0;
@@ -296,6 +299,62 @@ static void quant_q4_K(const float *x, blk_q4_K *y, int64_t k) {
     }
 }
 
+/* One 32-element Q5_K sub-block: the same importance weights, 32 levels, 16 candidates from rmin -0.5. */
+float orc_q5k_fit_subblock(const float *x, uint8_t *L, float *min_out) {
+    uint8_t Ltry[32];
+    float w[32], s2 = 0.f;
+    for (int l = 0; l < 32; l++) s2 += x[l] * x[l];
+    float av = sqrtf(s2 / 32.f);
+    for (int l = 0; l < 32; l++) w[l] = av + fabsf(x[l]);
+    return fit_scale_min(32, 31, x, w, L, min_out, Ltry, -0.5f, 0.1f, 15);
+}
+
+/* Q5_K: Q4_K's super-block with a fifth bit per weight.  Sub-block scales/mins are packed exactly as in
+ * Q4_K; the low four bits of the eight sub-blocks share qs like Q4_K's nibbles (sub-blocks 2c, 2c+1 in
+ * bytes 32c..32c+31), bit (2c) / (2c+1) of qh[l] is the fifth bit of element l of sub-block 2c / 2c+1. */
+static void quant_q5_K(const float *x, blk_q5_K *y, int64_t k) {
+    uint8_t L[QKK];
+    float mins[8], scales[8];
+    for (int64_t b = 0; b < k / QKK; b++) {
+        const float *xb = x + b * QKK;
+        float max_scale = 0.f, max_min = 0.f;
+        for (int j = 0; j < 8; j++) {
+            scales[j] = orc_q5k_fit_subblock(xb + 32 * j, L + 32 * j, &mins[j]);
+            if (scales[j] > max_scale) max_scale = scales[j];
+            if (mins[j] > max_min) max_min = mins[j];
+        }
+        float inv_scale = max_scale > 0.f ? 63.f / max_scale : 0.f;
+        float inv_min = max_min > 0.f ? 63.f / max_min : 0.f;
+        memset(y[b].scales, 0, 12);
+        for (int j = 0; j < 8; j++) {
+            uint8_t ls = (uint8_t)imin(63, orc_nearest_int(inv_scale * scales[j]));
+            uint8_t lm = (uint8_t)imin(63, orc_nearest_int(inv_min * mins[j]));
+            q4k_pack_scale_min(j, ls, lm, y[b].scales);
+        }
+        y[b].d = orc_fp32_to_fp16(max_scale / 63.f);
+        y[b].dmin = orc_fp32_to_fp16(max_min / 63.f);
+        uint8_t sc[8], mn[8];
+        orc_q4k_scale_min(y[b].scales, sc, mn);
+        for (int j = 0; j < 8; j++) {
+            float d = h2f(y[b].d) * (float)sc[j];
+            if (d == 0.f) continue;
+            float dm = h2f(y[b].dmin) * (float)mn[j];
+            for (int l = 0; l < 32; l++) {
+                int q = orc_nearest_int((xb[32 * j + l] + dm) / d);
+                L[32 * j + l] = (uint8_t)imax(0, imin(31, q));
+            }
+        }
+        memset(y[b].qh, 0, sizeof y[b].qh);
+        for (int c = 0; c < 4; c++)
+            for (int l = 0; l < 32; l++) {
+                int l1 = L[64 * c + l], l2 = L[64 * c + 32 + l];
+                if (l1 > 15) { l1 -= 16; y[b].qh[l] |= (uint8_t)(1u << (2 * c)); }
+                if (l2 > 15) { l2 -= 16; y[b].qh[l] |= (uint8_t)(2u << (2 * c)); }
+                y[b].qs[32 * c + l] = (uint8_t)(l1 | (l2 << 4));
+            }
+    }
+}
+
 /* symmetric fit x ~ scale*(L-nmax), L-nmax in [-nmax, nmax-1], weights x^2;
  * 19 candidate spacings around -nmax/max.  Published reference search for Q6_K. */
 static float fit_scale_sym(int n, int nmax, const float *x, int8_t *L) {
@@ -384,6 +443,7 @@ int32_t orc_quantize_row(int32_t t, const float *x, void *y, int64_t k) {
         case ORC_Q8_0: quant_q8_0(x, (blk_q8_0 *)y, k); return 0;
         case ORC_Q4_0: quant_q4_0(x, (blk_q4_0 *)y, k); return 0;
         case ORC_Q4_K: quant_q4_K(x, (blk_q4_K *)y, k); return 0;
+        case ORC_Q5_K: quant_q5_K(x, (blk_q5_K *)y, k); return 0;
         case ORC_Q6_K: quant_q6_K(x, (blk_q6_K *)y, k); return 0;
         case ORC_Q8_K: quant_q8_K(x, (blk_q8_K *)y, k); return 0;
         default: return -1;
@@ -432,6 +492,22 @@ static void deq_q4_K(const blk_q4_K *x, float *y, int64_t k) {
         }
     }
 }
+static void deq_q5_K(const blk_q5_K *x, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / QKK; b++) {
+        float d = h2f(x[b].d), dmin = h2f(x[b].dmin);
+        uint8_t sc[8], mn[8];
+        orc_q4k_scale_min(x[b].scales, sc, mn);
+        for (int c = 0; c < 4; c++) {
+            float d1 = d * (float)sc[2 * c], m1 = dmin * (float)mn[2 * c];
+            float d2 = d * (float)sc[2 * c + 1], m2 = dmin * (float)mn[2 * c + 1];
+            for (int l = 0; l < 32; l++) {
+                uint8_t q = x[b].qs[32 * c + l], h = x[b].qh[l];
+                y[b * QKK + 64 * c + l] = d1 * (float)((q & 0xF) + ((h >> (2 * c)) & 1) * 16) - m1;
+                y[b * QKK + 64 * c + 32 + l] = d2 * (float)((q >> 4) + ((h >> (2 * c + 1)) & 1) * 16) - m2;
+            }
+        }
+    }
+}
 static void deq_q6_K(const blk_q6_K *x, float *y, int64_t k) {
     for (int64_t b = 0; b < k / QKK; b++) {
         float d = h2f(x[b].d);
@@ -464,6 +540,7 @@ int32_t orc_dequantize_row(int32_t t, const void *x, float *y, int64_t k) {
         case ORC_Q8_0: deq_q8_0((const blk_q8_0 *)x, y, k); return 0;
         case ORC_Q4_0: deq_q4_0((const blk_q4_0 *)x, y, k); return 0;
         case ORC_Q4_K: deq_q4_K((const blk_q4_K *)x, y, k); return 0;
+        case ORC_Q5_K: deq_q5_K((const blk_q5_K *)x, y, k); return 0;
         case ORC_Q6_K: deq_q6_K((const blk_q6_K *)x, y, k); return 0;
         case ORC_Q8_K: deq_q8_K((const blk_q8_K *)x, y, k); return 0;
         default: return -1;
@@ -514,6 +591,27 @@ static float dot_q4_K_q8_K(const blk_q4_K *w, const blk_q8_K *x, int64_t k) {
     }
     return acc;
 }
+static float dot_q5_K_q8_K(const blk_q5_K *w, const blk_q8_K *x, int64_t k) {
+    float acc = 0.f;
+    for (int64_t b = 0; b < k / QKK; b++) {
+        uint8_t sc[8], mn[8];
+        orc_q4k_scale_min(w[b].scales, sc, mn);
+        int32_t isum = 0, msum = 0;
+        for (int c = 0; c < 4; c++) {
+            int32_t s_lo = 0, s_hi = 0;
+            for (int l = 0; l < 32; l++) {
+                uint8_t q = w[b].qs[32 * c + l], h = w[b].qh[l];
+                s_lo += (int)((q & 0xF) + ((h >> (2 * c)) & 1) * 16) * (int)x[b].qs[64 * c + l];
+                s_hi += (int)((q >> 4) + ((h >> (2 * c + 1)) & 1) * 16) * (int)x[b].qs[64 * c + 32 + l];
+            }
+            isum += (int32_t)sc[2 * c] * s_lo + (int32_t)sc[2 * c + 1] * s_hi;
+        }
+        for (int j = 0; j < 8; j++) msum += (int32_t)mn[j] * ((int32_t)x[b].bsums[2 * j] + (int32_t)x[b].bsums[2 * j + 1]);
+        float d = h2f(w[b].d) * x[b].d, dm = h2f(w[b].dmin) * x[b].d;
+        acc += d * (float)isum - dm * (float)msum;
+    }
+    return acc;
+}
 static float dot_q6_K_q8_K(const blk_q6_K *w, const blk_q8_K *x, int64_t k) {
     float acc = 0.f;
     for (int64_t b = 0; b < k / QKK; b++) {
@@ -545,6 +643,7 @@ float orc_vec_dot_q(int32_t t, const void *w, const void *xq, int64_t k) {
         case ORC_Q4_0: return dot_q4_0_q8_0((const blk_q4_0 *)w, (const blk_q8_0 *)xq, k);
         case ORC_Q8_0: return dot_q8_0_q8_0((const blk_q8_0 *)w, (const blk_q8_0 *)xq, k);
         case ORC_Q4_K: return dot_q4_K_q8_K((const blk_q4_K *)w, (const blk_q8_K *)xq, k);
+        case ORC_Q5_K: return dot_q5_K_q8_K((const blk_q5_K *)w, (const blk_q8_K *)xq, k);
         case ORC_Q6_K: return dot_q6_K_q8_K((const blk_q6_K *)w, (const blk_q8_K *)xq, k);
         default: return NAN;
     }
@@ -552,7 +651,7 @@ float orc_vec_dot_q(int32_t t, const void *w, const void *xq, int64_t k) {
 
 /* ---------------------------------------------------------------- matvec */
 
-static int is_weight_type(int32_t t) { return t == ORC_Q4_0 || t == ORC_Q8_0 || t == ORC_Q4_K || t == ORC_Q6_K; }
+static int is_weight_type(int32_t t) { return t == ORC_Q4_0 || t == ORC_Q8_0 || t == ORC_Q4_K || t == ORC_Q5_K || t == ORC_Q6_K; }
 static int32_t act_type_for(int32_t wt) { return (wt == ORC_Q4_0 || wt == ORC_Q8_0) ? ORC_Q8_0 : ORC_Q8_K; }
 
 int32_t orc_matvec(int32_t wt, int32_t scheme, const void *W, const float *x, float *y,

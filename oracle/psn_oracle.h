@@ -12,7 +12,7 @@
  * (/root/reference/docs/muse/muse-glimmer.md:112) and the `--backend cpu|cuda|metal`
  * switch (/root/reference/apps/pylon/docs/2026-06-09-pylon-qwen35-local-inference-roadmap.md:137-150).
  * The functions below therefore restate the PUBLISHED GGUF block formats
- * (Q8_0, Q4_0, Q4_K, Q6_K weights; Q8_0, Q8_K activations) and the published
+ * (Q8_0, Q4_0, Q4_K, Q5_K, Q6_K weights; Q8_0, Q8_K activations) and the published
  * reference quantizers / integer dot products for them.
  *
  * Parity status per function (what pins it, since the reference holds no
@@ -23,7 +23,8 @@
  *   Q8_K quantize ............ pinned: closed form + bsums invariant
  *   all dequantizers ......... pinned: independent bit-level packers (pack o unpack = id),
  *                              one-hot lane/nibble-order tests
- *   Q4_K / Q6_K quantize ..... pinned by what the mathematics fixes (tests/test_oracle_kquant_search.py):
+ *   Q4_K / Q5_K / Q6_K quantize  pinned by what the mathematics fixes (tests/test_oracle_kquant_search.py;
+ *                              Q5_K shares Q4_K's search code with 32 levels and 16 candidates from -0.5):
  *                              sub-blocks and whole super-blocks that lie on the format's grid round-trip
  *                              exactly (levels, 6-bit / int8 scales, fp16 d and dmin); the (scale, min)
  *                              returned for a set of levels is the weighted least-squares fit
@@ -49,7 +50,7 @@ extern "C" {
 #endif
 
 /* GGUF tensor type ids */
-enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q6_K = 14, ORC_Q8_K = 15 };
+enum { ORC_Q4_0 = 2, ORC_Q8_0 = 8, ORC_Q4_K = 12, ORC_Q5_K = 13, ORC_Q6_K = 14, ORC_Q8_K = 15 };
 /* activation schemes */
 enum { ORC_ACT_F32 = 0, ORC_ACT_Q8 = 1 };
 
@@ -78,6 +79,8 @@ void orc_q4k_scale_min(const uint8_t *scales12, uint8_t sc[8], uint8_t mn[8]);
  * Q6_K: x[16] ~ scale * (L - 32), L in 0..63, returns scale, writes L. */
 float orc_q4k_fit_subblock(const float *x32, uint8_t *L, float *min_out);
 float orc_q6k_fit_subblock(const float *x16, int8_t *L);
+/* Q5_K: as Q4_K with L in 0..31 */
+float orc_q5k_fit_subblock(const float *x32, uint8_t *L, float *min_out);
 
 /* integer dot of one quantized weight row with one quantized activation row */
 float orc_vec_dot_q(int32_t wtype, const void *w, const void *xq, int64_t k);

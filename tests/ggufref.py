@@ -105,6 +105,40 @@ def parse_q4_K(rows, k):
     return d, dmin, sc, mn, q
 
 
+# ---------------------------------------------------------------------- Q5_K
+
+def pack_q5_K(d, dmin, sc, mn, q):
+    """q[256] in 0..31 in element order.  Layout from the format's description: fp16 d, fp16 dmin, the
+    12-byte scale field of Q4_K, qh[32] (bit j of qh[l] = fifth bit of element l of sub-block j), qs[128]
+    (low nibble of byte 32c+l = element l of sub-block 2c, high nibble = element l of sub-block 2c+1)."""
+    out = np.zeros(176, dtype=np.uint8)
+    out[0:2] = f16_bytes(d)
+    out[2:4] = f16_bytes(dmin)
+    out[4:16] = pack_q4k_scales(sc, mn)
+    for e in range(256):
+        sb, l = divmod(e, 32)
+        v = int(q[e])
+        out[16 + l] |= np.uint8((v >> 4) << sb)
+        out[48 + 32 * (sb // 2) + l] |= np.uint8((v & 15) << (4 * (sb % 2)))
+    return out
+
+
+def expected_q5_K(d, dmin, sc, mn, q):
+    return expected_q4_K(d, dmin, sc, mn, q)          # same arithmetic, q runs to 31
+
+
+def parse_q5_K(rows, k):
+    """-> d, dmin float64 [n, nb]; sc, mn int64 [n, nb, 8]; q int64 [n, nb, 256] (element order, 0..31)."""
+    n = rows.shape[0]
+    nb = k // 256
+    b = rows.reshape(n, nb, 176)
+    as144 = np.concatenate([b[:, :, :16], b[:, :, 48:]], axis=2).reshape(n, nb * 144)
+    d, dmin, sc, mn, q4 = parse_q4_K(as144, k)
+    qh = b[:, :, 16:48].astype(np.int64)                                    # [n, nb, 32]
+    hi = np.stack([(qh >> j) & 1 for j in range(8)], axis=2).reshape(n, nb, 256)
+    return d, dmin, sc, mn, q4 + 16 * hi
+
+
 # ---------------------------------------------------------------------- Q6_K
 
 def pack_q6_K(d, scales, L):

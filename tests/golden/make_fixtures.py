@@ -17,7 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 N, K, BATCH, M = 8, 512, 2, 4
-FORMATS = {"q4_0": 2, "q8_0": 8, "q4_K": 12, "q6_K": 14}
+FORMATS = {"q4_0": 2, "q8_0": 8, "q4_K": 12, "q6_K": 14, "q5_K": 13}      # appended in this order: a format's seed is its position
 
 
 def inputs(seed):

@@ -16,7 +16,7 @@ def make_file(orc, path, alignment=32):
     k = 1024
     tensors, raw = [], {}
     for name, t, n in (("blk.0.attn_q.weight", orc.Q4_0, 48), ("blk.0.ffn_down.weight", orc.Q4_K, 40),
-                       ("output.weight", orc.Q6_K, 72), ("blk.0.attn_k.weight", orc.Q8_0, 16)):
+                       ("output.weight", orc.Q6_K, 72), ("blk.0.attn_k.weight", orc.Q8_0, 16), ("blk.0.ffn_up.weight", orc.Q5_K, 24)):
         blocks = orc.quantize(t, G.seeded_weights(1000 + n, n, k))
         raw[name] = (t, n, k, blocks)
         tensors.append((name, (k, n), t, blocks))
@@ -49,7 +49,7 @@ def test_round_trip_header_metadata_and_tensor_bytes(orc, tmp_path, alignment):
     assert np.array_equal(f.data("output_norm.weight").view(np.float32), norm)
     # the first bytes are exactly the documented header
     head = open(path, "rb").read(24)
-    assert head[:4] == b"GGUF" and struct.unpack("<IQQ", head[4:]) == (3, 5, 9 + (alignment != 32))
+    assert head[:4] == b"GGUF" and struct.unpack("<IQQ", head[4:]) == (3, 6, 9 + (alignment != 32))
 
 
 def test_malformed_files_are_rejected(orc, tmp_path):
@@ -90,8 +90,9 @@ def test_malformed_files_are_rejected(orc, tmp_path):
             gguf.tensor_nbytes(2, dims)
     with pytest.raises(gguf.GGUFError):
         gguf.write_gguf(str(tmp_path / "x.gguf"), {}, [("t", (100, 4), 2, np.zeros(10, np.uint8))])   # ragged row
+    assert gguf.tensor_nbytes(13, (256, 4)) == 4 * 176                                                # Q5_K
     with pytest.raises(gguf.GGUFError):
-        gguf.tensor_nbytes(13, (256, 4))                                                              # Q5_K: not supported
+        gguf.tensor_nbytes(10, (256, 4))                                                              # Q2_K: not supported
 
 
 @pytest.mark.gpu

@@ -12,7 +12,7 @@ import ggufref as G
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "psn_golden.npz")
 N, K = 8, 512
-FORMATS = {"q4_0": 2, "q8_0": 8, "q4_K": 12, "q6_K": 14}
+FORMATS = {"q4_0": 2, "q8_0": 8, "q4_K": 12, "q6_K": 14, "q5_K": 13}
 
 
 @pytest.fixture(scope="module")

@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 
 GATE = 1e-3          # the stated bar
 PARITY_TOL = 2e-5    # what is asserted
-FORMATS = ["Q4_0", "Q8_0", "Q4_K", "Q6_K"]
+FORMATS = ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"]
 
 
 def say(msg):
@@ -152,6 +152,19 @@ def test_q4_K_small_batch_shapes(hip, orc, n, k, batch):
     x = G.seeded_acts(421, batch, k)
     for scheme in (_ffi.ACT_Q8, _ffi.ACT_F32):
         err = G.max_rel_err(hip.matvec_host(orc.Q4_K, W, x, n, k, scheme), orc.matvec(orc.Q4_K, scheme, W, x, n, k))
+        say(f"  scheme={scheme} max_rel_err={err:.3e}")
+        assert err < PARITY_TOL
+
+
+@pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("batch", [1, 2, 4, 8])
+def test_q5_K_small_batch_shapes(hip, orc, n, k, batch):
+    """Q5_K at the Q4_K configuration's shapes and batches (the format the served models also use)."""
+    say(f"Q5_K n={n} k={k} batch={batch}")
+    W = weights(orc, "Q5_K", 425, n, k)
+    x = G.seeded_acts(426, batch, k)
+    for scheme in (_ffi.ACT_Q8, _ffi.ACT_F32):
+        err = G.max_rel_err(hip.matvec_host(orc.Q5_K, W, x, n, k, scheme), orc.matvec(orc.Q5_K, scheme, W, x, n, k))
         say(f"  scheme={scheme} max_rel_err={err:.3e}")
         assert err < PARITY_TOL
 
@@ -406,7 +419,7 @@ def test_graph_replay_matches_eager(hip, orc):
 
 # ------------------------------------------------------------------ streaming (direct-to-LDS) kernels
 
-@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_streaming_kernels_every_variant(hip, orc, qname):
     """Weights land in per-wave rings of LDS buffers (1 to 4 passes in flight); rows per pass =
     64 / lanes_per_row, so the matrices hold multiples of 8 rows.  k = 2048 fills 8-lane groups exactly,
@@ -517,6 +530,7 @@ def norm_ref(x, delta, w, eps):
     ("Q4_0", [4096, 1024, 1024], 4096),      # Q8_0 activations
     ("Q8_0", [1024, 1024], 2048),
     ("Q6_K", [4096], 4096),                  # an LM-head slice
+    ("Q5_K", [2048, 512, 512], 4096),
     ("Q4_K", [2048, 512], 8192),             # 512-thread staging
     ("Q4_K", [512, 256, 256], 512),          # two chunks per row
     ("Q4_K", [4096], 14336),                 # rows too long for the fused kernels: two launches

@@ -60,8 +60,8 @@ def test_nearest_int_half_even(orc):
 
 
 def test_block_sizes(orc):
-    assert [orc.block_bytes(t) for t in (orc.Q8_0, orc.Q4_0, orc.Q4_K, orc.Q6_K, orc.Q8_K)] == [34, 18, 144, 210, 292]
-    assert [orc.block_elems(t) for t in (orc.Q8_0, orc.Q4_0, orc.Q4_K, orc.Q6_K, orc.Q8_K)] == [32, 32, 256, 256, 256]
+    assert [orc.block_bytes(t) for t in (orc.Q8_0, orc.Q4_0, orc.Q4_K, orc.Q5_K, orc.Q6_K, orc.Q8_K)] == [34, 18, 144, 176, 210, 292]
+    assert [orc.block_elems(t) for t in (orc.Q8_0, orc.Q4_0, orc.Q4_K, orc.Q5_K, orc.Q6_K, orc.Q8_K)] == [32, 32, 256, 256, 256, 256]
     assert orc.row_bytes(orc.Q4_0, 4096) == 2304 and orc.row_bytes(orc.Q6_K, 4096) == 3360
     with pytest.raises(ValueError):
         orc.row_bytes(orc.Q4_K, 4096 + 32)
@@ -212,6 +212,59 @@ def test_q4_K_quantizer_validity_and_error(orc):
     assert not orc.quantize(orc.Q4_K, np.zeros(256, np.float32))[:4].any()
 
 
+# ---------------------------------------------------------------- Q5_K
+
+def test_q5_K_dequant_against_element_index_packer(orc):
+    rng = np.random.default_rng(12)
+    for _ in range(20):
+        sc = rng.integers(0, 64, 8)
+        mn = rng.integers(0, 64, 8)
+        q = rng.integers(0, 32, 256)
+        d, dmin = 0.0123, 0.0071
+        blk = G.pack_q5_K(d, dmin, sc, mn, q)
+        y = orc.dequantize(orc.Q5_K, blk, 256)
+        assert np.array_equal(y, G.expected_q5_K(d, dmin, sc, mn, q).astype(np.float32))
+        dd, mm, s2, m2, q2 = G.parse_q5_K(blk.reshape(1, -1), 256)
+        assert np.array_equal(q2[0, 0], q) and np.array_equal(s2[0, 0], sc) and np.array_equal(m2[0, 0], mn)
+
+
+def test_q5_K_one_hot_positions_and_fifth_bit(orc):
+    for e in (0, 31, 32, 63, 64, 100, 200, 255):
+        for v in (9, 16, 31):                         # low nibble only, fifth bit only, both
+            q = np.zeros(256, np.int64)
+            q[e] = v
+            blk = G.pack_q5_K(1.0, 0.0, np.arange(1, 9), np.zeros(8, np.int64), q)
+            y = orc.dequantize(orc.Q5_K, blk, 256)
+            want = np.zeros(256, np.float32)
+            want[e] = float(v) * (e // 32 + 1)
+            assert np.array_equal(y, want), (e, v)
+    # the fifth bits of element l of all eight sub-blocks share byte qh[l]
+    q = np.zeros(256, np.int64)
+    q[5::32] = 16
+    blk = G.pack_q5_K(1.0, 0.0, np.ones(8, np.int64), np.zeros(8, np.int64), q)
+    assert blk[16 + 5] == 0xFF and not np.delete(blk[16:48], 5).any() and not blk[48:].any()
+
+
+def test_q5_K_quantizer_validity_and_error(orc):
+    w = G.seeded_weights(22, 8, 1024)
+    rows = orc.quantize(orc.Q5_K, w)
+    d, dmin, sc, mn, q = G.parse_q5_K(rows, 1024)
+    assert np.all(d >= 0) and np.all(dmin >= 0) and np.all(np.isfinite(d)) and np.all(np.isfinite(dmin))
+    assert sc.max() == 63 and mn.max() <= 63 and q.max() == 31 and q.min() == 0
+    y = orc.dequantize(orc.Q5_K, rows, 1024)
+    rel_rms = np.sqrt(np.mean((y - w) ** 2)) / np.sqrt(np.mean(w ** 2))
+    assert rel_rms < 0.045                              # about half of Q4_K's: one more bit
+    step = (d[:, :, None] * sc).repeat(32, axis=2).reshape(8, 1024)
+    assert np.all(np.abs(y - w) <= step + 1e-6)
+    assert not orc.quantize(orc.Q5_K, np.zeros(256, np.float32))[:4].any()
+    # the quantizer's bytes follow from its own sub-block fits (the search shared with Q4_K, 32 levels)
+    blk = w[0, :256]
+    fits = [orc.q5k_fit_subblock(blk[32 * j:32 * j + 32]) for j in range(8)]
+    max_scale, max_min = max(f[0] for f in fits), max(f[1] for f in fits)
+    assert np.float16(np.float32(max_scale) / np.float32(63.0)) == np.float16(d[0, 0])
+    assert np.float16(np.float32(max_min) / np.float32(63.0)) == np.float16(dmin[0, 0])
+
+
 # ---------------------------------------------------------------- Q6_K
 
 def test_q6_K_dequant_against_element_index_packer(orc):
@@ -250,7 +303,7 @@ def test_q6_K_quantizer_validity_and_error(orc):
     assert not orc.quantize(orc.Q6_K, np.zeros(256, np.float32)).any()
 
 
-@pytest.mark.parametrize("qname", ["Q8_0", "Q4_0", "Q4_K", "Q6_K"])
+@pytest.mark.parametrize("qname", ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_requantizing_dequantized_rows_is_stable(orc, qname):
     """deq(quant(x)) lies on the format's grid, so quantizing it again must reproduce values
     within one ulp of the scale's fp16 rounding -- catches an encoder/decoder that disagree."""

@@ -36,20 +36,24 @@ def lstsq_scale_min(x, w, L):
 
 
 def q4k_search(x, w):
+    return kmin_search(x, w, 15, -1.0, 20)
+
+
+def kmin_search(x, w, nmax, rmin, nstep):
     """The published search, stated from its description in float64 with numpy.linalg.lstsq as the fit:
-    start from the plain grid of 15 steps over [min(x, 0), max]; then for s = 0..20 round x onto the grid
-    with 14 + 0.1*s steps over [current offset, max], refit (scale, offset) by weighted least squares
+    start from the plain grid of nmax steps over [min(x, 0), max]; then for s = 0..nstep round x onto the grid
+    with nmax + rmin + 0.1*s steps over [current offset, max] (Q4_K: 15, -1.0, 20; Q5_K: 31, -0.5, 15), refit (scale, offset) by weighted least squares
     (offset <= 0) and keep the refit if its weighted error is smaller -- the kept offset becomes the
     lower end of the grids that follow.  Returns (levels, scale, offset, error, error of the plain grid, last step kept)."""
     xd = x.astype(np.float64)
     lo = min(float(xd.min()), 0.0)
     hi = float(xd.max())
-    L = np.clip(np.rint(15.0 / (hi - lo) * (xd - lo)), 0, 15)
-    scale = (hi - lo) / 15.0
+    L = np.clip(np.rint(float(nmax) / (hi - lo) * (xd - lo)), 0, nmax)
+    scale = (hi - lo) / float(nmax)
     best = plain = werr(x, w, scale * L + lo)
     last = -1
-    for s in range(21):
-        Lc = np.clip(np.rint((14.0 + 0.1 * s) / (hi - lo) * (xd - lo)), 0, 15)
+    for s in range(nstep + 1):
+        Lc = np.clip(np.rint((nmax + rmin + 0.1 * s) / (hi - lo) * (xd - lo)), 0, nmax)
         if np.ptp(Lc) == 0:
             continue
         a, b = lstsq_scale_min(x, w, Lc)
@@ -209,6 +213,66 @@ def test_q4_K_row_fields_follow_from_the_subblock_fits(orc):
                 near = np.clip(np.rint(ideal), 0, 15)
                 tie = np.abs(ideal - np.floor(ideal) - 0.5) < 1e-4
                 assert np.array_equal(q[r, b, 32 * j:32 * j + 32][~tie], near[~tie])
+
+
+# ------------------------------------------------------------------------------------ Q5_K
+
+def test_q5k_exact_grid_roundtrips_exactly(orc):
+    """A sub-block that already lies on a 32-level arithmetic grid must come back as that grid."""
+    rng = np.random.default_rng(25)
+    for scale, mn in ((0.25, 1.0), (0.5, 0.0), (0.03125, 0.21875), (2.0, 7.0)):
+        L = rng.integers(0, 32, 32)
+        L[0], L[1] = 0, 31
+        x = (np.float32(scale) * L.astype(np.float32) - np.float32(mn)).astype(np.float32)
+        s, m, got = orc.q5k_fit_subblock(x)
+        assert np.array_equal(got, L)
+        assert s == pytest.approx(scale, rel=1e-6) and m == pytest.approx(mn, rel=1e-6, abs=1e-7)
+    s, m, L = orc.q5k_fit_subblock(np.full(32, -0.75, np.float32))
+    assert s == 0.0 and m == 0.75 and not L.any()
+
+
+def test_q5k_result_is_the_outcome_of_the_published_search(orc):
+    """Same statement of the search as Q4_K's with 32 levels and 16 candidate spacings 30.5 .. 32.0."""
+    same = improved = n = n_refit = 0
+    for x in sub_blocks(26, 1200, 32):
+        s, m, L = orc.q5k_fit_subblock(x)
+        assert m >= 0.0 and s >= 0.0 and L.max() <= 31
+        w = q4k_weights(x)
+        got = werr(x, w, s * L.astype(np.float64) - m)
+        Lr, a, b, err, plain, last = kmin_search(x, w, 31, -0.5, 15)
+        assert got <= plain * (1 + 1e-5) + 1e-12
+        n += 1
+        improved += err < plain * (1 - 1e-3)
+        if np.array_equal(L, Lr):
+            same += 1
+            assert s == pytest.approx(a, rel=2e-4) and -m == pytest.approx(b, rel=2e-3, abs=2e-6 * max(1.0, abs(a) * 31))
+            assert got == pytest.approx(err, rel=2e-3, abs=1e-12)
+            if last >= 0:
+                n_refit += 1
+                a2, b2 = lstsq_scale_min(x, w, L)                      # and that fit is the least-squares line of its levels
+                assert s == pytest.approx(a2, rel=2e-4)
+    assert same >= 0.95 * n and improved > 0.4 * n and n_refit > 0.4 * n, (same, improved, n_refit, n)
+
+
+def test_q5_K_block_on_exact_grids_roundtrips_bit_exactly(orc):
+    rng = np.random.default_rng(27)
+    for d0, m0 in ((2.0 ** -6, 2.0 ** -7), (2.0 ** -9, 2.0 ** -5), (0.0078125, 0.0)):
+        kj = rng.integers(1, 64, 8)
+        nj = rng.integers(0, 64, 8) if m0 else np.zeros(8, np.int64)
+        kj[rng.integers(8)] = 63
+        if m0:
+            nj[rng.integers(8)] = 63
+        L = rng.integers(0, 32, (8, 32))
+        L[:, 0] = 0
+        L[:, 1] = 31
+        x = (np.float32(d0) * kj[:, None].astype(np.float32) * L.astype(np.float32)
+             - np.float32(m0) * nj[:, None].astype(np.float32)).astype(np.float32).reshape(256)
+        blk = orc.quantize(orc.Q5_K, x)
+        d, dmin, sc, mn, q = G.parse_q5_K(blk.reshape(1, -1), 256)
+        assert d[0, 0] == d0 and dmin[0, 0] == m0
+        assert np.array_equal(sc[0, 0], kj) and np.array_equal(mn[0, 0], nj)
+        assert np.array_equal(q[0, 0], L.reshape(256))
+        assert np.array_equal(orc.dequantize(orc.Q5_K, blk, 256), x)
 
 
 # ------------------------------------------------------------------------------------ Q6_K

@@ -12,7 +12,7 @@ import pytest
 
 import ggufref as G
 
-FORMATS = ["Q8_0", "Q4_0", "Q4_K", "Q6_K"]
+FORMATS = ["Q8_0", "Q4_0", "Q4_K", "Q5_K", "Q6_K"]
 
 
 def deq_numpy(orc, t, rows, k):
@@ -23,8 +23,8 @@ def deq_numpy(orc, t, rows, k):
     if t == orc.Q8_0:
         d, q = G.parse_q8_0(rows, k)
         return (d[:, :, None] * q).reshape(rows.shape[0], k)
-    if t == orc.Q4_K:
-        d, dmin, sc, mn, q = G.parse_q4_K(rows, k)
+    if t in (orc.Q4_K, orc.Q5_K):
+        d, dmin, sc, mn, q = (G.parse_q4_K if t == orc.Q4_K else G.parse_q5_K)(rows, k)
         n, nb = d.shape
         scale = (d[:, :, None] * sc).repeat(32, axis=2)
         minv = (dmin[:, :, None] * mn).repeat(32, axis=2)
@@ -85,8 +85,8 @@ def q8_exact(orc, t, rows, x, k):
         else:
             dx, qx, bs = G.parse_q8_K(orc.quantize(orc.Q8_K, x[b]), k)   # Q8_K itself is pinned in test_oracle_formats
             nb = k // 256
-            if t == orc.Q4_K:
-                d, dmin, sc, mn, q = G.parse_q4_K(rows, k)
+            if t in (orc.Q4_K, orc.Q5_K):
+                d, dmin, sc, mn, q = (G.parse_q4_K if t == orc.Q4_K else G.parse_q5_K)(rows, k)
                 sub = np.einsum("nbsj,bsj->nbs", q.reshape(n, nb, 8, 32), qx.reshape(nb, 8, 32))
                 xs = qx.reshape(nb, 8, 32).sum(axis=2)               # explicit sums, not bsums
                 out[b] = ((d * dx[None]) * (sc * sub).sum(axis=2) - (dmin * dx[None]) * (mn * xs[None]).sum(axis=2)).sum(axis=1)

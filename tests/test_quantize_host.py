@@ -29,7 +29,7 @@ def special_rows(k):
     return w
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_native_quantizer_matches_oracle_bit_for_bit(orc, name):
     qt = getattr(_ffi, name)
     for k in (256, 2048):
@@ -39,7 +39,7 @@ def test_native_quantizer_matches_oracle_bit_for_bit(orc, name):
     assert np.array_equal(quantize.quantize(qt, x), orc.quantize(getattr(orc, name), x))
 
 
-@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q6_K"])
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_native_quantizer_is_the_same_on_any_number_of_threads(name):
     qt = getattr(_ffi, name)
     w = G.seeded_weights(702, 37, 512)                  # rows do not divide evenly over the threads
