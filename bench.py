@@ -32,11 +32,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each scaled by
-# what the same counter reads for a 256 MiB device-to-device copy: x1.9998 and x1.0000; the copies
-# are what --calibrate-copy adds to a run).
-MEASURED_TRAFFIC_BYTES = {"qkv": 14.465e6 + 24.0 * 1024, "o": 9.739e6 + 16.0 * 1024,
-                          "gate_up": 66.285e6 + 112.0 * 1024, "down": 33.684e6 + 17.0 * 1024}
+# HBM bytes per launch from hardware counters, not measured by this run: rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE over this same command (two runs), each scaled by what the same counter reads for a
+# 256 MiB device-to-device copy (x1.99979 and x1.0000; the copies are what --calibrate-copy adds).  The
+# figures and the commands are in profiles/matvec_q4_0_llama3_8b_step.md.
+MEASURED_TRAFFIC_BYTES = {"qkv": 14_517_000, "o": 9_781_300, "gate_up": 66_512_700, "down": 33_708_900}
+TRAFFIC_SOURCE = "profiles/matvec_q4_0_llama3_8b_step.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, copy-calibrated)"
 HIDDEN, KV, FFN, LAYERS = 4096, 1024, 14336, 32
 BPW_Q4_0 = 18.0 / 32.0
 
@@ -202,7 +203,8 @@ def main(argv=None):
     achieved = dom_bytes / dom_us / 1e3
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": int(sum(MEASURED_TRAFFIC_BYTES[n] for n in dom_names) / len(dom_names)), "kernel": dom_kernel,
+                "traffic": int(sum(MEASURED_TRAFFIC_BYTES[n] for n in dom_names) / len(dom_names)), "traffic_source": TRAFFIC_SOURCE,
+                "kernel": dom_kernel,
                 "avg_launch_us": round(dom_us, 3), "algo_bytes_per_launch": int(dom_bytes),
                 "launches_per_step": args.layers * len(dom_names),
                 "note": "average over the " + ", ".join(dom_names) + " launches, which share this kernel ("
