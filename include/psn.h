@@ -252,6 +252,9 @@ int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32
  *    4  four waves, every wave stages and multiplies (any tile);
  *   16  eight waves of which four only multiply and four only stage: X by direct-to-LDS loads three K
  *       steps ahead, weights decoded from registers one step ahead (64x64, 64x128, 128x128, 128x256);
+ *   32  the wide kernel for large M (256x256 tiles only): four waves, each with all 256 rows x 64 columns
+ *       in 256 accumulator registers; X and the raw GGUF bytes arrive in LDS rings by direct-to-LDS loads,
+ *       a wave decodes the operand of its own columns one K slice ahead, interleaved with its MFMAs;
  *   64  the weight-streaming kernel for M <= 64 (64x64 tiles): X and the raw GGUF bytes arrive in LDS
  *       rings by direct-to-LDS loads, every wave decodes its own MFMA operand, one barrier per 256 of K.
  * Host arithmetic only ... */

@@ -32,6 +32,7 @@ CODE_OBJECTS = [
     ("psn_mv_q5_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q5_K"]),
     ("psn_mv_q6_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q6_K"]),
     ("psn_pf_skinny", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=0"]),
+    ("psn_pf_wide", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=2"]),
     *[(f"psn_pf_{fmt}_{fam}", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", f"-DPSN_BUILD_PF={num}", f"-DPSN_BUILD_PF_{fmt.upper()}"])
       for fmt in ("q4_0", "q8_0") for num, fam in ((1, "ws"), (4, "base"))],
     ("psn_decode", "psn_decode.hip", []),

@@ -158,6 +158,11 @@ PSN_DEV u32 lds_read32(u32 addr) {
     asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr) : "memory");
     return v;
 }
+template <int OFF> PSN_DEV u32 lds_read32o(u32 addr) {
+    u32 v;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
 PSN_DEV u32 lds_read_u16(u32 addr) {
     u32 v;
     asm volatile("ds_read_u16 %0, %1" : "=v"(v) : "v"(addr) : "memory");

@@ -1077,9 +1077,10 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
  * many workgroups of that tile one compute unit holds (LDS and registers) */
 static const double k_prefill_step_us[] = {0.87, 1.10, 1.50, 2.00, 2.00, 2.44};
 static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
-/* the producer / consumer kernels (16 = four multiplying + four staging waves):
- * {tile index, kernel family, step cost, workgroups per compute unit} */
-static const struct { int tile; int waves; double step_us; int per_cu; } k_prefill_alt[] = {{3, 16, 1.20, 1}, {2, 16, 0.76, 1}};
+/* the producer / consumer kernels (16 = four multiplying + four staging waves) and the wide kernel (32:
+ * 256 x 256, four waves decoding their own operands from raw bytes):
+ * {tile index, kernel family, step cost, workgroups per compute unit, K steps a workgroup spends filling its load rings} */
+static const struct { int tile; int waves; double step_us; int per_cu; int fill; } k_prefill_alt[] = {{3, 16, 1.25, 1, 0}, {2, 16, 0.76, 1, 0}, {5, 32, 2.20, 1, 3}};
 
 extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
                                             int32_t *waves) {
@@ -1119,7 +1120,7 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
                 if (v.tile != i) continue;
                 const int64_t sl = (int64_t)cus * v.per_cu;
                 const int64_t r8 = (wgs + sl - 1) / sl;
-                double t8 = (double)r8 * steps * v.step_us + 5.0;
+                double t8 = (double)r8 * (steps + v.fill) * v.step_us + 5.0;
                 if (sp > 1) t8 += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;
                 if (t8 < best) { best = t8; bi = i; bs = sp; *waves = v.waves; }
             }
@@ -1139,18 +1140,23 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     /* waves == 64 selects the skinny kernel (M <= 64, 64 x 64 tiles, deep LDS rings) */
     const bool skinny = waves == 64;
     if (skinny && (bm != 64 || bn != 64 || M > 64)) return fail(PSN_E_UNSUPPORTED, "prefill: the skinny kernel serves M <= 64 with a 64x64 tile");
+    /* waves == 32 selects the wide kernel: 256 x 256 tiles, four waves with 128 x 128 each, weights decoded
+     * from raw bytes in LDS by the wave that multiplies them */
+    const bool wide = waves == 32;
+    if (wide && (bm != 256 || bn != 256)) return fail(PSN_E_UNSUPPORTED, "prefill: the wide kernel has a 256x256 tile");
     bool known = false;
     for (int i = 0; i < 6; ++i) known = known || (k_prefill_tiles[i][0] == bm && k_prefill_tiles[i][1] == bn);
     if (!known) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel with a %dx%d tile", bm, bn);
     /* 16: eight waves split into four multiplying and four staging ones */
     const bool has_ws = (bm == 64 && (bn == 64 || bn == 128)) || (bm == 128 && (bn == 128 || bn == 256));
-    if (!skinny && waves != 4 && !(waves == 16 && has_ws)) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel family %d for a %dx%d tile", waves, bm, bn);
+    if (!skinny && !wide && waves != 4 && !(waves == 16 && has_ws)) return fail(PSN_E_UNSUPPORTED, "prefill: no kernel family %d for a %dx%d tile", waves, bm, bn);
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
     /* the interleaved kernels carry their LDS as static arrays; the skinny kernel: rings of three X chunks
      * (64 rows x 256 k fp16) and three raw weight chunks (64 rows), reused for the final 8 x 16 KB reduction */
     const int skinny_rings = 3 * 32768 + 3 * 64 * (qtype == PSN_Q4_0 ? 144 : 272);
-    const int lds = skinny ? (skinny_rings > 8 * 16384 ? skinny_rings : 8 * 16384) : waves == 16 ? 0 : 2 * (bm + bn) * 128;
+    const int wide_rings = 3 * (32768 + 256 * (qtype == PSN_Q4_0 ? 36 : 68));   /* three stages of X (256 rows x 64 k) and of raw blocks (two per row) */
+    const int lds = skinny ? (skinny_rings > 8 * 16384 ? skinny_rings : 8 * 16384) : wide ? wide_rings : waves == 16 ? 0 : 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);
     if ((rc = bind(mod->ctx))) return rc;
     if (ksplit > 1) {
@@ -1177,6 +1183,10 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
         return launch(mod, s, name, (unsigned)(nt * ksplit), 512, (unsigned)lds, &a);
     }
     const int64_t blocks = 8 * ((nt + 7) / 8) * mt * ksplit;      /* the kernel spreads N tiles over 8 XCDs */
+    if (wide) {
+        snprintf(name, sizeof name, "psn_prefill_%s_wide", fmt_name(qtype));
+        return launch(mod, s, name, (unsigned)blocks, 256, (unsigned)lds, &a);
+    }
     snprintf(name, sizeof name, "psn_prefill_%s_m%d_n%d%s", fmt_name(qtype), bm, bn, waves == 16 ? "_ws" : "");
     return launch(mod, s, name, (unsigned)blocks, (unsigned)(64 * (waves == 16 ? 8 : 4)), (unsigned)lds, &a);
 }

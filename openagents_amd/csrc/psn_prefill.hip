@@ -639,6 +639,304 @@ PSN_DEV void prefill_skinny_body(const psn_prefill_args &a) {
     }
 }
 
+/* ---- wide variant (large M) --------------------------------------------------------------------------
+ * The kernels above move more bytes through LDS per MFMA than the LDS pipe can serve at the MFMA rate
+ * (fragment reads of 64 x 128 wave tiles plus the fp16 weight tile the producers write).  This one has
+ * four waves, one per SIMD, each holding all 256 rows x 64 columns of the workgroup's tile of Y in 256
+ * accumulator registers (a wave decodes only the two weight fragments of its own columns per K slice: no
+ * decode is done twice), and no fp16 weight tile at all:
+ *   - per 64 of K, X (256 rows, the swizzled tile layout of the other kernels) and the raw GGUF bytes of
+ *     the workgroup's 256 weight rows (two blocks per row: 36 or 68 bytes, copied dword by dword) arrive
+ *     by direct-to-LDS loads, in rings three stages deep: loads run two stages ahead and nobody spends
+ *     VALU time on staging;
+ *   - a wave decodes the eight weights per lane its own MFMA operand needs straight from the raw bytes
+ *     (aligned dword reads, shifted into place), one 16-wide K slice ahead of the MFMAs that use them, and
+ *     the decode instructions are interleaved with those MFMAs (measured on MI355X: an MFMA 32x32x16 keeps
+ *     the matrix pipe for 32 cycles but the issue port for about 13, so three to four VALU instructions
+ *     per MFMA ride along for free);
+ *   - one workgroup barrier per 64 of K; every wave first waits for its own share of the next stage's
+ *     loads (loads complete in issue order, so "at most n outstanding" identifies them). */
+template <int N> struct pf_int { static constexpr int value = N; };
+
+template <typename WF>
+PSN_DEV void prefill_wide_body(const psn_prefill_args &a) {
+    constexpr int BM = 256, BN = 256, TM = 8, TN = 2, NS = 3;     /* a wave: all 256 rows x 64 columns */
+    constexpr bool Q4 = WF::DW == 36;
+    constexpr int BB = WF::BYTES / 8;                       /* bytes of a GGUF block: 18 or 34 */
+    constexpr int SB = 2 * BB;                              /* raw bytes per row and stage */
+    constexpr int XBYTES = BM * 128, RBYTES = BN * SB;
+    constexpr int NX = XBYTES / 1024 / 4;                   /* X loads per wave and stage: 8 */
+    constexpr int NR = RBYTES / 4 / 64 / 4;                 /* raw dword loads per wave and stage: 9 or 17 */
+    extern __shared__ uint4 psn_smem[];
+    typedef __attribute__((address_space(3))) char lds_char;
+    lds_char *const lds_ptr = (lds_char *)psn_smem;
+    const u32 lds0 = (u32)(uintptr_t)lds_ptr;
+    const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wn = wave;
+    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
+
+    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+    const int S = a.ksplit;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_xcd_n = (nt + 7) >> 3;
+    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
+    const int tile_n = xcd + 8 * tn_local;
+    if (tn_local >= per_xcd_n || tile_n >= nt) return;            /* whole workgroup leaves together */
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int per_split = (C + S - 1) / S;
+    const int c_begin = split * per_split, c_end = min(c_begin + per_split, C);
+    if (c_begin >= c_end) return;
+    const int nsteps = (c_end - c_begin) * 4, g_base = c_begin * 4;
+
+    float16_t acc[TM][TN];
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    /* One stage = NX 16-byte words of X and NR dwords of raw weight bytes per thread, always at the same
+     * per-thread byte offsets from a base that moves with the stage (scalar arithmetic only).  Stages past
+     * the end of the K range repeat its last one (into ring slots nothing reads any more), so every step
+     * issues the same number of loads. */
+    u32 xoff_g[NX], woff_g[NR];
+    UNROLL for (int u = 0; u < NX; ++u) {
+        const int s_ = (wave * NX + u) * 64 + lane, row = s_ >> 3, chunk = (s_ & 7) ^ (row & 7);
+        xoff_g[u] = (u32)min(m0 + row, M - 1) * (u32)(K * 2) + (u32)(chunk * 16);
+    }
+    UNROLL for (int u = 0; u < NR; ++u) {
+        const int dw = (u * 4 + wave) * 64 + lane, row = dw / (SB / 4), off = dw % (SB / 4);
+        woff_g[u] = (u32)min(n0 + row, N - 1) * (u32)a.row_bytes + (u32)(off * 4);
+    }
+    auto issue = [&](int g) {
+        const int gg = g_base + min(g, nsteps - 1), slot = g % NS;
+        const char *xb = reinterpret_cast<const char *>(a.X) + (int64_t)gg * 128;
+        const char *wb = reinterpret_cast<const char *>(a.W) + (int64_t)gg * SB;
+        lds_char *xd = lds_ptr + slot * XBYTES, *rd = lds_ptr + NS * XBYTES + slot * RBYTES;
+        UNROLL for (int u = 0; u < NX; ++u)
+            __builtin_amdgcn_global_load_lds((const void *)(xb + xoff_g[u]), (__attribute__((address_space(3))) void *)(xd + (wave * NX + u) * 1024), 16, 0, 0);
+        UNROLL for (int u = 0; u < NR; ++u)
+            __builtin_amdgcn_global_load_lds((const void *)(wb + woff_g[u]), (__attribute__((address_space(3))) void *)(rd + (u * 4 + wave) * 256), 4, 0, 0);
+    };
+
+    /* per-lane LDS offsets: the X fragment of K slice kk (row base + swizzled 16-byte position; the four
+     * 32-row blocks of the wave's tile are 4096 bytes apart), the raw bytes of weight row block j */
+    u32 xsw[4], rrow[TN];
+    UNROLL for (int kk = 0; kk < 4; ++kk) xsw[kk] = (u32)((lane & 31) * 128) + ((((u32)(2 * kk + h)) ^ (u32)(lane & 7)) << 4);
+    UNROLL for (int j = 0; j < TN; ++j) rrow[j] = (u32)((wn * 64 + 32 * j + (lane & 31)) * SB);
+    const u32 hq = 8u * (u32)h;
+
+    /* Raw unit U: Q4_0 -- block U of the stage (its 8 quant bytes 8h.. carry both nibble planes, K slices
+     * 2U and 2U+1); Q8_0 -- K slice U (bytes 16*(U%2) + 8h.. of block U/2).  Blocks start on even bytes,
+     * not on dwords, and LDS reads that straddle dwords are slow: a stage's first block starts on a dword
+     * (scale in the low half, quants two bytes in: three dwords to shift), the second two bytes later. */
+    auto read_unit = [&](u32 rst, auto uc, u32 (&raw)[TN][3], u32 (&wd)[TN]) {
+        constexpr int U = decltype(uc)::value;
+        constexpr int blk = Q4 ? U : U >> 1, qo = Q4 ? 0 : 16 * (U & 1);
+        UNROLL for (int j = 0; j < TN; ++j) {
+            const u32 rb = rst + rrow[j];
+            if constexpr (blk == 0) {
+                wd[j] = lds_read32o<0>(rb);
+                raw[j][0] = lds_read32o<qo>(rb + hq);
+                raw[j][1] = lds_read32o<qo + 4>(rb + hq);
+                raw[j][2] = lds_read32o<qo + 8>(rb + hq);
+            } else {
+                wd[j] = lds_read32o<BB - 2>(rb);
+                raw[j][0] = lds_read32o<BB + 2 + qo>(rb + hq);
+                raw[j][1] = lds_read32o<BB + 6 + qo>(rb + hq);
+                raw[j][2] = 0;
+            }
+        }
+    };
+    auto tie_unit = [&](u32 (&raw)[TN][3], u32 (&wd)[TN]) {
+        UNROLL for (int j = 0; j < TN; ++j) { tie1(wd[j]); tie1(raw[j][0]); tie1(raw[j][1]); tie1(raw[j][2]); }
+    };
+    auto read_a = [&](u32 xst, int kk, u32x4 (&af)[TM]) {
+        const u32 ab = xst + xsw[kk];
+        af[0] = lds_read128<0>(ab);
+        af[1] = lds_read128<4096>(ab);
+        af[2] = lds_read128<8192>(ab);
+        af[3] = lds_read128<12288>(ab);
+        af[4] = lds_read128<16384>(ab);
+        af[5] = lds_read128<20480>(ab);
+        af[6] = lds_read128<24576>(ab);
+        af[7] = lds_read128<28672>(ab);
+    };
+    /* One K slice: the 16 MFMAs of slice `cur` (fragments af, bf), every second one followed by four VALU
+     * instructions of the decode of the NEXT slice's operand (K slice kn, out of its raw unit, into bn)
+     * -- a quarter of a fragment: perm, and, subtract the bias, multiply by the scale -- with the
+     * scheduler told not to move anything across the groups.  DEC false: the step's last slice, nothing left to decode. */
+    auto slice = [&](auto kc, auto decc, const u32x4 (&af)[TM], const u32x4 (&bf)[TN], const u32 (&raw)[TN][3], const u32 (&wd)[TN], u32x4 (&bn)[TN]) {
+        constexpr int kn = decltype(kc)::value;
+        constexpr bool DEC = decltype(decc)::value != 0;
+        UNROLL for (int j = 0; j < TN; ++j) {
+            u32 q[2] = {0, 0};
+            half2_t d2 = bits_h2(0);
+            if constexpr (DEC) {
+                u32 d;
+                if constexpr ((kn & 2) == 0) {
+                    q[0] = align2(raw[j][1], raw[j][0]);
+                    q[1] = align2(raw[j][2], raw[j][1]);
+                    d = wd[j] & 0xffffu;
+                } else {
+                    q[0] = raw[j][0];
+                    q[1] = raw[j][1];
+                    d = wd[j] >> 16;
+                }
+                d2 = bits_h2(d | (d << 16));
+                if constexpr (Q4) {
+                    if constexpr ((kn & 1) != 0) { q[0] >>= 4; q[1] >>= 4; }
+                } else {
+                    q[0] ^= 0x80808080u;
+                    q[1] ^= 0x80808080u;
+                }
+            }
+            u32 o[4];
+            UNROLL for (int t = 0; t < 4; ++t) {
+                acc[2 * t][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[2 * t]), __builtin_bit_cast(half8_t, bf[j]), acc[2 * t][j], 0, 0, 0);
+                if constexpr (DEC) {
+                    const u32 x = __builtin_amdgcn_perm(0x64646464u, q[t >> 1], (t & 1) ? 0x04030402u : 0x04010400u) & (Q4 ? 0x640f640fu : 0x64ff64ffu);
+                    o[t] = h2_bits((bits_h2(x) - bits_h2(Q4 ? 0x64086408u : 0x64806480u)) * d2);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                acc[2 * t + 1][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[2 * t + 1]), __builtin_bit_cast(half8_t, bf[j]), acc[2 * t + 1][j], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (DEC) bn[j] = (u32x4){o[0], o[1], o[2], o[3]};
+        }
+    };
+    /* The step's last slice multiplies out of registers only, so it runs AFTER the step's barrier, while the
+     * first reads of the next stage are on their way: eight MFMAs, then the wait for those reads, then the
+     * other eight, each followed by a quarter of the decode of the next step's first operand (raw -> bn). */
+    auto slice_last = [&](const u32x4 (&af)[TM], const u32x4 (&bf)[TN], const u32 (&raw)[TN][3], const u32 (&wd)[TN], u32x4 (&bn)[TN], auto &&arrive) {
+        UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int i = 0; i < 4; ++i) {
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[i]), __builtin_bit_cast(half8_t, bf[j]), acc[i][j], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        arrive();
+        UNROLL for (int j = 0; j < TN; ++j) {
+            u32 q[2] = {align2(raw[j][1], raw[j][0]), align2(raw[j][2], raw[j][1])};
+            const u32 d = wd[j] & 0xffffu;
+            const half2_t d2 = bits_h2(d | (d << 16));
+            if constexpr (!Q4) {
+                q[0] ^= 0x80808080u;
+                q[1] ^= 0x80808080u;
+            }
+            u32 o[4];
+            UNROLL for (int t = 0; t < 4; ++t) {
+                acc[4 + t][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[4 + t]), __builtin_bit_cast(half8_t, bf[j]), acc[4 + t][j], 0, 0, 0);
+                const u32 x = __builtin_amdgcn_perm(0x64646464u, q[t >> 1], (t & 1) ? 0x04030402u : 0x04010400u) & (Q4 ? 0x640f640fu : 0x64ff64ffu);
+                o[t] = h2_bits((bits_h2(x) - bits_h2(Q4 ? 0x64086408u : 0x64806480u)) * d2);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            bn[j] = (u32x4){o[0], o[1], o[2], o[3]};
+        }
+    };
+
+    /* Steady state at the top of step g: stage g's first raw unit(s) and first two X fragments sit in
+     * registers, the operand of its first slice is decoded; stages g+1 and g+2 are on their way. */
+    constexpr int RU = Q4 ? 2 : 3;                            /* raw register sets */
+    u32x4 af[4][TM], bf[2][TN];
+    u32 raw[RU][TN][3], wd[RU][TN];
+    issue(0);
+    issue(1);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NX + NR) : "memory");       /* my share of stage 0 */
+    lds_barrier();
+    issue(2);
+    {
+        const u32 xst = lds0, rst = lds0 + (u32)(NS * XBYTES);
+        read_unit(rst, pf_int<0>(), raw[0], wd[0]);
+        if constexpr (!Q4) read_unit(rst, pf_int<1>(), raw[1], wd[1]);
+        read_a(xst, 0, af[0]);
+        read_a(xst, 1, af[1]);
+        lds_wait();
+        tie_unit(raw[0], wd[0]);
+        if constexpr (!Q4) tie_unit(raw[1], wd[1]);
+        tie(af[0]);
+        tie(af[1]);
+        UNROLL for (int j = 0; j < TN; ++j) {
+            const u32 q0 = align2(raw[0][j][1], raw[0][j][0]), q1 = align2(raw[0][j][2], raw[0][j][1]), d = wd[0][j] & 0xffffu;
+            const half2_t d2 = bits_h2(d | (d << 16));
+            u32 o[4];
+            if constexpr (Q4) {
+                bytes_to_h4(q0, 0x640f640fu, bits_h2(0x64086408u), d2, o[0], o[1]);
+                bytes_to_h4(q1, 0x640f640fu, bits_h2(0x64086408u), d2, o[2], o[3]);
+            } else {
+                bytes_to_h4(q0 ^ 0x80808080u, 0x64ff64ffu, bits_h2(0x64806480u), d2, o[0], o[1]);
+                bytes_to_h4(q1 ^ 0x80808080u, 0x64ff64ffu, bits_h2(0x64806480u), d2, o[2], o[3]);
+            }
+            bf[0][j] = (u32x4){o[0], o[1], o[2], o[3]};
+        }
+    }
+    for (int g = 0; g < nsteps; ++g) {
+        const int slot = g % NS, nslot = (g + 1) % NS;
+        const u32 xst = lds0 + (u32)(slot * XBYTES), rst = lds0 + (u32)(NS * XBYTES + slot * RBYTES);
+        const u32 xsn = lds0 + (u32)(nslot * XBYTES), rsn = lds0 + (u32)(NS * XBYTES + nslot * RBYTES);
+        if constexpr (Q4) {
+            /* slice 0 multiplies, slice 1 (the other nibble plane of block 0) is decoded; block 1 and X of slice 2 arrive */
+            read_unit(rst, pf_int<1>(), raw[1], wd[1]);
+            read_a(xst, 2, af[2]);
+            slice(pf_int<1>(), pf_int<1>(), af[0], bf[0], raw[0], wd[0], bf[1]);
+            lds_wait();
+            tie_unit(raw[1], wd[1]);
+            tie(af[2]);
+            read_a(xst, 3, af[3]);
+            slice(pf_int<2>(), pf_int<1>(), af[1], bf[1], raw[1], wd[1], bf[0]);
+            lds_wait();
+            tie(af[3]);
+            slice(pf_int<3>(), pf_int<1>(), af[2], bf[0], raw[1], wd[1], bf[1]);
+        } else {
+            read_unit(rst, pf_int<2>(), raw[2], wd[2]);
+            read_a(xst, 2, af[2]);
+            slice(pf_int<1>(), pf_int<1>(), af[0], bf[0], raw[1], wd[1], bf[1]);
+            lds_wait();
+            tie_unit(raw[2], wd[2]);
+            tie(af[2]);
+            read_unit(rst, pf_int<3>(), raw[1], wd[1]);
+            read_a(xst, 3, af[3]);
+            slice(pf_int<2>(), pf_int<1>(), af[1], bf[1], raw[2], wd[2], bf[0]);
+            lds_wait();
+            tie_unit(raw[1], wd[1]);
+            tie(af[3]);
+            slice(pf_int<3>(), pf_int<1>(), af[2], bf[0], raw[1], wd[1], bf[1]);
+        }
+        /* my share of stage g+1 (stage g+2 may still be on its way); then nobody reads stage g any more */
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NX + NR) : "memory");
+        lds_barrier();
+        issue(g + 3);
+        read_unit(rsn, pf_int<0>(), raw[0], wd[0]);
+        if constexpr (!Q4) read_unit(rsn, pf_int<1>(), raw[1], wd[1]);
+        read_a(xsn, 0, af[0]);
+        read_a(xsn, 1, af[1]);
+        slice_last(af[3], bf[1], raw[0], wd[0], bf[0], [&]() {
+            lds_wait();
+            tie_unit(raw[0], wd[0]);
+            if constexpr (!Q4) tie_unit(raw[1], wd[1]);
+            tie(af[0]);
+            tie(af[1]);
+        });
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    int tid_out = threadIdx.x;
+    asm volatile("" : "+v"(tid_out));
+    const int wn_o = tid_out >> 6, lane_o = tid_out & 63;
+    const bool whole = m0 + BM <= M && n0 + BN <= N;              /* uniform: no element of the tile needs a bounds check */
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn_o * 64 + 32 * j + (lane_o & 31);
+        float *yc = a.Y + (int64_t)(m0 + 32 * i + 4 * (lane_o >> 5)) * N + col;
+        UNROLL for (int r = 0; r < 16; ++r) {
+            const int dr = 8 * (r >> 2) + (r & 3);
+            if (whole || (m0 + 32 * i + 4 * (lane_o >> 5) + dr < M && col < N)) {
+                if (S == 1) yc[(int64_t)dr * N] = acc[i][j][r];
+                else unsafeAtomicAdd(&yc[(int64_t)dr * N], acc[i][j][r]);
+            }
+        }
+    }
+}
+
+#define PSN_PREFILL_KERNEL_WIDE(fmt, WF)                                                                     \
+    extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_wide(const psn_prefill_args a) {   \
+        prefill_wide_body<WF>(a);                                                                            \
+    }
+
 #define PSN_PREFILL_KERNEL_SKINNY(fmt, WF)                                                                   \
     extern "C" __global__ void __launch_bounds__(512) psn_prefill_##fmt##_skinny(const psn_prefill_args a) { \
         prefill_skinny_body<WF>(a);                                                                          \
@@ -671,7 +969,7 @@ PSN_DEV void prefill_skinny_body(const psn_prefill_args &a) {
 
 /* The build compiles this file once per (format, kernel family) -- -DPSN_BUILD_ONLY -DPSN_BUILD_PF=<n>
  * -DPSN_BUILD_PF_Q4_0 or _Q8_0 -- so that the code objects build in parallel; without PSN_BUILD_ONLY
- * everything lands in one.  Family numbers: 0 skinny + fill, 1 ws (producer / consumer), 4 base (four waves). */
+ * everything lands in one.  Family numbers: 0 skinny + fill, 1 ws (producer / consumer), 2 wide, 4 base (four waves). */
 
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 0
 /* zero fill with plain vector stores (graph-safe stand-in for a memset node) */
@@ -682,6 +980,10 @@ extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_a
 }
 PSN_PREFILL_KERNEL_SKINNY(q4_0, PfQ4_0)
 PSN_PREFILL_KERNEL_SKINNY(q8_0, PfQ8_0)
+#endif
+#if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 2
+PSN_PREFILL_KERNEL_WIDE(q4_0, PfQ4_0)
+PSN_PREFILL_KERNEL_WIDE(q8_0, PfQ8_0)
 #endif
 #if !defined(PSN_BUILD_ONLY) || defined(PSN_BUILD_PF_Q4_0)
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 1

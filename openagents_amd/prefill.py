@@ -62,7 +62,7 @@ def main(argv=None):
                 tm, tn, sp, wv = prefill_plan(m, n, k, be.compute_units)
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
-                                  "kernel": f"psn_prefill_{fname}_skinny" if wv == 64 else f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}[wv],
+                                  "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide"}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),
                                   "ksplit": sp, "iters": args.iters}), flush=True)
             for w in ws:
                 w.buf.free()

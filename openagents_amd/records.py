@@ -166,7 +166,7 @@ def config3(be: HipBackend, samples: int = 9, seed: int = 31, weights=None) -> l
 
 def prefill_kernel_name(fmt: str, m: int, n: int, k: int, cus: int):
     tm, tn, sp, wv = prefill_plan(m, n, k, cus)
-    name = f"psn_prefill_{fmt}_skinny" if wv == 64 else f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}[wv]
+    name = {64: f"psn_prefill_{fmt}_skinny", 32: f"psn_prefill_{fmt}_wide"}.get(wv, f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, ""))
     return name, sp
 
 

@@ -143,6 +143,32 @@ def test_prefill_linearity_and_zero(hip, orc):
     assert not hip.matmul_host(t, W, np.zeros((m, k), np.float16), n, k).any()
 
 
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
+def test_wide_kernel_ragged_shapes(hip, orc, qname):
+    """The large-M kernel (waves code 32, 256 x 256 tiles, weights decoded from raw bytes by the multiplying
+    wave): ragged m and n against the tile, K ranges from one 256-chunk (the load rings are as deep as the
+    whole range) to many, with and without K split; the result without K split is the same on every run."""
+    t = getattr(orc, qname)
+    for m, n, k in ((256, 256, 256), (1, 70, 512), (300, 296, 1280), (512, 768, 2048), (257, 513, 4096), (640, 260, 3584)):
+        say(f"wide {qname} m={m} n={n} k={k}")
+        W = weights(orc, qname, 870, n, k)
+        X = G.seeded_acts(871 + m, m, k).astype(np.float16)
+        ref = orc.prefill(t, W, X, n, k)
+        for ksplit in (1, 2, 4):
+            if ksplit > 1 and ((m * n) % 4 or k // 256 < ksplit):
+                continue
+            y = hip.matmul_host(t, W, X, n, k, (256, 256, ksplit, 32))
+            err = G.max_rel_err(y, ref)
+            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (ksplit, m, n, k, err)
+    W = weights(orc, qname, 870, 513, 4096)
+    X = G.seeded_acts(871 + 257, 257, 4096).astype(np.float16)
+    ys = [hip.matmul_host(t, W, X, 513, 4096, (256, 256, 1, 32)) for _ in range(3)]
+    assert np.array_equal(ys[0], ys[1]) and np.array_equal(ys[0], ys[2])
+    with pytest.raises(backend.PsnError) as e:
+        hip.matmul_host(t, W, X, 513, 4096, (128, 256, 1, 32))          # the wide kernel has one tile
+    assert e.value.code == _ffi.E_UNSUPPORTED
+
+
 def test_prefill_errors(hip, orc):
     n, k = 64, 512
     W = weights(orc, "Q4_0", 850, n, k)
