@@ -459,139 +459,188 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
  * synchronization at all:
  *   - everything arrives by direct-to-LDS loads into rings of dynamic LDS, a whole 256-wide chunk of K
  *     at a time: X (64 rows x 256 k, four swizzled 64-k tiles) and the raw GGUF bytes of 64 weight rows
- *     exactly as they sit in memory; chunks are requested XR-1 / RS-1 iterations ahead;
- *   - eight waves multiply; a chunk is 16 k16-slices and wave w owns two of them in two of the four
- *     steps, for the whole 64 x 64 tile.  A wave decodes the eight weights per lane its own MFMA operand
- *     needs straight from the raw ring (8 bytes + the fp16 scale), so there is no fp16 weight tile, no
- *     decode stage and no producer wave; two waves per SIMD let one wave's decode run under the
- *     other's MFMAs;
- *   - one workgroup barrier per CHUNK (every wave waits for its own share of the next chunk's loads
- *     first -- loads complete in issue order, so a constant "at most n outstanding" identifies them);
+ *     exactly as they sit in memory.  X comes out of the L2 caches (every workgroup walks all of it) and
+ *     needs two chunks in flight; the weight bytes come from HBM and need as many bytes in flight as LDS
+ *     can hold.  Loads of one wave complete in issue order, so a wave can only wait for "all but the
+ *     youngest n" of its own loads: waves 0..3 issue the X loads and waves 4..7 the weight loads, each
+ *     ring with its own depth;
+ *   - eight waves multiply; a chunk is eight GGUF blocks and wave w owns block w (two k16 slices) of
+ *     every chunk, for the whole 64 x 64 tile.  A wave decodes the weights its own MFMA operands need
+ *     straight from the raw ring (16 bytes + the fp16 scale per lane and block; for Q4_0 the same eight
+ *     bytes carry both slices), so there is no fp16 weight tile, no decode stage and no producer wave;
+ *   - the two waves of a SIMD (w and w+4) run in opposite phases -- waves 0..3 decode a block and then
+ *     multiply it, waves 4..7 first multiply the block they decoded before -- so that one wave's decode
+ *     (VALU) runs under the other's MFMAs although a barrier lines them up once per chunk;
+ *   - one workgroup barrier per CHUNK (every wave waits for its own share of the next chunk's loads first);
  *   - the eight partial tiles are summed through LDS at the end, in a fixed order.
  * Loads past the end of the K range re-read its last chunk into ring slots nothing reads any more, so
  * every iteration issues the same number of loads and the outstanding-load count is a constant. */
-template <typename WF, bool WAVE0>
+template <typename WF> struct SkinnyRings {
+    static constexpr int XR = 3;                                /* X chunks in the ring */
+    static constexpr int RS = WF::DW == 36 ? 6 : 3;             /* raw weight chunks in the ring */
+    static constexpr int XBYTES = 4 * 64 * 128, RBYTES = 64 * WF::BYTES;
+    static constexpr int BYTES = XR * XBYTES + RS * RBYTES;
+};
+
+/* LOADER 0: waves 0..3 (X loads; decode, then multiply); 1: wave 4 (weight loads, one more than the others;
+ * multiply the block before, then decode); 2: waves 5..7.  EVEN: the wave's block index is even -- the
+ * block starts on a dword (scale in the low half of its first dword, quants two bytes in: aligned dwords
+ * are read and shifted; LDS reads that straddle dwords are very slow); an odd block starts two bytes
+ * later (scale in the high half of the dword before, quants aligned). */
+template <typename WF, int LOADER, bool EVEN>
 PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, int n0, int c_begin, int nq, int rot,
                                  u32 xs_base, u32 raw_base, __attribute__((address_space(3))) char *lds_ptr, u32 lds0, float16_t (&acc)[2][2]) {
-    constexpr int BN = 64, XR = 3, RS = 3;
-    constexpr int XBYTES = 4 * 64 * 128, RBYTES = BN * WF::BYTES;
+    typedef SkinnyRings<WF> R;
+    constexpr bool Q4 = WF::DW == 36;
+    constexpr int XR = R::XR, RS = R::RS, XBYTES = R::XBYTES, RBYTES = R::RBYTES;
     constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9 or 17 */
-    constexpr int CX = 4;                                   /* X loads per wave and chunk (32 KB over 8 waves) */
-    constexpr int CR = (RINSTR + (WAVE0 ? 7 : 0)) / 8;      /* raw loads per wave and chunk: wave 0 takes the odd one */
+    constexpr int CX = 8;                                   /* X loads per X wave and chunk (32 KB over 4 waves) */
+    constexpr int CR = RINSTR / 4 + (LOADER == 1 ? RINSTR % 4 : 0);   /* raw loads per weight wave and chunk */
+    constexpr int DEPTH = LOADER == 0 ? XR : RS, PER = LOADER == 0 ? CX : CR;
+    constexpr int BB = WF::BYTES / 8;                       /* bytes of a GGUF block: 18 or 34 */
+    constexpr int NP = Q4 ? 1 : 2;                          /* raw register sets per block: Q4_0 keeps both slices in the same bytes */
+    static_assert(RINSTR % 4 == 1, "wave 4 takes the one load that does not divide over four waves");
     const int M = a.M, N = a.N, K = a.K;
     auto chunk_of = [&](int q) { const int r = min(q, nq - 1) + rot; return c_begin + (r >= nq ? r - nq : r); };
-    auto issue_raw = [&](int q) {
+    auto issue = [&](int q) {
         const int c = chunk_of(q);
-        __attribute__((address_space(3))) char *dst = lds_ptr + (raw_base - lds0) + (q % RS) * RBYTES;
-        UNROLL for (int u = 0; u < CR; ++u) {
-            const int i = wave + 8 * u;                     /* instruction index; with WAVE0 the last one is index 8 or 16 */
-            const int word = i * 64 + lane, row = word / (WF::BYTES / 16), wd = word % (WF::BYTES / 16);
-            const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + (int64_t)c * WF::BYTES + wd * 16;
-            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
+        if constexpr (LOADER == 0) {
+            const int k0 = c * 256;
+            __attribute__((address_space(3))) char *dst = lds_ptr + (xs_base - lds0) + (q % XR) * XBYTES;
+            UNROLL for (int u = 0; u < CX; ++u) {
+                /* 16-byte word s_ of the stage in LDS order: step s_/512, row (s_%512)/8, position s_%8 holds chunk pos^(row&7) */
+                const int i = wave * CX + u, s_ = i * 64 + lane, step = s_ >> 9, row = (s_ >> 3) & 63, chunk = (s_ & 7) ^ (row & 7);
+                const uint16_t *src = a.X + (int64_t)min(row, M - 1) * K + k0 + step * 64 + chunk * 8;
+                __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
+            }
+        } else {
+            __attribute__((address_space(3))) char *dst = lds_ptr + (raw_base - lds0) + (q % RS) * RBYTES;
+            UNROLL for (int u = 0; u < CR; ++u) {
+                const int i = (wave - 4) + 4 * u;               /* instruction index; wave 4's last one is index 8 or 16 */
+                const int word = i * 64 + lane, row = word / (WF::BYTES / 16), wd = word % (WF::BYTES / 16);
+                const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + (int64_t)c * WF::BYTES + wd * 16;
+                __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
+            }
         }
     };
-    auto issue_x = [&](int q) {
-        const int k0 = chunk_of(q) * 256;
-        __attribute__((address_space(3))) char *dst = lds_ptr + (xs_base - lds0) + (q % XR) * XBYTES;
-        UNROLL for (int u = 0; u < CX; ++u) {
-            /* 16-byte word s_ of the stage in LDS order: step s_/512, row (s_%512)/8, position s_%8 holds chunk pos^(row&7) */
-            const int i = wave * CX + u, s_ = i * 64 + lane, step = s_ >> 9, row = (s_ >> 3) & 63, chunk = (s_ & 7) ^ (row & 7);
-            const uint16_t *src = a.X + (int64_t)min(row, M - 1) * K + k0 + step * 64 + chunk * 8;
-            __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
-        }
-    };
-    const int kk = wave & 3, sp = wave >> 2, h = lane >> 5;  /* this wave: k16 slice kk of steps sp and sp + 2 */
-    u32 xoff[2], roff[2];
-    UNROLL for (int i = 0; i < 2; ++i) {
-        xoff[i] = (u32)tile_off(32 * i + (lane & 31), 2 * kk + h);
-        /* GGUF block (2*step + kk/2) of the row; the 8 weights are plane kk%2, bytes 8h.. (Q4_0: nibble plane
-         * of bytes 8h..8h+7; Q8_0: the 8 int8 at 16*(kk%2) + 8h) */
-        roff[i] = (u32)((32 * i + (lane & 31)) * WF::BYTES + (kk >> 1) * (WF::BYTES / 8));
-    }
-    constexpr int BB = WF::BYTES / 8;                       /* bytes of a GGUF block: 18 or 34 */
-    const u32 qoff = WF::DW == 36 ? 2u + 8u * (u32)h : 2u + 16u * (u32)(kk & 1) + 8u * (u32)h;
+    /* this wave: block `wave` of the chunk = k16 slices 2*(wave&1) and 2*(wave&1)+1 of 64-k step wave/2.  Per-lane
+     * LDS offsets inside a ring slot: the two X fragments (rows 32.. sit 4096 bytes on), the row's block
+     * (rows 32.. sit 32 rows on) with and without the lane's quant offset 8h. */
+    const int h = lane >> 5;
+    u32 xlane[2];
+    UNROLL for (int sl = 0; sl < 2; ++sl) xlane[sl] = (u32)((wave >> 1) * 8192 + tile_off(lane & 31, 2 * (2 * (wave & 1) + sl) + h));
+    const u32 rlane = (u32)((lane & 31) * WF::BYTES + wave * BB), qlane = rlane + 8u * (u32)h;
+    constexpr int ROW32 = 32 * WF::BYTES;
 
-    for (int q = 0; q < RS - 1; ++q) issue_raw(q);
-    for (int q = 0; q < XR - 1; ++q) issue_x(q);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((XR - 2) * CX) : "memory");   /* my share of chunk 0 has landed */
-    lds_barrier();
-    for (int q = 0; q < nq; ++q) {
-        issue_raw(q + RS - 1);
-        issue_x(q + XR - 1);
-        const u32 xst = xs_base + (u32)((q % XR) * XBYTES), rst = raw_base + (u32)((q % RS) * RBYTES);
-        UNROLL for (int s2 = 0; s2 < 2; ++s2) {
-            const int step = sp + 2 * s2;
-            u32x4 xf[2];
-            u32 wq[2][2], wd[2];
-            UNROLL for (int i = 0; i < 2; ++i) xf[i] = lds_read128<0>(xst + (u32)(step * 8192) + xoff[i]);
-            /* GGUF blocks start on even bytes, not on dwords, and LDS reads that straddle dwords are very slow:
-             * read the aligned dwords around the eight quant bytes and shift them into place.  Block index
-             * 2*step + kk/2 is even or odd for the whole wave: an even block starts on a dword (scale in the
-             * low half, quants shifted by two bytes), an odd one two bytes later (scale in the high half of the
-             * dword before, quants aligned). */
-            u32 raw[2][3];
-            UNROLL for (int j = 0; j < 2; ++j) {
-                const u32 baddr = rst + roff[j] + (u32)(2 * step * BB);      /* block start */
-                if ((kk & 2) == 0) {
-                    wd[j] = lds_read32(baddr);                               /* scale | first two quant bytes */
-                    raw[j][0] = lds_read32(baddr + qoff - 2u);
-                    raw[j][1] = lds_read32(baddr + qoff + 2u);
-                    raw[j][2] = lds_read32(baddr + qoff + 6u);
-                } else {
-                    wd[j] = lds_read32(baddr - 2u);                          /* last two bytes of the block before | scale */
-                    raw[j][0] = lds_read32(baddr + qoff);
-                    raw[j][1] = lds_read32(baddr + qoff + 4u);
-                    raw[j][2] = 0;
-                }
+    struct unit { u32x4 xf[2][2]; u32 raw[NP][2][3], wd[2]; };
+    auto fetch = [&](u32 xst, u32 rst, unit &t) {
+        const u32 xa0 = xst + xlane[0], xa1 = xst + xlane[1], rw = rst + rlane, rq = rst + qlane;
+        t.xf[0][0] = lds_read128<0>(xa0);
+        t.xf[0][1] = lds_read128<4096>(xa0);
+        t.xf[1][0] = lds_read128<0>(xa1);
+        t.xf[1][1] = lds_read128<4096>(xa1);
+        if constexpr (EVEN) {
+            t.wd[0] = lds_read32o<0>(rw);                                    /* scale | first two quant bytes */
+            t.wd[1] = lds_read32o<ROW32>(rw);
+            UNROLL for (int p = 0; p < NP; ++p) {
+                t.raw[p][0][0] = p ? lds_read32o<16>(rq) : lds_read32o<0>(rq);
+                t.raw[p][0][1] = p ? lds_read32o<20>(rq) : lds_read32o<4>(rq);
+                t.raw[p][0][2] = p ? lds_read32o<24>(rq) : lds_read32o<8>(rq);
+                t.raw[p][1][0] = p ? lds_read32o<ROW32 + 16>(rq) : lds_read32o<ROW32>(rq);
+                t.raw[p][1][1] = p ? lds_read32o<ROW32 + 20>(rq) : lds_read32o<ROW32 + 4>(rq);
+                t.raw[p][1][2] = p ? lds_read32o<ROW32 + 24>(rq) : lds_read32o<ROW32 + 8>(rq);
             }
-            lds_wait();
-            tie(xf);
-            UNROLL for (int j = 0; j < 2; ++j) {
-                tie1(wd[j]); tie1(raw[j][0]); tie1(raw[j][1]); tie1(raw[j][2]);
-                if ((kk & 2) == 0) {
-                    wq[j][0] = align2(raw[j][1], raw[j][0]);
-                    wq[j][1] = align2(raw[j][2], raw[j][1]);
-                    wd[j] &= 0xffffu;
-                } else {
-                    wq[j][0] = raw[j][0];
-                    wq[j][1] = raw[j][1];
-                    wd[j] >>= 16;
-                }
+        } else {
+            t.wd[0] = lds_read32(rw - 2u);                                   /* last two bytes of the block before | scale */
+            t.wd[1] = lds_read32(rw + (u32)(ROW32 - 2));
+            UNROLL for (int p = 0; p < NP; ++p) {
+                t.raw[p][0][0] = p ? lds_read32o<18>(rq) : lds_read32o<2>(rq);
+                t.raw[p][0][1] = p ? lds_read32o<22>(rq) : lds_read32o<6>(rq);
+                t.raw[p][0][2] = 0;
+                t.raw[p][1][0] = p ? lds_read32o<ROW32 + 18>(rq) : lds_read32o<ROW32 + 2>(rq);
+                t.raw[p][1][1] = p ? lds_read32o<ROW32 + 22>(rq) : lds_read32o<ROW32 + 6>(rq);
+                t.raw[p][1][2] = 0;
             }
-            u32x4 wf[2];
-            UNROLL for (int j = 0; j < 2; ++j) {
-                const half2_t d2 = bits_h2(wd[j] | (wd[j] << 16));
-                u32 o[4];
-                if constexpr (WF::DW == 36) {
-                    const int sh = 4 * (kk & 1);
-                    bytes_to_h4(wq[j][0] >> sh, 0x640f640fu, bits_h2(0x64086408u), d2, o[0], o[1]);
-                    bytes_to_h4(wq[j][1] >> sh, 0x640f640fu, bits_h2(0x64086408u), d2, o[2], o[3]);
-                } else {
-                    bytes_to_h4(wq[j][0] ^ 0x80808080u, 0x64ff64ffu, bits_h2(0x64806480u), d2, o[0], o[1]);
-                    bytes_to_h4(wq[j][1] ^ 0x80808080u, 0x64ff64ffu, bits_h2(0x64806480u), d2, o[2], o[3]);
-                }
-                wf[j] = (u32x4){o[0], o[1], o[2], o[3]};
-            }
-            UNROLL for (int i = 0; i < 2; ++i) UNROLL for (int j = 0; j < 2; ++j)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, xf[i]), __builtin_bit_cast(half8_t, wf[j]), acc[i][j], 0, 0, 0);
         }
-        /* my share of chunk q+1: everything but this iteration's own loads */
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((XR - 2) * (CX + CR)) : "memory");
+    };
+    auto arrived = [&](unit &t) {
+        tie(t.xf[0]);
+        tie(t.xf[1]);
+        UNROLL for (int j = 0; j < 2; ++j) {
+            tie1(t.wd[j]);
+            UNROLL for (int p = 0; p < NP; ++p) { tie1(t.raw[p][j][0]); tie1(t.raw[p][j][1]); if (EVEN) tie1(t.raw[p][j][2]); }
+        }
+    };
+    /* MFMA operands of the block's two slices, column blocks j = 0, 1 */
+    auto decode = [&](const unit &t, u32x4 (&wf)[2][2]) {
+        UNROLL for (int j = 0; j < 2; ++j) {
+            const half2_t w2 = bits_h2(t.wd[j]);
+            const half2_t d2 = EVEN ? __builtin_shufflevector(w2, w2, 0, 0) : __builtin_shufflevector(w2, w2, 1, 1);
+            u32 q[NP][2];
+            UNROLL for (int p = 0; p < NP; ++p) {
+                q[p][0] = EVEN ? align2(t.raw[p][j][1], t.raw[p][j][0]) : t.raw[p][j][0];
+                q[p][1] = EVEN ? align2(t.raw[p][j][2], t.raw[p][j][1]) : t.raw[p][j][1];
+            }
+            UNROLL for (int sl = 0; sl < 2; ++sl) {
+                u32 o[4];
+                if constexpr (Q4) {
+                    bytes_to_h4((sl ? q[0][0] >> 4 : q[0][0]) & 0x0f0f0f0fu, 0xffffffffu, bits_h2(0x64086408u), d2, o[0], o[1]);
+                    bytes_to_h4((sl ? q[0][1] >> 4 : q[0][1]) & 0x0f0f0f0fu, 0xffffffffu, bits_h2(0x64086408u), d2, o[2], o[3]);
+                } else {
+                    bytes_to_h4(q[Q4 ? 0 : sl][0] ^ 0x80808080u, 0xffffffffu, bits_h2(0x64806480u), d2, o[0], o[1]);
+                    bytes_to_h4(q[Q4 ? 0 : sl][1] ^ 0x80808080u, 0xffffffffu, bits_h2(0x64806480u), d2, o[2], o[3]);
+                }
+                wf[sl][j] = (u32x4){o[0], o[1], o[2], o[3]};
+            }
+        }
+    };
+    auto multiply = [&](const u32x4 (&xf)[2][2], const u32x4 (&wf)[2][2]) {
+        UNROLL for (int sl = 0; sl < 2; ++sl) UNROLL for (int i = 0; i < 2; ++i) UNROLL for (int j = 0; j < 2; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, xf[sl][i]), __builtin_bit_cast(half8_t, wf[sl][j]), acc[i][j], 0, 0, 0);
+    };
+
+    for (int q = 0; q < DEPTH - 1; ++q) issue(q);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * PER) : "memory");   /* my share of chunk 0 has landed */
+    lds_barrier();
+    u32x4 xp[2][2], wp[2][2];                               /* LOADER != 0: the block decoded last */
+    UNROLL for (int sl = 0; sl < 2; ++sl) UNROLL for (int i = 0; i < 2; ++i) xp[sl][i] = wp[sl][i] = (u32x4){0, 0, 0, 0};
+    for (int q = 0; q < nq; ++q) {
+        issue(q + DEPTH - 1);
+        unit t;
+        fetch(xs_base + (u32)((q % XR) * XBYTES), raw_base + (u32)((q % RS) * RBYTES), t);
+        if constexpr (LOADER == 0) {
+            u32x4 wf[2][2];
+            lds_wait();
+            arrived(t);
+            decode(t, wf);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(t.xf, wf);
+        } else {
+            multiply(xp, wp);
+            __builtin_amdgcn_sched_barrier(0);
+            lds_wait();
+            arrived(t);
+            decode(t, wp);
+            UNROLL for (int sl = 0; sl < 2; ++sl) UNROLL for (int i = 0; i < 2; ++i) xp[sl][i] = t.xf[sl][i];
+        }
+        /* my share of chunk q+1: everything but the loads of the youngest DEPTH-2 iterations */
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((DEPTH - 2) * PER) : "memory");
         lds_barrier();
     }
+    if constexpr (LOADER != 0) multiply(xp, wp);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");        /* nothing lands in the rings any more ... */
     lds_barrier();                                          /* ... for any wave: they can hold the partial tiles */
 }
 
 template <typename WF>
 PSN_DEV void prefill_skinny_body(const psn_prefill_args &a) {
-    constexpr int BN = 64, XR = 3;
-    constexpr int XBYTES = 4 * 64 * 128;
+    typedef SkinnyRings<WF> R;
+    constexpr int BN = 64;
     extern __shared__ uint4 psn_smem[];
     typedef __attribute__((address_space(3))) char lds_char;
     lds_char *const lds_ptr = (lds_char *)psn_smem;
     const u32 lds0 = (u32)(uintptr_t)lds_ptr;
-    const u32 xs_base = lds0, raw_base = xs_base + XR * XBYTES;
+    const u32 xs_base = lds0, raw_base = xs_base + R::XR * R::XBYTES;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int M = a.M, N = a.N, C = a.K >> 8;
@@ -608,8 +657,18 @@ PSN_DEV void prefill_skinny_body(const psn_prefill_args &a) {
 
     float16_t acc[2][2];
     UNROLL for (int i = 0; i < 2; ++i) UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    if (wave == 0) prefill_skinny_loop<WF, true>(a, wave, lane, n0, c_begin, nq, rot, xs_base, raw_base, lds_ptr, lds0, acc);
-    else prefill_skinny_loop<WF, false>(a, wave, lane, n0, c_begin, nq, rot, xs_base, raw_base, lds_ptr, lds0, acc);
+#define PSN_SKINNY_LOOP(LOADER, EVEN) prefill_skinny_loop<WF, LOADER, EVEN>(a, wave, lane, n0, c_begin, nq, rot, xs_base, raw_base, lds_ptr, lds0, acc)
+    if (wave < 4) {
+        if ((wave & 1) == 0) PSN_SKINNY_LOOP(0, true);
+        else PSN_SKINNY_LOOP(0, false);
+    } else if (wave == 4) {
+        PSN_SKINNY_LOOP(1, true);
+    } else if ((wave & 1) == 0) {
+        PSN_SKINNY_LOOP(2, true);
+    } else {
+        PSN_SKINNY_LOOP(2, false);
+    }
+#undef PSN_SKINNY_LOOP
 
     /* partial tiles of the eight waves -> LDS (16 KB each, lane-contiguous); then wave w sums registers
      * 8*(w/4) .. +8 of tile w%4 over the eight waves, always in the order 0 .. 7 */
