@@ -26,7 +26,7 @@ class ActqInfo(C.Structure):
 
 class MatvecPlan(C.Structure):
     _fields_ = [("lanes_per_row", C.c_int32), ("rows_in_flight", C.c_int32), ("batch_tile", C.c_int32),
-                ("stage_lds", C.c_int32), ("blocks", C.c_int32), ("threads", C.c_int32), ("stream", C.c_int32), ("reserved", C.c_int32)]
+                ("stage_lds", C.c_int32), ("blocks", C.c_int32), ("threads", C.c_int32), ("stream", C.c_int32), ("mfma", C.c_int32)]
 
     def as_dict(self):
         return {k: int(getattr(self, k)) for k, _ in self._fields_}

@@ -31,6 +31,7 @@ CODE_OBJECTS = [
     ("psn_mv_q4_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q4_K"]),
     ("psn_mv_q5_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q5_K"]),
     ("psn_mv_q6_K", "psn_matvec.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_Q6_K"]),
+    ("psn_mvm", "psn_matvec_mfma.hip", []),
     ("psn_pf_skinny", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=0"]),
     ("psn_pf_wide", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=2"]),
     *[(f"psn_pf_{fmt}_{fam}", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", f"-DPSN_BUILD_PF={num}", f"-DPSN_BUILD_PF_{fmt.upper()}"])

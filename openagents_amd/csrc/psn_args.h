@@ -53,6 +53,8 @@ struct psn_matvec_args {
     const float *x_delta; /* [K] added to xf before the norm (may be null) */
     const float *norm_w;  /* [K] RMSNorm weights */
     float *h_out;         /* [K] receives xf + x_delta, written by workgroup 0 (may be null; must not alias xf or x_delta) */
+    int32_t kslices;      /* MFMA small-batch kernels: waves sharing a 16-row tile, each owning K / kslices of it */
+    int32_t pad0;
 };
 
 struct psn_prefill_args {

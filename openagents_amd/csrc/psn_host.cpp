@@ -694,6 +694,31 @@ static int32_t stream_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32
     return PSN_OK;
 }
 
+/* Can the small-batch MFMA kernel run this plan?  Fills in the dynamic LDS it needs. */
+static int32_t mfma_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32_t batch, const psn_matvec_plan *plan, const int64_t *n_rows,
+                               int32_t count, int max_lds, int64_t *lds_out) {
+    const int ks = plan->mfma;
+    const int64_t C = K / 256;
+    if (scheme != PSN_ACT_Q8 || (qtype != PSN_Q4_K && qtype != PSN_Q5_K)) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernels serve Q4_K and Q5_K with scheme Q8");
+    if (batch < 1 || batch > 8) return fail(PSN_E_UNSUPPORTED, "plan: batch=%d", batch);
+    if (plan->stage_lds != 1) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernels take quantized activations (stage_lds 1)");
+    if (plan->threads != 256 && plan->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", plan->threads);
+    const int waves = plan->threads / 64;
+    if (!(ks == 1 || ks == 2 || ks == 4 || ks == 8) || ks > waves) return fail(PSN_E_UNSUPPORTED, "plan: mfma=%d (1, 2, 4 or 8 waves per tile, at most the workgroup's)", ks);
+    if (C % ks || C / ks > 8) return fail(PSN_E_UNSUPPORTED, "plan: K=%lld does not split into %d slices of at most eight chunks", (long long)K, ks);
+    if (C * 8 > 2 * (int64_t)plan->threads) return fail(PSN_E_UNSUPPORTED, "plan: K=%lld is too long for %d threads to stage the activation sums", (long long)K, plan->threads);
+    for (int i = 0; n_rows && i < count; ++i)
+        if (n_rows[i] % 16) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernels need every matrix to hold a multiple of 16 rows");
+    if (plan->blocks < 1 || plan->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", plan->blocks);
+    const int64_t words = (C / ks) * (qtype == PSN_Q4_K ? 9 : 11), ni = (words + 3) / 4;
+    const int ring = plan->stream;
+    if (ring < 1 || ring > 4 || (ring - 1) * ni + ni - 1 > 63) return fail(PSN_E_UNSUPPORTED, "plan: stream=%d (with mfma: units in flight per wave, 1..4, at most 64 loads)", ring);
+    const int64_t total = C * 160 + (int64_t)waves * 1024 + (int64_t)waves * ring * ni * 1024;
+    if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernel needs %lld bytes of LDS, device offers %d", (long long)total, max_lds);
+    *lds_out = total;
+    return PSN_OK;
+}
+
 /* n_rows: the row counts of the matrices sharing the launch (count of them), or null when unknown */
 static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t cus, bool fuse_quantize,
                          const int64_t *n_rows, int32_t count, psn_matvec_plan *out) {
@@ -705,7 +730,7 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
     p.batch_tile = batch <= 1 ? 1 : batch <= 2 ? 2 : batch <= 4 ? 4 : 8;
     p.rows_in_flight = 1;
     p.stream = 0;
-    p.reserved = 0;
+    p.mfma = 0;
     /* the staged activations may take the whole 160 KB of a compute unit's LDS (batch 8 at K = 14336
      * needs 140 KB); re-quantizing inside the launch only pays up to batch 2 -- beyond that every
      * workgroup would redo batch x K of quantization, and one extra launch is cheaper (measured) */
@@ -751,6 +776,43 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
             return PSN_OK;
         }
         g_err[0] = 0;                                   /* not streamable after all: the register kernels take it */
+    }
+    /* Batch 2..8 of Q4_K / Q5_K on quantized activations: the int8-MFMA kernel, whose cost per weight
+     * does not grow with the batch.  Measured on MI355X: four-wave workgroups, two per compute unit,
+     * whose waves own slices of at most four chunks of one tile (K <= 4096); longer rows take eight
+     * waves with slices of up to eight chunks, one workgroup per compute unit.  One unit in flight per
+     * wave: deeper rings and more resident workgroups both measured slower. */
+    /* (fp32 input at batch 2 and short rows: quantizing inside a register-kernel launch still beats a
+     * quantize launch followed by this kernel -- 13.8 against 16.0 us at 14336 x 4096) */
+    const bool fused_wins = fuse_quantize && batch <= 2 && K <= 8192 && p.stage_lds == 2;
+    if (scheme == PSN_ACT_Q8 && batch >= 2 && !fused_wins && (qtype == PSN_Q4_K || qtype == PSN_Q5_K) && n_rows != nullptr) {
+        psn_matvec_plan q = p;
+        q.stage_lds = 1;
+        q.lanes_per_row = 16;
+        q.stream = 1;
+        q.batch_tile = 8;
+        q.blocks = 1;
+        int64_t lds = 0;
+        int32_t ok = PSN_E_UNSUPPORTED;
+        for (int pass = 0; pass < 2 && ok != PSN_OK; ++pass) {
+            const int waves_per_group = pass == 0 ? 4 : 8, max_slice = pass == 0 ? 4 : 8;
+            q.threads = 64 * waves_per_group;
+            for (int ks = 1; ks <= waves_per_group && ok != PSN_OK; ks *= 2) {
+                if (C % ks || C / ks > max_slice) continue;
+                q.mfma = ks;
+                ok = mfma_plan_check(qtype, scheme, K, batch, &q, n_rows, count, 160 * 1024, &lds);
+            }
+        }
+        if (ok == PSN_OK) {
+            const int64_t tpw = (q.threads / 64) / q.mfma, ntiles = N / 16;
+            int64_t b = (ntiles + tpw - 1) / tpw;
+            const int64_t cap = (q.threads == 256 ? 2 : 1) * (int64_t)cus;
+            if (b > cap) b = cap;
+            q.blocks = (int32_t)b;
+            *out = q;
+            return PSN_OK;
+        }
+        g_err[0] = 0;                                   /* shape not served: the register kernels take it */
     }
     if (p.stage_lds == 2) {
         /* Every workgroup re-quantizes x while staging it, a cost proportional to K: keep to about
@@ -829,7 +891,7 @@ struct norm_fusion {
 static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const seg_list &sg, const void *x,
                           int64_t K, int32_t batch, const psn_matvec_plan *plan, const norm_fusion *norm = nullptr) {
     int32_t lds = 0;
-    int32_t rc = plan_is_valid(plan, qtype, scheme, K, batch, mod->ctx->max_lds, &lds);
+    int32_t rc = plan->mfma ? PSN_OK : plan_is_valid(plan, qtype, scheme, K, batch, mod->ctx->max_lds, &lds);
     if (rc) return rc;
     psn_matvec_args a;
     memset(&a, 0, sizeof a);
@@ -849,6 +911,19 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
     a.threads = plan->threads;
     a.blocks = plan->blocks;
     char name[96];
+    if (plan->mfma) {
+        int64_t total = 0;
+        if ((rc = mfma_plan_check(qtype, scheme, K, batch, plan, sg.N, sg.count, mod->ctx->max_lds, &total))) return rc;
+        psn_actq_info li;
+        if ((rc = psn_actq_layout(psn_act_type_for(qtype), K, batch, &li))) return rc;
+        a.xqs = (const int8_t *)x + li.off_qs;
+        a.xd = (const float *)((const char *)x + li.off_d);
+        a.xs = (const char *)x + li.off_s;
+        a.kslices = plan->mfma;
+        a.ring = plan->stream;
+        snprintf(name, sizeof name, "psn_mvm_%s_q8", fmt_name(qtype));
+        return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)total, &a);
+    }
     if (plan->stream) {
         const int g = plan->lanes_per_row, rows = 64 / g, ring = plan->stream;
         int64_t total = 0;

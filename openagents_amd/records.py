@@ -29,7 +29,7 @@ import numpy as np
 
 from . import _ffi, quantize
 from ._ffi import ACT_Q8, Q4_0, Q4_K, Q6_K, Q8_0
-from .backend import HipBackend, matvec_plan, prefill_plan, row_bytes
+from .backend import HipBackend, act_type_for, matvec_plan, prefill_plan, row_bytes
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
@@ -87,6 +87,8 @@ def seeded_weights(seed: int, n: int, k: int) -> np.ndarray:
 def matvec_kernel_name(qtype: int, ns, k: int, batch: int, cus: int, x_is_f32: bool = True) -> str:
     p = matvec_plan(qtype, ACT_Q8, sum(ns), k, batch, cus, x_is_f32)
     f = FMT_NAME[qtype]
+    if p.mfma:
+        return f"psn_quantize_q8_K + psn_mvm_{f}_q8"
     if p.stream:
         return f"psn_mvs_{f}_q8_g{p.lanes_per_row}" + {1: "_lds", 2: "_xf"}[p.stage_lds] + f"_s{len(ns)}"
     return f"psn_mv_{f}_q8_g{p.lanes_per_row}_r{p.rows_in_flight}_b{p.batch_tile}" + {0: "", 1: "_lds", 2: "_xf"}[p.stage_lds]
@@ -114,13 +116,23 @@ def matvec_record(be: HipBackend, ws: list, blocks: np.ndarray, batch: int, op_r
     g = be.end_capture()
     st = stats(time_graph(be, g, copies, samples))
     be.destroy_graph(g)
+    extra = {}
+    if batch > 1:
+        # the same projection fed with activations that are already quantized (what a fused producer hands over)
+        xq = be.quantize_activations(x, k, batch, act_type_for(qtype))
+        be.begin_capture()
+        for w in ws:
+            be.quantized_matvec_q8(w, xq, y, batch)
+        g = be.end_capture()
+        extra["timing_prequantized_input"] = stats(time_graph(be, g, copies, samples))
+        be.destroy_graph(g)
     nbytes = n * row_bytes(qtype, k) + batch * 4 * (n + k)
     gbs = nbytes / st["median_us"] / 1e3
     return record(be, op_ref, matvec_kernel_name(qtype, [n], k, batch, be.compute_units),
                   graph_digest(f"{op_ref}:{FMT_NAME[qtype]}:n{n}:k{k}:b{batch}", blocks),
                   batch * 1e6 / st["median_us"], shape={"N": n, "K": k, "batch": batch, "format": FMT_NAME[qtype]},
                   timing=st, algorithmic_bytes=int(nbytes), GBps=round(gbs, 1), bound="hbm",
-                  frac_of_roofline=round(gbs / HBM_PEAK_GBS, 4), weight_copies=copies,
+                  frac_of_roofline=round(gbs / HBM_PEAK_GBS, 4), weight_copies=copies, **extra,
                   tokens_definition="activation columns through this one projection per second",
                   not_measured=["end-to-end model tokens/s (this record is one projection)", "host-side launch cost (graph replay)"])
 

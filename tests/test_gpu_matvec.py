@@ -461,6 +461,88 @@ def test_streaming_kernels_every_variant(hip, orc, qname):
     assert ran >= (20 if qname == "Q6_K" else 40)
 
 
+# ------------------------------------------------------------------ small-batch int8-MFMA kernels
+
+def mfma_plan(ks, threads, blocks, ring):
+    p = _ffi.MatvecPlan()
+    p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream, p.mfma = 16, 1, 8, 1, blocks, threads, ring, ks
+    return p
+
+
+@pytest.mark.parametrize("qname", ["Q4_K", "Q5_K"])
+def test_mfma_kernels_every_variant(hip, orc, qname):
+    """16-row tiles, K cut into `mfma` slices of at most eight chunks, one wave per (tile, slice).
+    k = 2560 gives slices of five chunks (a ragged last 1 KB load), k = 14336 slices of seven; several
+    matrices per launch with tile-aligned boundaries; few workgroups make every wave walk several units
+    (ring slots refilled, partial sums folded through LDS each time); every batch from 1 to 8 (columns
+    past the batch are zero operands whose results are dropped)."""
+    t = getattr(orc, qname)
+    ran = refused = 0
+    for k, ns, batches in ((2048, [80], (1, 2, 8)), (2560, [48, 16, 80, 32], (3, 8)), (4096, [1024, 256, 256], (2, 5, 7)), (14336, [64, 16], (4, 8))):
+        Ws = [weights(orc, qname, 950 + i, n, k) for i, n in enumerate(ns)]
+        ws = [hip.upload_weight(t, W, n, k) for W, n in zip(Ws, ns)]
+        for batch in batches:
+            x = G.seeded_acts(951 + batch, batch, k)
+            refs = [orc.matvec(t, orc.ACT_Q8, W, x, n, k) for W, n in zip(Ws, ns)]
+            xq = hip.quantize_activations(hip.upload(x), k, batch, _ffi.Q8_K)
+            for ks in (1, 2, 4, 8):
+                C = k // 256
+                if C % ks or C // ks > 8:
+                    continue
+                for threads, blocks, ring in ((256, 2, 1), (512, 1, 2), (512, 3, 3), (256, 5, 4), (512, 256, 1)):
+                    if ks > threads // 64:
+                        continue
+                    p = mfma_plan(ks, threads, blocks, ring)
+                    say(f"mfma {qname} k={k} ns={ns} batch={batch} {p.as_dict()}")
+                    ys = [hip.upload(np.full((batch, n), np.nan, np.float32)) for n in ns]
+                    try:
+                        hip.quantized_matvec_planned(ws, xq, ys, batch, _ffi.ACT_Q8, p)
+                    except backend.PsnError as e:
+                        # refused before anything is launched: the rings do not fit 160 KB of LDS or their loads
+                        # exceed the hardware's load counter
+                        assert e.code == _ffi.E_UNSUPPORTED and any(w in str(e) for w in ("LDS", "64 loads")), str(e)
+                        refused += 1
+                        continue
+                    ran += 1
+                    for y, ref, n in zip(ys, refs, ns):
+                        got = y.download(np.float32, (batch, n))
+                        err = G.max_rel_err(got, ref)
+                        assert np.all(np.isfinite(got)) and err < PARITY_TOL, (p.as_dict(), k, n, batch, err)
+    say(f"mfma {qname}: {ran} variants ran, {refused} refused")
+    assert ran >= 50
+
+
+def test_mfma_default_plan_and_refusals(hip, orc):
+    """psn_qmatvec picks the MFMA kernel for batch 2..8 of Q4_K / Q5_K where the shape allows and the
+    register kernels elsewhere; plans the kernel cannot run are refused before any launch."""
+    for qt, n, k in ((_ffi.Q4_K, 14336, 4096), (_ffi.Q4_K, 4096, 14336), (_ffi.Q5_K, 14336, 4096)):
+        for batch in (2, 4, 8):
+            p = backend.matvec_plan(qt, _ffi.ACT_Q8, n, k, batch)
+            assert p.mfma in (4, 8) and p.stage_lds == 1 and p.stream == 1, p.as_dict()
+    assert backend.matvec_plan(_ffi.Q5_K, _ffi.ACT_Q8, 4096, 14336, 4).mfma == 0         # eight 20 KB units exceed the LDS
+    assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_Q8, 1000, 4096, 4).mfma == 0          # 1000 rows: not whole tiles
+    assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_Q8, 4096, 11008, 4).mfma == 0         # 43 chunks do not split
+    assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_F32, 4096, 4096, 4).mfma == 0
+    assert backend.matvec_plan(_ffi.Q6_K, _ffi.ACT_Q8, 4096, 4096, 4).mfma == 0
+    k = 2048
+    x = G.seeded_acts(960, 2, k)
+    xq = hip.quantize_activations(hip.upload(x), k, 2, _ffi.Q8_K)
+    w_ok = hip.upload_weight(orc.Q4_K, weights(orc, "Q4_K", 961, 32, k), 32, k)
+    w_ragged = hip.upload_weight(orc.Q4_K, weights(orc, "Q4_K", 962, 40, k), 40, k)
+    w_q6 = hip.upload_weight(orc.Q6_K, weights(orc, "Q6_K", 963, 32, k), 32, k)
+    y = hip.alloc(2 * 40 * 4)
+    for w, p in ((w_ragged, mfma_plan(2, 256, 2, 1)), (w_q6, mfma_plan(2, 256, 2, 1)), (w_ok, mfma_plan(3, 256, 2, 1)),
+                 (w_ok, mfma_plan(8, 256, 2, 1)), (w_ok, mfma_plan(2, 256, 2, 0)), (w_ok, mfma_plan(2, 256, 2, 5)), (w_ok, mfma_plan(2, 128, 2, 1))):
+        with pytest.raises(backend.PsnError) as e:
+            hip.quantized_matvec_planned(w, xq, y, 2, _ffi.ACT_Q8, p)
+        assert e.value.code == _ffi.E_UNSUPPORTED, p.as_dict()
+    p = mfma_plan(2, 256, 2, 1)
+    p.stage_lds = 2                                          # fp32 input: this kernel does not quantize
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_planned(w_ok, hip.upload(x), y, 2, _ffi.ACT_Q8, p)
+    assert e.value.code == _ffi.E_UNSUPPORTED
+
+
 def test_streaming_plan_is_refused_where_it_cannot_run(hip, orc):
     k = 2560
     w6 = hip.upload_weight(orc.Q6_K, weights(orc, "Q6_K", 910, 80, k), 80, k)

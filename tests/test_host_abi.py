@@ -63,7 +63,7 @@ def test_activation_layout(lib):
 
 
 def test_matvec_plan_is_host_arithmetic(lib):
-    for qt in (_ffi.Q4_0, _ffi.Q8_0, _ffi.Q4_K, _ffi.Q6_K):
+    for qt in (_ffi.Q4_0, _ffi.Q8_0, _ffi.Q4_K, _ffi.Q5_K, _ffi.Q6_K):
         for (n, k) in ((4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336), (128256, 4096), (1, 256)):
             for batch in range(1, 9):
                 for scheme in (_ffi.ACT_F32, _ffi.ACT_Q8):
@@ -71,6 +71,7 @@ def test_matvec_plan_is_host_arithmetic(lib):
                     assert p.lanes_per_row in (8, 16, 32, 64) and p.rows_in_flight == 1
                     assert p.batch_tile >= batch and p.batch_tile in (1, 2, 4, 8)
                     assert 1 <= p.blocks <= 256 * 16 and p.threads in (256, 512)
+                    assert p.mfma in (0, 1, 2, 4, 8) and (p.mfma == 0 or (batch >= 2 and scheme == _ffi.ACT_Q8 and qt in (_ffi.Q4_K, _ffi.Q5_K)))
     for args, code in (((_ffi.Q4_0, 1, 0, 4096, 1), _ffi.E_SHAPE), ((_ffi.Q4_0, 1, 16, 4096 + 32, 1), _ffi.E_SHAPE),
                        ((_ffi.Q4_0, 1, 16, 4096, 9), _ffi.E_SHAPE), ((_ffi.Q8_K, 1, 16, 4096, 1), _ffi.E_UNSUPPORTED),
                        ((_ffi.Q4_0, 5, 16, 4096, 1), _ffi.E_UNSUPPORTED)):
