@@ -221,8 +221,9 @@ typedef struct psn_matvec_plan {
     int32_t mfma;           /* 0, or 1/2/4/8: the small-batch int8-MFMA kernel (Q4_K and Q5_K, scheme Q8, batch 1..8,
                                x already quantized: stage_lds 1) -- that many waves share a 16-row tile, each owning
                                K / mfma of it (a whole number of at most eight 256-weight chunks); every matrix a
-                               multiple of 16 rows; stream = 1..4 units in flight per wave; lanes_per_row,
-                               rows_in_flight and batch_tile are not used */
+                               multiple of 16 rows; stream = 1; slices of more than four chunks need one wave per
+                               (tile, slice): blocks * (threads / 64 / mfma) >= tiles; lanes_per_row, rows_in_flight
+                               and batch_tile are not used */
 } psn_matvec_plan;
 int32_t psn_qmatvec_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, int32_t batch, int32_t compute_units,
                          int32_t x_is_f32, psn_matvec_plan *out);

@@ -711,9 +711,15 @@ static int32_t mfma_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32_t
         if (n_rows[i] % 16) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernels need every matrix to hold a multiple of 16 rows");
     if (plan->blocks < 1 || plan->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", plan->blocks);
     const int64_t words = (C / ks) * (qtype == PSN_Q4_K ? 9 : 11), ni = (words + 3) / 4;
-    const int ring = plan->stream;
-    if (ring < 1 || ring > 4 || (ring - 1) * ni + ni - 1 > 63) return fail(PSN_E_UNSUPPORTED, "plan: stream=%d (with mfma: units in flight per wave, 1..4, at most 64 loads)", ring);
-    const int64_t total = C * 160 + (int64_t)waves * 1024 + (int64_t)waves * ring * ni * 1024;
+    if (plan->stream != 1) return fail(PSN_E_UNSUPPORTED, "plan: stream=%d (with mfma: 1)", plan->stream);
+    /* slices of more than four chunks run the kernel whose waves handle exactly one unit each */
+    if (C / ks > 4 && n_rows) {
+        int64_t tiles = 0;
+        for (int i = 0; i < count; ++i) tiles += n_rows[i] / 16;
+        if ((int64_t)plan->blocks * (waves / ks) < tiles)
+            return fail(PSN_E_UNSUPPORTED, "plan: slices of %lld chunks need one wave per unit (%lld tiles, %d workgroups of %d)", (long long)(C / ks), (long long)tiles, plan->blocks, waves / ks);
+    }
+    const int64_t total = C * 160 + (int64_t)waves * 1024 + (int64_t)waves * ni * 1024;
     if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernel needs %lld bytes of LDS, device offers %d", (long long)total, max_lds);
     *lds_out = total;
     return PSN_OK;
@@ -791,7 +797,7 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
         q.lanes_per_row = 16;
         q.stream = 1;
         q.batch_tile = 8;
-        q.blocks = 1;
+        q.blocks = 1 << 20;                             /* for the checks; set below */
         int64_t lds = 0;
         int32_t ok = PSN_E_UNSUPPORTED;
         for (int pass = 0; pass < 2 && ok != PSN_OK; ++pass) {
@@ -807,7 +813,7 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
             const int64_t tpw = (q.threads / 64) / q.mfma, ntiles = N / 16;
             int64_t b = (ntiles + tpw - 1) / tpw;
             const int64_t cap = (q.threads == 256 ? 2 : 1) * (int64_t)cus;
-            if (b > cap) b = cap;
+            if (b > cap && C / q.mfma <= 4) b = cap;    /* longer slices: one unit per wave, the grid covers every tile */
             q.blocks = (int32_t)b;
             *out = q;
             return PSN_OK;
@@ -920,8 +926,7 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
         a.xd = (const float *)((const char *)x + li.off_d);
         a.xs = (const char *)x + li.off_s;
         a.kslices = plan->mfma;
-        a.ring = plan->stream;
-        snprintf(name, sizeof name, "psn_mvm_%s_q8", fmt_name(qtype));
+        snprintf(name, sizeof name, "psn_mvm_%s_q8_%s", fmt_name(qtype), (K / 256) / plan->mfma > 4 ? "t8" : "p4");
         return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)total, &a);
     }
     if (plan->stream) {

@@ -75,7 +75,7 @@ struct LaneOffs {
 };
 
 template <typename F, int CI>
-PSN_DEV void mf_chunk(const LaneOffs &o, u32 xs_addr, u32 dx_addr, const u64 (&x)[8][8], bool first_quarter, float (&acc)[4]) {
+PSN_DEV void mf_chunk(const LaneOffs &o, u32 xs_addr, u32 dx_addr, const u64 (&x)[8], bool first_quarter, float (&acc)[4]) {
     constexpr int T0 = F::WORDS * CI;                       /* first word of the chunk in the slice */
     const u32x4 hdr = lds_read128<(T0 >> 2) * 1024>(o.hdr[T0 & 3]);
     u64 wq[4];
@@ -116,8 +116,8 @@ PSN_DEV void mf_chunk(const LaneOffs &o, u32 xs_addr, u32 dx_addr, const u64 (&x
             h0 |= ((q0 >> (2 * g + 1)) & 0x01010101u) << 4;
             h1 |= ((q1 >> (2 * g + 1)) & 0x01010101u) << 4;
         }
-        const v4i dl = mfma_i8(x[CI][2 * g], pack64(l0, l1));
-        const v4i dh = mfma_i8(x[CI][2 * g + 1], pack64(h0, h1));
+        const v4i dl = mfma_i8(x[2 * g], pack64(l0, l1));
+        const v4i dh = mfma_i8(x[2 * g + 1], pack64(h0, h1));
         const int s0 = (int)((sc[g >> 1] >> (16 * (g & 1))) & 0xffu), s1 = (int)((sc[g >> 1] >> (16 * (g & 1) + 8)) & 0xffu);
         UNROLL for (int i = 0; i < 4; ++i) { isum[i] += __mul24(s0, dl[i]); isum[i] += __mul24(s1, dh[i]); }
     }
@@ -129,8 +129,13 @@ PSN_DEV void mf_chunk(const LaneOffs &o, u32 xs_addr, u32 dx_addr, const u64 (&x
     }
 }
 
-template <typename F>
+/* SLMAX: chunks per slice the instantiation is unrolled for.  PERSIST: the regrouped activations of the
+ * whole slice stay in registers so that a wave can walk any number of units (SLMAX 4: 64 registers);
+ * without it they are regrouped chunk by chunk into the same 16 registers, and a wave handles exactly one
+ * unit (the host launches enough workgroups). */
+template <typename F, int SLMAX, bool PERSIST>
 PSN_DEV void mv_mfma(const psn_matvec_args &a) {
+#define PSN_XI(CI) (PERSIST ? ((CI) < SLMAX ? (CI) : 0) : 0)
     extern __shared__ uint4 psn_smem[];
     typedef __attribute__((address_space(3))) char lds_char;
     lds_char *const lds_ptr = (lds_char *)psn_smem;
@@ -142,140 +147,172 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     const int ks = wib % KS, tl = wib / KS;
     const int c0 = ks * SL;                                  /* first chunk of this wave's K slice */
     const int nw = SL * F::WORDS;                            /* 16-byte words per row of a slice */
-    const int NI = (nw + 3) >> 2;                            /* load instructions (1 KB each) per unit */
     const int ntiles = a.N >> 4;
     const int rb = (int)a.row_bytes;
     const int batch = a.batch;
+    const int NI = (nw + 3) >> 2;                            /* load instructions (1 KB each) per unit */
 
-    /* LDS: sub-block sums [C][8 columns][16 B], activation scales [C][8] floats, 1 KB per wave (regrouping
-     * of the activations at the start, partial sums [4][64] floats at the end), then `ring` buffers of
-     * NI KB per wave */
-    const int ring = a.ring;
+    /* LDS: sub-block sums [C][8 columns][16 B], activation scales [C][8] floats (every wave fills in and
+     * reads only its own chunks), 1 KB per wave (regrouping of the activations, later the partial sums
+     * [4][64] floats), then one buffer of NI KB per wave */
     const u32 xs_tab = lds0, dx_tab = xs_tab + (u32)C * 128u, red = dx_tab + (u32)C * 32u;
-    const u32 buf_off = (u32)C * 160u + (u32)wpb * 1024u + (u32)(wib * ring) * (u32)NI * 1024u;
+    const u32 buf_off = (u32)C * 160u + (u32)wpb * 1024u + (u32)wib * (u32)NI * 1024u;
     const u32 buf = lds0 + buf_off;
 
-    /* ---- loads go out in the order they are needed: table inputs, this wave's activations, weights ---- */
-    const int16_t *bs = reinterpret_cast<const int16_t *>(a.xs);
-    u32x4 tb0[2], tb1[2];
-    u32 tbd[2];
-    UNROLL for (int rd = 0; rd < 2; ++rd) {
-        const int item = threadIdx.x + rd * a.threads, c = item >> 3, m = item & 7;
-        tb0[rd] = tb1[rd] = (u32x4)(0u);
-        tbd[rd] = 0;
-        if (c < C && m < batch) {
-            const int16_t *p = bs + ((int64_t)m * C + c) * 16;
-            tb0[rd] = global_read128(p);
-            tb1[rd] = global_read128(p + 8);
-            tbd[rd] = global_read32(a.xd + m * C + c);
-        }
-    }
-    /* this wave's activations, fetched the way memory likes them: one instruction covers 256 contiguous
-     * bytes (a chunk) of each of four columns; they are regrouped into MFMA operands through LDS below */
-    u32x4 xt[8][2];
+    /* The matrices sharing the launch: lane i (< 4) of these registers holds matrix i's base addresses, first
+     * row and row count (v_readlane with the matrix index picks one: no block of scalar registers is tied up
+     * for the whole kernel, and no indexed read of the kernel arguments).  Row ends past the last matrix
+     * equal the total, so they never compare below a row. */
+    const int E0 = a.row_end[0], E1 = a.row_end[1], E2 = a.row_end[2];
+    u32 seg_w_lo, seg_w_hi, seg_y_lo, seg_y_hi, seg_first, seg_rows;
     {
-        const int col = lane >> 4;                           /* + 4 i */
-        const int8_t *xp = a.xqs + (int64_t)col * K + (int64_t)c0 * 256 + (lane & 15) * 16;
-        UNROLL for (int c = 0; c < 8; ++c) UNROLL for (int i = 0; i < 2; ++i) {
-            xt[c][i] = (u32x4)(0u);
-            if (c < SL && col + 4 * i < batch) xt[c][i] = global_read128(xp + (int64_t)(4 * i) * K + c * 256);
-        }
+        const int li = lane & 3;
+        /* (the empty asm keeps the compiler from turning the selects into an indexed load from a private
+         * copy of the arguments) */
+        const uint8_t *W0 = a.W[0], *W1 = a.W[1], *W2 = a.W[2], *W3 = a.W[3];
+        float *Y0 = a.y[0], *Y1 = a.y[1], *Y2 = a.y[2], *Y3 = a.y[3];
+        int E3 = a.row_end[3];
+        asm volatile("" : "+s"(W0), "+s"(W1), "+s"(W2), "+s"(W3), "+s"(Y0), "+s"(Y1), "+s"(Y2), "+s"(Y3), "+s"(E3));
+        const uint8_t *wv = li == 0 ? W0 : li == 1 ? W1 : li == 2 ? W2 : W3;
+        float *yv = li == 0 ? Y0 : li == 1 ? Y1 : li == 2 ? Y2 : Y3;
+        const int fv = li == 0 ? 0 : li == 1 ? E0 : li == 2 ? E1 : E2;
+        const int ev = li == 0 ? E0 : li == 1 ? E1 : li == 2 ? E2 : E3;
+        seg_w_lo = (u32)(uintptr_t)wv; seg_w_hi = (u32)((uintptr_t)wv >> 32);
+        seg_y_lo = (u32)(uintptr_t)yv; seg_y_hi = (u32)((uintptr_t)yv >> 32);
+        seg_first = (u32)fv; seg_rows = (u32)(ev - fv);
     }
-
-    const uint8_t *W0 = a.W[0], *W1 = a.W[1], *W2 = a.W[2], *W3 = a.W[3];
-    float *Y0 = a.y[0], *Y1 = a.y[1], *Y2 = a.y[2], *Y3 = a.y[3];
-    int E0 = a.row_end[0], E1 = a.row_end[1], E2 = a.row_end[2], E3 = a.row_end[3];
-    asm volatile("" : "+s"(W0), "+s"(W1), "+s"(W2), "+s"(W3), "+s"(Y0), "+s"(Y1), "+s"(Y2), "+s"(Y3), "+s"(E0), "+s"(E1), "+s"(E2), "+s"(E3));
-    const int nseg = a.nseg;
     /* a tile never straddles two matrices (every matrix holds a multiple of 16 rows) */
     auto tile_base = [&](int tile, const uint8_t *&w, float *&y, int &nrows) {
         const int row0 = tile << 4;
-        const uint8_t *wb = W0;
-        float *yb = Y0;
-        int first = 0, end = E0;
-        if (nseg > 1 && row0 >= E0) { wb = W1; yb = Y1; first = E0; end = E1; }
-        if (nseg > 2 && row0 >= E1) { wb = W2; yb = Y2; first = E1; end = E2; }
-        if (nseg > 3 && row0 >= E2) { wb = W3; yb = Y3; first = E2; end = E3; }
-        w = wb + (int64_t)(row0 - first) * rb;
-        y = yb + (row0 - first);
-        nrows = end - first;
+        const int si = (row0 >= E0) + (row0 >= E1) + (row0 >= E2);
+        const u64 wb = pack64(__builtin_amdgcn_readlane(seg_w_lo, si), __builtin_amdgcn_readlane(seg_w_hi, si));
+        const u64 yb = pack64(__builtin_amdgcn_readlane(seg_y_lo, si), __builtin_amdgcn_readlane(seg_y_hi, si));
+        const int first = __builtin_amdgcn_readlane(seg_first, si);
+        nrows = __builtin_amdgcn_readlane(seg_rows, si);
+        w = (const uint8_t *)(uintptr_t)wb + (int64_t)(row0 - first) * rb;
+        y = (float *)(uintptr_t)yb + (row0 - first);
     };
-    /* lane p fetches row p >> 2; in instruction i it owns word 4 i + ((p & 3) ^ (row >> 2)) */
+
+    /* ---- what a wave requests, in this order: its table inputs, then chunk by chunk the activations
+     *      (first unit only) and the weight words up to the chunk's end.  A compute unit keeps a bounded
+     *      number of bytes in flight and an issuing wave stalls until its request is accepted, so loads
+     *      are requested two chunks ahead of the arithmetic instead of all at once: while some waves sit
+     *      in a load instruction the others multiply. ---- */
+
+    /* table inputs: entry e = lane covers (column e & 7, chunk e >> 3) of this wave's slice */
+    const int te_m = lane & 7, te_c = lane >> 3;
+    const bool te_live = te_c < SL && te_m < batch;
+    u32x4 tb0 = (u32x4)(0u), tb1 = (u32x4)(0u);
+    u32 tbd = 0;
+    if (te_live) {
+        const int16_t *p = reinterpret_cast<const int16_t *>(a.xs) + ((int64_t)te_m * C + c0 + te_c) * 16;
+        tb0 = global_read128(p);
+        tb1 = global_read128(p + 8);
+        tbd = global_read32(a.xd + te_m * C + c0 + te_c);
+    }
+
+    /* activations: one instruction covers 256 contiguous bytes (a chunk) of each of four columns */
+    u32x4 xt[3][2];                                          /* chunks CI, CI + 1, CI + 2 are in flight: slot CI % 3 */
+    const int xcol = lane >> 4;                              /* + 4 i */
+    const int8_t *xp = a.xqs + (int64_t)xcol * K + (int64_t)c0 * 256 + (lane & 15) * 16;
+    const int nx = batch > 4 ? 2 : 1;
+    /* weights: lane p fetches row p >> 2; in instruction i it owns word 4 i + ((p & 3) ^ (row >> 2)) */
     const int lrow = lane >> 2, lword = (lane & 3) ^ (lrow >> 2);
     const int64_t lane_goff = (int64_t)lrow * rb + (int64_t)c0 * (F::WORDS * 16);
-    auto issue = [&](int tile, int b) {
-        const uint8_t *w;
-        float *y;
-        int nrows;
-        tile_base(tile, w, y, nrows);
-        const uint8_t *src = w + lane_goff;
-        lds_char *dst = lds_ptr + buf_off + b * (NI << 10);
-        int t = lword;
-        for (int i = 0; i < NI; ++i) {
-            __builtin_amdgcn_global_load_lds((const void *)(src + min(t, nw - 1) * 16), (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+    const uint8_t *wsrc_lane = nullptr;                      /* current unit's tile + lane_goff */
+    auto issue_w = [&](int i0, int i1) {                     /* load instructions i0 .. i1 of the current unit */
+        lds_char *dst = lds_ptr + buf_off + (i0 << 10);
+        int t = lword + 4 * i0;
+        for (int i = i0; i <= i1; ++i) {
+            __builtin_amdgcn_global_load_lds((const void *)(wsrc_lane + min(t, nw - 1) * 16), (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
             t += 4;
             dst += 1024;
         }
     };
+    bool first_unit = true;
+#define PSN_MF_ISSUE(CI)                                                                                     \
+    if (CI < SL) {                                                                                           \
+        if (first_unit) {                                                                                    \
+            UNROLL for (int i = 0; i < 2; ++i) {                                                             \
+                xt[(CI) % 3][i] = (u32x4)(0u);                                                                     \
+                if (4 * i < batch) {                                                                         \
+                    if (xcol + 4 * i < batch) xt[(CI) % 3][i] = global_read128(xp + (int64_t)(4 * i) * K + CI * 256); \
+                }                                                                                            \
+            }                                                                                                \
+        }                                                                                                    \
+        issue_w(CI == 0 ? 0 : ((F::WORDS * CI - 1) >> 2) + 1, min((F::WORDS * CI + F::WORDS - 1) >> 2, NI - 1)); \
+    }
 
     const int tiles_per_round = a.blocks * TPW;
-    const int iters = (ntiles + tiles_per_round - 1) / tiles_per_round;
+    const int iters = PERSIST ? (ntiles + tiles_per_round - 1) / tiles_per_round : 1;
     int tile = blockIdx.x * TPW + tl;
-    /* everything the ring holds goes in flight at once */
-    int issued = 0;
-    for (; issued < ring && tile + issued * tiles_per_round < ntiles; ++issued) issue(tile + issued * tiles_per_round, issued);
-
-    /* ---- tables: per chunk and column, the eight sub-block sums as (low 6 bits, signed rest) bytes and the scale ---- */
-    wait_vmcnt(issued * NI);
-    UNROLL for (int rd = 0; rd < 2; ++rd) {
-        asm volatile("" : "+v"(tb0[rd]), "+v"(tb1[rd]), "+v"(tbd[rd]));
-        const int item = threadIdx.x + rd * a.threads, c = item >> 3;
-        if (c < C) {
-            u32 lo[2] = {0, 0}, hi[2] = {0, 0};
-            UNROLL for (int j = 0; j < 8; ++j) {
-                const u32 v = j < 4 ? tb0[rd][j] : tb1[rd][j - 4];
-                const int s = (int)(int16_t)(v & 0xffffu) + ((int)v >> 16);
-                lo[j >> 2] |= (u32)(s & 63) << (8 * (j & 3));
-                hi[j >> 2] |= (u32)((s >> 6) & 0xff) << (8 * (j & 3));
-            }
-            u32x4 e;
-            e.x = lo[0]; e.y = lo[1]; e.z = hi[0]; e.w = hi[1];
-            lds_write128(xs_tab + (u32)item * 16u, e);
-            lds_write32(dx_tab + (u32)item * 4u, tbd[rd]);
-        }
+    const uint8_t *wtile;
+    float *ydst;
+    int nrows = 0;
+    if (tile < ntiles) {
+        tile_base(tile, wtile, ydst, nrows);
+        wsrc_lane = wtile + lane_goff;
+        PSN_MF_ISSUE(0)
+        PSN_MF_ISSUE(1)
     }
-    /* Regroup: lane (m = lane & 15, kq = lane >> 4) needs bytes 8 kq .. 8 kq + 7 of every sub-block of
-     * column m.  Four columns of one chunk pass through the wave's own 1 KB at a time: the 8-byte piece
-     * (column cq, sub-block sb, quarter kq) sits at
+
+    /* ---- this wave's table entries: the eight sub-block sums of (column, chunk) as (low 6 bits, signed
+     *      rest) bytes, and the activation scale ---- */
+    /* the last load instruction of the unit that chunk j needs */
+    auto w_last = [&](int j) { return min((F::WORDS * j + F::WORDS - 1) >> 2, NI - 1); };
+    {
+        const int g = min(2, SL);                            /* chunks requested so far */
+        wait_vmcnt(tile < ntiles ? g * nx + w_last(g - 1) + 1 : 0);
+    }
+    asm volatile("" : "+v"(tb0), "+v"(tb1), "+v"(tbd));
+    if (te_c < SL) {
+        u32 lo[2] = {0, 0}, hi[2] = {0, 0};
+        UNROLL for (int j = 0; j < 8; ++j) {
+            const u32 v = j < 4 ? tb0[j] : tb1[j - 4];
+            const int s16 = (int)(int16_t)(v & 0xffffu) + ((int)v >> 16);
+            lo[j >> 2] |= (u32)(s16 & 63) << (8 * (j & 3));
+            hi[j >> 2] |= (u32)((s16 >> 6) & 0xff) << (8 * (j & 3));
+        }
+        u32x4 e;
+        e.x = lo[0]; e.y = lo[1]; e.z = hi[0]; e.w = hi[1];
+        const u32 item = (u32)((c0 + te_c) * 8 + te_m);
+        lds_write128(xs_tab + item * 16u, e);
+        lds_write32(dx_tab + item * 4u, tbd);
+    }
+
+    /* Regrouping of a chunk's activations: lane (m = lane & 15, kq = lane >> 4) needs bytes 8 kq .. 8 kq + 7
+     * of every sub-block of column m.  Four columns pass through the wave's own 1 KB at a time: the 8-byte
+     * piece (column cq, sub-block sb, quarter kq) sits at
      *     cq * 256 + (((sb >> 1) ^ cq) & 3) * 64 + kq * 16 + (sb & 1) * 8,
      * so a lane picks up two sub-blocks per 16-byte read and the lanes of one read touch every bank
      * once.  One wave's LDS operations execute in order: no waits in between. */
-    u64 x[8][8];
-    UNROLL for (int c = 0; c < 8; ++c) UNROLL for (int sb = 0; sb < 8; ++sb) x[c][sb] = 0ull;
+    u64 x[PERSIST ? SLMAX : 1][8];
+    UNROLL for (int c = 0; c < (PERSIST ? SLMAX : 1); ++c) UNROLL for (int sb = 0; sb < 8; ++sb) x[c][sb] = 0ull;
+    const u32 scratch = red + (u32)wib * 1024u;
+    u32 rg_wr, rg_rd;
     {
-        const u32 scratch = red + (u32)wib * 1024u;
         const u32 cq_w = (u32)(lane >> 4), w = (u32)(lane & 15), sb_w = w >> 1;
-        const u32 wr = scratch + cq_w * 256u + ((((sb_w >> 1) ^ cq_w) & 3u) << 6) + (w & 1u) * 32u + (sb_w & 1u) * 8u;
-        const u32 cq_r = (u32)(n & 3);
-        const u32 rd = scratch + cq_r * 256u + (u32)kq * 16u;
-        UNROLL for (int c = 0; c < 8; ++c) UNROLL for (int i = 0; i < 2; ++i) {
-            if (c < SL && 4 * i < batch) {
-                asm volatile("" : "+v"(xt[c][i]));
-                lds_write64(wr, pack64(xt[c][i].x, xt[c][i].y));
-                lds_write64(wr + 16u, pack64(xt[c][i].z, xt[c][i].w));
-                if ((n >> 2) == i) {
-                    UNROLL for (u32 q = 0; q < 4; ++q) {
-                        const u32x4 v = lds_read128<0>(rd + (((q ^ cq_r) & 3u) << 6));
-                        x[c][2 * q] = pack64(v.x, v.y);
-                        x[c][2 * q + 1] = pack64(v.z, v.w);
-                    }
-                }
-            }
-        }
-        lds_wait();
-        UNROLL for (int c = 0; c < 8; ++c) UNROLL for (int sb = 0; sb < 8; ++sb) tie64(x[c][sb]);
+        rg_wr = scratch + cq_w * 256u + ((((sb_w >> 1) ^ cq_w) & 3u) << 6) + (w & 1u) * 32u + (sb_w & 1u) * 8u;
+        rg_rd = scratch + (u32)(n & 3) * 256u + (u32)kq * 16u;
     }
-    lds_barrier();
+    const u32 cq_r = (u32)(n & 3);
+#define PSN_MF_REGROUP(CI)                                                                                   \
+    UNROLL for (int i = 0; i < 2; ++i) {                                                                     \
+        if (4 * i < batch) {                                                                                 \
+            asm volatile("" : "+v"(xt[(CI) % 3][i]));                                                              \
+            lds_write64(rg_wr, pack64(xt[(CI) % 3][i].x, xt[(CI) % 3][i].y));                                            \
+            lds_write64(rg_wr + 16u, pack64(xt[(CI) % 3][i].z, xt[(CI) % 3][i].w));                                      \
+            if ((n >> 2) == i) {                                                                             \
+                UNROLL for (u32 q = 0; q < 4; ++q) {                                                         \
+                    const u32x4 v = lds_read128<0>(rg_rd + (((q ^ cq_r) & 3u) << 6));                        \
+                    x[PSN_XI(CI)][2 * q] = pack64(v.x, v.y);                                                         \
+                    x[PSN_XI(CI)][2 * q + 1] = pack64(v.z, v.w);                                                     \
+                }                                                                                            \
+            }                                                                                                \
+        }                                                                                                    \
+    }                                                                                                        \
+    lds_wait();                                                                                              \
+    UNROLL for (int sb = 0; sb < 8; ++sb) tie64(x[PSN_XI(CI)][sb]);
 
     LaneOffs o;
     {
@@ -292,37 +329,37 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     const u32 red_w = red + (u32)wib * 1024u + (u32)lane * 4u;
     const bool first_quarter = kq == 0;
 
-    int b = 0;                                               /* ring buffer of the current unit */
-    for (int it = 0; it < iters; ++it, tile += tiles_per_round) {
+    for (int it = 0; it < iters; ++it) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
         const bool live = tile < ntiles;
         if (live) {
-            /* the units issued after this one stay in flight; chunk CI of this one is complete once the
-             * instruction holding its last word has landed */
-            const int younger = (issued - it - 1) * NI + NI - 1;
-            LaneOffs ob;
-            const u32 boff = (u32)(b * (NI << 10));
-            UNROLL for (int k = 0; k < 4; ++k) { ob.hdr[k] = o.hdr[k] + boff; ob.w[k] = o.w[k] + boff; }
+            /* chunk CI: request chunk CI + 2, wait until CI's own requests have landed (everything
+             * requested later may stay in flight), regroup its activations (first unit), multiply */
 #define PSN_MF_CHUNK(CI)                                                                   \
-            if (CI < SL) {                                                                 \
-                wait_vmcnt(younger - ((F::WORDS * CI + F::WORDS - 1) >> 2));               \
-                mf_chunk<F, CI>(ob, xs_addr, dx_addr, x, first_quarter, acc);              \
+            if (CI < SLMAX && CI < SL) {                                                   \
+                if (CI + 2 < SLMAX) { PSN_MF_ISSUE((CI + 2 < 8 ? CI + 2 : 7)) }           \
+                {                                                                          \
+                    const int g = min(CI + 3, SL);       /* chunks requested so far */     \
+                    wait_vmcnt((g - CI - 1) * (first_unit ? nx : 0) + w_last(g - 1) - w_last(CI)); \
+                }                                                                          \
+                if (first_unit) { PSN_MF_REGROUP(CI) }                                     \
+                mf_chunk<F, CI>(o, xs_addr, dx_addr, x[PSN_XI(CI)], first_quarter, acc);   \
             }
             PSN_MF_CHUNK(0) PSN_MF_CHUNK(1) PSN_MF_CHUNK(2) PSN_MF_CHUNK(3)
             PSN_MF_CHUNK(4) PSN_MF_CHUNK(5) PSN_MF_CHUNK(6) PSN_MF_CHUNK(7)
 #undef PSN_MF_CHUNK
+            first_unit = false;
         }
-        const uint8_t *wsrc;
-        float *ydst;
-        int nrows = 0;
-        if (live) tile_base(tile, wsrc, ydst, nrows);
-        /* this buffer is free again: refill it with the unit `ring` steps ahead */
-        const int next = tile + ring * tiles_per_round;
-        if (live && next < ntiles) {
-            issue(next, b);
-            ++issued;
+        float *const ycur = ydst;
+        const int ncur = nrows;
+        /* the buffer is free: the next unit's first two chunks are requested while the partial sums are folded */
+        tile += tiles_per_round;
+        if (live && tile < ntiles) {
+            tile_base(tile, wtile, ydst, nrows);
+            wsrc_lane = wtile + lane_goff;
+            PSN_MF_ISSUE(0)
+            PSN_MF_ISSUE(1)
         }
-        b = b + 1 == ring ? 0 : b + 1;
         if (KS > 1) {
             UNROLL for (int i = 0; i < 4; ++i) lds_write32(red_w + (u32)i * 256u, __float_as_uint(acc[i]));
             lds_barrier();
@@ -338,12 +375,19 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
         if (live && ks == 0) {
             UNROLL for (int i = 0; i < 4; ++i) {
                 const int col = 4 * kq + i;
-                if (col < batch) ydst[(int64_t)col * nrows + n] = acc[i];
+                if (col < batch) ycur[(int64_t)col * ncur + n] = acc[i];
             }
         }
         if (KS > 1) lds_barrier();
     }
+#undef PSN_MF_ISSUE
+#undef PSN_MF_REGROUP
+#undef PSN_XI
 }
 
-extern "C" __global__ void __launch_bounds__(512) psn_mvm_q4_K_q8(const psn_matvec_args a) { mv_mfma<MfQ4_K>(a); }
-extern "C" __global__ void __launch_bounds__(512) psn_mvm_q5_K_q8(const psn_matvec_args a) { mv_mfma<MfQ5_K>(a); }
+/* psn_mvm_<fmt>_q8_p4: slices of at most four chunks, any number of units per wave;
+ * psn_mvm_<fmt>_q8_t8: slices of at most eight chunks, one unit per wave */
+extern "C" __global__ void __launch_bounds__(512) psn_mvm_q4_K_q8_p4(const psn_matvec_args a) { mv_mfma<MfQ4_K, 4, true>(a); }
+extern "C" __global__ void __launch_bounds__(512) psn_mvm_q4_K_q8_t8(const psn_matvec_args a) { mv_mfma<MfQ4_K, 8, false>(a); }
+extern "C" __global__ void __launch_bounds__(512) psn_mvm_q5_K_q8_p4(const psn_matvec_args a) { mv_mfma<MfQ5_K, 4, true>(a); }
+extern "C" __global__ void __launch_bounds__(512) psn_mvm_q5_K_q8_t8(const psn_matvec_args a) { mv_mfma<MfQ5_K, 8, false>(a); }

@@ -88,7 +88,7 @@ def matvec_kernel_name(qtype: int, ns, k: int, batch: int, cus: int, x_is_f32: b
     p = matvec_plan(qtype, ACT_Q8, sum(ns), k, batch, cus, x_is_f32)
     f = FMT_NAME[qtype]
     if p.mfma:
-        return f"psn_quantize_q8_K + psn_mvm_{f}_q8"
+        return f"psn_quantize_q8_K + psn_mvm_{f}_q8_" + ("t8" if (k // 256) // p.mfma > 4 else "p4")
     if p.stream:
         return f"psn_mvs_{f}_q8_g{p.lanes_per_row}" + {1: "_lds", 2: "_xf"}[p.stage_lds] + f"_s{len(ns)}"
     return f"psn_mv_{f}_q8_g{p.lanes_per_row}_r{p.rows_in_flight}_b{p.batch_tile}" + {0: "", 1: "_lds", 2: "_xf"}[p.stage_lds]

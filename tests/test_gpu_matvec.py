@@ -474,7 +474,7 @@ def test_mfma_kernels_every_variant(hip, orc, qname):
     """16-row tiles, K cut into `mfma` slices of at most eight chunks, one wave per (tile, slice).
     k = 2560 gives slices of five chunks (a ragged last 1 KB load), k = 14336 slices of seven; several
     matrices per launch with tile-aligned boundaries; few workgroups make every wave walk several units
-    (ring slots refilled, partial sums folded through LDS each time); every batch from 1 to 8 (columns
+    (buffer refilled, partial sums folded through LDS each time; slices of up to four chunks only); every batch from 1 to 8 (columns
     past the batch are zero operands whose results are dropped)."""
     t = getattr(orc, qname)
     ran = refused = 0
@@ -489,7 +489,7 @@ def test_mfma_kernels_every_variant(hip, orc, qname):
                 C = k // 256
                 if C % ks or C // ks > 8:
                     continue
-                for threads, blocks, ring in ((256, 2, 1), (512, 1, 2), (512, 3, 3), (256, 5, 4), (512, 256, 1)):
+                for threads, blocks, ring in ((256, 2, 1), (512, 1, 1), (512, 3, 1), (256, 5, 1), (512, 256, 1), (256, 300, 1)):
                     if ks > threads // 64:
                         continue
                     p = mfma_plan(ks, threads, blocks, ring)
@@ -498,9 +498,9 @@ def test_mfma_kernels_every_variant(hip, orc, qname):
                     try:
                         hip.quantized_matvec_planned(ws, xq, ys, batch, _ffi.ACT_Q8, p)
                     except backend.PsnError as e:
-                        # refused before anything is launched: the rings do not fit 160 KB of LDS or their loads
-                        # exceed the hardware's load counter
-                        assert e.code == _ffi.E_UNSUPPORTED and any(w in str(e) for w in ("LDS", "64 loads")), str(e)
+                        # refused before anything is launched: the buffers do not fit 160 KB of LDS, or slices of
+                        # more than four chunks were given fewer waves than units
+                        assert e.code == _ffi.E_UNSUPPORTED and any(w in str(e) for w in ("LDS", "one wave per unit")), str(e)
                         refused += 1
                         continue
                     ran += 1
@@ -532,7 +532,8 @@ def test_mfma_default_plan_and_refusals(hip, orc):
     w_q6 = hip.upload_weight(orc.Q6_K, weights(orc, "Q6_K", 963, 32, k), 32, k)
     y = hip.alloc(2 * 40 * 4)
     for w, p in ((w_ragged, mfma_plan(2, 256, 2, 1)), (w_q6, mfma_plan(2, 256, 2, 1)), (w_ok, mfma_plan(3, 256, 2, 1)),
-                 (w_ok, mfma_plan(8, 256, 2, 1)), (w_ok, mfma_plan(2, 256, 2, 0)), (w_ok, mfma_plan(2, 256, 2, 5)), (w_ok, mfma_plan(2, 128, 2, 1))):
+                 (w_ok, mfma_plan(8, 256, 2, 1)), (w_ok, mfma_plan(2, 256, 2, 0)), (w_ok, mfma_plan(2, 256, 2, 2)), (w_ok, mfma_plan(2, 128, 2, 1)),
+                 (w_ok, mfma_plan(1, 256, 0, 1))):
         with pytest.raises(backend.PsnError) as e:
             hip.quantized_matvec_planned(w, xq, y, 2, _ffi.ACT_Q8, p)
         assert e.value.code == _ffi.E_UNSUPPORTED, p.as_dict()
