@@ -196,7 +196,7 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     /* ---- what a wave requests, in this order: its table inputs, then chunk by chunk the activations
      *      (first unit only) and the weight words up to the chunk's end.  A compute unit keeps a bounded
      *      number of bytes in flight and an issuing wave stalls until its request is accepted, so loads
-     *      are requested two chunks ahead of the arithmetic instead of all at once: while some waves sit
+     *      are requested LA chunks ahead of the arithmetic instead of all at once: while some waves sit
      *      in a load instruction the others multiply. ---- */
 
     /* table inputs: entry e = lane covers (column e & 7, chunk e >> 3) of this wave's slice */
@@ -212,7 +212,9 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     }
 
     /* activations: one instruction covers 256 contiguous bytes (a chunk) of each of four columns */
-    u32x4 xt[3][2];                                          /* chunks CI, CI + 1, CI + 2 are in flight: slot CI % 3 */
+    constexpr int LA = 1;                                    /* chunks requested ahead of the one being multiplied (measured:
+                                                              * 0 is 20 % slower, 2 and 3 are 3-8 % slower than 1) */
+    u32x4 xt[LA + 1][2];                                     /* chunks CI .. CI + LA are in flight: slot CI % (LA + 1) */
     const int xcol = lane >> 4;                              /* + 4 i */
     const int8_t *xp = a.xqs + (int64_t)xcol * K + (int64_t)c0 * 256 + (lane & 15) * 16;
     const int nx = batch > 4 ? 2 : 1;
@@ -234,9 +236,9 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     if (CI < SL) {                                                                                           \
         if (first_unit) {                                                                                    \
             UNROLL for (int i = 0; i < 2; ++i) {                                                             \
-                xt[(CI) % 3][i] = (u32x4)(0u);                                                                     \
+                xt[(CI) % (LA + 1)][i] = (u32x4)(0u);                                                                     \
                 if (4 * i < batch) {                                                                         \
-                    if (xcol + 4 * i < batch) xt[(CI) % 3][i] = global_read128(xp + (int64_t)(4 * i) * K + CI * 256); \
+                    if (xcol + 4 * i < batch) xt[(CI) % (LA + 1)][i] = global_read128(xp + (int64_t)(4 * i) * K + CI * 256); \
                 }                                                                                            \
             }                                                                                                \
         }                                                                                                    \
@@ -252,8 +254,9 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     if (tile < ntiles) {
         tile_base(tile, wtile, ydst, nrows);
         wsrc_lane = wtile + lane_goff;
-        PSN_MF_ISSUE(0)
-        PSN_MF_ISSUE(1)
+        if (LA > 0) { PSN_MF_ISSUE(0) }
+        if (LA > 1) { PSN_MF_ISSUE(1) }
+        if (LA > 2) { PSN_MF_ISSUE(2) }
     }
 
     /* ---- this wave's table entries: the eight sub-block sums of (column, chunk) as (low 6 bits, signed
@@ -261,7 +264,7 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     /* the last load instruction of the unit that chunk j needs */
     auto w_last = [&](int j) { return min((F::WORDS * j + F::WORDS - 1) >> 2, NI - 1); };
     {
-        const int g = min(2, SL);                            /* chunks requested so far */
+        const int g = min(LA, SL);                           /* chunks requested so far */
         wait_vmcnt(tile < ntiles ? g * nx + w_last(g - 1) + 1 : 0);
     }
     asm volatile("" : "+v"(tb0), "+v"(tb1), "+v"(tbd));
@@ -299,9 +302,9 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
 #define PSN_MF_REGROUP(CI)                                                                                   \
     UNROLL for (int i = 0; i < 2; ++i) {                                                                     \
         if (4 * i < batch) {                                                                                 \
-            asm volatile("" : "+v"(xt[(CI) % 3][i]));                                                              \
-            lds_write64(rg_wr, pack64(xt[(CI) % 3][i].x, xt[(CI) % 3][i].y));                                            \
-            lds_write64(rg_wr + 16u, pack64(xt[(CI) % 3][i].z, xt[(CI) % 3][i].w));                                      \
+            asm volatile("" : "+v"(xt[(CI) % (LA + 1)][i]));                                                              \
+            lds_write64(rg_wr, pack64(xt[(CI) % (LA + 1)][i].x, xt[(CI) % (LA + 1)][i].y));                                            \
+            lds_write64(rg_wr + 16u, pack64(xt[(CI) % (LA + 1)][i].z, xt[(CI) % (LA + 1)][i].w));                                      \
             if ((n >> 2) == i) {                                                                             \
                 UNROLL for (u32 q = 0; q < 4; ++q) {                                                         \
                     const u32x4 v = lds_read128<0>(rg_rd + (((q ^ cq_r) & 3u) << 6));                        \
@@ -333,13 +336,13 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
         float acc[4] = {0.f, 0.f, 0.f, 0.f};
         const bool live = tile < ntiles;
         if (live) {
-            /* chunk CI: request chunk CI + 2, wait until CI's own requests have landed (everything
+            /* chunk CI: request chunk CI + LA, wait until CI's own requests have landed (everything
              * requested later may stay in flight), regroup its activations (first unit), multiply */
 #define PSN_MF_CHUNK(CI)                                                                   \
             if (CI < SLMAX && CI < SL) {                                                   \
-                if (CI + 2 < SLMAX) { PSN_MF_ISSUE((CI + 2 < 8 ? CI + 2 : 7)) }           \
+                if (CI + LA < SLMAX) { PSN_MF_ISSUE((CI + LA < 8 ? CI + LA : 7)) }         \
                 {                                                                          \
-                    const int g = min(CI + 3, SL);       /* chunks requested so far */     \
+                    const int g = min(CI + LA + 1, SL);  /* chunks requested so far */     \
                     wait_vmcnt((g - CI - 1) * (first_unit ? nx : 0) + w_last(g - 1) - w_last(CI)); \
                 }                                                                          \
                 if (first_unit) { PSN_MF_REGROUP(CI) }                                     \
@@ -352,13 +355,14 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
         }
         float *const ycur = ydst;
         const int ncur = nrows;
-        /* the buffer is free: the next unit's first two chunks are requested while the partial sums are folded */
+        /* the buffer is free: the next unit's first chunks are requested while the partial sums are folded */
         tile += tiles_per_round;
         if (live && tile < ntiles) {
             tile_base(tile, wtile, ydst, nrows);
             wsrc_lane = wtile + lane_goff;
-            PSN_MF_ISSUE(0)
-            PSN_MF_ISSUE(1)
+            if (LA > 0) { PSN_MF_ISSUE(0) }
+            if (LA > 1) { PSN_MF_ISSUE(1) }
+            if (LA > 2) { PSN_MF_ISSUE(2) }
         }
         if (KS > 1) {
             UNROLL for (int i = 0; i < 4; ++i) lds_write32(red_w + (u32)i * 256u, __float_as_uint(acc[i]));
