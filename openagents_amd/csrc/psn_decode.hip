@@ -156,39 +156,52 @@ extern "C" __global__ void __launch_bounds__(256) psn_rope_kv_store(const psn_ro
 }
 
 /* Attention of one new token over cache positions 0 .. n_ctx-1, head_dim 128.  Workgroup = (kv head,
- * 64 consecutive positions), one wave per query head of the group (up to 8).  A wave first scores
- * its head: lane p takes position p (one K row of 256 bytes in registers, the query read from LDS
- * as broadcasts); then the lanes switch to two output dims each and accumulate
- * exp(score - max) * V, the weights handed from lane to lane with v_readlane.  Everything the wave
- * needs from the cache -- its K row and its two dims of all 64 V rows -- is requested up front,
- * so the kernel pays one memory round trip.  Rows past the context re-read the last valid one and
- * get weight 0.  Writes the unnormalized partial output plus (max, sum) per head and split. */
+ * 64 consecutive positions), one wave per query head of the group (up to 8).  The 64 K rows and 64 V
+ * rows of the split (256 bytes each, n_kv_heads * 256 bytes apart) are fetched four rows per
+ * instruction, 16 lanes per row, 16 bytes per lane: lane (q = lane >> 4, s = lane & 15) holds dims
+ * 8 s .. 8 s + 7 of rows 4 j + q, j = 0 .. 15 -- every load instruction reads four contiguous 256-byte
+ * rows, and all 32 of them are requested before anything is used (one memory round trip).  A row's
+ * score is the sum over its 16 lanes of an eight-dim partial dot product (the lane's eight query dims
+ * stay in registers); the softmax weights of a lane's own rows are then already in its registers, so
+ * the weighted V sum needs no lane-to-lane traffic until the four row quarters are added at the end.
+ * Rows past the context re-read the last valid one and get weight 0.  Writes the unnormalized partial
+ * output plus (max, sum) per head and split. */
+PSN_DEV float quarters_sum(float v) {                        /* over lanes l, l ^ 16, l ^ 32, l ^ 48 */
+    v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
+    return v + __shfl_xor(v, 32, 64);
+}
+PSN_DEV float quarters_max(float v) {
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F)));
+    return fmaxf(v, __shfl_xor(v, 32, 64));
+}
+PSN_DEV u32 pack_h2(float lo, float hi) {
+    const f16 a = (f16)lo, b = (f16)hi;
+    return (u32)__builtin_bit_cast(unsigned short, a) | ((u32)__builtin_bit_cast(unsigned short, b) << 16);
+}
+
 template <bool ROPE>
 PSN_DEV void attn_partial_body(const psn_attn_args &a) {
     constexpr int D = 128;
     __shared__ float qs[8][D];
     __shared__ uint4 knew_row[16];                            /* the new token's rotated key row, fp16 */
     const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int quarter = lane >> 4, sub = lane & 15;
     const int kvh = blockIdx.x % a.n_kv_heads, split = blockIdx.x / a.n_kv_heads;
     const int group = a.n_heads / a.n_kv_heads;                  /* == blockDim.x / 64 */
     const int head = kvh * group + g;
-    const int p = split * 64 + lane;
-    const bool live = p < a.n_ctx;
     const int last = a.n_ctx - 1 - split * 64;                   /* last valid position of this split, >= 0 */
-    uint4 kreg[16];
+    uint4 kreg[16], vreg[16];
     {
-        const uint4 *krow = reinterpret_cast<const uint4 *>(reinterpret_cast<const f16 *>(a.k_cache) + ((int64_t)(split * 64 + min(lane, last)) * a.n_kv_heads + kvh) * D);
-        UNROLL for (int c = 0; c < 16; ++c) kreg[c] = krow[c];
-    }
-    u32 vreg[64];
-    {
-        const u32 *vbase = reinterpret_cast<const u32 *>(reinterpret_cast<const f16 *>(a.v_cache) + ((int64_t)split * 64 * a.n_kv_heads + kvh) * D) + lane;
-        const int64_t vstride = (int64_t)a.n_kv_heads * D / 2;   /* dwords between positions */
-        UNROLL for (int i = 0; i < 64; ++i) vreg[i] = vbase[(int64_t)min(i, last) * vstride];
+        const int64_t row16 = (int64_t)a.n_kv_heads * (D / 8);   /* 16-byte words between positions */
+        const uint4 *kb = reinterpret_cast<const uint4 *>(a.k_cache) + ((int64_t)split * 64 * a.n_kv_heads + kvh) * (D / 8) + sub;
+        const uint4 *vb = reinterpret_cast<const uint4 *>(a.v_cache) + ((int64_t)split * 64 * a.n_kv_heads + kvh) * (D / 8) + sub;
+        UNROLL for (int j = 0; j < 16; ++j) kreg[j] = kb[(int64_t)min(4 * j + quarter, last) * row16];
+        UNROLL for (int j = 0; j < 16; ++j) vreg[j] = vb[(int64_t)min(4 * j + quarter, last) * row16];
     }
     if constexpr (ROPE) {
-        /* lane i rotates pair i of this wave's query head; wave 0 also leaves the coefficients in LDS
-         * for the lane that has to rotate the new key row */
+        /* lane i rotates pair i of this wave's query head; wave 0 of the split that owns the token's
+         * position also rotates the new key row, rounds it to fp16 like a cached row, leaves it in LDS and
+         * appends it to the cache */
         const float2 tc = *reinterpret_cast<const float2 *>(a.rope_table + 2 * lane);
         const float cs = tc.x, sn = tc.y;
         float r0, r1;
@@ -197,14 +210,11 @@ PSN_DEV void attn_partial_body(const psn_attn_args &a) {
         qs[g][2 * lane] = r0;
         qs[g][2 * lane + 1] = r1;
         if (g == 0 && split == ((a.n_ctx - 1) >> 6)) {
-            /* wave 0 of the split that owns the token's position rotates the new key row, one pair per
-             * lane, rounds it to fp16 like a cached row, leaves it in LDS and appends it to the cache */
             const int pos = a.n_ctx - 1;
             const float2 kv = *reinterpret_cast<const float2 *>(a.k_new + kvh * D + 2 * lane);
             float k0, k1;
             rope_pair(kv.x, kv.y, cs, sn, k0, k1);
-            const f16 h0 = (f16)k0, h1 = (f16)k1;
-            const u32 packed = (u32)__builtin_bit_cast(unsigned short, h0) | ((u32)__builtin_bit_cast(unsigned short, h1) << 16);
+            const u32 packed = pack_h2(k0, k1);
             reinterpret_cast<u32 *>(knew_row)[lane] = packed;
             reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.k_cache_w) + ((int64_t)pos * a.n_kv_heads + kvh) * D)[lane] = packed;
         }
@@ -216,46 +226,61 @@ PSN_DEV void attn_partial_body(const psn_attn_args &a) {
     if constexpr (ROPE) {
         /* the token's own position is not in the cache yet: the split that owns it takes the key row from
          * LDS (see above) and the value row from the fresh projection, rounded to fp16 like a cached row;
-         * wave 0 appends the value row to the cache */
+         * wave 0 appends the value row to the cache.  Rows behind the token's position were loaded from
+         * cache rows that nothing has written yet: they get weight 0, but 0 * (a stale Inf/NaN pattern)
+         * would still poison the sum, so they are replaced as well. */
         const int pos = a.n_ctx - 1;
         const bool own = split == (pos >> 6);                    /* uniform */
-        const float2 vn = *reinterpret_cast<const float2 *>(a.v_new + kvh * D + 2 * lane);
-        const f16 v0 = (f16)vn.x, v1 = (f16)vn.y;
-        const u32 vpacked = (u32)__builtin_bit_cast(unsigned short, v0) | ((u32)__builtin_bit_cast(unsigned short, v1) << 16);
-        /* rows behind the token's position were loaded from cache rows that nothing has written yet:
-         * they get weight 0, but 0 * (a stale Inf/NaN pattern) would still poison the sum.  The first
-         * row to replace sits in a vector register (64 = none, for the other splits), so that each row
-         * is one compare and one select with no scalar masks to hold. */
-        int pl_v = own ? (pos & 63) : 64;
+        const float4 va = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub), vb4 = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub + 4);
+        uint4 vnew;
+        vnew.x = pack_h2(va.x, va.y); vnew.y = pack_h2(va.z, va.w); vnew.z = pack_h2(vb4.x, vb4.y); vnew.w = pack_h2(vb4.z, vb4.w);
+        int pl_v = own ? (pos & 63) : 64;                        /* first row to replace (64: none) */
         asm volatile("" : "+v"(pl_v));
-        UNROLL for (int i = 0; i < 64; ++i) vreg[i] = i >= pl_v ? vpacked : vreg[i];
+        UNROLL for (int j = 0; j < 16; ++j) {
+            const bool behind = 4 * j + quarter >= pl_v;
+            vreg[j].x = behind ? vnew.x : vreg[j].x; vreg[j].y = behind ? vnew.y : vreg[j].y;
+            vreg[j].z = behind ? vnew.z : vreg[j].z; vreg[j].w = behind ? vnew.w : vreg[j].w;
+        }
         if (own) {
-            if (lane == (pos & 63)) {
-                UNROLL for (int c = 0; c < 16; ++c) kreg[c] = knew_row[c];
+            const uint4 kn = knew_row[sub];
+            UNROLL for (int j = 0; j < 16; ++j) {
+                const bool mine = 4 * j + quarter == pl_v;
+                kreg[j].x = mine ? kn.x : kreg[j].x; kreg[j].y = mine ? kn.y : kreg[j].y;
+                kreg[j].z = mine ? kn.z : kreg[j].z; kreg[j].w = mine ? kn.w : kreg[j].w;
             }
-            if (g == 0) reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos * a.n_kv_heads + kvh) * D)[lane] = vpacked;
+            if (g == 0 && quarter == 0) reinterpret_cast<uint4 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos * a.n_kv_heads + kvh) * D)[sub] = vnew;
         }
     }
-    float s = 0.f;
-    UNROLL for (int c = 0; c < 16; ++c) {
-        const u32 kw[4] = {kreg[c].x, kreg[c].y, kreg[c].z, kreg[c].w};
-        const float4 qa = *reinterpret_cast<const float4 *>(&qs[g][8 * c]), qb = *reinterpret_cast<const float4 *>(&qs[g][8 * c + 4]);
-        s += h2f_lo(kw[0]) * qa.x + h2f_hi(kw[0]) * qa.y + h2f_lo(kw[1]) * qa.z + h2f_hi(kw[1]) * qa.w;
+    const float4 qa = *reinterpret_cast<const float4 *>(&qs[g][8 * sub]), qb = *reinterpret_cast<const float4 *>(&qs[g][8 * sub + 4]);
+    float sc[16];
+    float m = -INFINITY;
+    UNROLL for (int j = 0; j < 16; ++j) {
+        const u32 kw[4] = {kreg[j].x, kreg[j].y, kreg[j].z, kreg[j].w};
+        float s = h2f_lo(kw[0]) * qa.x + h2f_hi(kw[0]) * qa.y + h2f_lo(kw[1]) * qa.z + h2f_hi(kw[1]) * qa.w;
         s += h2f_lo(kw[2]) * qb.x + h2f_hi(kw[2]) * qb.y + h2f_lo(kw[3]) * qb.z + h2f_hi(kw[3]) * qb.w;
+        s = group_sum<16>(s);
+        sc[j] = 4 * j + quarter <= last ? s * a.scale : -INFINITY;
+        m = fmaxf(m, sc[j]);
     }
-    const float sc = live ? s * a.scale : -INFINITY;
-    const float m = group_max<64>(sc);
-    const float e = live ? __expf(sc - m) : 0.f;                 /* lane i holds the weight of position i */
-    const float sum = group_sum<64>(e);
-    float o0 = 0.f, o1 = 0.f;
-    UNROLL for (int i = 0; i < 64; ++i) {
-        const float w = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), i));
-        o0 += w * h2f_lo(vreg[i]);
-        o1 += w * h2f_hi(vreg[i]);
+    m = quarters_max(m);                                         /* row 0 of the split is always live: m is finite */
+    float sum = 0.f;
+    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    UNROLL for (int j = 0; j < 16; ++j) {
+        const float w = 4 * j + quarter <= last ? __expf(sc[j] - m) : 0.f;
+        sum += w;
+        const u32 vw[4] = {vreg[j].x, vreg[j].y, vreg[j].z, vreg[j].w};
+        UNROLL for (int t = 0; t < 4; ++t) {
+            o[2 * t] += w * h2f_lo(vw[t]);
+            o[2 * t + 1] += w * h2f_hi(vw[t]);
+        }
     }
+    sum = quarters_sum(sum);
+    UNROLL for (int t = 0; t < 8; ++t) o[t] = quarters_sum(o[t]);
     float *dst = a.partial + ((int64_t)head * a.n_splits + split) * (D + 2);
-    dst[2 * lane] = o0;
-    dst[2 * lane + 1] = o1;
+    if (quarter == 0) {
+        /* (D + 2) floats per split: rows start on 8-byte, not 16-byte, boundaries */
+        UNROLL for (int t = 0; t < 4; ++t) *reinterpret_cast<float2 *>(dst + 8 * sub + 2 * t) = make_float2(o[2 * t], o[2 * t + 1]);
+    }
     if (lane == 0) { dst[D] = m; dst[D + 1] = sum; }
 }
 
