@@ -53,10 +53,13 @@ def actq_layout(act_type: int, k: int, batch: int) -> _ffi.ActqInfo:
     return info
 
 
-def prefill_plan(m: int, n: int, k: int, compute_units: int = 256):
-    """(tile_m, tile_n, ksplit, waves) the library picks for a prefill shape."""
+def prefill_plan(m: int, n: int, k: int, compute_units: int = 256, qtype: int | None = None):
+    """(tile_m, tile_n, ksplit, waves) the library picks for a prefill shape (qtype None: the Q4_0 / Q8_0 plan)."""
     tm, tn, sp, wv = C.c_int32(), C.c_int32(), C.c_int32(), C.c_int32()
-    _check(_ffi.load().psn_qmatmul_prefill_plan(m, n, k, compute_units, C.byref(tm), C.byref(tn), C.byref(sp), C.byref(wv)))
+    if qtype is None:
+        _check(_ffi.load().psn_qmatmul_prefill_plan(m, n, k, compute_units, C.byref(tm), C.byref(tn), C.byref(sp), C.byref(wv)))
+    else:
+        _check(_ffi.load().psn_qmatmul_prefill_plan_for(qtype, m, n, k, compute_units, C.byref(tm), C.byref(tn), C.byref(sp), C.byref(wv)))
     return int(tm.value), int(tn.value), int(sp.value), int(wv.value)
 
 

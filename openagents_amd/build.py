@@ -36,6 +36,8 @@ CODE_OBJECTS = [
     ("psn_pf_wide", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=2"]),
     *[(f"psn_pf_{fmt}_{fam}", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", f"-DPSN_BUILD_PF={num}", f"-DPSN_BUILD_PF_{fmt.upper()}"])
       for fmt in ("q4_0", "q8_0") for num, fam in ((1, "ws"), (4, "base"))],
+    *[(f"psn_pf_{fmt}_base", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=4", f"-DPSN_BUILD_PF_{fmt.upper()}"])
+      for fmt in ("q4_K", "q5_K", "q6_K")],
     ("psn_decode", "psn_decode.hip", []),
     ("psn_calib", "psn_calib.hip", []),
 ]

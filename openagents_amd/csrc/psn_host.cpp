@@ -1142,7 +1142,7 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
                              psn_buf *Y, int64_t M, int64_t N, int64_t K) {
     int32_t rc = check_same_ctx(mod, s, W, X, Y, what);
     if (rc) return rc;
-    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) return fail(PSN_E_UNSUPPORTED, "%s: type %d (Q4_0 and Q8_0 have kernels)", what, qtype);
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "%s: type %d (Q4_0, Q8_0, Q4_K, Q5_K and Q6_K have kernels)", what, qtype);
     if (M <= 0 || N <= 0 || M > (1 << 20) || N > (1 << 24)) return fail(PSN_E_SHAPE, "%s: M=%lld N=%lld out of range", what, (long long)M, (long long)N);
     const int64_t rb = psn_row_bytes(qtype, K);
     if (rb < 0) return (int32_t)rb;
@@ -1212,11 +1212,48 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
     return PSN_OK;
 }
 
+/* The K-quants (Q4_K, Q5_K, Q6_K) have the four-wave family only: the same estimate over its six tiles
+ * (their dequantization is fp32 arithmetic per weight, about 1.6 x the step cost of the Q4_0 kernels). */
+static void prefill_plan_base(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit) {
+    if (cus <= 0) cus = 256;
+    double best = 1e300;
+    int bi = 0, bs = 1;
+    for (int i = 0; i < 6; ++i) {
+        const int bm = k_prefill_tiles[i][0], bn = k_prefill_tiles[i][1];
+        if (bm > 64 && M <= 64) continue;
+        const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
+        const int64_t slots = (int64_t)cus * (k_prefill_wgs_per_cu[i] > 2 ? 2 : k_prefill_wgs_per_cu[i]);
+        for (int sp = 1; sp <= 8; sp *= 2) {
+            if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
+            const int64_t wgs = mt * nt * sp, rounds = (wgs + slots - 1) / slots;
+            double t = (double)rounds * ((double)(K / 64) / sp) * k_prefill_step_us[i] * 1.6 + 5.0;
+            if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;
+            if (t < best) { best = t; bi = i; bs = sp; }
+        }
+    }
+    *tile_m = k_prefill_tiles[bi][0];
+    *tile_n = k_prefill_tiles[bi][1];
+    *ksplit = bs;
+}
+
+extern "C" int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n,
+                                                int32_t *ksplit, int32_t *waves) {
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "prefill: type %d", qtype);
+    if (qtype == PSN_Q4_0 || qtype == PSN_Q8_0) return psn_qmatmul_prefill_plan(M, N, K, cus, tile_m, tile_n, ksplit, waves);
+    if (!tile_m || !tile_n || !ksplit || !waves) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan_for: null output");
+    if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill plan: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    prefill_plan_base(M, N, K, cus, tile_m, tile_n, ksplit);
+    *waves = 4;
+    return PSN_OK;
+}
+
 extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X,
                                              psn_buf *Y, int64_t M, int64_t N, int64_t K, int32_t bm, int32_t bn, int32_t ksplit,
                                              int32_t waves) {
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4)
+        return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family only (waves = 4)", fmt_name(qtype));
     /* waves == 64 selects the skinny kernel (M <= 64, 64 x 64 tiles, deep LDS rings) */
     const bool skinny = waves == 64;
     if (skinny && (bm != 64 || bn != 64 || M > 64)) return fail(PSN_E_UNSUPPORTED, "prefill: the skinny kernel serves M <= 64 with a 64x64 tile");
@@ -1277,7 +1314,8 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
     int32_t bm = 0, bn = 0, sp = 1, wv = 4;
-    if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv))) return rc;
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) prefill_plan_base(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp);
+    else if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv))) return rc;
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }
 

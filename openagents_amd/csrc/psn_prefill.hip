@@ -1,6 +1,7 @@
 /*
  * psn_prefill.hip -- gfx950 quantized prefill matmul  Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k]
- * for GGUF Q4_0 / Q8_0 weights, fp16 activations, fp32 accumulation on v_mfma_f32_32x32x16_f16.
+ * for GGUF Q4_0 / Q8_0 weights (every kernel family) and Q4_K / Q5_K / Q6_K weights (the four-wave base family),
+ * fp16 activations, fp32 accumulation on v_mfma_f32_32x32x16_f16.
  *
  * A workgroup of 256 threads owns a BM x BN tile of Y and walks K in steps of 64.  Per step
  *   - the X tile (BM x 64 fp16) goes global -> LDS with 16-byte direct-to-LDS loads;
@@ -120,6 +121,104 @@ struct PfQ8_0 {
         const half2_t d2 = bits_h2(dbits | (dbits << 16));
         const half2_t bias = bits_h2(0x64806480u);
         UNROLL for (int i = 0; i < 4; ++i) bytes_to_h4(q[i] ^ 0x80808080u, 0x64ff64ffu, bias, d2, o[2 * i], o[2 * i + 1]);
+    }
+};
+
+/* ---- K-quant weights (Q4_K, Q5_K, Q6_K): a chunk is one super-block.  The reference dequantizes in fp32
+ *      with one rounding per operation (d * sc, then * q, then - dmin * m); the fp16 weight the MFMA sees is
+ *      that fp32 value rounded once more, so the same operations are spelled out here (no fused
+ *      multiply-add) and converted with round-to-nearest-even. ---- */
+PSN_DEV u32 pack_h2_rn(float a, float b) {
+    const half2_t v = {(_Float16)a, (_Float16)b};
+    return h2_bits(v);
+}
+PSN_DEV void pf_kq_scales(u32 s0, u32 s1, u32 s2, u32 (&sc)[2], u32 (&mn)[2]) {
+    sc[0] = s0 & 0x3f3f3f3fu;
+    mn[0] = s1 & 0x3f3f3f3fu;
+    sc[1] = (s2 & 0x0f0f0f0fu) | ((s0 >> 2) & 0x30303030u);
+    mn[1] = ((s2 >> 4) & 0x0f0f0f0fu) | ((s1 >> 2) & 0x30303030u);
+}
+template <int I> PSN_DEV float pf_byte(const u32 (&v)[2]) { return (float)((v[I >> 2] >> (8 * (I & 3))) & 0xffu); }
+/* four unsigned byte values of q -> d1 * q - m1, two packed pairs */
+PSN_DEV void pf_affine4(u32 q, float d1, float m1, u32 &lo, u32 &hi) {
+    const float v0 = __fsub_rn(__fmul_rn(d1, (float)(q & 0xffu)), m1), v1 = __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xffu)), m1);
+    const float v2 = __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xffu)), m1), v3 = __fsub_rn(__fmul_rn(d1, (float)(q >> 24)), m1);
+    lo = pack_h2_rn(v0, v1);
+    hi = pack_h2_rn(v2, v3);
+}
+
+/* Q4_K: dword 0 = d | dmin << 16, dwords 1..3 = scales, dwords 4..35 = nibbles (sub-block 2g in the low,
+ * 2g+1 in the high nibbles of bytes 32g .. 32g+31) */
+struct PfQ4_K {
+    static constexpr int DW = 36, BYTES = 144;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    template <int B>
+    static PSN_DEV void deq_block(const u32 (&w)[DW], u32 (&o)[16]) {
+        u32 sc[2], mn[2];
+        pf_kq_scales(w[1], w[2], w[3], sc, mn);
+        const float d1 = __fmul_rn(h2f_lo(w[0]), pf_byte<B>(sc)), m1 = __fmul_rn(h2f_hi(w[0]), pf_byte<B>(mn));
+        UNROLL for (int i = 0; i < 8; ++i)
+            pf_affine4((w[4 + 8 * (B >> 1) + i] >> (4 * (B & 1))) & 0x0f0f0f0fu, d1, m1, o[2 * i], o[2 * i + 1]);
+    }
+};
+
+/* Q5_K: dword 0 and the scales as Q4_K, dwords 4..11 = qh (bit j of byte l: fifth bit of element l of
+ * sub-block j), dwords 12..43 = nibbles laid out as Q4_K's */
+struct PfQ5_K {
+    static constexpr int DW = 44, BYTES = 176;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const uint4 *q = reinterpret_cast<const uint4 *>(p);
+        UNROLL for (int i = 0; i < 11; ++i) unpack4(q[i], &w[4 * i]);
+    }
+    template <int B>
+    static PSN_DEV void deq_block(const u32 (&w)[DW], u32 (&o)[16]) {
+        u32 sc[2], mn[2];
+        pf_kq_scales(w[1], w[2], w[3], sc, mn);
+        const float d1 = __fmul_rn(h2f_lo(w[0]), pf_byte<B>(sc)), m1 = __fmul_rn(h2f_hi(w[0]), pf_byte<B>(mn));
+        UNROLL for (int i = 0; i < 8; ++i) {
+            const u32 nib = (w[12 + 8 * (B >> 1) + i] >> (4 * (B & 1))) & 0x0f0f0f0fu;
+            const u32 top = ((w[4 + i] >> B) & 0x01010101u) << 4;
+            pf_affine4(nib | top, d1, m1, o[2 * i], o[2 * i + 1]);
+        }
+    }
+};
+
+/* Q6_K: 210 bytes: ql[128] (dwords 0..31), qh[64] (32..47), int8 scales[16] (48..51), fp16 d (dword 52).
+ * A super-block starts on an even byte, not on a dword: the loads are declared 2-byte aligned.  Element
+ * 128 h + 32 t + l: low four bits from ql[64 h + 32 (t & 1) + l] (high nibble for t >= 2), bits 4..5 from
+ * (qh[32 h + l] >> 2 t) & 3, minus 32, times d * scales[8 h + 2 t + l / 16]. */
+struct __attribute__((packed, aligned(2))) pf_u4_a2 { u32 x, y, z, w; };
+struct __attribute__((packed, aligned(2))) pf_u16_a2 { unsigned short v; };
+struct PfQ6_K {
+    static constexpr int DW = 53, BYTES = 210;
+    static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
+        const pf_u4_a2 *q = reinterpret_cast<const pf_u4_a2 *>(p);
+        UNROLL for (int i = 0; i < 13; ++i) {
+            const pf_u4_a2 v = q[i];
+            w[4 * i] = v.x; w[4 * i + 1] = v.y; w[4 * i + 2] = v.z; w[4 * i + 3] = v.w;
+        }
+        w[52] = reinterpret_cast<const pf_u16_a2 *>(p + 208)->v;
+    }
+    template <int B>
+    static PSN_DEV void deq_block(const u32 (&w)[DW], u32 (&o)[16]) {
+        constexpr int h = B >> 2, t = B & 3;
+        const float d = h2f_lo(w[52]);
+        constexpr int si = 8 * h + 2 * t;                       /* scale of elements l < 16; l >= 16: si + 1 */
+        const float ds0 = __fmul_rn(d, (float)(int)(int8_t)((w[48 + (si >> 2)] >> (8 * (si & 3))) & 0xffu));
+        const float ds1 = __fmul_rn(d, (float)(int)(int8_t)((w[48 + ((si + 1) >> 2)] >> (8 * ((si + 1) & 3))) & 0xffu));
+        UNROLL for (int i = 0; i < 8; ++i) {
+            const u32 nib = (w[16 * h + 8 * (t & 1) + i] >> (4 * (t >> 1))) & 0x0f0f0f0fu;
+            const u32 top = ((w[32 + 8 * h + i] >> (2 * t)) & 0x03030303u) << 4;
+            const u32 q = nib | top;
+            const float ds = i < 4 ? ds0 : ds1;
+            const float v0 = __fmul_rn(ds, (float)((int)(q & 0xffu) - 32)), v1 = __fmul_rn(ds, (float)((int)((q >> 8) & 0xffu) - 32));
+            const float v2 = __fmul_rn(ds, (float)((int)((q >> 16) & 0xffu) - 32)), v3 = __fmul_rn(ds, (float)((int)(q >> 24) - 32));
+            o[2 * i] = pack_h2_rn(v0, v1);
+            o[2 * i + 1] = pack_h2_rn(v2, v3);
+        }
     }
 };
 
@@ -1059,4 +1158,14 @@ PSN_PREFILL_FAMILY_WS(q8_0, PfQ8_0)
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 4
 PSN_PREFILL_FAMILY_BASE(q8_0, PfQ8_0)
 #endif
+#endif
+/* K-quants: the four-wave family only (-DPSN_BUILD_PF=4 -DPSN_BUILD_PF_Q4_K / _Q5_K / _Q6_K) */
+#if !defined(PSN_BUILD_ONLY) || (defined(PSN_BUILD_PF_Q4_K) && PSN_BUILD_PF == 4)
+PSN_PREFILL_FAMILY_BASE(q4_K, PfQ4_K)
+#endif
+#if !defined(PSN_BUILD_ONLY) || (defined(PSN_BUILD_PF_Q5_K) && PSN_BUILD_PF == 4)
+PSN_PREFILL_FAMILY_BASE(q5_K, PfQ5_K)
+#endif
+#if !defined(PSN_BUILD_ONLY) || (defined(PSN_BUILD_PF_Q6_K) && PSN_BUILD_PF == 4)
+PSN_PREFILL_FAMILY_BASE(q6_K, PfQ6_K)
 #endif

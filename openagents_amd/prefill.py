@@ -1,4 +1,4 @@
-"""Quantized prefill matmul benchmark: Q4_0 / Q8_0 weights 4096->14336 and 14336->4096, fp16
+"""Quantized prefill matmul benchmark: Q4_0 / Q8_0 (default) or Q4_K / Q5_K / Q6_K weights 4096->14336 and 14336->4096, fp16
 activations for M = 64, 512, 2048 tokens (seeded N(0,0.02) weights quantized on the host).
 
     python -m openagents_amd.prefill [--iters 20] [--formats q4_0,q8_0] [--m 64,512,2048]
@@ -16,7 +16,7 @@ import sys
 import numpy as np
 
 from . import quantize
-from ._ffi import Q4_0, Q8_0
+from ._ffi import Q4_0, Q4_K, Q5_K, Q6_K, Q8_0
 from .backend import HipBackend, prefill_plan, row_bytes
 
 MFMA_PEAK_TFLOPS = 2500.0
@@ -31,7 +31,8 @@ def main(argv=None):
     ap.add_argument("--m", default="64,512,2048")
     ap.add_argument("--seed", type=int, default=7)
     args = ap.parse_args(argv)
-    fmts = {"q4_0": (Q4_0, quantize.quantize_q4_0), "q8_0": (Q8_0, quantize.quantize_q8_0)}
+    fmts = {"q4_0": (Q4_0, quantize.quantize_q4_0), "q8_0": (Q8_0, quantize.quantize_q8_0), "q4_K": (Q4_K, quantize.quantize_q4_K),
+            "q5_K": (Q5_K, quantize.quantize_q5_K), "q6_K": (Q6_K, quantize.quantize_q6_K)}
     be = HipBackend(0)
     rng = np.random.default_rng(args.seed)
     for fname in args.formats.split(","):
@@ -59,7 +60,7 @@ def main(argv=None):
                 tflops, gbs = flops / us / 1e6, nbytes / us / 1e3
                 bound = "mfma" if flops / nbytes >= MFMA_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "hbm"
                 frac = tflops / MFMA_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS
-                tm, tn, sp, wv = prefill_plan(m, n, k, be.compute_units)
+                tm, tn, sp, wv = prefill_plan(m, n, k, be.compute_units, qt)
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
                                   "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide"}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),

@@ -56,6 +56,47 @@ def test_every_tile_ragged_shapes(hip, orc, qname, tile):
                 assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, waves, m, n, k, err)
 
 
+@pytest.mark.parametrize("qname", ["Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("tile", TILES)
+def test_k_quant_prefill_every_tile_ragged_shapes(hip, orc, qname, tile):
+    """The K-quants run the four-wave family: weights dequantized in fp32 exactly as the reference does
+    (one rounding per operation) and rounded to fp16 for the MFMA.  Ragged m and n against every tile; k of
+    three and five super-blocks exercises the partial last round of the register chunks; Q6_K's 210-byte
+    super-blocks put every second one on an odd dword boundary."""
+    t = getattr(orc, qname)
+    for m, n, k in ((1, 70, 768), (37, 300, 1280), (200, 130, 512), (333, 516, 1024)):
+        say(f"prefill {qname} tile={tile} m={m} n={n} k={k}")
+        W = weights(orc, qname, 830, n, k)
+        X = G.seeded_acts(831 + m, m, k).astype(np.float16)
+        ref = orc.prefill(t, W, X, n, k)
+        for ksplit in (1, 2, 4):
+            if ksplit > 1 and (m * n) % 4:
+                continue
+            y = hip.matmul_host(t, W, X, n, k, tile + (ksplit, 4))
+            err = G.max_rel_err(y, ref)
+            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, m, n, k, err)
+
+
+@pytest.mark.parametrize("qname", ["Q4_K", "Q5_K", "Q6_K"])
+def test_k_quant_prefill_default_plan_and_refusals(hip, orc, qname):
+    """psn_qmatmul_prefill picks a four-wave tile by itself for the K-quants (a slice of the 4096 -> 14336
+    projection at M = 64 and M = 512); the other kernel families exist for Q4_0 / Q8_0 only."""
+    t = getattr(orc, qname)
+    n, k = 1024, 4096
+    W = weights(orc, qname, 840, n, k)
+    for m in (64, 512):
+        say(f"prefill {qname} default plan m={m} n={n} k={k}")
+        X = G.seeded_acts(841 + m, m, k).astype(np.float16)
+        err = G.max_rel_err(hip.matmul_host(t, W, X, n, k), orc.prefill(t, W, X, n, k))
+        say(f"  max_rel_err={err:.3e}")
+        assert err < PARITY_TOL
+    X = G.seeded_acts(842, 64, k).astype(np.float16)
+    for tile in ((64, 64, 1, 64), (128, 256, 1, 16), (256, 256, 1, 32)):
+        with pytest.raises(backend.PsnError) as e:
+            hip.matmul_host(t, W, X, n, k, tile)
+        assert e.value.code == _ffi.E_UNSUPPORTED
+
+
 @pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
 def test_skinny_kernel_ragged_shapes(hip, orc, qname):
     """The M <= 64 kernel (waves code 64): every combination of ragged m and n, K ranges of one to many
