@@ -247,8 +247,8 @@ int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, i
 /* Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k]; X fp16 [M][K], Y fp32 [M][N], weight tiles are
  * dequantized to fp16 (h = round to nearest even) in LDS and fed to fp16 MFMA with fp32
  * accumulation.  qtype PSN_Q4_0 or PSN_Q8_0 (every kernel family below), PSN_Q4_K, PSN_Q5_K or PSN_Q6_K
- * (family 4 only, chosen without consulting psn_qmatmul_prefill_plan; their fp32 dequantization is restated
- * operation by operation before the rounding to fp16).  Replaces the CUDA backend's quantized prefill
+ * (family 4, and for Q4_K / Q5_K family 16 on the 128x256 tile; planned by psn_qmatmul_prefill_plan_for;
+ * their fp32 dequantization is restated operation by operation before the rounding to fp16).  Replaces the CUDA backend's quantized prefill
  * matmul op. */
 int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
                             const psn_buf *X_f16, psn_buf *Y_f32, int64_t M, int64_t N, int64_t K);
@@ -268,7 +268,7 @@ int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32
 int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m, int32_t *tile_n,
                                  int32_t *ksplit, int32_t *waves);
 /* The same for a given weight type: what psn_qmatmul_prefill runs (Q4_0 / Q8_0: the plan above; the
- * K-quants: a family-4 tile). */
+ * K-quants: a family-4 tile or the 128x256 family-16 kernel). */
 int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m,
                                      int32_t *tile_n, int32_t *ksplit, int32_t *waves);
 /* ... and the same matmul with a caller-chosen shape (auto-tuners, benchmarks). */

@@ -1160,6 +1160,11 @@ static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
 /* the producer / consumer kernels (16 = four multiplying + four staging waves) and the wide kernel (32:
  * 256 x 256, four waves decoding their own operands from raw bytes):
  * {tile index, kernel family, step cost, workgroups per compute unit, K steps a workgroup spends filling its load rings} */
+/* the K-quants' four-wave kernels per tile (measured for the 128- and 256-row tiles, scaled from the Q4_0
+ * figures for the 64-row ones) and their 128 x 256 producer / consumer kernel (one round of workgroups,
+ * several rounds) */
+static const double k_kquant_step_us[] = {1.22, 1.54, 2.08, 2.08, 1.90, 2.77};
+static const double k_kquant_ws_step_us[2] = {1.75, 3.4};
 static const struct { int tile; int waves; double step_us; int per_cu; int fill; } k_prefill_alt[] = {{3, 16, 1.25, 1, 0}, {2, 16, 0.76, 1, 0}, {5, 32, 2.20, 1, 3}};
 
 extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
@@ -1212,12 +1217,15 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
     return PSN_OK;
 }
 
-/* The K-quants (Q4_K, Q5_K, Q6_K) have the four-wave family only: the same estimate over its six tiles
- * (their dequantization is fp32 arithmetic per weight, about 1.6 x the step cost of the Q4_0 kernels). */
-static void prefill_plan_base(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit) {
+/* The K-quants (Q4_K, Q5_K, Q6_K) have the four-wave family (the same estimate over its six tiles with step costs of
+ * their own: the dequantization is fp32 arithmetic per weight) and, Q4_K and
+ * Q5_K, the 128 x 256 producer / consumer kernel (its staging waves decode while the others multiply). */
+static void prefill_plan_kquant(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
+                                int32_t *waves) {
     if (cus <= 0) cus = 256;
     double best = 1e300;
     int bi = 0, bs = 1;
+    *waves = 4;
     for (int i = 0; i < 6; ++i) {
         const int bm = k_prefill_tiles[i][0], bn = k_prefill_tiles[i][1];
         if (bm > 64 && M <= 64) continue;
@@ -1226,9 +1234,15 @@ static void prefill_plan_base(int64_t M, int64_t N, int64_t K, int32_t cus, int3
         for (int sp = 1; sp <= 8; sp *= 2) {
             if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
             const int64_t wgs = mt * nt * sp, rounds = (wgs + slots - 1) / slots;
-            double t = (double)rounds * ((double)(K / 64) / sp) * k_prefill_step_us[i] * 1.6 + 5.0;
-            if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;
-            if (t < best) { best = t; bi = i; bs = sp; }
+            double t = (double)rounds * ((double)(K / 64) / sp) * k_kquant_step_us[i] + 5.0;
+            if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 / 3.0e6 + sp / 1.6e6) + 4.0   /* zero fill + atomic adds (measured 1.6 TB/s) + a launch */;
+            if (t < best) { best = t; bi = i; bs = sp; *waves = 4; }
+            if (i == 3 && qtype != PSN_Q6_K && M > 64) {
+                const int64_t r16 = (wgs + cus - 1) / cus;
+                double t16 = (double)r16 * ((double)(K / 64) / sp) * (r16 > 1 ? k_kquant_ws_step_us[1] : k_kquant_ws_step_us[0]) + 5.0;
+                if (sp > 1) t16 += (double)(M * N) * 4.0 * (1.0 / 3.0e6 + sp / 1.6e6) + 4.0   /* zero fill + atomic adds (measured 1.6 TB/s) + a launch */;
+                if (t16 < best) { best = t16; bi = i; bs = sp; *waves = 16; }
+            }
         }
     }
     *tile_m = k_prefill_tiles[bi][0];
@@ -1242,8 +1256,7 @@ extern "C" int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_
     if (qtype == PSN_Q4_0 || qtype == PSN_Q8_0) return psn_qmatmul_prefill_plan(M, N, K, cus, tile_m, tile_n, ksplit, waves);
     if (!tile_m || !tile_n || !ksplit || !waves) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan_for: null output");
     if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill plan: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-    prefill_plan_base(M, N, K, cus, tile_m, tile_n, ksplit);
-    *waves = 4;
+    prefill_plan_kquant(qtype, M, N, K, cus, tile_m, tile_n, ksplit, waves);
     return PSN_OK;
 }
 
@@ -1252,8 +1265,9 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
                                              int32_t waves) {
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
-    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4)
-        return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family only (waves = 4)", fmt_name(qtype));
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !(waves == 16 && bm == 128 && bn == 256 && qtype != PSN_Q6_K))
+        return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family%s", fmt_name(qtype),
+                    qtype == PSN_Q6_K ? " only (waves = 4)" : " and the 128x256 producer / consumer kernel (waves = 16)");
     /* waves == 64 selects the skinny kernel (M <= 64, 64 x 64 tiles, deep LDS rings) */
     const bool skinny = waves == 64;
     if (skinny && (bm != 64 || bn != 64 || M > 64)) return fail(PSN_E_UNSUPPORTED, "prefill: the skinny kernel serves M <= 64 with a 64x64 tile");
@@ -1314,7 +1328,7 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
     int32_t bm = 0, bn = 0, sp = 1, wv = 4;
-    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) prefill_plan_base(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp);
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) prefill_plan_kquant(qtype, M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv);
     else if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv))) return rc;
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }

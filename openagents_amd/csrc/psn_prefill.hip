@@ -44,6 +44,7 @@ PSN_DEV void bytes_to_h4(u32 v, u32 keep, half2_t bias, half2_t d2, u32 &lo, u32
 
 struct PfQ4_0 {
     static constexpr int DW = 36, BYTES = 144;
+    static constexpr bool KQ = false;
     static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
@@ -87,6 +88,7 @@ struct PfQ4_0 {
 
 struct PfQ8_0 {
     static constexpr int DW = 68, BYTES = 272;
+    static constexpr bool KQ = false;
     static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 17; ++i) unpack4(q[i], &w[4 * i]);
@@ -151,6 +153,7 @@ PSN_DEV void pf_affine4(u32 q, float d1, float m1, u32 &lo, u32 &hi) {
  * 2g+1 in the high nibbles of bytes 32g .. 32g+31) */
 struct PfQ4_K {
     static constexpr int DW = 36, BYTES = 144;
+    static constexpr bool KQ = true;                          /* super-block format: deq_block is all there is */
     static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 9; ++i) unpack4(q[i], &w[4 * i]);
@@ -163,12 +166,22 @@ struct PfQ4_K {
         UNROLL for (int i = 0; i < 8; ++i)
             pf_affine4((w[4 + 8 * (B >> 1) + i] >> (4 * (B & 1))) & 0x0f0f0f0fu, d1, m1, o[2 * i], o[2 * i + 1]);
     }
+    /* elements 16 H .. 16 H + 15 of block B */
+    template <int B, int H>
+    static PSN_DEV void deq_half(const u32 (&w)[DW], u32 (&o)[8]) {
+        u32 sc[2], mn[2];
+        pf_kq_scales(w[1], w[2], w[3], sc, mn);
+        const float d1 = __fmul_rn(h2f_lo(w[0]), pf_byte<B>(sc)), m1 = __fmul_rn(h2f_hi(w[0]), pf_byte<B>(mn));
+        UNROLL for (int i = 0; i < 4; ++i)
+            pf_affine4((w[4 + 8 * (B >> 1) + 4 * H + i] >> (4 * (B & 1))) & 0x0f0f0f0fu, d1, m1, o[2 * i], o[2 * i + 1]);
+    }
 };
 
 /* Q5_K: dword 0 and the scales as Q4_K, dwords 4..11 = qh (bit j of byte l: fifth bit of element l of
  * sub-block j), dwords 12..43 = nibbles laid out as Q4_K's */
 struct PfQ5_K {
     static constexpr int DW = 44, BYTES = 176;
+    static constexpr bool KQ = true;
     static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
         const uint4 *q = reinterpret_cast<const uint4 *>(p);
         UNROLL for (int i = 0; i < 11; ++i) unpack4(q[i], &w[4 * i]);
@@ -184,6 +197,17 @@ struct PfQ5_K {
             pf_affine4(nib | top, d1, m1, o[2 * i], o[2 * i + 1]);
         }
     }
+    template <int B, int H>
+    static PSN_DEV void deq_half(const u32 (&w)[DW], u32 (&o)[8]) {
+        u32 sc[2], mn[2];
+        pf_kq_scales(w[1], w[2], w[3], sc, mn);
+        const float d1 = __fmul_rn(h2f_lo(w[0]), pf_byte<B>(sc)), m1 = __fmul_rn(h2f_hi(w[0]), pf_byte<B>(mn));
+        UNROLL for (int i = 0; i < 4; ++i) {
+            const u32 nib = (w[12 + 8 * (B >> 1) + 4 * H + i] >> (4 * (B & 1))) & 0x0f0f0f0fu;
+            const u32 top = ((w[4 + 4 * H + i] >> B) & 0x01010101u) << 4;
+            pf_affine4(nib | top, d1, m1, o[2 * i], o[2 * i + 1]);
+        }
+    }
 };
 
 /* Q6_K: 210 bytes: ql[128] (dwords 0..31), qh[64] (32..47), int8 scales[16] (48..51), fp16 d (dword 52).
@@ -194,6 +218,7 @@ struct __attribute__((packed, aligned(2))) pf_u4_a2 { u32 x, y, z, w; };
 struct __attribute__((packed, aligned(2))) pf_u16_a2 { unsigned short v; };
 struct PfQ6_K {
     static constexpr int DW = 53, BYTES = 210;
+    static constexpr bool KQ = true;
     static PSN_DEV void load(const uint8_t *p, u32 (&w)[DW]) {
         const pf_u4_a2 *q = reinterpret_cast<const pf_u4_a2 *>(p);
         UNROLL for (int i = 0; i < 13; ++i) {
@@ -395,6 +420,29 @@ template <typename WF> PSN_DEV void deq16(const u32 (&q)[8], u32 dbits, int H, u
 /* the part of K step SUB (blocks 2*SUB, 2*SUB+1 of the chunk) that thread part `q` of P owns -> LDS */
 template <typename WF, int SUB, int P>
 PSN_DEV void stage_part(const u32 (&w)[WF::DW], char *tile, int row, int part) {
+    if constexpr (WF::KQ) {
+        /* K-quants: one producer thread per weight row (128 x 256 tile), both blocks of the step */
+        static_assert(P == 1, "the K-quants have the 128 x 256 producer / consumer kernel only");
+        /* (the scheduler is kept from interleaving the four halves: it would hold all 64 results at once) */
+        u32 o[8];
+        WF::template deq_half<2 * SUB, 0>(w, o);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 0)) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 1)) = make_uint4(o[4], o[5], o[6], o[7]);
+        __builtin_amdgcn_sched_barrier(0);
+        WF::template deq_half<2 * SUB, 1>(w, o);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 2)) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 3)) = make_uint4(o[4], o[5], o[6], o[7]);
+        __builtin_amdgcn_sched_barrier(0);
+        WF::template deq_half<2 * SUB + 1, 0>(w, o);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 4)) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 5)) = make_uint4(o[4], o[5], o[6], o[7]);
+        __builtin_amdgcn_sched_barrier(0);
+        WF::template deq_half<2 * SUB + 1, 1>(w, o);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 6)) = make_uint4(o[0], o[1], o[2], o[3]);
+        *reinterpret_cast<uint4 *>(tile + tile_off(row, 7)) = make_uint4(o[4], o[5], o[6], o[7]);
+        __builtin_amdgcn_sched_barrier(0);
+        return;
+    } else {
     u32 qa[8], qb[8], da, db;
     raw_block<2 * SUB>(w, qa, da);
     raw_block<2 * SUB + 1>(w, qb, db);
@@ -426,6 +474,7 @@ PSN_DEV void stage_part(const u32 (&w)[WF::DW], char *tile, int row, int part) {
             *reinterpret_cast<uint4 *>(tile + tile_off(row, 2 * part)) = make_uint4(o[0], o[1], o[2], o[3]);
             *reinterpret_cast<uint4 *>(tile + tile_off(row, 2 * part + 1)) = make_uint4(o[4], o[5], o[6], o[7]);
         }
+    }
     }
 }
 
@@ -1159,12 +1208,15 @@ PSN_PREFILL_FAMILY_WS(q8_0, PfQ8_0)
 PSN_PREFILL_FAMILY_BASE(q8_0, PfQ8_0)
 #endif
 #endif
-/* K-quants: the four-wave family only (-DPSN_BUILD_PF=4 -DPSN_BUILD_PF_Q4_K / _Q5_K / _Q6_K) */
+/* K-quants: the four-wave family, and for Q4_K / Q5_K the 128 x 256 producer / consumer kernel
+ * (-DPSN_BUILD_PF=4 -DPSN_BUILD_PF_Q4_K / _Q5_K / _Q6_K) */
 #if !defined(PSN_BUILD_ONLY) || (defined(PSN_BUILD_PF_Q4_K) && PSN_BUILD_PF == 4)
 PSN_PREFILL_FAMILY_BASE(q4_K, PfQ4_K)
+PSN_PREFILL_KERNEL_WS(q4_K, PfQ4_K, 128, 256)
 #endif
 #if !defined(PSN_BUILD_ONLY) || (defined(PSN_BUILD_PF_Q5_K) && PSN_BUILD_PF == 4)
 PSN_PREFILL_FAMILY_BASE(q5_K, PfQ5_K)
+PSN_PREFILL_KERNEL_WS(q5_K, PfQ5_K, 128, 256)
 #endif
 #if !defined(PSN_BUILD_ONLY) || (defined(PSN_BUILD_PF_Q6_K) && PSN_BUILD_PF == 4)
 PSN_PREFILL_FAMILY_BASE(q6_K, PfQ6_K)

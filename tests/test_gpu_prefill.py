@@ -69,12 +69,14 @@ def test_k_quant_prefill_every_tile_ragged_shapes(hip, orc, qname, tile):
         W = weights(orc, qname, 830, n, k)
         X = G.seeded_acts(831 + m, m, k).astype(np.float16)
         ref = orc.prefill(t, W, X, n, k)
-        for ksplit in (1, 2, 4):
-            if ksplit > 1 and (m * n) % 4:
-                continue
-            y = hip.matmul_host(t, W, X, n, k, tile + (ksplit, 4))
-            err = G.max_rel_err(y, ref)
-            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, m, n, k, err)
+        families = (4, 16) if tile == (128, 256) and qname != "Q6_K" else (4,)   # Q4_K / Q5_K: also the producer / consumer kernel
+        for waves in families:
+            for ksplit in (1, 2, 4):
+                if ksplit > 1 and (m * n) % 4:
+                    continue
+                y = hip.matmul_host(t, W, X, n, k, tile + (ksplit, waves))
+                err = G.max_rel_err(y, ref)
+                assert np.all(np.isfinite(y)) and err < PARITY_TOL, (tile, ksplit, waves, m, n, k, err)
 
 
 @pytest.mark.parametrize("qname", ["Q4_K", "Q5_K", "Q6_K"])
@@ -91,7 +93,7 @@ def test_k_quant_prefill_default_plan_and_refusals(hip, orc, qname):
         say(f"  max_rel_err={err:.3e}")
         assert err < PARITY_TOL
     X = G.seeded_acts(842, 64, k).astype(np.float16)
-    for tile in ((64, 64, 1, 64), (128, 256, 1, 16), (256, 256, 1, 32)):
+    for tile in ((64, 64, 1, 64), (128, 128, 1, 16), (256, 256, 1, 32)):
         with pytest.raises(backend.PsnError) as e:
             hip.matmul_host(t, W, X, n, k, tile)
         assert e.value.code == _ffi.E_UNSUPPORTED
