@@ -1,8 +1,9 @@
-"""GPU parity of the quantized prefill matmul (Q4_0 / Q8_0 weights, fp16 activations, fp16 MFMA with
-fp32 accumulation) against the CPU oracle, through the C ABI.
+"""GPU parity of the quantized prefill matmul (Q4_0 / Q8_0 and Q4_K / Q5_K / Q6_K weights, fp16 activations,
+fp16 MFMA with fp32 accumulation) against the CPU oracle, through the C ABI.
 
 Oracle definition: Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k] with h = round-to-nearest-even to fp16 and
-fp32 accumulation.  The kernel forms h(d*q) bit-exactly, so only the accumulation order differs.
+fp32 accumulation.  The kernels form the fp16 weight bit-exactly (h(d*q); for the K-quants the reference's
+fp32 dequantization operation by operation, then h), so only the accumulation order differs.
 Gate (north_star): max|y - ref| / max|ref| <= 1e-3; asserted: PARITY_TOL.
 """
 import sys
