@@ -15,12 +15,15 @@
  *
  * Work unit: 16 rows x SL chunks (a "slice", SL <= 8).  A workgroup of 8 (or 4) waves holds
  * waves/KS row tiles at a time, the KS waves of a tile each own one K slice of it and never change
- * slice: their columns' activations (SL x 256 int8 per column) stay in registers for the whole
- * launch.  Partial sums of the KS waves meet in LDS.
+ * slice: their columns' activations (256 int8 per chunk and column, fetched 256 contiguous bytes at a
+ * time and regrouped into MFMA operands through LDS) are read once per wave.  Partial sums of the KS
+ * waves meet in LDS.
  *
- * The weights arrive by 16-byte direct-to-LDS loads, one buffer per wave, all of a unit's loads in
- * flight before the first is used.  A load instruction fetches four consecutive 16-byte words (64
- * contiguous bytes) of each of the 16 rows; word t of row r lands at
+ * The weights arrive by 16-byte direct-to-LDS loads, one buffer per wave, requested one chunk ahead of
+ * the arithmetic (a compute unit's memory path accepts a bounded number of bytes and stalls the issuing
+ * wave, so a wave that requests its whole unit up front multiplies nothing meanwhile).  A load
+ * instruction fetches four consecutive 16-byte words (64 contiguous bytes) of each of the 16 rows; word t
+ * of row r lands at
  *     (t >> 2) * 1024 + (4 r + ((t ^ (r >> 2)) & 3)) * 16
  * so that the 16 rows of one word sit in 16 different 16-byte columns of the LDS banks (the reads
  * below are conflict-free) while the four lanes of a row still fetch one contiguous 64 bytes.
