@@ -710,7 +710,6 @@ static int32_t mfma_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32_t
     for (int i = 0; n_rows && i < count; ++i)
         if (n_rows[i] % 16) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernels need every matrix to hold a multiple of 16 rows");
     if (plan->blocks < 1 || plan->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", plan->blocks);
-    const int64_t words = (C / ks) * (qtype == PSN_Q4_K ? 9 : 11), ni = (words + 3) / 4;
     if (plan->stream != 1) return fail(PSN_E_UNSUPPORTED, "plan: stream=%d (with mfma: 1)", plan->stream);
     /* slices of more than four chunks run the kernel whose waves handle exactly one unit each */
     if (C / ks > 4 && n_rows) {
@@ -719,7 +718,8 @@ static int32_t mfma_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32_t
         if ((int64_t)plan->blocks * (waves / ks) < tiles)
             return fail(PSN_E_UNSUPPORTED, "plan: slices of %lld chunks need one wave per unit (%lld tiles, %d workgroups of %d)", (long long)(C / ks), (long long)tiles, plan->blocks, waves / ks);
     }
-    const int64_t total = C * 160 + (int64_t)waves * 1024 + (int64_t)waves * ni * 1024;
+    /* tables, 1 KB per wave, and per wave a ring of four chunks (9 or 11 KB) */
+    const int64_t total = C * 160 + (int64_t)waves * 1024 + (int64_t)waves * (qtype == PSN_Q4_K ? 9 : 11) * 1024;
     if (total > max_lds) return fail(PSN_E_UNSUPPORTED, "plan: the MFMA kernel needs %lld bytes of LDS, device offers %d", (long long)total, max_lds);
     *lds_out = total;
     return PSN_OK;
@@ -783,39 +783,45 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
         }
         g_err[0] = 0;                                   /* not streamable after all: the register kernels take it */
     }
-    /* Batch 2..8 of Q4_K / Q5_K on quantized activations: the int8-MFMA kernel, whose cost per weight
-     * does not grow with the batch.  Measured on MI355X: four-wave workgroups, two per compute unit,
-     * whose waves own slices of at most four chunks of one tile (K <= 4096); longer rows take eight
-     * waves with slices of up to eight chunks, one workgroup per compute unit.  One unit in flight per
-     * wave: deeper rings and more resident workgroups both measured slower. */
-    /* (fp32 input at batch 2 and short rows: quantizing inside a register-kernel launch still beats a
-     * quantize launch followed by this kernel -- 13.8 against 16.0 us at 14336 x 4096) */
-    const bool fused_wins = fuse_quantize && batch <= 2 && K <= 8192 && p.stage_lds == 2;
-    if (scheme == PSN_ACT_Q8 && batch >= 2 && !fused_wins && (qtype == PSN_Q4_K || qtype == PSN_Q5_K) && n_rows != nullptr) {
-        psn_matvec_plan q = p;
+    /* Batch 3..8 of Q4_K / Q5_K on quantized activations: the int8-MFMA kernel, whose cost per weight
+     * does not grow with the batch (measured on MI355X against the register kernels over nine shapes:
+     * 1.1-2.1 x faster at batch 8, 0.75-0.95 x at batch 2 -- so batch 2 stays with the register kernels,
+     * except fp32 input with rows longer than 8192, where a quantize launch + this kernel beats
+     * re-quantizing in every workgroup, 14.3 against 20.7 us at 4096 x 14336).
+     * Candidates: four waves (two workgroups per compute unit) or eight (one), any slice count that
+     * leaves whole slices of at most eight chunks and fits the LDS.  Preferred: the one that gives every
+     * compute unit a workgroup, then slices of at most four chunks (the kernel whose waves may walk
+     * several units), then four-wave workgroups.  One unit in flight per wave: deeper rings and more
+     * resident workgroups both measured slower. */
+    const bool mfma_batch = batch >= 3 || (batch == 2 && fuse_quantize && K > 8192);
+    if (scheme == PSN_ACT_Q8 && mfma_batch && (qtype == PSN_Q4_K || qtype == PSN_Q5_K) && n_rows != nullptr) {
+        psn_matvec_plan q = p, best_q = p;
         q.stage_lds = 1;
         q.lanes_per_row = 16;
         q.stream = 1;
         q.batch_tile = 8;
-        q.blocks = 1 << 20;                             /* for the checks; set below */
-        int64_t lds = 0;
-        int32_t ok = PSN_E_UNSUPPORTED;
-        for (int pass = 0; pass < 2 && ok != PSN_OK; ++pass) {
-            const int waves_per_group = pass == 0 ? 4 : 8, max_slice = pass == 0 ? 4 : 8;
-            q.threads = 64 * waves_per_group;
-            for (int ks = 1; ks <= waves_per_group && ok != PSN_OK; ks *= 2) {
-                if (C % ks || C / ks > max_slice) continue;
+        const int64_t ntiles = N / 16;
+        int64_t best_score = -1;
+        for (int threads = 256; threads <= 512; threads *= 2) {
+            for (int ks = 1; ks <= threads / 64; ks *= 2) {
+                if (C % ks || C / ks > 8) continue;
+                q.threads = threads;
                 q.mfma = ks;
-                ok = mfma_plan_check(qtype, scheme, K, batch, &q, n_rows, count, 160 * 1024, &lds);
+                const int64_t tpw = (threads / 64) / ks, cap = (threads == 256 ? 2 : 1) * (int64_t)cus;
+                int64_t b = (ntiles + tpw - 1) / tpw;
+                const bool short_slices = C / ks <= 4;
+                if (b > cap && short_slices) b = cap;       /* longer slices: one unit per wave, the grid covers every tile */
+                q.blocks = (int32_t)b;
+                int64_t lds = 0;
+                if (mfma_plan_check(qtype, scheme, K, batch, &q, n_rows, count, 160 * 1024, &lds) != PSN_OK) continue;
+                const int64_t busy = b < cus ? b : cus;     /* compute units with a workgroup */
+                const int64_t score = busy * 8 + (short_slices ? 4 : 0) + (threads == 256 ? 2 : 0) + (ks <= 4 ? 1 : 0);
+                if (score > best_score) { best_score = score; best_q = q; }
             }
         }
-        if (ok == PSN_OK) {
-            const int64_t tpw = (q.threads / 64) / q.mfma, ntiles = N / 16;
-            int64_t b = (ntiles + tpw - 1) / tpw;
-            const int64_t cap = (q.threads == 256 ? 2 : 1) * (int64_t)cus;
-            if (b > cap && C / q.mfma <= 4) b = cap;    /* longer slices: one unit per wave, the grid covers every tile */
-            q.blocks = (int32_t)b;
-            *out = q;
+        g_err[0] = 0;
+        if (best_score >= 0) {
+            *out = best_q;
             return PSN_OK;
         }
         g_err[0] = 0;                                   /* shape not served: the register kernels take it */

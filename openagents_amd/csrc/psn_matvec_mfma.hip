@@ -79,7 +79,7 @@ struct LaneOffs {
 
 template <typename F, int CI>
 PSN_DEV void mf_chunk(const LaneOffs &o, u32 xs_addr, u32 dx_addr, const u64 (&x)[8], bool first_quarter, float (&acc)[4]) {
-    constexpr int T0 = F::WORDS * CI;                       /* first word of the chunk in the slice */
+    constexpr int T0 = F::WORDS * (CI & 3);                 /* first word of the chunk in the wave's buffer, a ring of four chunks */
     const u32x4 hdr = lds_read128<(T0 >> 2) * 1024>(o.hdr[T0 & 3]);
     u64 wq[4];
     constexpr int TA = T0 + F::NIB0, TB = TA + 2, TC = TA + 4, TD = TA + 6;
@@ -157,9 +157,10 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
 
     /* LDS: sub-block sums [C][8 columns][16 B], activation scales [C][8] floats (every wave fills in and
      * reads only its own chunks), 1 KB per wave (regrouping of the activations, later the partial sums
-     * [4][64] floats), then one buffer of NI KB per wave */
+     * [4][64] floats), then one buffer per wave: a ring of four chunks (4 x WORDS words = WORDS load
+     * instructions of 1 KB; load instruction i of a unit lands in slot i % WORDS) */
     const u32 xs_tab = lds0, dx_tab = xs_tab + (u32)C * 128u, red = dx_tab + (u32)C * 32u;
-    const u32 buf_off = (u32)C * 160u + (u32)wpb * 1024u + (u32)wib * (u32)NI * 1024u;
+    const u32 buf_off = (u32)C * 160u + (u32)wpb * 1024u + (u32)wib * (u32)(F::WORDS << 10);
     const u32 buf = lds0 + buf_off;
 
     /* The matrices sharing the launch: lane i (< 4) of these registers holds matrix i's base addresses, first
@@ -226,12 +227,13 @@ PSN_DEV void mv_mfma(const psn_matvec_args &a) {
     const int64_t lane_goff = (int64_t)lrow * rb + (int64_t)c0 * (F::WORDS * 16);
     const uint8_t *wsrc_lane = nullptr;                      /* current unit's tile + lane_goff */
     auto issue_w = [&](int i0, int i1) {                     /* load instructions i0 .. i1 of the current unit */
-        lds_char *dst = lds_ptr + buf_off + (i0 << 10);
+        int slot = i0 % F::WORDS;
         int t = lword + 4 * i0;
         for (int i = i0; i <= i1; ++i) {
+            lds_char *dst = lds_ptr + buf_off + (slot << 10);
             __builtin_amdgcn_global_load_lds((const void *)(wsrc_lane + min(t, nw - 1) * 16), (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
             t += 4;
-            dst += 1024;
+            slot = slot + 1 == F::WORDS ? 0 : slot + 1;
         }
     };
     bool first_unit = true;

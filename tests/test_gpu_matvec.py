@@ -513,13 +513,16 @@ def test_mfma_kernels_every_variant(hip, orc, qname):
 
 
 def test_mfma_default_plan_and_refusals(hip, orc):
-    """psn_qmatvec picks the MFMA kernel for batch 2..8 of Q4_K / Q5_K where the shape allows and the
+    """psn_qmatvec picks the MFMA kernel for batch 3..8 of Q4_K / Q5_K where the shape allows and the
     register kernels elsewhere; plans the kernel cannot run are refused before any launch."""
     for qt, n, k in ((_ffi.Q4_K, 14336, 4096), (_ffi.Q4_K, 4096, 14336), (_ffi.Q5_K, 14336, 4096)):
-        for batch in (2, 4, 8):
+        for batch in (3, 4, 8):
             p = backend.matvec_plan(qt, _ffi.ACT_Q8, n, k, batch)
             assert p.mfma in (4, 8) and p.stage_lds == 1 and p.stream == 1, p.as_dict()
-    assert backend.matvec_plan(_ffi.Q5_K, _ffi.ACT_Q8, 4096, 14336, 4).mfma == 0         # eight 20 KB units exceed the LDS
+        assert backend.matvec_plan(qt, _ffi.ACT_Q8, n, k, 2).mfma == 0                   # batch 2: the register kernels are faster
+    assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_Q8, 4096, 14336, 2, 256, True).mfma == 8   # ... unless long rows of fp32 input would be re-quantized per workgroup
+    assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_Q8, 4096, 8192, 8).as_dict()["blocks"] == 256   # every compute unit gets a workgroup
+    assert backend.matvec_plan(_ffi.Q5_K, _ffi.ACT_Q8, 4096, 14336, 4).mfma == 8         # a wave's buffer is a ring of four chunks, whatever the slice
     assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_Q8, 1000, 4096, 4).mfma == 0          # 1000 rows: not whole tiles
     assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_Q8, 4096, 11008, 4).mfma == 0         # 43 chunks do not split
     assert backend.matvec_plan(_ffi.Q4_K, _ffi.ACT_F32, 4096, 4096, 4).mfma == 0
