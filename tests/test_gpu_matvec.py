@@ -547,6 +547,23 @@ def test_mfma_default_plan_and_refusals(hip, orc):
     assert e.value.code == _ffi.E_UNSUPPORTED
 
 
+@pytest.mark.parametrize("qname", ["Q4_K", "Q5_K"])
+def test_small_batch_default_path_odd_shapes(hip, orc, qname):
+    """psn_qmatvec (fp32 in) at batch 3..8 over shapes at the edges of what the MFMA kernels serve: one
+    tile, one chunk, slice counts of every kind, K that does not split (nine chunks: register kernels),
+    row counts that are not whole tiles (register kernels) -- whatever runs must match the oracle."""
+    t = getattr(orc, qname)
+    for n, k in ((16, 256), (48, 512), (32, 768), (4112, 1024), (80, 2304), (100, 1024), (64, 5120), (16, 14336), (272, 8192)):
+        W = weights(orc, qname, 970, n, k)
+        for batch in (3, 8):
+            p = backend.matvec_plan(t, _ffi.ACT_Q8, n, k, batch)
+            say(f"small-batch default {qname} n={n} k={k} batch={batch} mfma={p.mfma} threads={p.threads} blocks={p.blocks}")
+            x = G.seeded_acts(971 + batch, batch, k)
+            y = hip.matvec_host(t, W, x, n, k, _ffi.ACT_Q8)
+            err = G.max_rel_err(y, orc.matvec(t, _ffi.ACT_Q8, W, x, n, k))
+            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (n, k, batch, p.as_dict(), err)
+
+
 def test_streaming_plan_is_refused_where_it_cannot_run(hip, orc):
     k = 2560
     w6 = hip.upload_weight(orc.Q6_K, weights(orc, "Q6_K", 910, 80, k), 80, k)

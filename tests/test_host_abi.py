@@ -80,6 +80,29 @@ def test_matvec_plan_is_host_arithmetic(lib):
         assert e.value.code == code, args
 
 
+def test_matvec_plans_are_consistent_over_many_shapes(lib):
+    """Host arithmetic only: every plan the library returns over a grid of shapes and batches is one its own
+    kernels accept (thread counts, slice arithmetic of the MFMA kernels, enough workgroups for one-unit waves)."""
+    for qt in (_ffi.Q4_0, _ffi.Q8_0, _ffi.Q4_K, _ffi.Q5_K, _ffi.Q6_K):
+        for k in (256, 512, 768, 1024, 2048, 2304, 4096, 5120, 8192, 11008, 14336, 16384, 28672):
+            for n in (1, 16, 17, 48, 1000, 1024, 4096, 14336, 128256):
+                for batch in (1, 2, 3, 5, 8):
+                    for x_is_f32 in (False, True):
+                        p = backend.matvec_plan(qt, _ffi.ACT_Q8, n, k, batch, 256, x_is_f32)
+                        assert p.threads in (256, 512) and 1 <= p.blocks <= 1 << 20, p.as_dict()
+                        if p.mfma:
+                            c, waves = k // 256, p.threads // 64
+                            assert qt in (_ffi.Q4_K, _ffi.Q5_K) and batch >= 2 and n % 16 == 0, p.as_dict()
+                            assert p.mfma in (1, 2, 4, 8) and p.mfma <= waves and c % p.mfma == 0 and c // p.mfma <= 8, p.as_dict()
+                            assert p.stage_lds == 1 and p.stream == 1, p.as_dict()
+                            if c // p.mfma > 4:
+                                assert p.blocks * (waves // p.mfma) >= n // 16, p.as_dict()      # one wave per unit
+                            lds = c * 160 + waves * 1024 + waves * (9 if qt == _ffi.Q4_K else 11) * 1024
+                            assert lds <= 160 * 1024, p.as_dict()
+                        elif p.stream:
+                            assert batch == 1 and p.stage_lds in (1, 2) and k // 256 <= p.lanes_per_row, p.as_dict()
+
+
 def test_null_handles_are_rejected_without_a_device(lib):
     assert lib.psn_stream_sync(None) == _ffi.E_INVALID_ARG
     assert lib.psn_buf_free(None) == _ffi.E_INVALID_ARG
