@@ -84,6 +84,13 @@ int64_t psn_row_bytes(int32_t qtype, int64_t k);
  * quantize pass a loader runs when a checkpoint arrives as fp32/fp16. */
 int32_t psn_quantize_rows(int32_t qtype, const float *x, int64_t n, int64_t k, void *out, size_t out_bytes, int32_t threads);
 
+/* The inverse on the host: n rows of GGUF blocks -> fp32 out[n][k] (out_elems floats available), the
+ * published dequantize_row_* formulas in their fp32 operation order.  A loader reads a token's row of a
+ * quantized embedding table with it (the one tensor of a model file that is looked up, not multiplied);
+ * the activation formats are refused.  Replaces the per-row decode the reference's GGUF loader applies
+ * to such tensors (the formats are those /root/reference/docs/muse/muse-glimmer.md:112 names). */
+int32_t psn_dequantize_rows(int32_t qtype, const void *blocks, int64_t n, int64_t k, float *out, size_t out_elems);
+
 /* ---- context, module, stream, event, buffer  (the "module load, buffer alloc, launch and
  *      stream sync" surface; replaces the CUDA backend's context/module/stream/buffer wrappers) -- */
 

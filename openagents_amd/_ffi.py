@@ -44,6 +44,7 @@ SIGNATURES = {
     "psn_block_bytes": (_i32, [_i32]),
     "psn_row_bytes": (_i64, [_i32, _i64]),
     "psn_quantize_rows": (_i32, [_i32, _vp, _i64, _i64, _vp, _sz, _i32]),
+    "psn_dequantize_rows": (_i32, [_i32, _vp, _i64, _i64, _vp, _sz]),
     "psn_ctx_create": (_i32, [_i32, _pp]),
     "psn_ctx_destroy": (_i32, [_vp]),
     "psn_ctx_info": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_i64), C.c_char_p, _sz]),

@@ -111,6 +111,22 @@ extern "C" int32_t psn_quantize_rows(int32_t qtype, const float *x, int64_t n, i
     return PSN_OK;
 }
 
+int psn_dequantize_rows_impl(int32_t qtype, const uint8_t *in, int64_t n, int64_t k, float *out, int64_t row_bytes);
+
+extern "C" int32_t psn_dequantize_rows(int32_t qtype, const void *blocks, int64_t n, int64_t k, float *out, size_t out_elems) {
+    if (!blocks || !out) return fail(PSN_E_INVALID_ARG, "psn_dequantize_rows: null pointer");
+    if (qtype == PSN_Q8_K) return fail(PSN_E_UNSUPPORTED, "psn_dequantize_rows: Q8_K is an activation format");
+    const int64_t rb = psn_row_bytes(qtype, k);
+    if (rb < 0) return (int32_t)rb;
+    if (n <= 0) return fail(PSN_E_SHAPE, "psn_dequantize_rows: n=%lld", (long long)n);
+    if ((uint64_t)n * (uint64_t)k > out_elems)
+        return fail(PSN_E_INVALID_ARG, "psn_dequantize_rows: output holds %zu floats, %lld rows of %lld need %lld", out_elems, (long long)n,
+                    (long long)k, (long long)(n * k));
+    if (psn_dequantize_rows_impl(qtype, static_cast<const uint8_t *>(blocks), n, k, out, rb) != 0)
+        return fail(PSN_E_UNSUPPORTED, "psn_dequantize_rows: type %d has no dequantizer", qtype);
+    return PSN_OK;
+}
+
 static bool is_weight_type(int32_t t) { return t == PSN_Q4_0 || t == PSN_Q8_0 || t == PSN_Q4_K || t == PSN_Q5_K || t == PSN_Q6_K; }
 static const char *fmt_name(int32_t t) {
     switch (t) {

@@ -1,4 +1,5 @@
-/* Host-side GGUF weight quantizer of the library: fp32 rows -> Q4_0 / Q8_0 / Q4_K / Q5_K / Q6_K blocks.
+/* Host-side GGUF weight quantizer of the library: fp32 rows -> Q4_0 / Q8_0 / Q4_K / Q5_K / Q6_K blocks,
+ * and the dequantizer back to fp32 (a token's embedding row, a check of what a file holds).
  *
  * This is the import step of the path (fp32 or fp16 checkpoints become the quantized tensors that
  * psn_weight_upload takes), restating the published ggml reference quantizers so that a tensor
@@ -306,6 +307,75 @@ void row_q6_K(const float *x, uint8_t *out, int64_t k) {
     }
 }
 
+/* ---- the inverse direction: blocks -> fp32, the published dequantize_row_* formulas in their fp32
+ *      operation order (value = (d * sub-block scale) * level - (dmin * sub-block min)) ---------- */
+inline float half_at(const uint8_t *p) {
+    uint16_t u;
+    std::memcpy(&u, p, 2);
+    return from_half_bits(u);
+}
+
+void deq_q4_0(const uint8_t *in, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / 32; ++b, in += 18, y += 32) {
+        const float d = half_at(in);
+        for (int j = 0; j < 16; ++j) {
+            y[j] = (float)((in[2 + j] & 15) - 8) * d;
+            y[j + 16] = (float)((in[2 + j] >> 4) - 8) * d;
+        }
+    }
+}
+
+void deq_q8_0(const uint8_t *in, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / 32; ++b, in += 34, y += 32) {
+        const float d = half_at(in);
+        for (int j = 0; j < 32; ++j) y[j] = (float)(int8_t)in[2 + j] * d;
+    }
+}
+
+/* Q4_K (HIGH false: levels at 16) and Q5_K (fifth bits at 16, low nibbles at 48) */
+template <bool HIGH>
+void deq_q45_K(const uint8_t *in, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / 256; ++b, in += HIGH ? 176 : 144, y += 256) {
+        const float d = half_at(in), dmin = half_at(in + 2);
+        const uint8_t *qh = in + 16, *qs = in + (HIGH ? 48 : 16);
+        for (int c = 0; c < 4; ++c) {
+            int s1, m1, s2, m2;
+            unpack6(in + 4, 2 * c, s1, m1);
+            unpack6(in + 4, 2 * c + 1, s2, m2);
+            const float d1 = d * (float)s1, n1 = dmin * (float)m1, d2 = d * (float)s2, n2 = dmin * (float)m2;
+            for (int l = 0; l < 32; ++l) {
+                int a = qs[32 * c + l] & 15, e = qs[32 * c + l] >> 4;
+                if (HIGH) {
+                    a += ((qh[l] >> (2 * c)) & 1) << 4;
+                    e += ((qh[l] >> (2 * c + 1)) & 1) << 4;
+                }
+                y[64 * c + l] = d1 * (float)a - n1;
+                y[64 * c + 32 + l] = d2 * (float)e - n2;
+            }
+        }
+    }
+}
+
+void deq_q6_K(const uint8_t *in, float *y, int64_t k) {
+    for (int64_t b = 0; b < k / 256; ++b, in += 210, y += 256) {
+        const uint8_t *ql = in, *qh = in + 128;
+        const int8_t *sc = reinterpret_cast<const int8_t *>(in + 192);
+        const float d = half_at(in + 208);
+        for (int h = 0; h < 2; ++h)
+            for (int l = 0; l < 32; ++l) {
+                const int g = 8 * h + l / 16, hb = qh[32 * h + l];
+                const int q1 = ((ql[64 * h + l] & 15) | ((hb & 3) << 4)) - 32;
+                const int q2 = ((ql[64 * h + 32 + l] & 15) | (((hb >> 2) & 3) << 4)) - 32;
+                const int q3 = ((ql[64 * h + l] >> 4) | (((hb >> 4) & 3) << 4)) - 32;
+                const int q4 = ((ql[64 * h + 32 + l] >> 4) | (((hb >> 6) & 3) << 4)) - 32;
+                y[128 * h + l] = d * (float)sc[g] * (float)q1;
+                y[128 * h + 32 + l] = d * (float)sc[g + 2] * (float)q2;
+                y[128 * h + 64 + l] = d * (float)sc[g + 4] * (float)q3;
+                y[128 * h + 96 + l] = d * (float)sc[g + 6] * (float)q4;
+            }
+    }
+}
+
 using row_fn = void (*)(const float *, uint8_t *, int64_t);
 
 row_fn row_quantizer(int32_t qtype) {
@@ -338,5 +408,21 @@ int psn_quantize_rows_impl(int32_t qtype, const float *x, int64_t n, int64_t k, 
             for (int64_t r = n * t / nt; r < n * (t + 1) / nt; ++r) fn(x + r * k, out + r * row_bytes, k);
         });
     for (auto &th : pool) th.join();
+    return 0;
+}
+
+/* rows [n][row_bytes] blocks -> [n][k] fp32; returns 0, or -1 when the type has no dequantizer.
+ * The caller (psn_dequantize_rows in psn_host.cpp) has checked the shape and the buffer size. */
+int psn_dequantize_rows_impl(int32_t qtype, const uint8_t *in, int64_t n, int64_t k, float *out, int64_t row_bytes) {
+    void (*fn)(const uint8_t *, float *, int64_t) = nullptr;
+    switch (qtype) {
+        case PSN_Q4_0: fn = deq_q4_0; break;
+        case PSN_Q8_0: fn = deq_q8_0; break;
+        case PSN_Q4_K: fn = deq_q45_K<false>; break;
+        case PSN_Q5_K: fn = deq_q45_K<true>; break;
+        case PSN_Q6_K: fn = deq_q6_K; break;
+        default: return -1;
+    }
+    for (int64_t r = 0; r < n; ++r) fn(in + r * row_bytes, out + r * k, k);
     return 0;
 }

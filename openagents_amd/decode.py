@@ -10,6 +10,11 @@ SwiGLU -> down; then the final norm and the LM head.  Every op is a call into th
 runs the Llama-3-8B-shaped synthetic step (Q4_K projections, Q6_K LM head, random-init weights from
 the host quantizers, KV cache pre-filled with fp16 N(0,1)) and prints one JSON record with tokens/s
 and the matvec share of the step time.
+
+`load_gguf_model(backend, path)` builds the same step from a model file: the llama-family metadata keys
+and tensor names of the GGUF convention, any mix of the five weight formats per tensor (a file whose
+attn_v / ffn_down switch format between layers, as the K-quant mixes do, simply gets one launch per
+format where matrices share an input).
 """
 from __future__ import annotations
 
@@ -22,6 +27,7 @@ from dataclasses import dataclass, field
 import numpy as np
 
 from ._ffi import ACT_Q8, Q4_K, Q6_K
+from . import gguf as _gguf
 from .backend import DeviceBuffer, HipBackend, QuantizedTensor, act_type_for, actq_layout, row_bytes
 
 
@@ -62,6 +68,17 @@ class ModelWeights:
     lm_head: QuantizedTensor
 
 
+def _by_format(ws, ys):
+    """Matrices sharing an input, split into the groups one launch can take (same format and K), in
+    first-seen order: [([weights], [outputs]), ...]."""
+    groups = {}
+    for w, y in zip(ws, ys):
+        g = groups.setdefault((w.qtype, w.k), ([], []))
+        g[0].append(w)
+        g[1].append(y)
+    return list(groups.values())
+
+
 class DecodeStep:
     """Owns the activations, KV caches and scratch of one sequence and enqueues one token step."""
 
@@ -97,38 +114,55 @@ class DecodeStep:
         self.k_cache = [be.alloc(cache_bytes) for _ in range(s.n_layers)]
         self.v_cache = [be.alloc(cache_bytes) for _ in range(s.n_layers)]
         be.reserve(max(s.hidden, s.ffn), 1)
+        self.qkv_launches = [len(_by_format([lw.wq, lw.wk, lw.wv], [0, 1, 2])) for lw in weights.layers]
+        self.gate_up_launches = [len(_by_format([lw.w_gate, lw.w_up], [0, 1])) for lw in weights.layers]
         if self.fused:
-            l0 = weights.layers[0]
-            kinds = {act_type_for(t.qtype) for t in (l0.wq, l0.wo, l0.w_gate, l0.w_down, weights.lm_head)}
-            if len(kinds) != 1:
-                raise ValueError("fused quantization needs one activation type for all projections")
-            self.act_type = kinds.pop()
-            self.xq_h = be.alloc(int(actq_layout(self.act_type, s.hidden, 1).bytes))
-            self.xq_attn = be.alloc(int(actq_layout(self.act_type, s.hidden, 1).bytes))
-            self.xq_f = be.alloc(int(actq_layout(self.act_type, s.ffn, 1).bytes))
+            # the producers of wo's and w_down's inputs write the activation blocks those matrices read, so the
+            # activation type may change from layer to layer; matrices fed by a norm launch of their own
+            # (fused_norm off) share its one quantized copy and must agree on the type
+            kinds = {act_type_for(t.qtype) for lw in weights.layers for t in (lw.wq, lw.wk, lw.wv, lw.wo, lw.w_gate, lw.w_up, lw.w_down)}
+            kinds.add(act_type_for(weights.lm_head.qtype))
+            if not self.fused_norm and len(kinds) != 1:
+                raise ValueError("with the norm as its own launch, fused quantization needs one activation type for all projections")
+            self.act_type = act_type_for(weights.layers[0].wo.qtype)
+            self.xq_h = be.alloc(max(int(actq_layout(a, s.hidden, 1).bytes) for a in kinds))
+            self.xq_attn = be.alloc(max(int(actq_layout(a, s.hidden, 1).bytes) for a in kinds))
+            self.xq_f = be.alloc(max(int(actq_layout(a, s.ffn, 1).bytes) for a in kinds))
             self.rope_tab = be.alloc(s.head_dim * 4)
 
     @property
     def launches_per_layer(self) -> int:
+        """Launches of a layer whose q|k|v and gate|up each share one format."""
         return 7 if self.fused_norm else 9 if self.fused else 10
 
     @property
     def launches_outside_layers(self) -> int:
         return 2 if self.fused_norm else 3 if self.fused else 2
 
+    @property
+    def launches_per_token(self) -> int:
+        """Every launch of one step, counting one extra per additional format among q|k|v and gate|up."""
+        extra = sum(n - 1 for n in self.qkv_launches) + sum(n - 1 for n in self.gate_up_launches)
+        return len(self.w.layers) * self.launches_per_layer + self.launches_outside_layers + extra
+
+    def _norm_multi(self, ws, x, delta, norm, h_out, ys):
+        """ys = ws . q(rmsnorm(x + delta) * norm): one launch per weight format, each redoing the add and the norm
+        from the same x and delta (h_out, written by the first, is a different buffer)."""
+        for gi, (gw, gy) in enumerate(_by_format(ws, ys)):
+            self.be.quantized_matvec_norm_multi(gw, x, delta, norm, h_out if gi == 0 else None, gy, self.shape.eps)
+
     def _enqueue_norm_fused(self, pos: int):
         """Seven launches per layer: q|k|v (with add + norm), attention partial, combine, o, gate|up (with
         add + norm), SwiGLU, down.  The residual stream moves self.x -> self.x2 -> self.x within a layer."""
-        be, s, at = self.be, self.shape, self.act_type
+        be, s = self.be, self.shape
         be.rope_table(self.rope_tab, s.head_dim, pos, s.rope_theta)
         for li, lw in enumerate(self.w.layers):
-            be.quantized_matvec_norm_multi([lw.wq, lw.wk, lw.wv], self.x, self.down if li > 0 else None, lw.attn_norm, self.x2,
-                                           [self.q, self.k, self.v], s.eps)
-            be.attention_decode_rope(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn, at,
-                                     s.n_heads, s.n_kv_heads, s.head_dim, pos, self.rope_tab)
+            self._norm_multi([lw.wq, lw.wk, lw.wv], self.x, self.down if li > 0 else None, lw.attn_norm, self.x2, [self.q, self.k, self.v])
+            be.attention_decode_rope(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn,
+                                     act_type_for(lw.wo.qtype), s.n_heads, s.n_kv_heads, s.head_dim, pos, self.rope_tab)
             be.quantized_matvec_q8(lw.wo, self.xq_attn, self.o, 1)
-            be.quantized_matvec_norm_multi([lw.w_gate, lw.w_up], self.x2, self.o, lw.ffn_norm, self.x, [self.gate, self.up], s.eps)
-            be.swiglu_q8(self.gate, self.up, None, self.xq_f, at, s.ffn)
+            self._norm_multi([lw.w_gate, lw.w_up], self.x2, self.o, lw.ffn_norm, self.x, [self.gate, self.up])
+            be.swiglu_q8(self.gate, self.up, None, self.xq_f, act_type_for(lw.w_down.qtype), s.ffn)
             be.quantized_matvec_q8(lw.w_down, self.xq_f, self.down, 1)
         be.quantized_matvec_norm_multi([self.w.lm_head], self.x, self.down, self.w.final_norm, None, [self.logits], s.eps)
 
@@ -142,14 +176,16 @@ class DecodeStep:
         for li, lw in enumerate(self.w.layers):
             if glue:
                 be.add_rmsnorm_q8(self.x, self.down if li > 0 else None, lw.attn_norm, None, self.xq_h, at, s.hidden, s.eps)
-            be.quantized_matvec_q8_multi([lw.wq, lw.wk, lw.wv], self.xq_h, [self.q, self.k, self.v], 1)
+            for gw, gy in _by_format([lw.wq, lw.wk, lw.wv], [self.q, self.k, self.v]):
+                be.quantized_matvec_q8_multi(gw, self.xq_h, gy, 1)
             if glue:
                 be.attention_decode_rope(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn, at,
                                          s.n_heads, s.n_kv_heads, s.head_dim, pos, self.rope_tab)
             be.quantized_matvec_q8(lw.wo, self.xq_attn, self.o, 1)
             if glue:
                 be.add_rmsnorm_q8(self.x, self.o, lw.ffn_norm, None, self.xq_h, at, s.hidden, s.eps)
-            be.quantized_matvec_q8_multi([lw.w_gate, lw.w_up], self.xq_h, [self.gate, self.up], 1)
+            for gw, gy in _by_format([lw.w_gate, lw.w_up], [self.gate, self.up]):
+                be.quantized_matvec_q8_multi(gw, self.xq_h, gy, 1)
             if glue:
                 be.swiglu_q8(self.gate, self.up, None, self.xq_f, at, s.ffn)
             be.quantized_matvec_q8(lw.w_down, self.xq_f, self.down, 1)
@@ -167,14 +203,16 @@ class DecodeStep:
         for li, lw in enumerate(self.w.layers):
             if glue:
                 be.add_rmsnorm(self.x, self.down if li > 0 else None, lw.attn_norm, self.xn, s.hidden, s.eps)
-            be.quantized_matvec_multi([lw.wq, lw.wk, lw.wv], self.xn, [self.q, self.k, self.v], 1, sch)
+            for gw, gy in _by_format([lw.wq, lw.wk, lw.wv], [self.q, self.k, self.v]):
+                be.quantized_matvec_multi(gw, self.xn, gy, 1, sch)
             if glue:
                 be.rope_kv_store(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], s.n_heads, s.n_kv_heads, s.head_dim, pos, s.rope_theta)
                 be.attention_decode(self.q, self.k_cache[li], self.v_cache[li], self.attn_ws, self.attn, s.n_heads, s.n_kv_heads, s.head_dim, pos + 1)
             be.quantized_matvec(lw.wo, self.attn, self.o, 1, sch)
             if glue:
                 be.add_rmsnorm(self.x, self.o, lw.ffn_norm, self.xn, s.hidden, s.eps)
-            be.quantized_matvec_multi([lw.w_gate, lw.w_up], self.xn, [self.gate, self.up], 1, sch)
+            for gw, gy in _by_format([lw.w_gate, lw.w_up], [self.gate, self.up]):
+                be.quantized_matvec_multi(gw, self.xn, gy, 1, sch)
             if glue:
                 be.swiglu(self.gate, self.up, self.act, s.ffn)
             be.quantized_matvec(lw.w_down, self.act, self.down, 1, sch)
@@ -235,6 +273,141 @@ def synthetic_weights(be: HipBackend, shape: LlamaShape, seed: int = 0, unique_l
     return ModelWeights(layers, be.upload(np.ones(s.hidden, np.float32)), be.upload_weight(Q6_K, head_full, s.vocab, s.hidden))
 
 
+class TokenEmbedding:
+    """The embedding table of a model file, left on the host in the file's mapping: one row is
+    dequantized per token (psn_dequantize_rows), which is all a decode step reads of it."""
+
+    def __init__(self, gf: "_gguf.GGUFFile", name: str = "token_embd.weight"):
+        t = gf.tensors[name]
+        self.info, self.bytes = t, gf.data(name)
+        self.hidden, self.vocab = t.k, t.n
+        self.row_nbytes = t.nbytes // t.n
+
+    def row(self, token: int) -> np.ndarray:
+        if not 0 <= token < self.vocab:
+            raise IndexError(f"token {token} outside the vocabulary of {self.vocab}")
+        raw = self.bytes[token * self.row_nbytes:(token + 1) * self.row_nbytes]
+        if self.info.ggml_type == 0:
+            return np.array(raw.view(np.float32))
+        if self.info.ggml_type == 1:
+            return raw.view(np.float16).astype(np.float32)
+        from . import quantize
+        return quantize.dequantize(self.info.ggml_type, raw, self.hidden)[0]
+
+
+@dataclass
+class GGUFModel:
+    shape: LlamaShape
+    weights: ModelWeights
+    embedding: TokenEmbedding
+    file: "_gguf.GGUFFile"
+
+
+_LAYER_TENSORS = {"wq": "attn_q", "wk": "attn_k", "wv": "attn_v", "wo": "attn_output", "w_gate": "ffn_gate", "w_up": "ffn_up", "w_down": "ffn_down"}
+
+
+def load_gguf_model(be: HipBackend, path: str) -> GGUFModel:
+    """Read a llama-architecture GGUF file into device weights.
+
+    Metadata: general.architecture = "llama", llama.{block_count, embedding_length, feed_forward_length,
+    attention.head_count, attention.head_count_kv (default head_count), attention.key_length (default
+    embedding_length / head_count), attention.layer_norm_rms_epsilon (default 1e-5), rope.freq_base
+    (default 10000)}.  Tensors: token_embd, output_norm, output (absent = tied to token_embd),
+    blk.N.{attn_norm, attn_q, attn_k, attn_v, attn_output, ffn_norm, ffn_gate, ffn_up, ffn_down}.weight;
+    projections in any of Q4_0 / Q8_0 / Q4_K / Q5_K / Q6_K, norms in F32 or F16.  What this step does not
+    compute is refused rather than ignored: another architecture, projection biases, rotary scaling."""
+    gf = _gguf.GGUFFile(path)
+    md = gf.metadata
+    arch = md.get("general.architecture")
+    if arch != "llama":
+        raise _gguf.GGUFError(f"general.architecture = {arch!r}: only the llama layer structure is implemented")
+
+    def need(key):
+        if f"llama.{key}" not in md:
+            raise _gguf.GGUFError(f"metadata key llama.{key} is missing")
+        return md[f"llama.{key}"]
+
+    hidden, n_heads = int(need("embedding_length")), int(need("attention.head_count"))
+    n_kv = md.get("llama.attention.head_count_kv", n_heads)
+    if isinstance(n_kv, list):
+        if len(set(n_kv)) != 1:
+            raise _gguf.GGUFError("per-layer head_count_kv values differ")
+        n_kv = n_kv[0]
+    if n_heads <= 0 or hidden % n_heads:
+        raise _gguf.GGUFError(f"embedding_length {hidden} is not a multiple of head_count {n_heads}")
+    head_dim = int(md.get("llama.attention.key_length", hidden // n_heads))
+    scaling = md.get("llama.rope.scaling.type", "none")
+    if scaling not in ("none", "") or "rope_freqs.weight" in gf.tensors:
+        raise _gguf.GGUFError("rotary frequency scaling (rope.scaling / rope_freqs) is not implemented")
+    if int(md.get("llama.rope.dimension_count", head_dim)) != head_dim:
+        raise _gguf.GGUFError("partial rotary embedding (rope.dimension_count < head size) is not implemented")
+    if "token_embd.weight" not in gf.tensors:
+        raise _gguf.GGUFError("tensor token_embd.weight is missing")
+    emb = TokenEmbedding(gf)
+    head_name = "output.weight" if "output.weight" in gf.tensors else "token_embd.weight"
+    shape = LlamaShape(hidden=hidden, n_heads=n_heads, n_kv_heads=int(n_kv), head_dim=head_dim, ffn=int(need("feed_forward_length")),
+                       vocab=gf.tensors[head_name].n, n_layers=int(need("block_count")),
+                       rope_theta=float(md.get("llama.rope.freq_base", 10000.0)), eps=float(md.get("llama.attention.layer_norm_rms_epsilon", 1e-5)))
+    if n_heads * head_dim != hidden or shape.n_kv_heads <= 0 or n_heads % shape.n_kv_heads:
+        raise _gguf.GGUFError(f"head layout {n_heads} x {head_dim} (kv {shape.n_kv_heads}) does not match embedding_length {hidden}")
+    if emb.hidden != hidden:
+        raise _gguf.GGUFError(f"token_embd rows hold {emb.hidden} values, embedding_length is {hidden}")
+
+    def matrix(name, n, k):
+        if name not in gf.tensors:
+            raise _gguf.GGUFError(f"tensor {name} is missing")
+        t = gf.tensors[name]
+        if (t.n, t.k) != (n, k):
+            raise _gguf.GGUFError(f"tensor {name} is [{t.n}, {t.k}], the metadata implies [{n}, {k}]")
+        return gf.upload(be, name)
+
+    def vector(name, n):
+        if name not in gf.tensors:
+            raise _gguf.GGUFError(f"tensor {name} is missing")
+        t = gf.tensors[name]
+        if t.ggml_type not in (0, 1) or (t.n, t.k) != (1, n):
+            raise _gguf.GGUFError(f"tensor {name}: want {n} F32 or F16 values")
+        raw = gf.data(name)
+        return be.upload(np.array(raw.view(np.float32)) if t.ggml_type == 0 else raw.view(np.float16).astype(np.float32))
+
+    dims = {"wq": (hidden, hidden), "wk": (shape.kv_dim, hidden), "wv": (shape.kv_dim, hidden), "wo": (hidden, hidden),
+            "w_gate": (shape.ffn, hidden), "w_up": (shape.ffn, hidden), "w_down": (hidden, shape.ffn)}
+    layers = []
+    for li in range(shape.n_layers):
+        for bias in ("attn_q", "attn_k", "attn_v", "attn_output"):
+            if f"blk.{li}.{bias}.bias" in gf.tensors:
+                raise _gguf.GGUFError(f"blk.{li}.{bias}.bias: projection biases are not implemented")
+        t = {field_: matrix(f"blk.{li}.{stem}.weight", *dims[field_]) for field_, stem in _LAYER_TENSORS.items()}
+        layers.append(LayerWeights(**t, attn_norm=vector(f"blk.{li}.attn_norm.weight", hidden), ffn_norm=vector(f"blk.{li}.ffn_norm.weight", hidden)))
+    weights = ModelWeights(layers, vector("output_norm.weight", hidden), matrix(head_name, shape.vocab, hidden))
+    return GGUFModel(shape, weights, emb, gf)
+
+
+def greedy_tokens(model: GGUFModel, step: "DecodeStep", prompt, n_new: int):
+    """Feed `prompt` (token ids) one position at a time from an empty cache, then extend it by n_new
+    arg-max tokens.  Returns (all tokens, the logits that chose the last one; with n_new = 0 the logits after
+    the prompt).  A plain host loop: embedding row to the device, one step's launches, logits back."""
+    tokens = [int(t) for t in prompt]
+    if not tokens:
+        raise ValueError("need at least one prompt token")
+    if len(tokens) + n_new > step.max_ctx:
+        raise ValueError(f"{len(tokens)} prompt + {n_new} new tokens exceed the context of {step.max_ctx}")
+    pos = 0
+    while True:
+        step.x.upload(model.embedding.row(tokens[pos]))
+        step.enqueue(pos)
+        if pos == len(tokens) - 1:                     # the newest token: its logits choose the next one
+            logits = step.logits.download(np.float32, (model.shape.vocab,))
+            if n_new == 0:
+                break
+            tokens.append(int(np.argmax(logits)))
+            n_new -= 1
+            if n_new == 0:
+                break
+        pos += 1
+    return tokens, logits
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--layers", type=int, default=32)
@@ -288,7 +461,7 @@ def main(argv=None):
            "config": {"layers": shape.n_layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,
                       "ffn": shape.ffn, "vocab": shape.vocab, "context": args.ctx, "weights": "Q4_K projections, Q6_K LM head",
                       "activation_scheme": "Q8 (Q8_K blocks, " + ("written by the producing kernel)" if step.fused else "quantized inside the matvec launch)"),
-                      "launches_per_token": shape.n_layers * step.launches_per_layer + step.launches_outside_layers, "graph_replay": True},
+                      "launches_per_token": step.launches_per_token, "graph_replay": True},
            "data": "synthetic random-init weights (one unique layer copied to every layer's own allocation), fp16 N(0,1) KV cache",
            "logits_finite": bool(np.all(np.isfinite(logits))), "steps": args.steps, "setup_s": round(setup_s, 1),
            "not_measured": ["sampling", "tokenizer", "host loop"]}

@@ -60,3 +60,20 @@ def quantize_q5_K(x: np.ndarray, threads: int | None = None) -> np.ndarray:
 
 def quantize_q6_K(x: np.ndarray, threads: int | None = None) -> np.ndarray:
     return quantize(Q6_K, x, threads)
+
+
+def dequantize(qtype: int, blocks: np.ndarray, k: int) -> np.ndarray:
+    """uint8 [n, psn_row_bytes(qtype, k)] (or one flat row) -> fp32 [n, k], the reference's dequantize_row_* values."""
+    lib = _ffi.load()
+    rb = lib.psn_row_bytes(qtype, k)
+    if rb < 0:
+        raise ValueError(lib.psn_last_error().decode(errors="replace"))
+    b = np.ascontiguousarray(blocks, dtype=np.uint8).reshape(-1)
+    if b.size == 0 or b.size % rb:
+        raise ValueError(f"{b.size} bytes is not a whole number of {rb}-byte rows")
+    n = b.size // rb
+    out = np.empty((n, k), dtype=np.float32)
+    rc = lib.psn_dequantize_rows(qtype, C.c_void_p(b.ctypes.data), n, k, C.c_void_p(out.ctypes.data), out.size)
+    if rc < 0:
+        raise ValueError(lib.psn_last_error().decode(errors="replace"))
+    return out

@@ -252,7 +252,7 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
     t_full, t_mv = st_full["median_us"], st_mv["median_us"]
     digest = graph_digest(f"decode-step:l{layers}:ctx{ctx}:h{shape.hidden}:ffn{shape.ffn}:v{shape.vocab}",
                           *[protos[name] for name in sorted(protos)])
-    launches = shape.n_layers * step.launches_per_layer + step.launches_outside_layers
+    launches = step.launches_per_token
     rec = record(be, "decode.step.q4_K.b1", f"psn decode-step graph ({launches} launches: psn_mvs_q4_K_q8_g*_xn_s*, psn_mvs_q4_K_q8_g*_lds_s1, "
                  "psn_mvs_q6_K_q8_g16_xn_s1, psn_attn_partial_rope, psn_attn_combine, psn_swiglu, psn_rope_table)",
                  digest, 1e6 / t_full, shape={"layers": layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,

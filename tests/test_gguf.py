@@ -109,3 +109,89 @@ def test_tensors_from_a_file_reach_the_kernels_unchanged(hip, orc, tmp_path):
         assert G.max_rel_err(y.download(np.float32, (1, n)), orc.matvec(t, orc.ACT_Q8, blocks, x, n, k)) < 2e-5
     with pytest.raises(gguf.GGUFError):
         f.upload(hip, "output_norm.weight")
+
+
+class RecordingBackend:
+    """Stands in for the device in host-only tests of the loader: remembers what would be uploaded."""
+
+    def __init__(self):
+        self.weights, self.vectors = [], []
+
+    def upload_weight(self, qtype, blocks, n, k):
+        self.weights.append((qtype, n, k, np.array(blocks)))
+        return self.weights[-1]
+
+    def upload(self, arr):
+        self.vectors.append(np.array(arr))
+        return self.vectors[-1]
+
+
+DIMS = dict(hidden=256, n_heads=2, n_kv_heads=1, ffn=512, vocab=96, rope_theta=500000.0, eps=1e-5)
+
+
+def test_model_loader_reads_the_llama_convention(orc, tmp_path):
+    from decoderef import write_llama_file
+    from openagents_amd.decode import load_gguf_model
+    path = tmp_path / "m.gguf"
+    host = write_llama_file(orc, path, DIMS, [{"attn_v": "Q6_K"}, {"ffn_down": "Q8_0"}], embd_format="Q5_K", seed=5, norm_types=[0, 1])
+    be = RecordingBackend()
+    model = load_gguf_model(be, str(path))
+    s = model.shape
+    assert (s.hidden, s.n_heads, s.n_kv_heads, s.head_dim, s.kv_dim, s.ffn, s.vocab, s.n_layers) == (256, 2, 1, 128, 128, 512, 96, 2)
+    assert s.rope_theta == 500000.0
+    l0, l1 = model.weights.layers
+    assert (l0.wv[0], l0.wv[1], l0.wv[2]) == (orc.Q6_K, 128, 256) and np.array_equal(l0.wv[3].reshape(-1), host["layers"][0]["attn_v"][1].reshape(-1))
+    assert (l1.w_down[0], l1.w_down[1], l1.w_down[2]) == (orc.Q8_0, 256, 512)
+    assert np.array_equal(l1.attn_norm, host["layers"][1]["attn_norm"])          # stored as F16, widened on load
+    assert np.array_equal(model.weights.final_norm, host["final_norm"])
+    assert model.weights.lm_head[0] == orc.Q6_K and model.weights.lm_head[1] == 96
+    # the embedding table stays on the host: a row is dequantized per token, bit-equal to the oracle's values
+    table = orc.dequantize(orc.Q5_K, host["embd"][1], 256)
+    for tok in (0, 41, 95):
+        assert np.array_equal(model.embedding.row(tok).view(np.uint32), table[tok].view(np.uint32))
+    with pytest.raises(IndexError):
+        model.embedding.row(96)
+    assert not any(w[1] == 96 and w[0] == orc.Q5_K for w in be.weights)           # ... and was not uploaded as a matrix
+
+
+def test_model_loader_refuses_what_the_step_does_not_compute(orc, tmp_path):
+    from decoderef import write_llama_file
+    from openagents_amd.decode import load_gguf_model
+    be = RecordingBackend()
+
+    def refused(match, **kw):
+        path = tmp_path / "bad.gguf"
+        write_llama_file(orc, path, kw.pop("dims", DIMS), kw.pop("formats", [{}]), **kw)
+        with pytest.raises(gguf.GGUFError, match=match):
+            load_gguf_model(be, str(path))
+
+    refused("architecture", extra_metadata={"general.architecture": (gguf.STRING, "qwen2")})
+    refused("embedding_length is missing", extra_metadata={"llama.embedding_length": None})
+    refused("rotary frequency scaling", extra_metadata={"llama.rope.scaling.type": (gguf.STRING, "linear")})
+    refused("rotary frequency scaling", extra_tensors=[("rope_freqs.weight", (64,), 0, np.ones(64, np.float32).view(np.uint8))])
+    refused("partial rotary", extra_metadata={"llama.rope.dimension_count": (gguf.U32, 64)})
+    refused("biases", extra_tensors=[("blk.0.attn_q.bias", (256,), 0, np.zeros(256, np.float32).view(np.uint8))])
+    refused("blk.0.ffn_up.weight is missing", omit=("blk.0.ffn_up.weight",))
+    refused("token_embd.weight is missing", omit=("token_embd.weight",))
+    refused("metadata implies", extra_metadata={"llama.feed_forward_length": (gguf.U32, 768)})
+    refused("not a multiple", extra_metadata={"llama.attention.head_count": (gguf.U32, 3)})
+    refused("head layout", extra_metadata={"llama.attention.head_count_kv": (gguf.U32, 0)})
+    # per-layer kv-head arrays are accepted when they agree, refused when they differ
+    path = tmp_path / "ok.gguf"
+    write_llama_file(orc, path, DIMS, [{}, {}], extra_metadata={"llama.attention.head_count_kv": (gguf.ARRAY, (gguf.U32, [1, 1]))})
+    assert load_gguf_model(be, str(path)).shape.n_kv_heads == 1
+    refused("head_count_kv values differ", formats=[{}, {}], extra_metadata={"llama.attention.head_count_kv": (gguf.ARRAY, (gguf.U32, [1, 2]))})
+    # a norm stored in a quantized format is not a vector this loader takes
+    q = orc.quantize(orc.Q8_0, np.ones((1, 256), np.float32))
+    refused("F32 or F16", omit=("output_norm.weight",), extra_tensors=[("output_norm.weight", (256,), 8, q)])
+
+
+def test_tied_head_uses_the_embedding_table(orc, tmp_path):
+    from decoderef import write_llama_file
+    from openagents_amd.decode import load_gguf_model
+    path = tmp_path / "tied.gguf"
+    host = write_llama_file(orc, path, DIMS, [{}], embd_format="Q8_0", head_format=None)
+    be = RecordingBackend()
+    model = load_gguf_model(be, str(path))
+    assert model.weights.lm_head[0] == orc.Q8_0 and model.weights.lm_head[1:3] == (96, 256)
+    assert np.array_equal(model.weights.lm_head[3].reshape(-1), host["embd"][1].reshape(-1))

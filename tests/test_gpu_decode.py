@@ -13,6 +13,7 @@ import numpy as np
 import pytest
 
 import ggufref as G
+from decoderef import attention_ref, ref_step, rmsnorm_ref, rope_ref, write_llama_file
 from openagents_amd import _ffi, backend
 from openagents_amd.decode import DecodeStep, LayerWeights, LlamaShape, ModelWeights
 
@@ -22,35 +23,6 @@ pytestmark = pytest.mark.gpu
 def say(msg):
     print(msg, flush=True)
     sys.stdout.flush()
-
-
-def rmsnorm_ref(x, w, eps):
-    x = x.astype(np.float64)
-    return (x / np.sqrt(np.mean(x * x) + eps) * w).astype(np.float32)
-
-
-def rope_ref(vec, n_heads, head_dim, pos, theta):
-    v = vec.astype(np.float64).reshape(n_heads, head_dim // 2, 2)
-    i = np.arange(head_dim // 2)
-    ang = pos * theta ** (-2.0 * i / head_dim)
-    c, s = np.cos(ang), np.sin(ang)
-    out = np.empty_like(v)
-    out[:, :, 0] = v[:, :, 0] * c - v[:, :, 1] * s
-    out[:, :, 1] = v[:, :, 0] * s + v[:, :, 1] * c
-    return out.reshape(-1).astype(np.float32)
-
-
-def attention_ref(q, kc, vc, n_heads, n_kv, d, n_ctx):
-    q = q.astype(np.float64).reshape(n_heads, d)
-    k = kc[:n_ctx].astype(np.float64).reshape(n_ctx, n_kv, d)
-    v = vc[:n_ctx].astype(np.float64).reshape(n_ctx, n_kv, d)
-    out = np.empty((n_heads, d))
-    for h in range(n_heads):
-        g = h // (n_heads // n_kv)
-        s = k[:, g, :] @ q[h] / np.sqrt(d)
-        p = np.exp(s - s.max())
-        out[h] = (p / p.sum()) @ v[:, g, :]
-    return out.reshape(-1).astype(np.float32)
 
 
 def test_add_rmsnorm(hip):
@@ -314,6 +286,81 @@ def test_whole_small_decode_step_eager_and_graph(hip, orc):
             hip.sync()
     finally:
         hip.destroy_graph(graph)
+
+
+def test_model_file_with_mixed_formats_decodes_like_the_reference(hip, orc, tmp_path):
+    """A llama-architecture GGUF file whose tensors mix all five weight formats (v and down switching
+    format between layers, gate and up even disagreeing on the activation type; norms in F32 and F16)
+    -> load_gguf_model -> a few greedy tokens from an empty cache, against the numpy + oracle step."""
+    from openagents_amd.decode import greedy_tokens, load_gguf_model
+    dims = dict(hidden=512, n_heads=4, n_kv_heads=2, ffn=1024, vocab=768, rope_theta=10000.0, eps=1e-6)
+    formats = [{"attn_v": "Q6_K", "ffn_down": "Q6_K"},
+               {"attn_q": "Q5_K", "attn_k": "Q5_K", "attn_v": "Q5_K", "attn_output": "Q8_0", "ffn_up": "Q4_0", "ffn_down": "Q4_0"},
+               {"attn_q": "Q8_0", "attn_k": "Q4_0", "attn_v": "Q8_0", "attn_output": "Q6_K", "ffn_gate": "Q5_K", "ffn_up": "Q5_K", "ffn_down": "Q5_K"}]
+    path = tmp_path / "mixed.gguf"
+    host = write_llama_file(orc, path, dims, formats, embd_format="Q4_K", head_format="Q6_K", seed=77, norm_types=[0, 1, 0])
+    model = load_gguf_model(hip, str(path))
+    s = model.shape
+    assert (s.hidden, s.n_heads, s.n_kv_heads, s.head_dim, s.ffn, s.vocab, s.n_layers) == (512, 4, 2, 128, 1024, 768, 3)
+    assert s.rope_theta == 10000.0 and abs(s.eps - 1e-6) < 1e-12
+    assert [t.qtype for t in (model.weights.layers[1].wq, model.weights.layers[1].wo, model.weights.layers[1].w_up)] == [orc.Q5_K, orc.Q8_0, orc.Q4_0]
+    ctx = 8
+    step = DecodeStep(hip, s, model.weights, ctx)
+    assert step.fused_norm
+    assert step.qkv_launches == [2, 1, 2] and step.gate_up_launches == [1, 2, 1]
+    assert step.launches_per_token == 3 * 7 + 2 + 3
+    with pytest.raises(ValueError):
+        DecodeStep(hip, s, model.weights, ctx, fused_norm=False)       # one quantized copy cannot serve Q8_0 and Q8_K readers
+
+    prompt, n_new = [5, 700, 31], 2
+    tokens, logits = greedy_tokens(model, step, prompt, n_new)
+    kc = [np.zeros((ctx, s.kv_dim), np.float16) for _ in range(s.n_layers)]
+    vc = [np.zeros((ctx, s.kv_dim), np.float16) for _ in range(s.n_layers)]
+    embd = orc.dequantize(orc.Q4_K, host["embd"][1], s.hidden)
+    ref_tokens = list(prompt)
+    for pos in range(len(prompt) + n_new - 1):
+        assert np.array_equal(model.embedding.row(ref_tokens[pos]), embd[ref_tokens[pos]])
+        ref_logits = ref_step(orc, dims, host, embd[ref_tokens[pos]], kc, vc, pos)
+        if pos >= len(prompt) - 1:
+            ref_tokens.append(int(np.argmax(ref_logits)))
+    err = G.max_rel_err(logits, ref_logits)
+    say(f"mixed-format model file: tokens {tokens} (reference {ref_tokens}), last logits max_rel_err={err:.3e}")
+    assert tokens == ref_tokens
+    assert err < 1e-3
+    # the caches the steps filled are the reference's rows (fp16 roundings of values that agree to ~1e-5)
+    last = len(tokens) - 2
+    for li in range(s.n_layers):
+        got = step.k_cache[li].download(np.float16, (ctx, s.kv_dim))[:last + 1].astype(np.float32)
+        assert np.max(np.abs(got - kc[li][:last + 1].astype(np.float32))) < 2e-2 * max(1.0, float(np.max(np.abs(kc[li].astype(np.float32)))))
+
+    # the unfused path (every matvec quantizes its own fp32 input) takes the same file
+    plain = DecodeStep(hip, s, model.weights, ctx, fused_quant=False)
+    t2, l2 = greedy_tokens(model, plain, prompt, n_new)
+    assert t2 == tokens and G.max_rel_err(l2, logits) < 1e-3
+
+    # one captured graph of the last position replays to the eager logits
+    pos = len(tokens) - 2
+    step.x.upload(model.embedding.row(tokens[pos]))
+    graph = step.capture(pos)
+    try:
+        for _ in range(2):
+            step.x.upload(model.embedding.row(tokens[pos]))
+            hip.launch_graph(graph)
+            assert np.array_equal(step.logits.download(np.float32, (s.vocab,)), logits)
+            hip.sync()
+    finally:
+        hip.destroy_graph(graph)
+
+    # a tied LM head (no output.weight): the embedding table is also the last matrix
+    tied_path = tmp_path / "tied.gguf"
+    tied_host = write_llama_file(orc, tied_path, dims, [{}], embd_format="Q8_0", head_format=None, seed=78)
+    tied = load_gguf_model(hip, str(tied_path))
+    assert tied.weights.lm_head.qtype == orc.Q8_0 and tied.shape.vocab == 768
+    st = DecodeStep(hip, tied.shape, tied.weights, 4)
+    _, lg = greedy_tokens(tied, st, [9], 0)
+    e8 = orc.dequantize(orc.Q8_0, tied_host["embd"][1], 512)
+    ref = ref_step(orc, dims, tied_host, e8[9], [np.zeros((4, 256), np.float16)], [np.zeros((4, 256), np.float16)], 0)
+    assert G.max_rel_err(lg, ref) < 1e-3
 
 
 def test_llama3_8b_shaped_step_properties(hip):

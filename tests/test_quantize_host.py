@@ -62,3 +62,44 @@ def test_native_quantizer_argument_errors():
     assert lib.psn_error_name(lib.psn_quantize_rows(_ffi.Q4_K, None, 2, 256, C.c_void_p(out.ctypes.data), out.nbytes, 1)) == b"PSN_E_INVALID_ARG"
     with pytest.raises(ValueError):
         quantize.quantize(_ffi.Q4_0, np.zeros((2, 48), np.float32))
+
+
+@pytest.mark.parametrize("name", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
+def test_native_dequantizer_matches_oracle_and_the_element_layout(orc, name):
+    """The library's host dequantizer against the oracle's (itself pinned by independent bit-level packers),
+    bit for bit: on quantizer output and on random BYTES (every bit pattern of scales, levels and high
+    bits, not only what a quantizer emits)."""
+    qt, ot = getattr(_ffi, name), getattr(orc, name)
+    for k in (256, 2048):
+        blocks = orc.quantize(ot, special_rows(k))
+        got = quantize.dequantize(qt, blocks, k)
+        assert got.shape == (24, k)
+        assert np.array_equal(got.view(np.uint32), orc.dequantize(ot, blocks, k).view(np.uint32)), (name, k)
+    rng = np.random.default_rng(703)
+    k = 512
+    rb = int(_ffi.load().psn_row_bytes(qt, k))
+    raw = rng.integers(0, 256, (5, rb), dtype=np.uint8)
+    bb = int(_ffi.load().psn_block_bytes(qt))
+    half_at = {"Q4_0": (0,), "Q8_0": (0,), "Q4_K": (0, 2), "Q5_K": (0, 2), "Q6_K": (208,)}[name]
+    for off in half_at:                                   # keep the fp16 scales finite
+        raw.reshape(5, -1, bb)[:, :, off + 1] &= 0x3b
+    got = quantize.dequantize(qt, raw, k)
+    assert np.array_equal(got.view(np.uint32), orc.dequantize(ot, raw, k).view(np.uint32))
+    one = quantize.dequantize(qt, raw[3], k)              # a flat single row, as an embedding lookup passes it
+    assert one.shape == (1, k) and np.array_equal(one[0], got[3])
+
+
+def test_native_dequantizer_argument_errors():
+    lib = _ffi.load()
+    blocks = np.zeros(2 * 144, np.uint8)
+    out = np.zeros(2 * 256, np.float32)
+    call = lambda qt, n, k, elems: lib.psn_dequantize_rows(qt, C.c_void_p(blocks.ctypes.data), n, k, C.c_void_p(out.ctypes.data), elems)
+    assert call(_ffi.Q4_K, 2, 256, out.size) == 0
+    assert lib.psn_error_name(call(_ffi.Q4_K, 2, 256, out.size - 1)) == b"PSN_E_INVALID_ARG"
+    assert lib.psn_error_name(call(_ffi.Q4_K, 2, 250, out.size)) == b"PSN_E_SHAPE"
+    assert lib.psn_error_name(call(_ffi.Q4_K, 0, 256, out.size)) == b"PSN_E_SHAPE"
+    assert lib.psn_error_name(call(_ffi.Q8_K, 2, 256, out.size)) == b"PSN_E_UNSUPPORTED"
+    assert lib.psn_error_name(call(7, 2, 256, out.size)) == b"PSN_E_UNSUPPORTED"
+    assert lib.psn_error_name(lib.psn_dequantize_rows(_ffi.Q4_K, None, 2, 256, C.c_void_p(out.ctypes.data), out.size)) == b"PSN_E_INVALID_ARG"
+    with pytest.raises(ValueError):
+        quantize.dequantize(_ffi.Q4_K, np.zeros(100, np.uint8), 256)
