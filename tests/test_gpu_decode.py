@@ -74,6 +74,37 @@ def test_attention_decode(hip, nh, nkv):
         assert G.max_rel_err(got, attention_ref(q, kc, vc, nh, nkv, d, n_ctx)) < 2e-5
 
 
+def test_attention_over_changing_shapes_on_one_stream(hip):
+    """Head layouts beyond the parametrized ones (odd groups, one kv head per query head, a single
+    position), interleaved on one stream and each run twice: against the fp64 restatement, and the
+    quantized output against psn_act_quantize of the fp32 one."""
+    rng = np.random.default_rng(903)
+    d = 128
+    shapes = [(6, 2, 200), (32, 8, 2048), (6, 2, 64), (8, 2, 1), (12, 4, 777), (32, 8, 130), (2, 1, 65), (16, 16, 300), (32, 8, 2048)]
+    for rep, (nh, nkv, n_ctx) in enumerate(shapes * 2):
+        say(f"attention paths heads={nh}/{nkv} ctx={n_ctx} rep={rep}")
+        q = rng.standard_normal(nh * d, dtype=np.float32)
+        kc = rng.standard_normal((n_ctx, nkv * d), dtype=np.float32).astype(np.float16)
+        vc = rng.standard_normal((n_ctx, nkv * d), dtype=np.float32).astype(np.float16)
+        ws = hip.alloc(nh * ((n_ctx + 63) // 64) * 130 * 4)
+        ref = attention_ref(q, kc, vc, nh, nkv, d, n_ctx)
+        qb, kb, vb = hip.upload(q), hip.upload(kc), hip.upload(vc)
+        plain = hip.alloc(nh * d * 4)
+        hip.attention_decode(qb, kb, vb, ws, plain, nh, nkv, d, n_ctx)
+        got = plain.download(np.float32, (nh * d,))
+        assert G.max_rel_err(got, ref) < 2e-5
+        for at in (_ffi.Q8_K, _ffi.Q8_0):
+            out, outq = hip.alloc(nh * d * 4), hip.alloc(int(backend.actq_layout(at, nh * d, 1).bytes))
+            hip.attention_decode_q8(qb, kb, vb, ws, out, outq, at, nh, nkv, d, n_ctx)
+            assert np.array_equal(out.download(np.float32, (nh * d,)), got)
+            want = hip.quantize_activations(out, nh * d, 1, at)
+            n = nh * d
+            li = backend.actq_layout(at, n, 1)
+            a, b = outq.download(np.uint8, (int(li.bytes),)), want.download(np.uint8, (int(li.bytes),))
+            for off, ln in ((0, n), (int(li.off_d), n // (32 if at == _ffi.Q8_0 else 256) * 4), (int(li.off_s), n // 32 * 4 if at == _ffi.Q8_0 else n // 16 * 2)):
+                assert np.array_equal(a[off:off + ln], b[off:off + ln])
+
+
 @pytest.mark.parametrize("pos", [0, 63, 64, 149, 2047])
 def test_rope_fused_into_attention_matches_separate_launches(hip, pos):
     """Two launches (attention that rotates and appends itself, combine) against three (rotary + append,
