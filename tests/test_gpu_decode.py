@@ -394,6 +394,19 @@ def test_model_file_with_mixed_formats_decodes_like_the_reference(hip, orc, tmp_
     assert G.max_rel_err(lg, ref) < 1e-3
 
 
+def test_decode_cli_generates_from_a_model_file(orc, tmp_path, capsys):
+    import json
+    from openagents_amd import decode
+    dims = dict(hidden=256, n_heads=2, n_kv_heads=1, ffn=512, vocab=320, rope_theta=10000.0, eps=1e-5)
+    path = tmp_path / "cli.gguf"
+    write_llama_file(orc, path, dims, [{"attn_v": "Q6_K"}, {}], embd_format="Q8_0", head_format=None, seed=91)
+    assert decode.main(["--gguf", str(path), "--prompt", "5,300", "--new", "3", "--ctx", "16"]) == 0
+    rec = json.loads(capsys.readouterr().out.strip().splitlines()[-1])
+    assert rec["prompt_tokens"] == 2 and rec["new_tokens"] == 3 and len(rec["tokens"]) == 5 and rec["tokens"][:2] == [5, 300]
+    assert all(0 <= t < 320 for t in rec["tokens"]) and rec["logits_finite"]
+    assert rec["formats"] == ["Q4_K", "Q6_K", "Q8_0"] and rec["config"]["layers"] == 2
+
+
 def test_llama3_8b_shaped_step_properties(hip):
     """Config 5 at its real shape (32 layers, hidden 4096, 32/8 heads, FFN 14336, context 2048, Q4_K
     projections, Q6_K 128256-row LM head).  No CPU restatement at this size; instead: the captured graph
