@@ -17,6 +17,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 N, K, BATCH, M = 8, 512, 2, 4
+NB = 32                                   # rows of the batch-8 fixtures
 FORMATS = {"q4_0": 2, "q8_0": 8, "q4_K": 12, "q6_K": 14, "q5_K": 13}      # appended in this order: a format's seed is its position
 
 
@@ -40,9 +41,17 @@ def build():
         out[f"{name}_deq"] = oracle.dequantize(t, blocks, K)
         out[f"{name}_y_q8"] = oracle.matvec(t, oracle.ACT_Q8, blocks, x, N, K, nthreads=1)
         out[f"{name}_y_f32"] = oracle.matvec(t, oracle.ACT_F32, blocks, x, N, K, nthreads=1)
-        if name in ("q4_0", "q8_0"):
-            out[f"{name}_xh"] = xh
-            out[f"{name}_y_prefill"] = oracle.prefill(t, blocks, xh, N, K, nthreads=1)
+        out[f"{name}_xh"] = xh
+        out[f"{name}_y_prefill"] = oracle.prefill(t, blocks, xh, N, K, nthreads=1)
+    # 32 rows x 8 activation columns: the shape class the small-batch (batch 2..8) kernels of Q4_K / Q5_K serve
+    for i, name in enumerate(("q4_K", "q5_K")):
+        rng = np.random.default_rng(7200 + i)
+        w = rng.standard_normal((NB, K), dtype=np.float32) * np.float32(0.02)
+        x = rng.standard_normal((8, K), dtype=np.float32)
+        blocks = oracle.quantize(FORMATS[name], w, nthreads=1)
+        out[f"batch8_{name}_blocks"] = blocks
+        out[f"batch8_{name}_x"] = x
+        out[f"batch8_{name}_y_q8"] = oracle.matvec(FORMATS[name], oracle.ACT_Q8, blocks, x, NB, K, nthreads=1)
     _, x, _ = inputs(7100)
     out["act_x"] = x
     out["act_q8_0"] = oracle.quantize(oracle.Q8_0, x, nthreads=1)

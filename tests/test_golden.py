@@ -34,6 +34,13 @@ def test_oracle_reproduces_golden_blocks_and_outputs(orc, gold, name):
         assert G.max_rel_err(orc.prefill(t, blocks, gold[f"{name}_xh"], N, K), gold[f"{name}_y_prefill"]) < 2e-6
 
 
+@pytest.mark.parametrize("name", ["q4_K", "q5_K"])
+def test_oracle_reproduces_golden_batch8_outputs(orc, gold, name):
+    t = FORMATS[name]
+    blocks, x = gold[f"batch8_{name}_blocks"], gold[f"batch8_{name}_x"]
+    assert np.array_equal(orc.matvec(t, orc.ACT_Q8, blocks, x, 32, K, nthreads=1), gold[f"batch8_{name}_y_q8"])
+
+
 def test_oracle_reproduces_golden_activation_blocks(orc, gold):
     assert np.array_equal(orc.quantize(orc.Q8_0, gold["act_x"]), gold["act_q8_0"])
     assert np.array_equal(orc.quantize(orc.Q8_K, gold["act_x"]), gold["act_q8_K"])
@@ -67,6 +74,19 @@ def test_gpu_matches_golden(hip, gold, name):
     if f"{name}_xh" in gold:
         y = hip.matmul_host(t, blocks, gold[f"{name}_xh"], N, K)
         assert G.max_rel_err(y, gold[f"{name}_y_prefill"]) < 2e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["q4_K", "q5_K"])
+def test_gpu_small_batch_kernels_match_golden(hip, gold, name):
+    """Batch 8 and batch 4 of a 32-row matrix: the default plan puts these on the int8-MFMA kernels."""
+    from openagents_amd import _ffi, backend
+    t = FORMATS[name]
+    blocks, x, want = gold[f"batch8_{name}_blocks"], gold[f"batch8_{name}_x"], gold[f"batch8_{name}_y_q8"]
+    assert backend.matvec_plan(t, _ffi.ACT_Q8, 32, K, 8, hip.compute_units, True).mfma > 0
+    for b in (8, 4):
+        y = hip.matvec_host(t, blocks, x[:b], 32, K, _ffi.ACT_Q8)
+        assert G.max_rel_err(y, want[:b]) < 2e-5
 
 
 @pytest.mark.gpu
