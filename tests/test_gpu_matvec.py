@@ -697,3 +697,29 @@ def test_norm_fused_projection_argument_errors(hip, orc):
     with pytest.raises(backend.PsnError) as e:
         hip.quantized_matvec_norm_multi([w], hip.alloc(k * 2), None, wn, None, [y])
     assert e.value.name == "PSN_E_INVALID_ARG"
+
+
+def test_default_plans_over_seeded_random_shapes(hip, orc):
+    """Whatever the planner picks for shapes nobody tuned for (odd row counts, one to 56 chunks per row,
+    every batch, both schemes, fp32 and pre-quantized input) must match the oracle."""
+    rng = np.random.default_rng(5150)
+    ks = [256, 512, 768, 1024, 1536, 2048, 2816, 4096, 5120, 8192, 11008, 14336]
+    for case in range(48):
+        qname = FORMATS[case % 5]
+        qt = getattr(orc, qname)
+        k = int(ks[int(rng.integers(len(ks)))])
+        n = int(rng.integers(1, 700)) if rng.random() < 0.5 else int(rng.integers(1, 40)) * 16
+        batch = int(rng.integers(1, 9))
+        scheme = _ffi.ACT_F32 if case % 7 == 3 else _ffi.ACT_Q8
+        say(f"random default plan #{case}: {qname} n={n} k={k} batch={batch} scheme={scheme}")
+        b = orc.quantize(qt, G.seeded_weights(5200 + case, n, k))
+        x = G.seeded_acts(5300 + case, batch, k)
+        ref = orc.matvec(qt, scheme, b, x, n, k)
+        got = hip.matvec_host(qt, b, x, n, k, scheme)
+        assert G.max_rel_err(got, ref) < (2e-5 if scheme == _ffi.ACT_Q8 else 1e-4), (qname, n, k, batch, scheme)
+        if scheme == _ffi.ACT_Q8:
+            w = hip.upload_weight(qt, b, n, k)
+            xq = hip.quantize_activations(hip.upload(x), k, batch, backend.act_type_for(qt))
+            y = hip.alloc(batch * n * 4)
+            hip.quantized_matvec_q8(w, xq, y, batch)
+            assert G.max_rel_err(y.download(np.float32, (batch, n)), ref) < 2e-5, (qname, n, k, batch, "q8 in")

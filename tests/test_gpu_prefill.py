@@ -231,3 +231,20 @@ def test_prefill_errors(hip, orc):
     assert e.value.code == _ffi.E_UNSUPPORTED
     hip.quantized_matmul(w, x, y, 4)
     hip.sync()
+
+
+def test_prefill_default_plans_over_seeded_random_shapes(hip, orc):
+    """The planner's own choice of family, tile and K split for shapes nobody tuned for, all five formats."""
+    rng = np.random.default_rng(6150)
+    for case in range(30):
+        qname = ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"][case % 5]
+        qt = getattr(orc, qname)
+        k = int(rng.choice([256, 512, 1024, 1536, 2048, 4096]))
+        n = int(rng.integers(1, 900))
+        m = int(rng.choice([1, 3, 17, 64, 65, 100, 128, 257, 300, 520]))
+        say(f"random prefill #{case}: {qname} m={m} n={n} k={k} plan={backend.prefill_plan(m, n, k, hip.compute_units, qt)}")
+        b = orc.quantize(qt, G.seeded_weights(6200 + case, n, k))
+        x = G.seeded_acts(6300 + case, m, k).astype(np.float16)
+        ref = orc.prefill(qt, b, x, n, k)
+        got = hip.matmul_host(qt, b, x, n, k)
+        assert G.max_rel_err(got, ref) < 2e-5, (qname, m, n, k)
