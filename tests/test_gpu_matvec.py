@@ -116,7 +116,7 @@ def test_every_kernel_variant_small(hip, orc, qname, scheme, batch):
         assert np.all(np.isfinite(y)) and err < PARITY_TOL, (p.as_dict(), err)
 
 
-# ------------------------------------------------------------------ matvec: BASELINE shapes, default plan
+# ------------------------------------------------------------------ matvec: the benchmark shapes, default plan
 
 SHAPES = [(4096, 4096), (1024, 4096), (14336, 4096), (4096, 14336)]
 
