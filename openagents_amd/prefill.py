@@ -6,12 +6,21 @@ activations for M = 64, 512, 2048 tokens (seeded N(0,0.02) weights quantized on 
 Prints one JSON record per (format, shape, M): microseconds, TFLOP/s, GB/s and the fraction of the
 roofline that binds (fp16 MFMA 2.5 PFLOP/s, or HBM 8 TB/s when the arithmetic intensity is below
 the ridge of 312.5 FLOP/B).  Weight copies rotate so that the HBM-bound cases stream from memory.
+
+With --sample-clock S every cell is additionally run back to back for S seconds while a thread reads the
+shader clock from `rocm-smi --showclocks` five times a second; the record then carries the median clock
+under that load and the fraction of the MFMA rate at that clock (2.5 PFLOP/s is quoted at 2.4 GHz, and the
+device lowers its clock under sustained matrix work on real data).
 """
 from __future__ import annotations
 
 import argparse
 import json
+import re
+import subprocess
 import sys
+import threading
+import time
 
 import numpy as np
 
@@ -20,7 +29,39 @@ from ._ffi import Q4_0, Q4_K, Q5_K, Q6_K, Q8_0
 from .backend import HipBackend, prefill_plan, row_bytes
 
 MFMA_PEAK_TFLOPS = 2500.0
+MFMA_PEAK_CLOCK_MHZ = 2400.0
 HBM_PEAK_GBS = 8000.0
+
+
+class ClockSampler:
+    """Reads the current shader clock (MHz) from rocm-smi in a thread until stopped."""
+
+    def __init__(self, period_s: float = 0.2):
+        self.period, self.samples, self._stop = period_s, [], threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    def _run(self):
+        while not self._stop.is_set():
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=5).stdout
+                m = re.search(r"sclk clock level[^\n]*\((\d+)Mhz\)", out)
+                if m:
+                    self.samples.append(int(m.group(1)))
+            except (OSError, subprocess.SubprocessError):
+                pass
+            self._stop.wait(self.period)
+
+    def __enter__(self):
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join()
+
+    def median(self):
+        s = sorted(self.samples[1:] or self.samples)          # the first sample may predate the ramp
+        return s[len(s) // 2] if s else None
 
 
 def main(argv=None):
@@ -30,6 +71,7 @@ def main(argv=None):
     ap.add_argument("--formats", default="q4_0,q8_0")
     ap.add_argument("--m", default="64,512,2048")
     ap.add_argument("--seed", type=int, default=7)
+    ap.add_argument("--sample-clock", type=float, default=0.0, metavar="S", help="also run each cell for S seconds and report the shader clock under that load")
     args = ap.parse_args(argv)
     fmts = {"q4_0": (Q4_0, quantize.quantize_q4_0), "q8_0": (Q8_0, quantize.quantize_q8_0), "q4_K": (Q4_K, quantize.quantize_q4_K),
             "q5_K": (Q5_K, quantize.quantize_q5_K), "q6_K": (Q6_K, quantize.quantize_q6_K)}
@@ -61,10 +103,29 @@ def main(argv=None):
                 bound = "mfma" if flops / nbytes >= MFMA_PEAK_TFLOPS * 1e3 / HBM_PEAK_GBS else "hbm"
                 frac = tflops / MFMA_PEAK_TFLOPS if bound == "mfma" else gbs / HBM_PEAK_GBS
                 tm, tn, sp, wv = prefill_plan(m, n, k, be.compute_units, qt)
+                sustained = {}
+                if args.sample_clock > 0:
+                    with ClockSampler() as cs:
+                        t0, launches = time.time(), 0
+                        s0, s1 = be.event(), be.event()
+                        be.record(s0)
+                        while time.time() - t0 < args.sample_clock:
+                            for i in range(16):
+                                be.quantized_matmul(ws[i % copies], x, y, m)
+                            be.sync()
+                            launches += 16
+                        be.record(s1)
+                        sus_us = be.elapsed_us(s0, s1) / launches
+                        be.destroy_event(s0)
+                        be.destroy_event(s1)
+                    mhz = cs.median()
+                    sustained = {"sustained_us": round(sus_us, 1), "sustained_TFLOPs": round(flops / sus_us / 1e6, 1), "sclk_MHz_under_load": mhz}
+                    if mhz and bound == "mfma":
+                        sustained["frac_of_mfma_rate_at_that_clock"] = round(flops / sus_us / 1e6 / (MFMA_PEAK_TFLOPS * mhz / MFMA_PEAK_CLOCK_MHZ), 4)
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
                                   "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide"}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),
-                                  "ksplit": sp, "iters": args.iters}), flush=True)
+                                  "ksplit": sp, "iters": args.iters, **sustained}), flush=True)
             for w in ws:
                 w.buf.free()
     return 0
