@@ -94,6 +94,7 @@ def main(argv=None):
     from openagents_amd.backend import HipBackend, matvec_plan
 
     be = HipBackend(0)
+    be.reserve_prefill(14336, 4096)      # workspace of the dense prefill family (config 4 records), sized before any graph is captured
     t_setup = time.time()
     layer = make_layer(args.seed)
     rng = np.random.default_rng(args.seed + 1)

@@ -335,6 +335,10 @@ class HipBackend:
     def reserve(self, k: int, batch: int = 1):
         _check(self.lib.psn_stream_reserve(self.stream, k, batch))
 
+    def reserve_prefill(self, n: int, k: int):
+        """Size the stream's workspace for the dense prefill family on an [n, k] matrix (before a capture)."""
+        _check(self.lib.psn_prefill_reserve(self.stream, n, k))
+
     def begin_capture(self):
         _check(self.lib.psn_graph_begin_capture(self.stream))
         self._capturing = True

@@ -34,6 +34,7 @@ CODE_OBJECTS = [
     ("psn_mvm", "psn_matvec_mfma.hip", []),
     ("psn_pf_skinny", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=0"]),
     ("psn_pf_wide", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=2"]),
+    ("psn_pf_dense", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=5"]),
     *[(f"psn_pf_{fmt}_{fam}", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", f"-DPSN_BUILD_PF={num}", f"-DPSN_BUILD_PF_{fmt.upper()}"])
       for fmt in ("q4_0", "q8_0") for num, fam in ((1, "ws"), (4, "base"))],
     *[(f"psn_pf_{fmt}_base", "psn_prefill.hip", ["-DPSN_BUILD_ONLY", "-DPSN_BUILD_PF=4", f"-DPSN_BUILD_PF_{fmt.upper()}"])

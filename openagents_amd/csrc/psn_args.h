@@ -66,6 +66,14 @@ struct psn_prefill_args {
     int64_t row_bytes;
 };
 
+/* weights -> fp16 fragments for the dense prefill kernel (psn_prefill_<fmt>_unpack) */
+struct psn_unpack_args {
+    const uint8_t *W;     /* [N][row_bytes] GGUF blocks */
+    uint16_t *out;        /* fragment-major fp16: [ceil(N/32)][K/16][64 lanes][8] */
+    int32_t N, K;
+    int64_t row_bytes;
+};
+
 struct psn_fill_args {
     uint32_t *p;          /* 16-byte aligned */
     int64_t n16;          /* number of 16-byte words to zero */

@@ -1189,10 +1189,35 @@ static const double k_kquant_step_us[] = {1.22, 1.54, 2.08, 2.08, 1.90, 2.77};
 static const double k_kquant_ws_step_us[2] = {1.75, 3.4};
 static const struct { int tile; int waves; double step_us; int per_cu; int fill; } k_prefill_alt[] = {{3, 16, 1.25, 1, 0}, {2, 16, 0.76, 1, 0}, {5, 32, 2.20, 1, 3}};
 
+/* The dense family's estimate: one pass that rewrites the matrix as fp16 (0.45 us per million weights + a
+ * launch, measured) and the multiply on 256 x 256 tiles, whose 64-wide K step costs 1.85 us with most
+ * compute units busy and 1.4 us on a mostly empty chip (the clock is higher then). */
+static double dense_estimate(int64_t M, int64_t N, int64_t K, int32_t cus, int *ksplit_out) {
+    const int64_t mt = (M + 255) / 256, nt = (N + 255) / 256;
+    const double unpack = 4.0 + (double)N * (double)K * 0.45e-6;
+    double best = 1e300;
+    for (int sp = 1; sp <= 4; sp *= 2) {
+        if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
+        const int64_t wgs = mt * nt * sp, rounds = (wgs + cus - 1) / cus;
+        const bool busy = wgs * 4 >= (int64_t)cus * 3;
+        double t = unpack + (double)rounds * ((double)(K / 64) / sp) * (busy ? 1.85 : 1.4) + 5.0;
+        if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;   /* zero fill and atomic adds + a launch */
+        if (t < best) { best = t; *ksplit_out = sp; }
+    }
+    return best;
+}
+
+static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit, int32_t *waves,
+                              double *t_best);
 extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
                                             int32_t *waves) {
+    return psn_qmatmul_prefill_plan_for(PSN_Q4_0, M, N, K, cus, tile_m, tile_n, ksplit, waves);
+}
+static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit, int32_t *waves,
+                              double *t_best) {
     if (!tile_m || !tile_n || !ksplit || !waves) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: out is null");
     *waves = 4;
+    *t_best = 0.0;
     if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
     if (cus <= 0) cus = 256;
     if (M <= 64) {
@@ -1236,13 +1261,14 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
     *tile_m = k_prefill_tiles[bi][0];
     *tile_n = k_prefill_tiles[bi][1];
     *ksplit = bs;
+    *t_best = best;
     return PSN_OK;
 }
 
 /* The K-quants (Q4_K, Q5_K, Q6_K) have the four-wave family (the same estimate over its six tiles with step costs of
  * their own: the dequantization is fp32 arithmetic per weight) and, Q4_K and
  * Q5_K, the 128 x 256 producer / consumer kernel (its staging waves decode while the others multiply). */
-static void prefill_plan_kquant(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
+static double prefill_plan_kquant(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
                                 int32_t *waves) {
     if (cus <= 0) cus = 256;
     double best = 1e300;
@@ -1270,16 +1296,48 @@ static void prefill_plan_kquant(int32_t qtype, int64_t M, int64_t N, int64_t K, 
     *tile_m = k_prefill_tiles[bi][0];
     *tile_n = k_prefill_tiles[bi][1];
     *ksplit = bs;
+    return best;
+}
+
+/* the plan for any format; with allow_dense the dense family (needs the stream's workspace) competes */
+static int32_t prefill_plan_any(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t cus, bool allow_dense, int32_t *tile_m, int32_t *tile_n,
+                                int32_t *ksplit, int32_t *waves) {
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "prefill: type %d", qtype);
+    if (!tile_m || !tile_n || !ksplit || !waves) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: null output");
+    if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill plan: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
+    if (cus <= 0) cus = 256;
+    double best = 0.0;
+    if (qtype == PSN_Q4_0 || qtype == PSN_Q8_0) {
+        int32_t rc = plan_q4_0_q8_0(M, N, K, cus, tile_m, tile_n, ksplit, waves, &best);
+        if (rc) return rc;
+        if (M <= 64) return PSN_OK;                              /* the weight-streaming kernel */
+        if (qtype == PSN_Q8_0) best *= 1.15;                     /* the step costs above were measured on Q4_0; Q8_0 stages twice the bytes */
+    } else {
+        best = prefill_plan_kquant(qtype, M, N, K, cus, tile_m, tile_n, ksplit, waves);
+    }
+    if (allow_dense && M > 64) {
+        int sp = 1;
+        if (dense_estimate(M, N, K, cus, &sp) < 0.95 * best) {   /* two more launches and a workspace: only for a clear gain */
+            *tile_m = 256;
+            *tile_n = 256;
+            *ksplit = sp;
+            *waves = 128;
+        }
+    }
+    return PSN_OK;
 }
 
 extern "C" int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n,
                                                 int32_t *ksplit, int32_t *waves) {
-    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "prefill: type %d", qtype);
-    if (qtype == PSN_Q4_0 || qtype == PSN_Q8_0) return psn_qmatmul_prefill_plan(M, N, K, cus, tile_m, tile_n, ksplit, waves);
-    if (!tile_m || !tile_n || !ksplit || !waves) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan_for: null output");
-    if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill plan: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
-    prefill_plan_kquant(qtype, M, N, K, cus, tile_m, tile_n, ksplit, waves);
-    return PSN_OK;
+    return prefill_plan_any(qtype, M, N, K, cus, true, tile_m, tile_n, ksplit, waves);
+}
+
+extern "C" int32_t psn_prefill_reserve(psn_stream *s, int64_t N, int64_t K) {
+    if (!s) return fail(PSN_E_INVALID_ARG, "stream is null");
+    if (N <= 0 || K <= 0 || K % 256 || N > (1 << 30) || K > (1 << 24)) return fail(PSN_E_SHAPE, "psn_prefill_reserve: N=%lld K=%lld", (long long)N, (long long)K);
+    int32_t rc = bind(s->ctx);
+    if (rc) return rc;
+    return ensure_workspace(s, (N + 255) / 256 * 256 * K * 2);
 }
 
 extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X,
@@ -1287,6 +1345,48 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
                                              int32_t waves) {
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
+    /* waves == 128 selects the dense family (any format): the whole matrix is dequantized to fp16 fragments in
+     * the stream's workspace (psn_prefill_<fmt>_unpack), then psn_prefill_dense_f16 multiplies 256 x 256 tiles */
+    if (waves == 128) {
+        if (bm != 256 || bn != 256) return fail(PSN_E_UNSUPPORTED, "prefill: the dense kernel has a 256x256 tile");
+        if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
+        if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
+        const int64_t nt = (N + 255) / 256, mt = (M + 255) / 256, C = K / 256;
+        const int64_t ws_bytes = nt * 256 * K * 2;
+        if ((rc = bind(mod->ctx))) return rc;
+        if ((rc = ensure_workspace(s, ws_bytes))) return rc;
+        bool cap = false;
+        if ((rc = is_capturing(s, &cap))) return rc;
+        if (cap) s->ws_in_graph = true;
+        psn_unpack_args u;
+        memset(&u, 0, sizeof u);
+        u.W = (const uint8_t *)W->p;
+        u.out = (uint16_t *)s->ws;
+        u.N = (int32_t)N;
+        u.K = (int32_t)K;
+        u.row_bytes = psn_row_bytes(qtype, K);
+        char name[96];
+        snprintf(name, sizeof name, "psn_prefill_%s_unpack", fmt_name(qtype));
+        if ((rc = launch(mod, s, name, (unsigned)(nt * C), 256, 0, &u))) return rc;
+        if (ksplit > 1) {
+            psn_fill_args f;
+            f.p = (uint32_t *)Y->p;
+            f.n16 = M * N / 4;
+            const int64_t fb = (f.n16 + 255) / 256;
+            if ((rc = launch(mod, s, "psn_fill_zero", (unsigned)(fb > 2048 ? 2048 : fb), 256, 0, &f))) return rc;
+        }
+        psn_prefill_args a;
+        memset(&a, 0, sizeof a);
+        a.W = (const uint8_t *)s->ws;
+        a.X = (const uint16_t *)X->p;
+        a.Y = (float *)Y->p;
+        a.M = (int32_t)M;
+        a.N = (int32_t)N;
+        a.K = (int32_t)K;
+        a.ksplit = ksplit;
+        a.row_bytes = K * 2;
+        return launch(mod, s, "psn_prefill_dense_f16", (unsigned)(8 * ((nt + 7) / 8) * mt * ksplit), 256, 4 * 16384, &a);
+    }
     if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !(waves == 16 && bm == 128 && bn == 256 && qtype != PSN_Q6_K))
         return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family%s", fmt_name(qtype),
                     qtype == PSN_Q6_K ? " only (waves = 4)" : " and the 128x256 producer / consumer kernel (waves = 16)");
@@ -1350,8 +1450,13 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
     int32_t bm = 0, bn = 0, sp = 1, wv = 4;
-    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0) prefill_plan_kquant(qtype, M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv);
-    else if ((rc = psn_qmatmul_prefill_plan(M, N, K, mod->ctx->compute_units, &bm, &bn, &sp, &wv))) return rc;
+    /* the dense family needs nt * 256 * K fp16 values of workspace on this stream: it competes when that is
+     * there already or may still be allocated (not while capturing, not once a graph holds the workspace) */
+    bool cap = false;
+    if ((rc = is_capturing(s, &cap))) return rc;
+    const int64_t dense_ws = (N + 255) / 256 * 256 * K * 2;
+    const bool dense_ok = s->ws_bytes >= (size_t)dense_ws || (!cap && !s->ws_in_graph);
+    if ((rc = prefill_plan_any(qtype, M, N, K, mod->ctx->compute_units, dense_ok, &bm, &bn, &sp, &wv))) return rc;
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }
 

@@ -1139,6 +1139,157 @@ PSN_DEV void prefill_wide_body(const psn_prefill_args &a) {
     }
 }
 
+/* ------------------------------------------------------------------------------------------
+ * Dense family: dequantize once, multiply as plain fp16.
+ *
+ * A workgroup of any other family dequantizes its weight tile again for every M tile that needs it; from
+ * a few thousand rows of X on (and from 2048 for the K-quants, whose dequantization is fp32 arithmetic per
+ * weight) it is cheaper to turn the whole matrix into fp16 once per call and run a matmul with no decode
+ * in its loop.  psn_prefill_<fmt>_unpack writes h(deq(W)) -- the same fp16 values every other family
+ * feeds the MFMA -- in the order the multiply kernel consumes them: fragment (32-row block nb, 16-wide K
+ * slice ks) is 1 KB, lane (h = lane >> 5, n = lane & 31) holding W[32 nb + n][16 ks + 8 h .. + 7], i.e.
+ * exactly one B operand of v_mfma_f32_32x32x16_f16.  psn_prefill_dense_f16 (256 x 256 tile, four waves,
+ * each all 256 rows x 64 columns as in the wide kernel) then fetches its weight fragments with plain
+ * 16-byte loads straight into registers, four 32-wide K stages ahead, so that LDS carries only X: a
+ * stage of X is 256 rows of 64 bytes, the four 16-byte pieces of a row stored at piece ^ ((row >> 2) & 3)
+ * (conflict-free fragment reads), filled by direct-to-LDS loads into a ring of four slots; one barrier
+ * per stage, placed between the stage's two K slices so that both batches of fragment reads hide under
+ * sixteen MFMAs.
+ * ------------------------------------------------------------------------------------------ */
+template <typename WF>
+PSN_DEV void prefill_unpack_body(const psn_unpack_args &a) {
+    const int C = a.K >> 8, KF = a.K >> 4;
+    const int rb = (int)(blockIdx.x / (unsigned)C), chunk = (int)(blockIdx.x % (unsigned)C);
+    const int row = rb * 256 + (int)threadIdx.x;
+    if (row >= a.N) return;                                   /* rows of the last 256-row panel past N stay unwritten: their columns are never stored */
+    u32 w[WF::DW];
+    WF::load(a.W + (int64_t)row * a.row_bytes + (int64_t)chunk * WF::BYTES, w);
+    uint4 *frag = reinterpret_cast<uint4 *>(a.out) + ((int64_t)(row >> 5) * KF + chunk * 16) * 64 + (row & 31);
+    auto put = [&](auto bc) {
+        constexpr int B = decltype(bc)::value;
+        u32 o[16];
+        WF::template deq_block<B>(w, o);
+        UNROLL for (int i = 0; i < 4; ++i)                    /* elements 8 i .. 8 i + 7 of the sub-block: K slice 2 B + (i >> 1), half i & 1 */
+            frag[(2 * B + (i >> 1)) * 64 + (i & 1) * 32] = make_uint4(o[4 * i], o[4 * i + 1], o[4 * i + 2], o[4 * i + 3]);
+    };
+    put(pf_int<0>()); put(pf_int<1>()); put(pf_int<2>()); put(pf_int<3>());
+    put(pf_int<4>()); put(pf_int<5>()); put(pf_int<6>()); put(pf_int<7>());
+}
+
+PSN_DEV void prefill_dense_body(const psn_prefill_args &a) {
+    constexpr int BM = 256, BN = 256, TM = 8, TN = 2, NS = 4;
+    constexpr int KS = 32;                                   /* k per stage */
+    constexpr int XB = BM * KS * 2;                          /* bytes of X per stage: 16 KB */
+    constexpr int NL = 4 + 2 * TN;                           /* loads per wave and stage: 4 of X, 4 of W */
+    extern __shared__ uint4 psn_smem[];
+    typedef __attribute__((address_space(3))) char lds_char;
+    lds_char *const lds_ptr = (lds_char *)psn_smem;
+    const u32 lds0 = (u32)(uintptr_t)lds_ptr;
+    const int tid = threadIdx.x, lane = tid & 63, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int M = a.M, N = a.N, K = a.K, C = K >> 8;
+    const int mt = (M + BM - 1) / BM, nt = (N + BN - 1) / BN;
+    const int S = a.ksplit;
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_xcd_n = (nt + 7) >> 3;
+    const int tile_m = local % mt, split = (local / mt) % S, tn_local = local / (mt * S);
+    const int tile_n = xcd + 8 * tn_local;
+    if (tn_local >= per_xcd_n || tile_n >= nt) return;            /* whole workgroup leaves together */
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int per_split = (C + S - 1) / S;
+    const int c_begin = split * per_split, c_end = min(c_begin + per_split, C);
+    if (c_begin >= c_end) return;
+    const int nsteps = (c_end - c_begin) * (256 / KS), g_base = c_begin * (256 / KS);   /* a multiple of NS */
+
+    float16_t acc[TM][TN];
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    /* X: load instruction u of wave w fills LDS bytes [(4 w + u) * 1024, + 1024) of the stage's slot; the
+     * lane picks the global piece that belongs at its LDS position.  Stages past the end of the K range
+     * repeat its last one (into slots nothing reads any more), so every stage issues the same loads. */
+    u32 xoff_g[4];
+    UNROLL for (int u = 0; u < 4; ++u) {
+        const int s_ = (wave * 4 + u) * 64 + lane, row = s_ >> 2, piece = (s_ & 3) ^ ((row >> 2) & 3);
+        xoff_g[u] = (u32)min(m0 + row, M - 1) * (u32)(K * 2) + (u32)(piece * 16);
+    }
+    const int KF = K >> 4;                                   /* fragments per 32-row block */
+    const char *wfrag = reinterpret_cast<const char *>(a.W) + ((int64_t)((n0 >> 5) + wave * 2) * KF) * 1024 + lane * 16;
+    const int64_t wjump = (int64_t)KF * 1024;                /* the wave's second 32-row block */
+    u32x4 bq[NS][2][TN];
+    auto issue_x = [&](int g) {
+        const int gg = g_base + min(g, nsteps - 1), slot = g % NS;
+        const char *xb = reinterpret_cast<const char *>(a.X) + (int64_t)gg * (KS * 2);
+        lds_char *xd = lds_ptr + slot * XB;
+        UNROLL for (int u = 0; u < 4; ++u)
+            __builtin_amdgcn_global_load_lds((const void *)(xb + xoff_g[u]), (__attribute__((address_space(3))) void *)(xd + (wave * 4 + u) * 1024), 16, 0, 0);
+    };
+    auto issue_b = [&](int g, u32x4 (&dst)[2][TN]) {
+        const int gg = g_base + min(g, nsteps - 1);
+        const char *p = wfrag + (int64_t)gg * 2048;
+        UNROLL for (int kk = 0; kk < 2; ++kk) UNROLL for (int j = 0; j < TN; ++j) dst[kk][j] = global_read128(p + kk * 1024 + j * wjump);
+    };
+    u32 fsw[2];                                              /* per-lane offset of the fragment of K slice kk inside a 32-row block of X */
+    UNROLL for (int kk = 0; kk < 2; ++kk) fsw[kk] = (u32)((lane & 31) * 64) + ((((u32)(2 * kk + h)) ^ (u32)((lane >> 2) & 3)) << 4);
+    auto read_a = [&](u32 st, int kk, u32x4 (&af)[TM]) {
+        const u32 ab = st + fsw[kk];
+        af[0] = lds_read128<0>(ab);
+        af[1] = lds_read128<2048>(ab);
+        af[2] = lds_read128<4096>(ab);
+        af[3] = lds_read128<6144>(ab);
+        af[4] = lds_read128<8192>(ab);
+        af[5] = lds_read128<10240>(ab);
+        af[6] = lds_read128<12288>(ab);
+        af[7] = lds_read128<14336>(ab);
+    };
+    auto mfmas = [&](const u32x4 (&af)[TM], const u32x4 (&bf)[TN]) {
+        UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int i = 0; i < TM; ++i)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, af[i]), __builtin_bit_cast(half8_t, bf[j]), acc[i][j], 0, 0, 0);
+    };
+    u32x4 a0[TM], a1[TM];
+    UNROLL for (int s = 0; s < NS; ++s) { issue_x(s); issue_b(s, bq[s]); }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 1) * NL) : "memory");        /* my share of stage 0 */
+    lds_barrier();
+    read_a(lds0, 0, a0);
+    lds_wait();
+    tie(a0);
+    for (int g = 0; g < nsteps; g += NS) {
+        UNROLL for (int s = 0; s < NS; ++s) {
+            const u32 st = lds0 + (u32)(s * XB), sn = lds0 + (u32)(((s + 1) % NS) * XB);
+            read_a(st, 1, a1);
+            mfmas(a0, bq[s][0]);
+            /* stage g + s + 1 has landed (the two after it may still be on their way); my reads of this stage are done */
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 2) * NL) : "memory");
+            lds_barrier();
+            tie(a1);
+            tie(bq[s][1]);
+            issue_x(g + s + NS);                             /* into this stage's slot: nobody reads it any more */
+            read_a(sn, 0, a0);
+            mfmas(a1, bq[s][1]);
+            issue_b(g + s + NS, bq[s]);                      /* both of the stage's fragment sets have been multiplied */
+            lds_wait();
+            tie(a0);
+            tie(bq[(s + 1) % NS][0]);
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+    int tid_out = threadIdx.x;
+    asm volatile("" : "+v"(tid_out));
+    const int wn_o = tid_out >> 6, lane_o = tid_out & 63;
+    const bool whole = m0 + BM <= M && n0 + BN <= N;              /* uniform: no element of the tile needs a bounds check */
+    UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn_o * 64 + 32 * j + (lane_o & 31);
+        float *yc = a.Y + (int64_t)(m0 + 32 * i + 4 * (lane_o >> 5)) * N + col;
+        UNROLL for (int r = 0; r < 16; ++r) {
+            const int dr = 8 * (r >> 2) + (r & 3);
+            if (whole || (m0 + 32 * i + 4 * (lane_o >> 5) + dr < M && col < N)) {
+                if (S == 1) yc[(int64_t)dr * N] = acc[i][j][r];
+                else unsafeAtomicAdd(&yc[(int64_t)dr * N], acc[i][j][r]);
+            }
+        }
+    }
+}
+
 #define PSN_PREFILL_KERNEL_WIDE(fmt, WF)                                                                     \
     extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_wide(const psn_prefill_args a) {   \
         prefill_wide_body<WF>(a);                                                                            \
@@ -1176,7 +1327,8 @@ PSN_DEV void prefill_wide_body(const psn_prefill_args &a) {
 
 /* The build compiles this file once per (format, kernel family) -- -DPSN_BUILD_ONLY -DPSN_BUILD_PF=<n>
  * -DPSN_BUILD_PF_Q4_0 or _Q8_0 -- so that the code objects build in parallel; without PSN_BUILD_ONLY
- * everything lands in one.  Family numbers: 0 skinny + fill, 1 ws (producer / consumer), 2 wide, 4 base (four waves). */
+ * everything lands in one.  Family numbers: 0 skinny + fill, 1 ws (producer / consumer), 2 wide, 4 base (four waves),
+ * 5 dense (unpack kernels of all formats + the fp16 multiply). */
 
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 0
 /* zero fill with plain vector stores (graph-safe stand-in for a memset node) */
@@ -1207,6 +1359,16 @@ PSN_PREFILL_FAMILY_WS(q8_0, PfQ8_0)
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 4
 PSN_PREFILL_FAMILY_BASE(q8_0, PfQ8_0)
 #endif
+#endif
+#if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 5
+extern "C" __global__ void __launch_bounds__(256) psn_prefill_dense_f16(const psn_prefill_args a) { prefill_dense_body(a); }
+#define PSN_PREFILL_KERNEL_UNPACK(fmt, WF) \
+    extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_unpack(const psn_unpack_args a) { prefill_unpack_body<WF>(a); }
+PSN_PREFILL_KERNEL_UNPACK(q4_0, PfQ4_0)
+PSN_PREFILL_KERNEL_UNPACK(q8_0, PfQ8_0)
+PSN_PREFILL_KERNEL_UNPACK(q4_K, PfQ4_K)
+PSN_PREFILL_KERNEL_UNPACK(q5_K, PfQ5_K)
+PSN_PREFILL_KERNEL_UNPACK(q6_K, PfQ6_K)
 #endif
 /* K-quants: the four-wave family, and for Q4_K / Q5_K the 128 x 256 producer / consumer kernel
  * (-DPSN_BUILD_PF=4 -DPSN_BUILD_PF_Q4_K / _Q5_K / _Q6_K) */

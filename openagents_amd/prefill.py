@@ -124,7 +124,7 @@ def main(argv=None):
                         sustained["frac_of_mfma_rate_at_that_clock"] = round(flops / sus_us / 1e6 / (MFMA_PEAK_TFLOPS * mhz / MFMA_PEAK_CLOCK_MHZ), 4)
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
-                                  "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide"}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),
+                                  "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide", 128: f"psn_prefill_{fname}_unpack + psn_prefill_dense_f16"}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),
                                   "ksplit": sp, "iters": args.iters, **sustained}), flush=True)
             for w in ws:
                 w.buf.free()

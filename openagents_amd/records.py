@@ -178,7 +178,7 @@ def config3(be: HipBackend, samples: int = 9, seed: int = 31, weights=None) -> l
 
 def prefill_kernel_name(fmt: str, m: int, n: int, k: int, cus: int):
     tm, tn, sp, wv = prefill_plan(m, n, k, cus)
-    name = {64: f"psn_prefill_{fmt}_skinny", 32: f"psn_prefill_{fmt}_wide"}.get(wv, f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, ""))
+    name = {64: f"psn_prefill_{fmt}_skinny", 32: f"psn_prefill_{fmt}_wide", 128: f"psn_prefill_{fmt}_unpack + psn_prefill_dense_f16"}.get(wv, f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, ""))
     return name, sp
 
 
@@ -305,6 +305,7 @@ def main(argv=None):
     args = ap.parse_args(argv)
     os.makedirs(args.out, exist_ok=True)
     be = HipBackend(0)
+    be.reserve_prefill(14336, 4096)      # the dense prefill family's workspace, before any graph refers to the stream's workspace
     recs = []
     todo = set(args.configs.split(","))
     if "1" in todo:

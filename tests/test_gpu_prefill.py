@@ -248,3 +248,71 @@ def test_prefill_default_plans_over_seeded_random_shapes(hip, orc):
         ref = orc.prefill(qt, b, x, n, k)
         got = hip.matmul_host(qt, b, x, n, k)
         assert G.max_rel_err(got, ref) < 2e-5, (qname, m, n, k)
+
+
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
+def test_dense_family_ragged_shapes(hip, orc, qname):
+    """Family 128: the matrix is rewritten as fp16 fragments once (psn_prefill_<fmt>_unpack), then multiplied
+    on 256 x 256 tiles.  Ragged m and n against the tile and against the 32-row fragment blocks, one to
+    sixteen chunks of K, every K split the shape allows; the fp16 values are those of the other families,
+    so the same tolerance holds."""
+    t = getattr(orc, qname)
+    for m, n, k in ((1, 40, 256), (37, 300, 1280), (260, 700, 2048), (333, 516, 1024), (257, 256, 512), (520, 33, 4096)):
+        W = weights(orc, qname, 820, n, k)
+        X = G.seeded_acts(821 + m, m, k).astype(np.float16)
+        ref = orc.prefill(t, W, X, n, k)
+        for ksplit in (1, 2, 4):
+            if ksplit > 1 and ((m * n) % 4 or k // 256 < ksplit):
+                continue
+            say(f"dense prefill {qname} m={m} n={n} k={k} ksplit={ksplit}")
+            y = hip.matmul_host(t, W, X, n, k, (256, 256, ksplit, 128))
+            err = G.max_rel_err(y, ref)
+            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (qname, ksplit, m, n, k, err)
+    with pytest.raises(backend.PsnError) as e:
+        hip.matmul_host(t, W, X, n, k, (128, 256, 1, 128))                      # the dense kernel has one tile
+    assert e.value.name == "PSN_E_UNSUPPORTED"
+
+
+def test_dense_family_in_graphs_needs_its_workspace_first(hip, orc):
+    """Large M takes the dense family by default.  Its fp16 copy of the matrix lives in the stream's
+    workspace, which cannot be allocated during a capture: on a stream that has none the default plan falls
+    back to the other families (same result), a forced dense launch is refused, and after psn_prefill_reserve
+    the capture contains the dense launches and replays to the eager result."""
+    t, n, k, m = orc.Q4_K, 3000, 1024, 1500
+    assert backend.prefill_plan(m, n, k, hip.compute_units, t)[3] == 128
+    assert backend.prefill_plan(64, n, k, hip.compute_units, t)[3] != 128
+    W = weights(orc, "Q4_K", 830, n, k)
+    X = G.seeded_acts(831, m, k).astype(np.float16)
+    ref = orc.prefill(t, W, X, n, k)
+    w, x = hip.upload_weight(t, W, n, k), hip.upload(X)
+    y = hip.alloc(m * n * 4)
+    s2 = hip.new_stream()
+    try:
+        with hip.on_stream(s2):
+            hip.begin_capture()
+            try:
+                hip.quantized_matmul(w, x, y, m)                                  # no workspace on this stream: not dense
+                with pytest.raises(backend.PsnError) as e:
+                    hip.quantized_matmul(w, x, y, m, (256, 256, 1, 128))
+                assert e.value.name == "PSN_E_INVALID_ARG"
+            finally:
+                g = hip.end_capture()
+            hip.launch_graph(g)
+            hip.sync()
+            assert G.max_rel_err(y.download(np.float32, (m, n)), ref) < PARITY_TOL
+            hip.destroy_graph(g)
+            hip.reserve_prefill(n, k)
+            y.fill_zero()
+            hip.begin_capture()
+            try:
+                hip.quantized_matmul(w, x, y, m)                                  # dense now
+                hip.quantized_matmul(w, x, y, m, (256, 256, 2, 128))
+            finally:
+                g = hip.end_capture()
+            for _ in range(3):
+                hip.launch_graph(g)
+                hip.sync()
+                assert G.max_rel_err(y.download(np.float32, (m, n)), ref) < PARITY_TOL
+            hip.destroy_graph(g)
+    finally:
+        hip.destroy_stream(s2)
