@@ -176,8 +176,8 @@ def config3(be: HipBackend, samples: int = 9, seed: int = 31, weights=None) -> l
     return out
 
 
-def prefill_kernel_name(fmt: str, m: int, n: int, k: int, cus: int):
-    tm, tn, sp, wv = prefill_plan(m, n, k, cus)
+def prefill_kernel_name(fmt: str, m: int, n: int, k: int, cus: int, qtype: int | None = None):
+    tm, tn, sp, wv = prefill_plan(m, n, k, cus, qtype)
     name = {64: f"psn_prefill_{fmt}_skinny", 32: f"psn_prefill_{fmt}_wide", 128: f"psn_prefill_{fmt}_unpack + psn_prefill_dense_f16"}.get(wv, f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, ""))
     return name, sp
 
@@ -206,7 +206,7 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
                 t_us = st["median_us"]
                 bound_us = max(flops / (MFMA_F16_PEAK_TFLOPS * 1e6), nbytes / (HBM_PEAK_GBS * 1e3))
                 bound = "mfma" if flops / (MFMA_F16_PEAK_TFLOPS * 1e6) >= nbytes / (HBM_PEAK_GBS * 1e3) else "hbm"
-                kname, sp = prefill_kernel_name(fmt, m, n, k, be.compute_units)
+                kname, sp = prefill_kernel_name(fmt, m, n, k, be.compute_units, qtype)
                 out.append(record(be, f"prefill.{fmt}.{k}x{n}.m{m}", kname, digest, m * 1e6 / t_us,
                                   shape={"M": m, "N": n, "K": k, "format": fmt, "ksplit": sp}, timing=st,
                                   TFLOPs=round(flops / t_us / 1e6, 1), GBps=round(nbytes / t_us / 1e3, 1),
