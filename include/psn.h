@@ -288,6 +288,16 @@ int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_t N, int64_
 /* Sizes the stream's workspace for the dense family on an [N][K] matrix (and keeps whatever the decode
  * matvecs reserved: the workspace only grows).  Call before capturing a graph that should contain it. */
 int32_t psn_prefill_reserve(psn_stream *s, int64_t N, int64_t K);
+/* The dense family with the dequantization hoisted out of the call: psn_prefill_pack writes h(deq(W)) once
+ * into a caller-owned buffer of psn_prefill_packed_bytes(N, K) bytes (2 bytes per weight, rows padded to whole
+ * 256-row panels; a deployment with HBM to spare keeps one per matrix beside the GGUF blocks the decode
+ * matvec reads), psn_qmatmul_prefill_packed multiplies any number of X against it -- the same result as
+ * psn_qmatmul_prefill_tiled(..., 256, 256, ksplit, 128) without the 35-48 us pass per call.  No stream
+ * workspace is involved.  No counterpart in the reference, which dequantizes inside every call. */
+int64_t psn_prefill_packed_bytes(int64_t N, int64_t K);
+int32_t psn_prefill_pack(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, psn_buf *packed, int64_t N, int64_t K);
+int32_t psn_qmatmul_prefill_packed(psn_module *mod, psn_stream *s, const psn_buf *packed, const psn_buf *X_f16, psn_buf *Y_f32,
+                                   int64_t M, int64_t N, int64_t K);
 /* ... and the same matmul with a caller-chosen shape (auto-tuners, benchmarks). */
 int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X_f16,
                                   psn_buf *Y_f32, int64_t M, int64_t N, int64_t K, int32_t tile_m, int32_t tile_n,

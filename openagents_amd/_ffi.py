@@ -90,6 +90,9 @@ SIGNATURES = {
     "psn_qmatmul_prefill_plan_for": (_i32, [_i32, _i64, _i64, _i64, _i32, C.POINTER(_i32), C.POINTER(_i32), C.POINTER(_i32), C.POINTER(_i32)]),
     "psn_qmatmul_prefill_tiled": (_i32, [_vp, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i32, _i32, _i32, _i32]),
     "psn_prefill_reserve": (_i32, [_vp, _i64, _i64]),
+    "psn_prefill_packed_bytes": (_i64, [_i64, _i64]),
+    "psn_prefill_pack": (_i32, [_vp, _vp, _i32, _vp, _vp, _i64, _i64]),
+    "psn_qmatmul_prefill_packed": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64]),
     "psn_add_rmsnorm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, C.c_float]),
     "psn_rope_kv_store": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, C.c_float]),
     "psn_attention_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32]),

@@ -335,6 +335,18 @@ class HipBackend:
     def reserve(self, k: int, batch: int = 1):
         _check(self.lib.psn_stream_reserve(self.stream, k, batch))
 
+    def pack_for_prefill(self, w: QuantizedTensor) -> DeviceBuffer:
+        """h(deq(w)) as fp16 MFMA fragments in a buffer of its own (2 bytes per weight): dequantized once, multiplied many times."""
+        nbytes = int(self.lib.psn_prefill_packed_bytes(w.n, w.k))
+        if nbytes < 0:
+            _check(nbytes)
+        packed = self.alloc(nbytes)
+        _check(self.lib.psn_prefill_pack(self.module, self.stream, w.qtype, w.buf.handle, packed.handle, w.n, w.k))
+        return packed
+
+    def quantized_matmul_packed(self, packed: DeviceBuffer, x_f16: DeviceBuffer, y: DeviceBuffer, m: int, n: int, k: int):
+        _check(self.lib.psn_qmatmul_prefill_packed(self.module, self.stream, packed.handle, x_f16.handle, y.handle, m, n, k))
+
     def reserve_prefill(self, n: int, k: int):
         """Size the stream's workspace for the dense prefill family on an [n, k] matrix (before a capture)."""
         _check(self.lib.psn_prefill_reserve(self.stream, n, k))

@@ -1332,12 +1332,83 @@ extern "C" int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_
     return prefill_plan_any(qtype, M, N, K, cus, true, tile_m, tile_n, ksplit, waves);
 }
 
+static int32_t need(const psn_buf *b, int64_t bytes, const char *what, const char *name);
+/* the dense family's two steps: GGUF blocks -> fp16 MFMA fragments ([ceil(N/32)][K/16][64 lanes][8 halves], rows
+ * padded to whole 256-row panels), and the fp16 multiply on 256 x 256 tiles over such a buffer */
+static int64_t packed_bytes(int64_t N, int64_t K) { return (N + 255) / 256 * 256 * K * 2; }
+static int32_t launch_unpack(psn_module *mod, psn_stream *s, int32_t qtype, const void *W, void *out, int64_t N, int64_t K) {
+    psn_unpack_args u;
+    memset(&u, 0, sizeof u);
+    u.W = (const uint8_t *)W;
+    u.out = (uint16_t *)out;
+    u.N = (int32_t)N;
+    u.K = (int32_t)K;
+    u.row_bytes = psn_row_bytes(qtype, K);
+    char name[96];
+    snprintf(name, sizeof name, "psn_prefill_%s_unpack", fmt_name(qtype));
+    return launch(mod, s, name, (unsigned)((N + 255) / 256 * (K / 256)), 256, 0, &u);
+}
+static int32_t launch_dense(psn_module *mod, psn_stream *s, const void *packed, const psn_buf *X, psn_buf *Y, int64_t M, int64_t N, int64_t K,
+                            int32_t ksplit) {
+    int32_t rc;
+    if (ksplit > 1) {
+        psn_fill_args f;
+        f.p = (uint32_t *)Y->p;
+        f.n16 = M * N / 4;
+        const int64_t fb = (f.n16 + 255) / 256;
+        if ((rc = launch(mod, s, "psn_fill_zero", (unsigned)(fb > 2048 ? 2048 : fb), 256, 0, &f))) return rc;
+    }
+    const int64_t nt = (N + 255) / 256, mt = (M + 255) / 256;
+    psn_prefill_args a;
+    memset(&a, 0, sizeof a);
+    a.W = (const uint8_t *)packed;
+    a.X = (const uint16_t *)X->p;
+    a.Y = (float *)Y->p;
+    a.M = (int32_t)M;
+    a.N = (int32_t)N;
+    a.K = (int32_t)K;
+    a.ksplit = ksplit;
+    a.row_bytes = K * 2;
+    return launch(mod, s, "psn_prefill_dense_f16", (unsigned)(8 * ((nt + 7) / 8) * mt * ksplit), 256, 4 * 16384, &a);
+}
+
+extern "C" int64_t psn_prefill_packed_bytes(int64_t N, int64_t K) {
+    if (N <= 0 || K <= 0 || K % 256 || N > (1 << 30) || K > (1 << 24)) return fail(PSN_E_SHAPE, "psn_prefill_packed_bytes: N=%lld K=%lld", (long long)N, (long long)K);
+    return packed_bytes(N, K);
+}
+extern "C" int32_t psn_prefill_pack(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, psn_buf *packed, int64_t N, int64_t K) {
+    if (!mod || !s || !W || !packed) return fail(PSN_E_INVALID_ARG, "psn_prefill_pack: null handle");
+    if (s->ctx != mod->ctx || W->ctx != mod->ctx || packed->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "psn_prefill_pack: handles belong to different contexts");
+    if (!is_weight_type(qtype)) return fail(PSN_E_UNSUPPORTED, "psn_prefill_pack: type %d", qtype);
+    if (N <= 0 || N > (1 << 30) || K <= 0 || K % 256 || K > (1 << 24)) return fail(PSN_E_SHAPE, "psn_prefill_pack: N=%lld K=%lld (K must be a multiple of 256)", (long long)N, (long long)K);
+    int32_t rc;
+    if ((rc = need(W, N * psn_row_bytes(qtype, K), "psn_prefill_pack", "W")) || (rc = need(packed, packed_bytes(N, K), "psn_prefill_pack", "packed"))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    return launch_unpack(mod, s, qtype, W->p, packed->p, N, K);
+}
+extern "C" int32_t psn_qmatmul_prefill_packed(psn_module *mod, psn_stream *s, const psn_buf *packed, const psn_buf *X, psn_buf *Y, int64_t M,
+                                              int64_t N, int64_t K) {
+    if (!mod || !s || !packed || !X || !Y) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_packed: null handle");
+    if (s->ctx != mod->ctx || packed->ctx != mod->ctx || X->ctx != mod->ctx || Y->ctx != mod->ctx)
+        return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_packed: handles belong to different contexts");
+    if (M <= 0 || M > (1 << 24) || N <= 0 || N > (1 << 30) || K <= 0 || K % 256 || K > (1 << 24))
+        return fail(PSN_E_SHAPE, "psn_qmatmul_prefill_packed: M=%lld N=%lld K=%lld (K must be a multiple of 256)", (long long)M, (long long)N, (long long)K);
+    int32_t rc;
+    if ((rc = need(packed, packed_bytes(N, K), "psn_qmatmul_prefill_packed", "packed")) || (rc = need(X, M * K * 2, "psn_qmatmul_prefill_packed", "X")) ||
+        (rc = need(Y, M * N * 4, "psn_qmatmul_prefill_packed", "Y")))
+        return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    int sp = 1;
+    (void)dense_estimate(M, N, K, mod->ctx->compute_units, &sp);
+    return launch_dense(mod, s, packed->p, X, Y, M, N, K, sp);
+}
+
 extern "C" int32_t psn_prefill_reserve(psn_stream *s, int64_t N, int64_t K) {
     if (!s) return fail(PSN_E_INVALID_ARG, "stream is null");
     if (N <= 0 || K <= 0 || K % 256 || N > (1 << 30) || K > (1 << 24)) return fail(PSN_E_SHAPE, "psn_prefill_reserve: N=%lld K=%lld", (long long)N, (long long)K);
     int32_t rc = bind(s->ctx);
     if (rc) return rc;
-    return ensure_workspace(s, (N + 255) / 256 * 256 * K * 2);
+    return ensure_workspace(s, packed_bytes(N, K));
 }
 
 extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int32_t qtype, const psn_buf *W, const psn_buf *X,
@@ -1351,41 +1422,13 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
         if (bm != 256 || bn != 256) return fail(PSN_E_UNSUPPORTED, "prefill: the dense kernel has a 256x256 tile");
         if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
         if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
-        const int64_t nt = (N + 255) / 256, mt = (M + 255) / 256, C = K / 256;
-        const int64_t ws_bytes = nt * 256 * K * 2;
         if ((rc = bind(mod->ctx))) return rc;
-        if ((rc = ensure_workspace(s, ws_bytes))) return rc;
+        if ((rc = ensure_workspace(s, packed_bytes(N, K)))) return rc;
         bool cap = false;
         if ((rc = is_capturing(s, &cap))) return rc;
         if (cap) s->ws_in_graph = true;
-        psn_unpack_args u;
-        memset(&u, 0, sizeof u);
-        u.W = (const uint8_t *)W->p;
-        u.out = (uint16_t *)s->ws;
-        u.N = (int32_t)N;
-        u.K = (int32_t)K;
-        u.row_bytes = psn_row_bytes(qtype, K);
-        char name[96];
-        snprintf(name, sizeof name, "psn_prefill_%s_unpack", fmt_name(qtype));
-        if ((rc = launch(mod, s, name, (unsigned)(nt * C), 256, 0, &u))) return rc;
-        if (ksplit > 1) {
-            psn_fill_args f;
-            f.p = (uint32_t *)Y->p;
-            f.n16 = M * N / 4;
-            const int64_t fb = (f.n16 + 255) / 256;
-            if ((rc = launch(mod, s, "psn_fill_zero", (unsigned)(fb > 2048 ? 2048 : fb), 256, 0, &f))) return rc;
-        }
-        psn_prefill_args a;
-        memset(&a, 0, sizeof a);
-        a.W = (const uint8_t *)s->ws;
-        a.X = (const uint16_t *)X->p;
-        a.Y = (float *)Y->p;
-        a.M = (int32_t)M;
-        a.N = (int32_t)N;
-        a.K = (int32_t)K;
-        a.ksplit = ksplit;
-        a.row_bytes = K * 2;
-        return launch(mod, s, "psn_prefill_dense_f16", (unsigned)(8 * ((nt + 7) / 8) * mt * ksplit), 256, 4 * 16384, &a);
+        if ((rc = launch_unpack(mod, s, qtype, W->p, s->ws, N, K))) return rc;
+        return launch_dense(mod, s, s->ws, X, Y, M, N, K, ksplit);
     }
     if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !(waves == 16 && bm == 128 && bn == 256 && qtype != PSN_Q6_K))
         return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family%s", fmt_name(qtype),
@@ -1454,7 +1497,7 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
      * there already or may still be allocated (not while capturing, not once a graph holds the workspace) */
     bool cap = false;
     if ((rc = is_capturing(s, &cap))) return rc;
-    const int64_t dense_ws = (N + 255) / 256 * 256 * K * 2;
+    const int64_t dense_ws = packed_bytes(N, K);
     const bool dense_ok = s->ws_bytes >= (size_t)dense_ws || (!cap && !s->ws_in_graph);
     if ((rc = prefill_plan_any(qtype, M, N, K, mod->ctx->compute_units, dense_ok, &bm, &bn, &sp, &wv))) return rc;
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);

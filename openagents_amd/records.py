@@ -207,6 +207,23 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
                 bound_us = max(flops / (MFMA_F16_PEAK_TFLOPS * 1e6), nbytes / (HBM_PEAK_GBS * 1e3))
                 bound = "mfma" if flops / (MFMA_F16_PEAK_TFLOPS * 1e6) >= nbytes / (HBM_PEAK_GBS * 1e3) else "hbm"
                 kname, sp = prefill_kernel_name(fmt, m, n, k, be.compute_units, qtype)
+                packed_extra = {}
+                if m >= 2048:
+                    # the same projection with the dequantization hoisted out of the call (psn_prefill_pack once, then
+                    # psn_qmatmul_prefill_packed): three packed copies rotate (2 bytes per weight each)
+                    packs = [be.pack_for_prefill(w) for w in ws[:3]]
+                    be.begin_capture()
+                    for pk in packs:
+                        be.quantized_matmul_packed(pk, x, y, m, n, k)
+                    gp = be.end_capture()
+                    sp_ = stats(time_graph(be, gp, len(packs), samples, replays=2))
+                    be.destroy_graph(gp)
+                    for pk in packs:
+                        pk.free()
+                    packed_extra = {"timing_packed_weights": {**sp_, "TFLOPs": round(flops / sp_["median_us"] / 1e6, 1),
+                                                              "frac_of_mfma_peak": round(flops / sp_["median_us"] / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
+                                                              "kernelRef": "psn_prefill_dense_f16",
+                                                              "note": "weights dequantized to fp16 fragments once beforehand (psn_prefill_pack, 2 bytes per weight resident)"}}
                 out.append(record(be, f"prefill.{fmt}.{k}x{n}.m{m}", kname, digest, m * 1e6 / t_us,
                                   shape={"M": m, "N": n, "K": k, "format": fmt, "ksplit": sp}, timing=st,
                                   TFLOPs=round(flops / t_us / 1e6, 1), GBps=round(nbytes / t_us / 1e3, 1),
@@ -215,7 +232,7 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
                                   frac_of_mfma_peak=round(flops / t_us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), weight_copies=copies,
                                   tokens_definition="prompt rows through this one projection per second",
                                   not_measured=["end-to-end prefill tokens/s (this record is one projection)",
-                                                "host-side launch cost (graph replay)"]))
+                                                "host-side launch cost (graph replay)"], **packed_extra))
                 x.free()
                 y.free()
             for w in ws:

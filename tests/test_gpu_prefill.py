@@ -278,7 +278,7 @@ def test_dense_family_in_graphs_needs_its_workspace_first(hip, orc):
     workspace, which cannot be allocated during a capture: on a stream that has none the default plan falls
     back to the other families (same result), a forced dense launch is refused, and after psn_prefill_reserve
     the capture contains the dense launches and replays to the eager result."""
-    t, n, k, m = orc.Q4_K, 3000, 1024, 1500
+    t, n, k, m = orc.Q4_K, 3000, 768, 3000
     assert backend.prefill_plan(m, n, k, hip.compute_units, t)[3] == 128
     assert backend.prefill_plan(64, n, k, hip.compute_units, t)[3] != 128
     W = weights(orc, "Q4_K", 830, n, k)
@@ -316,3 +316,29 @@ def test_dense_family_in_graphs_needs_its_workspace_first(hip, orc):
             hip.destroy_graph(g)
     finally:
         hip.destroy_stream(s2)
+
+
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
+def test_packed_weights_multiply_like_the_dense_family(hip, orc, qname):
+    """psn_prefill_pack once, psn_qmatmul_prefill_packed for several X of different heights: the oracle's
+    result each time, and the dense family's (same fragments, same multiply) up to the order of the K ranges' sums."""
+    t = getattr(orc, qname)
+    n, k = 700, 2048
+    W = weights(orc, qname, 840, n, k)
+    w = hip.upload_weight(t, W, n, k)
+    packed = hip.pack_for_prefill(w)
+    assert packed.nbytes >= 768 * k * 2
+    for m in (1, 260, 37):
+        X = G.seeded_acts(841 + m, m, k).astype(np.float16)
+        y = hip.alloc(m * n * 4)
+        hip.quantized_matmul_packed(packed, hip.upload(X), y, m, n, k)
+        got = y.download(np.float32, (m, n))
+        assert G.max_rel_err(got, orc.prefill(t, W, X, n, k)) < PARITY_TOL, (qname, m)
+        same = hip.matmul_host(t, W, X, n, k, (256, 256, 1, 128))
+        assert G.max_rel_err(got, same) < 2e-6                                          # the library may cut K (atomic adds): not bit for bit
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matmul_packed(hip.alloc(1024), hip.upload(X), y, m, n, k)          # not a packed buffer of this shape
+    assert e.value.name == "PSN_E_INVALID_ARG"
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matmul_packed(packed, hip.upload(X), y, m, n, 2000)
+    assert e.value.name == "PSN_E_SHAPE"
