@@ -125,8 +125,9 @@ int32_t psn_graph_destroy(psn_graph *g);
 int32_t psn_stream_wait_stream(psn_stream *waiter, psn_stream *signaler);
 /* Sizes the stream's activation workspace for psn_qmatvec / psn_qmatvec_multi with scheme Q8 up to
  * [batch][K], so later calls (and captures) never allocate.  A graph captured from a call that uses the
- * workspace holds its address: from then on the workspace cannot grow (calls that would need a larger
- * one fail with PSN_E_INVALID_ARG), so reserve the largest K x batch before the first capture. */
+ * workspace holds its address: while such a graph exists the workspace cannot grow (calls that would need
+ * a larger one fail with PSN_E_INVALID_ARG; destroying the graphs lifts this), so reserve the largest
+ * K x batch before the first capture. */
 int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch);
 
 int32_t psn_event_create(psn_ctx *ctx, psn_event **out);
@@ -280,7 +281,7 @@ int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t comput
                                  int32_t *ksplit, int32_t *waves);
 /* The same for a given weight type: what psn_qmatmul_prefill runs when the dense family's workspace is
  * available (psn_qmatmul_prefill_plan answers for Q4_0 / Q8_0; the K-quants have families 4, 16 on the
- * 128x256 tile, and 128).  While a stream is capturing, or once a captured graph refers to its workspace,
+ * 128x256 tile, and 128).  While a stream is capturing, or while a captured graph refers to its workspace,
  * the workspace cannot grow: psn_qmatmul_prefill then takes the best plan without family 128 unless
  * psn_prefill_reserve (or an earlier dense call of that size) has sized it. */
 int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m,

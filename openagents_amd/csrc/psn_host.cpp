@@ -18,6 +18,7 @@
 #include <new>
 #include <string>
 #include <unordered_map>
+#include <memory>
 #include <vector>
 
 /* code objects linked into the library (generated table, see build.py) */
@@ -175,7 +176,8 @@ struct psn_stream {
     hipStream_t s;
     void *ws;          /* activation workspace of psn_qmatvec (scheme Q8) */
     size_t ws_bytes;
-    bool ws_in_graph;  /* a captured graph holds the address of ws: it must never move again */
+    bool ws_in_capture;                 /* the capture in progress has baked the address of ws into a node */
+    std::shared_ptr<int> ws_graph_refs; /* live graphs that hold the address of ws: it must not move while any exists */
     hipEvent_t join_ev; /* created on first use by psn_stream_wait_stream */
 };
 struct psn_buf {
@@ -191,6 +193,7 @@ struct psn_graph {
     psn_ctx *ctx;
     hipGraph_t g;
     hipGraphExec_t exec;
+    std::shared_ptr<int> ws_refs;       /* set when the graph holds the address of its stream's workspace */
 };
 struct psn_module {
     psn_ctx *ctx;
@@ -332,7 +335,8 @@ extern "C" int32_t psn_stream_create(psn_ctx *c, psn_stream **out) {
     st->s = s;
     st->ws = nullptr;
     st->ws_bytes = 0;
-    st->ws_in_graph = false;
+    st->ws_in_capture = false;
+    st->ws_graph_refs = std::make_shared<int>(0);
     st->join_ev = nullptr;
     *out = st;
     return PSN_OK;
@@ -376,7 +380,7 @@ static int32_t ensure_workspace(psn_stream *s, int64_t bytes) {
     int32_t rc = is_capturing(s, &cap);
     if (rc) return rc;
     if (cap) return fail(PSN_E_INVALID_ARG, "activation workspace must grow to %lld bytes during capture: call psn_stream_reserve first", (long long)bytes);
-    if (s->ws_in_graph)
+    if (s->ws_in_capture || *s->ws_graph_refs > 0)
         return fail(PSN_E_INVALID_ARG, "activation workspace (%zu bytes) is referenced by a captured graph and cannot grow to %lld bytes: "
                     "reserve the largest K x batch with psn_stream_reserve before the first capture", s->ws_bytes, (long long)bytes);
     /* earlier launches may still read the old workspace */
@@ -417,6 +421,7 @@ extern "C" int32_t psn_graph_begin_capture(psn_stream *s) {
     int32_t rc = bind(s->ctx);
     if (rc) return rc;
     HIP_TRY(hipStreamBeginCapture(s->s, hipStreamCaptureModeThreadLocal));
+    s->ws_in_capture = false;
     return PSN_OK;
 }
 extern "C" int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out) {
@@ -425,6 +430,8 @@ extern "C" int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out) {
     int32_t rc = bind(s->ctx);
     if (rc) return rc;
     hipGraph_t g = nullptr;
+    const bool holds_ws = s->ws_in_capture;
+    s->ws_in_capture = false;
     HIP_TRY(hipStreamEndCapture(s->s, &g));
     if (!g) return fail(PSN_E_HIP, "hipStreamEndCapture returned no graph (capture was invalidated)");
     hipGraphExec_t ex = nullptr;
@@ -435,6 +442,10 @@ extern "C" int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out) {
     gr->ctx = s->ctx;
     gr->g = g;
     gr->exec = ex;
+    if (holds_ws) {
+        gr->ws_refs = s->ws_graph_refs;
+        ++*gr->ws_refs;
+    }
     *out = gr;
     return PSN_OK;
 }
@@ -452,6 +463,7 @@ extern "C" int32_t psn_graph_destroy(psn_graph *g) {
     if (rc) return rc;
     (void)hipGraphExecDestroy(g->exec);
     (void)hipGraphDestroy(g->g);
+    if (g->ws_refs) --*g->ws_refs;
     delete g;
     return PSN_OK;
 }
@@ -1087,7 +1099,7 @@ extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qty
     if ((rc = ensure_workspace(s, li.bytes))) return rc;
     bool cap = false;
     if ((rc = is_capturing(s, &cap))) return rc;
-    if (cap) s->ws_in_graph = true;      /* the graph being recorded bakes the workspace address into its nodes */
+    if (cap) s->ws_in_capture = true;    /* the graph being recorded bakes the workspace address into its nodes */
     if ((rc = quantize_into(mod, s, at, (const float *)x->p, s->ws, K, batch))) return rc;
     return run_matvec(mod, s, qtype, scheme, sg, s->ws, K, batch, &plan);
 }
@@ -1426,7 +1438,7 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
         if ((rc = ensure_workspace(s, packed_bytes(N, K)))) return rc;
         bool cap = false;
         if ((rc = is_capturing(s, &cap))) return rc;
-        if (cap) s->ws_in_graph = true;
+        if (cap) s->ws_in_capture = true;
         if ((rc = launch_unpack(mod, s, qtype, W->p, s->ws, N, K))) return rc;
         return launch_dense(mod, s, s->ws, X, Y, M, N, K, ksplit);
     }
@@ -1498,7 +1510,7 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     bool cap = false;
     if ((rc = is_capturing(s, &cap))) return rc;
     const int64_t dense_ws = packed_bytes(N, K);
-    const bool dense_ok = s->ws_bytes >= (size_t)dense_ws || (!cap && !s->ws_in_graph);
+    const bool dense_ok = s->ws_bytes >= (size_t)dense_ws || (!cap && *s->ws_graph_refs == 0);
     if ((rc = prefill_plan_any(qtype, M, N, K, mod->ctx->compute_units, dense_ok, &bm, &bn, &sp, &wv))) return rc;
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }
@@ -1611,7 +1623,7 @@ extern "C" int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_
     if ((rc = ensure_workspace(s, li.bytes))) return rc;
     bool cap = false;
     if ((rc = is_capturing(s, &cap))) return rc;
-    if (cap) s->ws_in_graph = true;
+    if (cap) s->ws_in_capture = true;
     psn_actq_out qo;
     qo.qs = (int8_t *)s->ws + li.off_qs;
     qo.d = (float *)((char *)s->ws + li.off_d);

@@ -42,7 +42,7 @@ def test_uploads_downloads_and_memsets_are_refused_while_capturing(hip):
 def test_workspace_cannot_grow_once_a_graph_refers_to_it(orc):
     """Q6_K at batch 4 quantizes in a separate launch into the stream's workspace.  After such a call has
     been captured, a larger eager call on the same stream must fail instead of freeing memory the graph
-    still points at; the graph keeps replaying correctly."""
+    still points at; the graph keeps replaying correctly; once the graph is destroyed the workspace may grow."""
     with backend.HipBackend(0) as be:
         n, k_small, k_big, batch = 8, 1024, 327680, 4        # the workspace grows in 1 MiB steps: 4 x 327680 int8 exceed one
         Ws, Wb = orc.quantize(orc.Q6_K, G.seeded_weights(970, n, k_small)), orc.quantize(orc.Q6_K, G.seeded_weights(971, n, k_big))
@@ -63,3 +63,6 @@ def test_workspace_cannot_grow_once_a_graph_refers_to_it(orc):
         be.launch_graph(graph)
         assert G.max_rel_err(y.download(np.float32, (batch, n)), ref) < 2e-5
         be.destroy_graph(graph)
+        # no graph refers to the workspace any more: it may grow again
+        be.quantized_matvec(wb, dxb, y, batch, _ffi.ACT_Q8)
+        assert G.max_rel_err(y.download(np.float32, (batch, n)), orc.matvec(orc.Q6_K, orc.ACT_Q8, Wb, xb, n, k_big)) < 2e-5
