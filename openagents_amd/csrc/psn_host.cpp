@@ -1181,6 +1181,9 @@ static int32_t check_prefill(const char *what, psn_module *mod, psn_stream *s, i
     const int64_t rb = psn_row_bytes(qtype, K);
     if (rb < 0) return (int32_t)rb;
     if (K % 256 || K > (1 << 24)) return fail(PSN_E_SHAPE, "%s: K=%lld must be a multiple of 256", what, (long long)K);
+    /* several kernel families address X and W with 32-bit byte offsets */
+    if (M * K * 2 > (int64_t)UINT32_MAX || N * rb > (int64_t)UINT32_MAX)
+        return fail(PSN_E_SHAPE, "%s: X (%lld bytes) and W (%lld bytes) must each stay below 4 GiB", what, (long long)(M * K * 2), (long long)(N * rb));
     if ((int64_t)W->bytes < N * rb) return fail(PSN_E_INVALID_ARG, "%s: W holds %zu bytes, need %lld", what, W->bytes, (long long)(N * rb));
     if ((int64_t)X->bytes < M * K * 2) return fail(PSN_E_INVALID_ARG, "%s: X holds %zu bytes, need %lld", what, X->bytes, (long long)(M * K * 2));
     if ((int64_t)Y->bytes < M * N * 4) return fail(PSN_E_INVALID_ARG, "%s: Y holds %zu bytes, need %lld", what, Y->bytes, (long long)(M * N * 4));
@@ -1405,6 +1408,7 @@ extern "C" int32_t psn_qmatmul_prefill_packed(psn_module *mod, psn_stream *s, co
         return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_packed: handles belong to different contexts");
     if (M <= 0 || M > (1 << 24) || N <= 0 || N > (1 << 30) || K <= 0 || K % 256 || K > (1 << 24))
         return fail(PSN_E_SHAPE, "psn_qmatmul_prefill_packed: M=%lld N=%lld K=%lld (K must be a multiple of 256)", (long long)M, (long long)N, (long long)K);
+    if (M * K * 2 > (int64_t)UINT32_MAX) return fail(PSN_E_SHAPE, "psn_qmatmul_prefill_packed: X (%lld bytes) must stay below 4 GiB", (long long)(M * K * 2));
     int32_t rc;
     if ((rc = need(packed, packed_bytes(N, K), "psn_qmatmul_prefill_packed", "packed")) || (rc = need(X, M * K * 2, "psn_qmatmul_prefill_packed", "X")) ||
         (rc = need(Y, M * N * 4, "psn_qmatmul_prefill_packed", "Y")))

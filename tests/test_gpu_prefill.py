@@ -342,3 +342,16 @@ def test_packed_weights_multiply_like_the_dense_family(hip, orc, qname):
     with pytest.raises(backend.PsnError) as e:
         hip.quantized_matmul_packed(packed, hip.upload(X), y, m, n, 2000)
     assert e.value.name == "PSN_E_SHAPE"
+
+
+def test_prefill_refuses_operands_beyond_32_bit_offsets(hip, orc):
+    """Several families address X and W with 32-bit byte offsets: shapes that would overflow them are
+    refused by the host before any buffer is looked at."""
+    w = hip.upload_weight(orc.Q4_0, weights(orc, "Q4_0", 850, 64, 4096), 64, 4096)
+    x, y = hip.alloc(1 << 20), hip.alloc(1 << 20)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matmul(w, x, y, 1 << 20)                       # X would be 8 GiB
+    assert e.value.name == "PSN_E_SHAPE" and "4 GiB" in str(e.value)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matmul_packed(x, x, y, 1 << 20, 64, 4096)
+    assert e.value.name == "PSN_E_SHAPE"
