@@ -1202,21 +1202,29 @@ static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
  * several rounds) */
 static const double k_kquant_step_us[] = {1.22, 1.54, 2.08, 2.08, 1.90, 2.77};
 static const double k_kquant_ws_step_us[2] = {1.75, 3.4};
-static const struct { int tile; int waves; double step_us; int per_cu; int fill; } k_prefill_alt[] = {{3, 16, 1.25, 1, 0}, {2, 16, 0.76, 1, 0}, {5, 32, 2.20, 1, 3}};
+static const struct { int tile; int waves; double step_us; int per_cu; int fill; } k_prefill_alt[] = {{3, 16, 1.25, 1, 2}, {2, 16, 0.82, 1, 1}, {5, 32, 2.20, 1, 3}};
 
+/* zero fill of Y and the atomic adds of `sp` partial sums per element, plus a launch: with few ranges the adds overlap
+ * the multiply well enough to count at the fill's 3 TB/s; from `slow_from` ranges on (eight; four for the wide kernel,
+ * whose four waves hold a whole 256 x 256 tile) they run at the measured 1.6 TB/s */
+static double ksplit_overhead_us(int64_t M, int64_t N, int sp, int slow_from = 8) {
+    const double bytes = (double)(M * N) * 4.0;
+    return (sp >= slow_from ? bytes * (1.0 / 3.0e6 + sp / 1.6e6) : bytes * (1.0 + sp) / 3.0e6) + 4.0;
+}
 /* The dense family's estimate: one pass that rewrites the matrix as fp16 (0.45 us per million weights + a
- * launch, measured) and the multiply on 256 x 256 tiles, whose 64-wide K step costs 1.85 us with most
- * compute units busy and 1.4 us on a mostly empty chip (the clock is higher then). */
+ * launch, measured) and the multiply on 256 x 256 tiles, round by round of workgroups. */
 static double dense_estimate(int64_t M, int64_t N, int64_t K, int32_t cus, int *ksplit_out) {
     const int64_t mt = (M + 255) / 256, nt = (N + 255) / 256;
     const double unpack = 4.0 + (double)N * (double)K * 0.45e-6;
     double best = 1e300;
     for (int sp = 1; sp <= 4; sp *= 2) {
         if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
-        const int64_t wgs = mt * nt * sp, rounds = (wgs + cus - 1) / cus;
-        const bool busy = wgs * 4 >= (int64_t)cus * 3;
-        double t = unpack + (double)rounds * ((double)(K / 64) / sp) * (busy ? 1.85 : 1.4) + 5.0;
-        if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;   /* zero fill and atomic adds + a launch */
+        const int64_t wgs = mt * nt * sp, full = wgs / cus, rest = wgs % cus;
+        const double steps = (double)(K / 64) / sp;
+        /* a round that fills the chip costs 1.85 us per step; a partly filled one runs at a higher clock */
+        const double fill = (double)rest / cus;
+        double t = unpack + (double)full * steps * 1.85 + (rest ? steps * (fill >= 0.8 ? 1.85 : fill >= 0.6 ? 1.5 : 1.4) : 0.0) + 5.0;
+        if (sp > 1) t += ksplit_overhead_us(M, N, sp);
         if (t < best) { best = t; *ksplit_out = sp; }
     }
     return best;
@@ -1260,15 +1268,18 @@ static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int3
             const int64_t wgs = mt * nt * sp;
             const int64_t rounds = (wgs + slots - 1) / slots;
             const double steps = (double)(K / 64) / sp;
-            double t = (double)rounds * steps * k_prefill_step_us[i] + 5.0;
-            if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;   /* bytes / (3 TB/s) in us, + a launch */
+            /* the step costs are those of one workgroup per compute unit; workgroups that share one slow each
+             * other down (measured: 1.45 x with three of the small tiles resident) */
+            const int64_t resident = ((wgs < slots ? wgs : slots) + cus - 1) / cus;
+            double t = (double)rounds * steps * k_prefill_step_us[i] * (1.0 + 0.225 * (double)(resident - 1)) + 5.0;
+            if (sp > 1) t += ksplit_overhead_us(M, N, sp);
             if (t < best) { best = t; bi = i; bs = sp; *waves = 4; }
             for (const auto &v : k_prefill_alt) {
                 if (v.tile != i) continue;
                 const int64_t sl = (int64_t)cus * v.per_cu;
                 const int64_t r8 = (wgs + sl - 1) / sl;
                 double t8 = (double)r8 * (steps + v.fill) * v.step_us + 5.0;
-                if (sp > 1) t8 += (double)(M * N) * 4.0 * (1.0 + sp) / 3.0e6 + 4.0;
+                if (sp > 1) t8 += ksplit_overhead_us(M, N, sp, v.waves == 32 ? 4 : 8);
                 if (t8 < best) { best = t8; bi = i; bs = sp; *waves = v.waves; }
             }
         }
