@@ -1197,15 +1197,17 @@ static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
 /* the producer / consumer kernels (16 = four multiplying + four staging waves) and the wide kernel (32:
  * 256 x 256, four waves decoding their own operands from raw bytes):
  * {tile index, kernel family, step cost, workgroups per compute unit, K steps a workgroup spends filling its load rings} */
-/* the K-quants' four-wave kernels per tile (measured for the 128- and 256-row tiles, scaled from the Q4_0
- * figures for the 64-row ones) and their 128 x 256 producer / consumer kernel (one round of workgroups,
- * several rounds) */
-static const double k_kquant_step_us[] = {1.22, 1.54, 2.08, 2.08, 1.90, 2.77};
-static const double k_kquant_ws_step_us[2] = {1.75, 3.4};
+/* the K-quants' four-wave kernels per tile, one workgroup per compute unit (measured over three projection shapes,
+ * M = 128 .. 1024, every K split; Q5_K takes Q4_K's figures), what each further workgroup on the same compute unit adds
+ * (Q6_K's decode keeps the vector ALUs busy, so two resident workgroups take turns), and the 128 x 256 producer /
+ * consumer kernel of Q4_K and Q5_K (one round of workgroups, several rounds) */
+static const double k_q45_K_step_us[] = {0.76, 1.14, 1.33, 1.91, 1.71, 2.60};
+static const double k_q6_K_step_us[] = {0.95, 1.33, 1.51, 2.43, 1.96, 3.10};
+static const double k_kquant_ws_step_us[2] = {1.45, 3.4};
 static const struct { int tile; int waves; double step_us; int per_cu; int fill; } k_prefill_alt[] = {{3, 16, 1.25, 1, 2}, {2, 16, 0.82, 1, 1}, {5, 32, 2.20, 1, 3}};
 
 /* zero fill of Y and the atomic adds of `sp` partial sums per element, plus a launch: with few ranges the adds overlap
- * the multiply well enough to count at the fill's 3 TB/s; from `slow_from` ranges on (eight; four for the wide kernel,
+ * the multiply well enough to count at the fill's 3 TB/s; from `slow_from` ranges on (eight; four for the kernels
  * whose four waves hold a whole 256 x 256 tile) they run at the measured 1.6 TB/s */
 static double ksplit_overhead_us(int64_t M, int64_t N, int sp, int slow_from = 8) {
     const double bytes = (double)(M * N) * 4.0;
@@ -1224,7 +1226,7 @@ static double dense_estimate(int64_t M, int64_t N, int64_t K, int32_t cus, int *
         /* a round that fills the chip costs 1.85 us per step; a partly filled one runs at a higher clock */
         const double fill = (double)rest / cus;
         double t = unpack + (double)full * steps * 1.85 + (rest ? steps * (fill >= 0.8 ? 1.85 : fill >= 0.6 ? 1.5 : 1.4) : 0.0) + 5.0;
-        if (sp > 1) t += ksplit_overhead_us(M, N, sp);
+        if (sp > 1) t += ksplit_overhead_us(M, N, sp, 4);
         if (t < best) { best = t; *ksplit_out = sp; }
     }
     return best;
@@ -1272,7 +1274,7 @@ static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int3
              * other down (measured: 1.45 x with three of the small tiles resident) */
             const int64_t resident = ((wgs < slots ? wgs : slots) + cus - 1) / cus;
             double t = (double)rounds * steps * k_prefill_step_us[i] * (1.0 + 0.225 * (double)(resident - 1)) + 5.0;
-            if (sp > 1) t += ksplit_overhead_us(M, N, sp);
+            if (sp > 1) t += ksplit_overhead_us(M, N, sp, i == 5 ? 4 : 8);
             if (t < best) { best = t; bi = i; bs = sp; *waves = 4; }
             for (const auto &v : k_prefill_alt) {
                 if (v.tile != i) continue;
@@ -1297,6 +1299,8 @@ static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int3
 static double prefill_plan_kquant(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit,
                                 int32_t *waves) {
     if (cus <= 0) cus = 256;
+    const double *step_us = qtype == PSN_Q6_K ? k_q6_K_step_us : k_q45_K_step_us;
+    const double shared = qtype == PSN_Q6_K ? 1.0 : 0.35;
     double best = 1e300;
     int bi = 0, bs = 1;
     *waves = 4;
@@ -1308,13 +1312,14 @@ static double prefill_plan_kquant(int32_t qtype, int64_t M, int64_t N, int64_t K
         for (int sp = 1; sp <= 8; sp *= 2) {
             if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
             const int64_t wgs = mt * nt * sp, rounds = (wgs + slots - 1) / slots;
-            double t = (double)rounds * ((double)(K / 64) / sp) * k_kquant_step_us[i] + 5.0;
-            if (sp > 1) t += (double)(M * N) * 4.0 * (1.0 / 3.0e6 + sp / 1.6e6) + 4.0   /* zero fill + atomic adds (measured 1.6 TB/s) + a launch */;
+            const int64_t resident = ((wgs < slots ? wgs : slots) + cus - 1) / cus;
+            double t = (double)rounds * ((double)(K / 64) / sp) * step_us[i] * (1.0 + shared * (double)(resident - 1)) + 5.0;
+            if (sp > 1) t += ksplit_overhead_us(M, N, sp, i == 5 ? 4 : 8);
             if (t < best) { best = t; bi = i; bs = sp; *waves = 4; }
             if (i == 3 && qtype != PSN_Q6_K && M > 64) {
                 const int64_t r16 = (wgs + cus - 1) / cus;
-                double t16 = (double)r16 * ((double)(K / 64) / sp) * (r16 > 1 ? k_kquant_ws_step_us[1] : k_kquant_ws_step_us[0]) + 5.0;
-                if (sp > 1) t16 += (double)(M * N) * 4.0 * (1.0 / 3.0e6 + sp / 1.6e6) + 4.0   /* zero fill + atomic adds (measured 1.6 TB/s) + a launch */;
+                double t16 = (double)r16 * ((double)(K / 64) / sp + 2.0) * (r16 > 1 ? k_kquant_ws_step_us[1] : k_kquant_ws_step_us[0]) + 5.0;
+                if (sp > 1) t16 += ksplit_overhead_us(M, N, sp);
                 if (t16 < best) { best = t16; bi = i; bs = sp; *waves = 16; }
             }
         }

@@ -1,7 +1,7 @@
 """Quantized prefill matmul benchmark: Q4_0 / Q8_0 (default) or Q4_K / Q5_K / Q6_K weights 4096->14336 and 14336->4096, fp16
 activations for M = 64, 512, 2048 tokens (seeded N(0,0.02) weights quantized on the host).
 
-    python -m openagents_amd.prefill [--iters 20] [--formats q4_0,q8_0] [--m 64,512,2048]
+    python -m openagents_amd.prefill [--iters 20] [--formats q4_0,q8_0] [--m 64,512,2048] [--shapes 14336x4096,4096x14336]
 
 Prints one JSON record per (format, shape, M): microseconds, TFLOP/s, GB/s and the fraction of the
 roofline that binds (fp16 MFMA 2.5 PFLOP/s, or HBM 8 TB/s when the arithmetic intensity is below
@@ -11,6 +11,10 @@ With --sample-clock S every cell is additionally run back to back for S seconds 
 shader clock from `rocm-smi --showclocks` five times a second; the record then carries the median clock
 under that load and the fraction of the MFMA rate at that clock (2.5 PFLOP/s is quoted at 2.4 GHz, and the
 device lowers its clock under sustained matrix work on real data).
+
+With --compare-plans every cell is also timed under each explicit (tile_m, tile_n, ksplit, family) plan that accepts
+the shape; the record then names the fastest of them beside the planner's default, which is how the planner's cost
+model is checked.
 """
 from __future__ import annotations
 
@@ -26,8 +30,15 @@ import numpy as np
 
 from . import quantize
 from ._ffi import Q4_0, Q4_K, Q5_K, Q6_K, Q8_0
-from .backend import HipBackend, prefill_plan, row_bytes
+from .backend import HipBackend, PsnError, prefill_plan, row_bytes
 
+# (tile_m, tile_n, ksplit, family): the explicit plans --compare-plans tries (family 4 = four waves, 16 = producer / consumer,
+# 32 = wide, 128 = dense)
+EXPLICIT_PLANS = [(64, 64, 2, 4), (64, 64, 4, 4), (64, 64, 8, 4), (64, 128, 2, 4), (64, 128, 4, 4), (64, 128, 8, 4), (256, 128, 2, 4), (256, 128, 4, 4), (256, 128, 8, 4),
+                  (128, 128, 1, 4), (256, 128, 1, 4), (256, 256, 1, 4), (256, 256, 2, 4), (256, 256, 4, 4),
+                  (128, 128, 1, 16), (128, 128, 2, 16), (128, 128, 4, 16), (128, 128, 8, 16),
+                  (128, 256, 1, 16), (128, 256, 2, 16), (128, 256, 4, 16), (128, 256, 8, 16),
+                  (256, 256, 1, 32), (256, 256, 2, 32), (256, 256, 4, 32), (256, 256, 1, 128), (256, 256, 2, 128), (256, 256, 4, 128)]
 MFMA_PEAK_TFLOPS = 2500.0
 MFMA_PEAK_CLOCK_MHZ = 2400.0
 HBM_PEAK_GBS = 8000.0
@@ -72,6 +83,8 @@ def main(argv=None):
     ap.add_argument("--m", default="64,512,2048")
     ap.add_argument("--seed", type=int, default=7)
     ap.add_argument("--sample-clock", type=float, default=0.0, metavar="S", help="also run each cell for S seconds and report the shader clock under that load")
+    ap.add_argument("--shapes", default="14336x4096,4096x14336", help="weight shapes as NxK, comma separated")
+    ap.add_argument("--compare-plans", action="store_true", help="also time every explicit plan and name the fastest")
     args = ap.parse_args(argv)
     fmts = {"q4_0": (Q4_0, quantize.quantize_q4_0), "q8_0": (Q8_0, quantize.quantize_q8_0), "q4_K": (Q4_K, quantize.quantize_q4_K),
             "q5_K": (Q5_K, quantize.quantize_q5_K), "q6_K": (Q6_K, quantize.quantize_q6_K)}
@@ -79,24 +92,41 @@ def main(argv=None):
     rng = np.random.default_rng(args.seed)
     for fname in args.formats.split(","):
         qt, quant = fmts[fname]
-        for n, k in ((14336, 4096), (4096, 14336)):
+        for n, k in (tuple(int(v) for v in t.split("x")) for t in args.shapes.split(",")):
             blocks = quant(rng.standard_normal((n, k), dtype=np.float32) * np.float32(0.02))
             copies = max(2, int(300e6 // blocks.nbytes) + 1)
             ws = [be.upload_weight(qt, blocks, n, k) for _ in range(copies)]
             for m in (int(v) for v in args.m.split(",")):
                 x = be.upload(rng.standard_normal((m, k), dtype=np.float32).astype(np.float16))
                 y = be.alloc(m * n * 4)
-                for i in range(args.warmup):
-                    be.quantized_matmul(ws[i % copies], x, y, m)
-                be.sync()
-                e0, e1 = be.event(), be.event()
-                be.record(e0)
-                for i in range(args.iters):
-                    be.quantized_matmul(ws[i % copies], x, y, m)
-                be.record(e1)
-                us = be.elapsed_us(e0, e1) / args.iters
-                be.destroy_event(e0)
-                be.destroy_event(e1)
+                def timed(tile=None):
+                    for i in range(args.warmup):
+                        be.quantized_matmul(ws[i % copies], x, y, m, tile)
+                    be.sync()
+                    e0, e1 = be.event(), be.event()
+                    be.record(e0)
+                    for i in range(args.iters):
+                        be.quantized_matmul(ws[i % copies], x, y, m, tile)
+                    be.record(e1)
+                    t = be.elapsed_us(e0, e1) / args.iters
+                    be.destroy_event(e0)
+                    be.destroy_event(e1)
+                    return t
+
+                us = timed()
+                compared = {}
+                if args.compare_plans:
+                    tried = []
+                    for tile in EXPLICIT_PLANS:
+                        try:
+                            tried.append((timed(tile), tile))
+                        except PsnError:                         # this plan does not take this shape or format
+                            continue
+                    if tried:
+                        bt, bp = min(tried)
+                        for _ in range(2):                       # the two contenders again, alternating, under the same clocks
+                            bt, us = min(bt, timed(bp)), min(us, timed())
+                        compared = {"best_explicit_plan": list(bp), "best_explicit_us": round(bt, 1), "default_over_best": round(us / bt, 3)}
                 flops = 2.0 * m * n * k
                 nbytes = n * row_bytes(qt, k) + m * k * 2 + m * n * 4
                 tflops, gbs = flops / us / 1e6, nbytes / us / 1e3
@@ -125,7 +155,7 @@ def main(argv=None):
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
                                   "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide", 128: f"psn_prefill_{fname}_unpack + psn_prefill_dense_f16"}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),
-                                  "ksplit": sp, "iters": args.iters, **sustained}), flush=True)
+                                  "ksplit": sp, "iters": args.iters, **sustained, **compared}), flush=True)
             for w in ws:
                 w.buf.free()
     return 0
