@@ -272,7 +272,7 @@ int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32
  *       a wave decodes the operand of its own columns one K slice ahead, interleaved with its MFMAs;
  *   64  the weight-streaming kernel for M <= 64 (64x64 tiles): X and the raw GGUF bytes arrive in LDS
  *       rings by direct-to-LDS loads, every wave decodes its own MFMA operand, one barrier per 256 of K;
- *  128  the dense family for large M (256x256 tiles, every format): one pass writes h(deq(W)) for the whole
+ *  128  the dense family for large M (256x256 or 128x256 tiles, every format): one pass writes h(deq(W)) for the whole
  *       matrix as fp16 into the stream's workspace (ceil(N/256) * 256 * K * 2 bytes, see
  *       psn_prefill_reserve), in the order the multiply kernel's MFMA operands are read; that kernel has no
  *       decode in its loop.  Same fp16 values as every other family, two launches (three with K cut).

@@ -1214,20 +1214,27 @@ static double ksplit_overhead_us(int64_t M, int64_t N, int sp, int slow_from = 8
     return (sp >= slow_from ? bytes * (1.0 / 3.0e6 + sp / 1.6e6) : bytes * (1.0 + sp) / 3.0e6) + 4.0;
 }
 /* The dense family's estimate: one pass that rewrites the matrix as fp16 (0.45 us per million weights + a
- * launch, measured) and the multiply on 256 x 256 tiles, round by round of workgroups. */
-static double dense_estimate(int64_t M, int64_t N, int64_t K, int32_t cus, int *ksplit_out) {
-    const int64_t mt = (M + 255) / 256, nt = (N + 255) / 256;
-    const double unpack = 4.0 + (double)N * (double)K * 0.45e-6;
+ * launch, measured; none when the caller holds packed weights) and the multiply on 256 x 256 or 128 x 256 tiles,
+ * round by round of workgroups. */
+static const double k_dense_step_us[2][3] = {{1.85, 1.5, 1.4}, {0.96, 0.78, 0.72}};   /* {256, 128 rows} x {full round, 60-80 % filled, emptier} */
+static double dense_estimate(int64_t M, int64_t N, int64_t K, int32_t cus, bool with_unpack, int *bm_out, int *ksplit_out) {
+    const int64_t nt = (N + 255) / 256;
+    const double unpack = with_unpack ? 4.0 + (double)N * (double)K * 0.45e-6 : 0.0;
     double best = 1e300;
-    for (int sp = 1; sp <= 4; sp *= 2) {
-        if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
-        const int64_t wgs = mt * nt * sp, full = wgs / cus, rest = wgs % cus;
-        const double steps = (double)(K / 64) / sp;
-        /* a round that fills the chip costs 1.85 us per step; a partly filled one runs at a higher clock */
-        const double fill = (double)rest / cus;
-        double t = unpack + (double)full * steps * 1.85 + (rest ? steps * (fill >= 0.8 ? 1.85 : fill >= 0.6 ? 1.5 : 1.4) : 0.0) + 5.0;
-        if (sp > 1) t += ksplit_overhead_us(M, N, sp, 4);
-        if (t < best) { best = t; *ksplit_out = sp; }
+    for (int v = 0; v < 2; ++v) {
+        const int bm = v ? 128 : 256;
+        const int64_t mt = (M + bm - 1) / bm;
+        for (int sp = 1; sp <= 4; sp *= 2) {
+            if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
+            const int64_t wgs = mt * nt * sp, full = wgs / cus, rest = wgs % cus;
+            const double steps = (double)(K / 64) / sp;
+            /* a round that fills the chip runs at a lower clock than a partly filled one */
+            const double fill = (double)rest / cus;
+            double t = unpack + (double)full * steps * k_dense_step_us[v][0] +
+                       (rest ? steps * k_dense_step_us[v][fill >= 0.8 ? 0 : fill >= 0.6 ? 1 : 2] : 0.0) + 5.0;
+            if (sp > 1) t += ksplit_overhead_us(M, N, sp, v ? 8 : 4);
+            if (t < best) { best = t; *bm_out = bm; *ksplit_out = sp; }
+        }
     }
     return best;
 }
@@ -1347,9 +1354,9 @@ static int32_t prefill_plan_any(int32_t qtype, int64_t M, int64_t N, int64_t K, 
         best = prefill_plan_kquant(qtype, M, N, K, cus, tile_m, tile_n, ksplit, waves);
     }
     if (allow_dense && M > 64) {
-        int sp = 1;
-        if (dense_estimate(M, N, K, cus, &sp) < 0.95 * best) {   /* two more launches and a workspace: only for a clear gain */
-            *tile_m = 256;
+        int sp = 1, bm = 256;
+        if (dense_estimate(M, N, K, cus, true, &bm, &sp) < 0.95 * best) {   /* two more launches and a workspace: only for a clear gain */
+            *tile_m = bm;
             *tile_n = 256;
             *ksplit = sp;
             *waves = 128;
@@ -1380,7 +1387,7 @@ static int32_t launch_unpack(psn_module *mod, psn_stream *s, int32_t qtype, cons
     return launch(mod, s, name, (unsigned)((N + 255) / 256 * (K / 256)), 256, 0, &u);
 }
 static int32_t launch_dense(psn_module *mod, psn_stream *s, const void *packed, const psn_buf *X, psn_buf *Y, int64_t M, int64_t N, int64_t K,
-                            int32_t ksplit) {
+                            int32_t bm, int32_t ksplit) {
     int32_t rc;
     if (ksplit > 1) {
         psn_fill_args f;
@@ -1389,7 +1396,7 @@ static int32_t launch_dense(psn_module *mod, psn_stream *s, const void *packed, 
         const int64_t fb = (f.n16 + 255) / 256;
         if ((rc = launch(mod, s, "psn_fill_zero", (unsigned)(fb > 2048 ? 2048 : fb), 256, 0, &f))) return rc;
     }
-    const int64_t nt = (N + 255) / 256, mt = (M + 255) / 256;
+    const int64_t nt = (N + 255) / 256, mt = (M + bm - 1) / bm;
     psn_prefill_args a;
     memset(&a, 0, sizeof a);
     a.W = (const uint8_t *)packed;
@@ -1400,7 +1407,8 @@ static int32_t launch_dense(psn_module *mod, psn_stream *s, const void *packed, 
     a.K = (int32_t)K;
     a.ksplit = ksplit;
     a.row_bytes = K * 2;
-    return launch(mod, s, "psn_prefill_dense_f16", (unsigned)(8 * ((nt + 7) / 8) * mt * ksplit), 256, 4 * 16384, &a);
+    /* LDS: a ring of four stages of X, bm rows x 32 k fp16 each */
+    return launch(mod, s, bm == 128 ? "psn_prefill_dense_f16_m128" : "psn_prefill_dense_f16", (unsigned)(8 * ((nt + 7) / 8) * mt * ksplit), 256, 4 * bm * 64, &a);
 }
 
 extern "C" int64_t psn_prefill_packed_bytes(int64_t N, int64_t K) {
@@ -1430,9 +1438,9 @@ extern "C" int32_t psn_qmatmul_prefill_packed(psn_module *mod, psn_stream *s, co
         (rc = need(Y, M * N * 4, "psn_qmatmul_prefill_packed", "Y")))
         return rc;
     if ((rc = bind(mod->ctx))) return rc;
-    int sp = 1;
-    (void)dense_estimate(M, N, K, mod->ctx->compute_units, &sp);
-    return launch_dense(mod, s, packed->p, X, Y, M, N, K, sp);
+    int sp = 1, bm = 256;
+    (void)dense_estimate(M, N, K, mod->ctx->compute_units, false, &bm, &sp);
+    return launch_dense(mod, s, packed->p, X, Y, M, N, K, bm, sp);
 }
 
 extern "C" int32_t psn_prefill_reserve(psn_stream *s, int64_t N, int64_t K) {
@@ -1449,9 +1457,10 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     int32_t rc = check_prefill("psn_qmatmul_prefill", mod, s, qtype, W, X, Y, M, N, K);
     if (rc) return rc;
     /* waves == 128 selects the dense family (any format): the whole matrix is dequantized to fp16 fragments in
-     * the stream's workspace (psn_prefill_<fmt>_unpack), then psn_prefill_dense_f16 multiplies 256 x 256 tiles */
+     * the stream's workspace (psn_prefill_<fmt>_unpack), then psn_prefill_dense_f16(_m128) multiplies 256 x 256 or
+     * 128 x 256 tiles */
     if (waves == 128) {
-        if (bm != 256 || bn != 256) return fail(PSN_E_UNSUPPORTED, "prefill: the dense kernel has a 256x256 tile");
+        if ((bm != 256 && bm != 128) || bn != 256) return fail(PSN_E_UNSUPPORTED, "prefill: the dense kernels have 256x256 and 128x256 tiles");
         if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
         if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
         if ((rc = bind(mod->ctx))) return rc;
@@ -1460,7 +1469,7 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
         if ((rc = is_capturing(s, &cap))) return rc;
         if (cap) s->ws_in_capture = true;
         if ((rc = launch_unpack(mod, s, qtype, W->p, s->ws, N, K))) return rc;
-        return launch_dense(mod, s, s->ws, X, Y, M, N, K, ksplit);
+        return launch_dense(mod, s, s->ws, X, Y, M, N, K, bm, ksplit);
     }
     if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !(waves == 16 && bm == 128 && bn == 256 && qtype != PSN_Q6_K))
         return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family%s", fmt_name(qtype),

@@ -1149,9 +1149,11 @@ PSN_DEV void prefill_wide_body(const psn_prefill_args &a) {
  * feeds the MFMA -- in the order the multiply kernel consumes them: fragment (32-row block nb, 16-wide K
  * slice ks) is 1 KB, lane (h = lane >> 5, n = lane & 31) holding W[32 nb + n][16 ks + 8 h .. + 7], i.e.
  * exactly one B operand of v_mfma_f32_32x32x16_f16.  psn_prefill_dense_f16 (256 x 256 tile, four waves,
- * each all 256 rows x 64 columns as in the wide kernel) then fetches its weight fragments with plain
+ * each all 256 rows x 64 columns as in the wide kernel) and psn_prefill_dense_f16_m128 (128 x 256 tile: half the
+ * rows and accumulators per wave, twice the workgroups -- shapes whose 256-row tiles leave compute units idle or
+ * end on a mostly empty round) then fetch their weight fragments with plain
  * 16-byte loads straight into registers, four 32-wide K stages ahead, so that LDS carries only X: a
- * stage of X is 256 rows of 64 bytes, the four 16-byte pieces of a row stored at piece ^ ((row >> 2) & 3)
+ * stage of X is 256 (128) rows of 64 bytes, the four 16-byte pieces of a row stored at piece ^ ((row >> 2) & 3)
  * (conflict-free fragment reads), filled by direct-to-LDS loads into a ring of four slots; one barrier
  * per stage, placed between the stage's two K slices so that both batches of fragment reads hide under
  * sixteen MFMAs.
@@ -1176,11 +1178,13 @@ PSN_DEV void prefill_unpack_body(const psn_unpack_args &a) {
     put(pf_int<4>()); put(pf_int<5>()); put(pf_int<6>()); put(pf_int<7>());
 }
 
-PSN_DEV void prefill_dense_body(const psn_prefill_args &a) {
-    constexpr int BM = 256, BN = 256, TM = 8, TN = 2, NS = 4;
+template <int TM> PSN_DEV void prefill_dense_body(const psn_prefill_args &a) {
+    static_assert(TM == 4 || TM == 8, "128 or 256 rows of X per workgroup");
+    constexpr int BM = 32 * TM, BN = 256, TN = 2, NS = 4;
     constexpr int KS = 32;                                   /* k per stage */
-    constexpr int XB = BM * KS * 2;                          /* bytes of X per stage: 16 KB */
-    constexpr int NL = 4 + 2 * TN;                           /* loads per wave and stage: 4 of X, 4 of W */
+    constexpr int XB = BM * KS * 2;                          /* bytes of X per stage: 8 or 16 KB */
+    constexpr int XL = XB / 4096;                            /* X loads per wave and stage: 2 or 4 */
+    constexpr int NL = XL + 2 * TN;                          /* loads per wave and stage: those of X and 4 of W */
     extern __shared__ uint4 psn_smem[];
     typedef __attribute__((address_space(3))) char lds_char;
     lds_char *const lds_ptr = (lds_char *)psn_smem;
@@ -1204,12 +1208,12 @@ PSN_DEV void prefill_dense_body(const psn_prefill_args &a) {
     float16_t acc[TM][TN];
     UNROLL for (int i = 0; i < TM; ++i) UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    /* X: load instruction u of wave w fills LDS bytes [(4 w + u) * 1024, + 1024) of the stage's slot; the
+    /* X: load instruction u of wave w fills LDS bytes [(XL w + u) * 1024, + 1024) of the stage's slot; the
      * lane picks the global piece that belongs at its LDS position.  Stages past the end of the K range
      * repeat its last one (into slots nothing reads any more), so every stage issues the same loads. */
-    u32 xoff_g[4];
-    UNROLL for (int u = 0; u < 4; ++u) {
-        const int s_ = (wave * 4 + u) * 64 + lane, row = s_ >> 2, piece = (s_ & 3) ^ ((row >> 2) & 3);
+    u32 xoff_g[XL];
+    UNROLL for (int u = 0; u < XL; ++u) {
+        const int s_ = (wave * XL + u) * 64 + lane, row = s_ >> 2, piece = (s_ & 3) ^ ((row >> 2) & 3);
         xoff_g[u] = (u32)min(m0 + row, M - 1) * (u32)(K * 2) + (u32)(piece * 16);
     }
     const int KF = K >> 4;                                   /* fragments per 32-row block */
@@ -1220,8 +1224,8 @@ PSN_DEV void prefill_dense_body(const psn_prefill_args &a) {
         const int gg = g_base + min(g, nsteps - 1), slot = g % NS;
         const char *xb = reinterpret_cast<const char *>(a.X) + (int64_t)gg * (KS * 2);
         lds_char *xd = lds_ptr + slot * XB;
-        UNROLL for (int u = 0; u < 4; ++u)
-            __builtin_amdgcn_global_load_lds((const void *)(xb + xoff_g[u]), (__attribute__((address_space(3))) void *)(xd + (wave * 4 + u) * 1024), 16, 0, 0);
+        UNROLL for (int u = 0; u < XL; ++u)
+            __builtin_amdgcn_global_load_lds((const void *)(xb + xoff_g[u]), (__attribute__((address_space(3))) void *)(xd + (wave * XL + u) * 1024), 16, 0, 0);
     };
     auto issue_b = [&](int g, u32x4 (&dst)[2][TN]) {
         const int gg = g_base + min(g, nsteps - 1);
@@ -1236,10 +1240,12 @@ PSN_DEV void prefill_dense_body(const psn_prefill_args &a) {
         af[1] = lds_read128<2048>(ab);
         af[2] = lds_read128<4096>(ab);
         af[3] = lds_read128<6144>(ab);
-        af[4] = lds_read128<8192>(ab);
-        af[5] = lds_read128<10240>(ab);
-        af[6] = lds_read128<12288>(ab);
-        af[7] = lds_read128<14336>(ab);
+        if constexpr (TM == 8) {
+            af[4] = lds_read128<8192>(ab);
+            af[5] = lds_read128<10240>(ab);
+            af[6] = lds_read128<12288>(ab);
+            af[7] = lds_read128<14336>(ab);
+        }
     };
     auto mfmas = [&](const u32x4 (&af)[TM], const u32x4 (&bf)[TN]) {
         UNROLL for (int j = 0; j < TN; ++j) UNROLL for (int i = 0; i < TM; ++i)
@@ -1361,7 +1367,8 @@ PSN_PREFILL_FAMILY_BASE(q8_0, PfQ8_0)
 #endif
 #endif
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 5
-extern "C" __global__ void __launch_bounds__(256) psn_prefill_dense_f16(const psn_prefill_args a) { prefill_dense_body(a); }
+extern "C" __global__ void __launch_bounds__(256) psn_prefill_dense_f16(const psn_prefill_args a) { prefill_dense_body<8>(a); }
+extern "C" __global__ void __launch_bounds__(256) psn_prefill_dense_f16_m128(const psn_prefill_args a) { prefill_dense_body<4>(a); }
 #define PSN_PREFILL_KERNEL_UNPACK(fmt, WF) \
     extern "C" __global__ void __launch_bounds__(256) psn_prefill_##fmt##_unpack(const psn_unpack_args a) { prefill_unpack_body<WF>(a); }
 PSN_PREFILL_KERNEL_UNPACK(q4_0, PfQ4_0)

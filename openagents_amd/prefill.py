@@ -38,7 +38,7 @@ EXPLICIT_PLANS = [(64, 64, 2, 4), (64, 64, 4, 4), (64, 64, 8, 4), (64, 128, 2, 4
                   (128, 128, 1, 4), (256, 128, 1, 4), (256, 256, 1, 4), (256, 256, 2, 4), (256, 256, 4, 4),
                   (128, 128, 1, 16), (128, 128, 2, 16), (128, 128, 4, 16), (128, 128, 8, 16),
                   (128, 256, 1, 16), (128, 256, 2, 16), (128, 256, 4, 16), (128, 256, 8, 16),
-                  (256, 256, 1, 32), (256, 256, 2, 32), (256, 256, 4, 32), (256, 256, 1, 128), (256, 256, 2, 128), (256, 256, 4, 128)]
+                  (256, 256, 1, 32), (256, 256, 2, 32), (256, 256, 4, 32), (256, 256, 1, 128), (256, 256, 2, 128), (256, 256, 4, 128), (128, 256, 1, 128), (128, 256, 2, 128), (128, 256, 4, 128)]
 MFMA_PEAK_TFLOPS = 2500.0
 MFMA_PEAK_CLOCK_MHZ = 2400.0
 HBM_PEAK_GBS = 8000.0
@@ -154,7 +154,7 @@ def main(argv=None):
                         sustained["frac_of_mfma_rate_at_that_clock"] = round(flops / sus_us / 1e6 / (MFMA_PEAK_TFLOPS * mhz / MFMA_PEAK_CLOCK_MHZ), 4)
                 print(json.dumps({"op": "quantized prefill matmul", "format": fname, "M": m, "N": n, "K": k, "us": round(us, 1),
                                   "TFLOPs": round(tflops, 1), "GBps": round(gbs, 1), "bound": bound, "frac_of_roofline": round(frac, 4),
-                                  "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide", 128: f"psn_prefill_{fname}_unpack + psn_prefill_dense_f16"}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),
+                                  "kernel": {64: f"psn_prefill_{fname}_skinny", 32: f"psn_prefill_{fname}_wide", 128: f"psn_prefill_{fname}_unpack + psn_prefill_dense_f16" + ("_m128" if tm == 128 else "")}.get(wv, f"psn_prefill_{fname}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, "")),
                                   "ksplit": sp, "iters": args.iters, **sustained, **compared}), flush=True)
             for w in ws:
                 w.buf.free()

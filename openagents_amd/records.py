@@ -178,7 +178,7 @@ def config3(be: HipBackend, samples: int = 9, seed: int = 31, weights=None) -> l
 
 def prefill_kernel_name(fmt: str, m: int, n: int, k: int, cus: int, qtype: int | None = None):
     tm, tn, sp, wv = prefill_plan(m, n, k, cus, qtype)
-    name = {64: f"psn_prefill_{fmt}_skinny", 32: f"psn_prefill_{fmt}_wide", 128: f"psn_prefill_{fmt}_unpack + psn_prefill_dense_f16"}.get(wv, f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, ""))
+    name = {64: f"psn_prefill_{fmt}_skinny", 32: f"psn_prefill_{fmt}_wide", 128: f"psn_prefill_{fmt}_unpack + psn_prefill_dense_f16" + ("_m128" if tm == 128 else "")}.get(wv, f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, ""))
     return name, sp
 
 

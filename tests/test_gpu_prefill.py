@@ -253,9 +253,9 @@ def test_prefill_default_plans_over_seeded_random_shapes(hip, orc):
 @pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_dense_family_ragged_shapes(hip, orc, qname):
     """Family 128: the matrix is rewritten as fp16 fragments once (psn_prefill_<fmt>_unpack), then multiplied
-    on 256 x 256 tiles.  Ragged m and n against the tile and against the 32-row fragment blocks, one to
-    sixteen chunks of K, every K split the shape allows; the fp16 values are those of the other families,
-    so the same tolerance holds."""
+    on 256 x 256 or 128 x 256 tiles.  Ragged m and n against the tiles and against the 32-row fragment blocks,
+    one to sixteen chunks of K, every K split the shape allows; the fp16 values are those of the other
+    families, so the same tolerance holds."""
     t = getattr(orc, qname)
     for m, n, k in ((1, 40, 256), (37, 300, 1280), (260, 700, 2048), (333, 516, 1024), (257, 256, 512), (520, 33, 4096)):
         W = weights(orc, qname, 820, n, k)
@@ -264,12 +264,13 @@ def test_dense_family_ragged_shapes(hip, orc, qname):
         for ksplit in (1, 2, 4):
             if ksplit > 1 and ((m * n) % 4 or k // 256 < ksplit):
                 continue
-            say(f"dense prefill {qname} m={m} n={n} k={k} ksplit={ksplit}")
-            y = hip.matmul_host(t, W, X, n, k, (256, 256, ksplit, 128))
-            err = G.max_rel_err(y, ref)
-            assert np.all(np.isfinite(y)) and err < PARITY_TOL, (qname, ksplit, m, n, k, err)
+            for bm in (256, 128):
+                say(f"dense prefill {qname} m={m} n={n} k={k} rows per tile={bm} ksplit={ksplit}")
+                y = hip.matmul_host(t, W, X, n, k, (bm, 256, ksplit, 128))
+                err = G.max_rel_err(y, ref)
+                assert np.all(np.isfinite(y)) and err < PARITY_TOL, (qname, bm, ksplit, m, n, k, err)
     with pytest.raises(backend.PsnError) as e:
-        hip.matmul_host(t, W, X, n, k, (128, 256, 1, 128))                      # the dense kernel has one tile
+        hip.matmul_host(t, W, X, n, k, (128, 128, 1, 128))                      # the dense kernels' tiles are 256 columns wide
     assert e.value.name == "PSN_E_UNSUPPORTED"
 
 
