@@ -222,7 +222,7 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
                         pk.free()
                     packed_extra = {"timing_packed_weights": {**sp_, "TFLOPs": round(flops / sp_["median_us"] / 1e6, 1),
                                                               "frac_of_mfma_peak": round(flops / sp_["median_us"] / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
-                                                              "kernelRef": "psn_prefill_dense_f16",
+                                                              "kernelRef": "psn_prefill_dense_f16 or psn_prefill_dense_f16_m128 (by shape)",
                                                               "note": "weights dequantized to fp16 fragments once beforehand (psn_prefill_pack, 2 bytes per weight resident)"}}
                 out.append(record(be, f"prefill.{fmt}.{k}x{n}.m{m}", kname, digest, m * 1e6 / t_us,
                                   shape={"M": m, "N": n, "K": k, "format": fmt, "ksplit": sp}, timing=st,
