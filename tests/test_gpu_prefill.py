@@ -329,7 +329,7 @@ def test_packed_weights_multiply_like_the_dense_family(hip, orc, qname):
     w = hip.upload_weight(t, W, n, k)
     packed = hip.pack_for_prefill(w)
     assert packed.nbytes >= 768 * k * 2
-    for m in (1, 260, 37):
+    for m in (1, 260, 37, 384, 1100):                                                    # heights served by either tile of the multiply
         X = G.seeded_acts(841 + m, m, k).astype(np.float16)
         y = hip.alloc(m * n * 4)
         hip.quantized_matmul_packed(packed, hip.upload(X), y, m, n, k)
