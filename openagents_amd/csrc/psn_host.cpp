@@ -1273,7 +1273,8 @@ static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int3
         const int64_t mt = (M + bm - 1) / bm, nt = (N + bn - 1) / bn;
         const int64_t slots = (int64_t)cus * k_prefill_wgs_per_cu[i];
         for (int sp = 1; sp <= 8; sp *= 2) {
-            if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 4 * sp)) continue;
+            if (sp > 1 && ((M * N) % 4 != 0 || K / 256 < 2 * sp)) continue;
+            const bool short_range = sp > 1 && K / 256 < 4 * sp;    /* two or three chunks per range: the producer / consumer kernels only */
             const int64_t wgs = mt * nt * sp;
             const int64_t rounds = (wgs + slots - 1) / slots;
             const double steps = (double)(K / 64) / sp;
@@ -1282,9 +1283,9 @@ static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int3
             const int64_t resident = ((wgs < slots ? wgs : slots) + cus - 1) / cus;
             double t = (double)rounds * steps * k_prefill_step_us[i] * (1.0 + 0.225 * (double)(resident - 1)) + 5.0;
             if (sp > 1) t += ksplit_overhead_us(M, N, sp, i == 5 ? 4 : 8);
-            if (t < best) { best = t; bi = i; bs = sp; *waves = 4; }
+            if (!short_range && t < best) { best = t; bi = i; bs = sp; *waves = 4; }
             for (const auto &v : k_prefill_alt) {
-                if (v.tile != i) continue;
+                if (v.tile != i || (short_range && v.waves != 16)) continue;
                 const int64_t sl = (int64_t)cus * v.per_cu;
                 const int64_t r8 = (wgs + sl - 1) / sl;
                 double t8 = (double)r8 * (steps + v.fill) * v.step_us + 5.0;
