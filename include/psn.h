@@ -98,6 +98,9 @@ int32_t psn_ctx_create(int32_t device, psn_ctx **out);
 int32_t psn_ctx_destroy(psn_ctx *ctx);
 /* device facts: compute units, bytes of device memory, arch name copied into name[0..n) */
 int32_t psn_ctx_info(psn_ctx *ctx, int32_t *compute_units, int64_t *total_mem, char *name, size_t n);
+/* free and total bytes of device memory right now (hipMemGetInfo; either pointer may be NULL): what a caller
+ * compares before and after a call to see that it allocated nothing */
+int32_t psn_ctx_mem_info(psn_ctx *ctx, int64_t *free_bytes, int64_t *total_bytes);
 
 /* load a gfx950 code object from memory / the one built into the library */
 int32_t psn_module_load(psn_ctx *ctx, const void *code_object, size_t len, psn_module **out);
@@ -108,7 +111,17 @@ int32_t psn_module_has_kernel(psn_module *mod, const char *kernel_name);
 
 int32_t psn_stream_create(psn_ctx *ctx, psn_stream **out);
 int32_t psn_stream_sync(psn_stream *s);
+/* Destroys the stream.  Its workspace (psn_stream_reserve, psn_prefill_reserve) is freed with it unless
+ * captured graphs still hold the workspace's address: then the memory stays alive until the last such graph
+ * is destroyed, so those graphs remain launchable on other streams. */
 int32_t psn_stream_destroy(psn_stream *s);
+
+/* The names of the distinct kernels this thread has launched since psn_launch_log_clear(), in order of first
+ * launch, each followed by ';' (a thread-local buffer of 1 KB; when it is full the log ends in "...;").  Throughput
+ * records cite it as the kernel that actually ran (the `kernelRef` of the reference's KernelThroughputRecord,
+ * /root/reference/packages/tassadar-executor/src/kernel-optimization-parity.ts:27-59). */
+const char *psn_launch_log(void);
+void psn_launch_log_clear(void);
 
 /* Stream capture into a replayable graph (hipGraph): everything launched on `s` between begin and
  * end is recorded instead of run; psn_graph_launch replays it on a stream.  Calls that would have
@@ -129,6 +142,9 @@ int32_t psn_stream_wait_stream(psn_stream *waiter, psn_stream *signaler);
  * a larger one fail with PSN_E_INVALID_ARG; destroying the graphs lifts this), so reserve the largest
  * K x batch before the first capture. */
 int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch);
+/* The workspace belongs to the stream it was reserved on, also inside a capture: a launch on a side stream
+ * that was forked into a capture (psn_stream_wait_stream) uses -- and pins -- the side stream's workspace, and
+ * the graph that the capture's origin stream ends holds every workspace the capture touched. */
 
 int32_t psn_event_create(psn_ctx *ctx, psn_event **out);
 int32_t psn_event_destroy(psn_event *e);
@@ -199,7 +215,9 @@ int32_t psn_qmatvec_q8_multi(psn_module *mod, psn_stream *s, int32_t qtype, int3
 /* psn_qmatvec for callers that cannot allocate device memory (code under graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  This entry point has no counterpart in the reference: it exists
  * for those callers only.  Same arguments and results as psn_qmatvec, but nothing is allocated or freed,
- * on the device or through any allocating library routine: with scheme Q8 the quantized activations go
+ * on the device or through any allocating library routine (the first launch of a kernel name on a module
+ * looks the kernel up and remembers it in a host-side table; later calls do no host allocation either):
+ * with scheme Q8 the quantized activations go
  * into a static array in the library's device image (psn_noalloc_max_bytes() bytes per GPU, held until
  * the process ends) instead of the stream's workspace.  Shapes whose quantized activations
  * (psn_actq_layout(...).bytes) exceed that size fail with PSN_E_SHAPE.  Every call on a GPU shares that
@@ -341,7 +359,8 @@ int32_t psn_swiglu_q8(psn_module *mod, psn_stream *s, const psn_buf *gate, const
  * workgroup 0 also stores h to h_out (may be NULL), which must not alias x or delta -- a decoder
  * alternates two residual buffers.  Shapes the fused kernels do not serve (rows longer than 8192, more
  * than three matrices, row counts that are not whole passes) run the norm kernel and the pre-quantized
- * matvec as two launches with the same result.  No counterpart in the reference's CPU path, which
+ * matvec as two launches with the same result.  x and delta are never written on either path: h goes to
+ * h_out or nowhere, so several calls (one per weight format among q|k|v) may share x and delta.  No counterpart in the reference's CPU path, which
  * normalizes, quantizes and multiplies as separate steps; the arithmetic per element is the same. */
 int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t count,
                                const psn_buf *const *W, const psn_buf *x, const psn_buf *delta, const psn_buf *norm_weight,

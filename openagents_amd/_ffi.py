@@ -48,6 +48,9 @@ SIGNATURES = {
     "psn_ctx_create": (_i32, [_i32, _pp]),
     "psn_ctx_destroy": (_i32, [_vp]),
     "psn_ctx_info": (_i32, [_vp, C.POINTER(_i32), C.POINTER(_i64), C.c_char_p, _sz]),
+    "psn_ctx_mem_info": (_i32, [_vp, C.POINTER(_i64), C.POINTER(_i64)]),
+    "psn_launch_log": (C.c_char_p, []),
+    "psn_launch_log_clear": (None, []),
     "psn_module_load": (_i32, [_vp, _vp, _sz, _pp]),
     "psn_module_load_builtin": (_i32, [_vp, _pp]),
     "psn_module_unload": (_i32, [_vp]),

@@ -105,6 +105,8 @@ struct psn_norm_args {
     float eps;
     struct psn_actq_out qout;
     float *x_out;         /* when set, x + delta goes here and x is left alone */
+    int32_t keep_x;       /* nonzero: x + delta is stored nowhere unless x_out is set (x is never written) */
+    int32_t pad1;
 };
 struct psn_rope_args {
     float *q;             /* [n_heads][head_dim], rotated in place */

@@ -52,7 +52,7 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
     const int n4 = a.n >> 2, nt = blockDim.x;
     const float4 *x4 = reinterpret_cast<const float4 *>(a.x);
     float4 *xo4 = reinterpret_cast<float4 *>(a.x_out ? a.x_out : a.x);      /* where x + delta goes */
-    const bool store_sum = a.delta != nullptr || a.x_out != nullptr;
+    const bool store_sum = a.x_out != nullptr || (a.delta != nullptr && !a.keep_x);
     const float4 *d4 = reinterpret_cast<const float4 *>(a.delta);
     const float4 *w4 = reinterpret_cast<const float4 *>(a.weight);
     float4 *y4 = reinterpret_cast<float4 *>(a.y);
@@ -100,7 +100,12 @@ extern "C" __global__ void __launch_bounds__(1024) psn_add_rmsnorm(const psn_nor
         }
     } else {
         for (int i = threadIdx.x; i < n4; i += nt) {
-            const float4 t = store_sum ? xo4[i] : x4[i], ww = w4[i];
+            float4 t = store_sum ? xo4[i] : x4[i];
+            const float4 ww = w4[i];
+            if (!store_sum && d4) {                    /* the sum was not stored: add the delta again */
+                const float4 d = d4[i];
+                t.x += d.x; t.y += d.y; t.z += d.z; t.w += d.w;
+            }
             const float4 o = make_float4(t.x * scale * ww.x, t.y * scale * ww.y, t.z * scale * ww.z, t.w * scale * ww.w);
             if (y4) y4[i] = o;
             if (a.qout.qs) quantize_out4(a.qout, i, o);

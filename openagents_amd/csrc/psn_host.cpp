@@ -14,11 +14,14 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <map>
+#include <memory>
 #include <mutex>
+#include <exception>
 #include <new>
 #include <string>
+#include <string_view>
 #include <unordered_map>
-#include <memory>
 #include <vector>
 
 /* code objects linked into the library (generated table, see build.py) */
@@ -107,8 +110,16 @@ extern "C" int32_t psn_quantize_rows(int32_t qtype, const float *x, int64_t n, i
     if ((uint64_t)n * (uint64_t)rb > out_bytes)
         return fail(PSN_E_INVALID_ARG, "psn_quantize_rows: output holds %zu bytes, %lld rows of %lld bytes need %lld", out_bytes,
                     (long long)n, (long long)rb, (long long)(n * rb));
-    if (psn_quantize_rows_impl(qtype, x, n, k, static_cast<uint8_t *>(out), rb, threads < 1 ? 1 : threads) != 0)
-        return fail(PSN_E_UNSUPPORTED, "psn_quantize_rows: type %d has no quantizer", qtype);
+    /* more threads than 256 help nobody; thread creation or allocation failures must not unwind through the C boundary */
+    const int32_t nthreads = threads < 1 ? 1 : threads > 256 ? 256 : threads;
+    try {
+        if (psn_quantize_rows_impl(qtype, x, n, k, static_cast<uint8_t *>(out), rb, nthreads) != 0)
+            return fail(PSN_E_UNSUPPORTED, "psn_quantize_rows: type %d has no quantizer", qtype);
+    } catch (const std::bad_alloc &) {
+        return fail(PSN_E_OOM, "psn_quantize_rows: host allocation failed");
+    } catch (const std::exception &e) {
+        return fail(PSN_E_INVALID_ARG, "psn_quantize_rows: %s (threads=%d)", e.what(), nthreads);
+    }
     return PSN_OK;
 }
 
@@ -171,13 +182,22 @@ struct psn_ctx {
     int max_lds;
     char arch[64];
 };
+/* A stream's workspace (quantized activations of psn_qmatvec, the dense prefill family's fp16 matrix).  Graph
+ * nodes bake its address in, so the memory is owned jointly by the stream and by every graph recorded from a
+ * launch that used it: it neither moves nor is freed while such a graph, or a capture that may become one,
+ * exists.  Whoever lets go last (stream destroyed, last graph destroyed) frees it. */
+struct ws_state {
+    void *p = nullptr;
+    size_t bytes = 0;
+    int graph_refs = 0;    /* live graphs whose nodes hold p */
+    int capture_refs = 0;  /* captures in progress that have recorded a node holding p */
+    bool orphaned = false; /* the owning stream is gone; the last graph frees p */
+    int device = 0;
+};
 struct psn_stream {
     psn_ctx *ctx;
     hipStream_t s;
-    void *ws;          /* activation workspace of psn_qmatvec (scheme Q8) */
-    size_t ws_bytes;
-    bool ws_in_capture;                 /* the capture in progress has baked the address of ws into a node */
-    std::shared_ptr<int> ws_graph_refs; /* live graphs that hold the address of ws: it must not move while any exists */
+    std::shared_ptr<ws_state> ws;
     hipEvent_t join_ev; /* created on first use by psn_stream_wait_stream */
 };
 struct psn_buf {
@@ -193,14 +213,20 @@ struct psn_graph {
     psn_ctx *ctx;
     hipGraph_t g;
     hipGraphExec_t exec;
-    std::shared_ptr<int> ws_refs;       /* set when the graph holds the address of its stream's workspace */
+    std::vector<std::shared_ptr<ws_state>> ws_held;   /* workspaces (of any stream that took part in the capture) whose address the nodes hold */
 };
 struct psn_module {
     psn_ctx *ctx;
     std::vector<hipModule_t> m;   /* one per code object; kernels are looked up across all */
     std::mutex mu;
-    std::unordered_map<std::string, hipFunction_t> fn;
+    std::map<std::string, hipFunction_t, std::less<>> fn;   /* transparent comparator: a lookup by C string builds no std::string */
 };
+
+/* Workspaces touched by captures in progress, keyed by the capture's id (every stream that has joined a capture
+ * reports the same id), so that psn_graph_end_capture on the origin stream also finds the workspaces of forked
+ * side streams. */
+static std::mutex g_cap_mu;
+static std::unordered_map<unsigned long long, std::vector<std::shared_ptr<ws_state>>> g_cap_touched;
 
 static int32_t bind(psn_ctx *c) {
     if (!c) return fail(PSN_E_INVALID_ARG, "context is null");
@@ -240,6 +266,16 @@ extern "C" int32_t psn_ctx_info(psn_ctx *c, int32_t *cus, int64_t *mem, char *na
     if (cus) *cus = c->compute_units;
     if (mem) *mem = c->total_mem;
     if (name && n) snprintf(name, n, "%s", c->arch);
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_ctx_mem_info(psn_ctx *c, int64_t *free_bytes, int64_t *total_bytes) {
+    int32_t rc = bind(c);
+    if (rc) return rc;
+    size_t f = 0, t = 0;
+    HIP_TRY(hipMemGetInfo(&f, &t));
+    if (free_bytes) *free_bytes = (int64_t)f;
+    if (total_bytes) *total_bytes = (int64_t)t;
     return PSN_OK;
 }
 
@@ -301,7 +337,7 @@ extern "C" int32_t psn_module_unload(psn_module *mod) {
 }
 static int32_t get_fn(psn_module *mod, const char *name, hipFunction_t *out) {
     std::lock_guard<std::mutex> lk(mod->mu);
-    auto it = mod->fn.find(name);
+    auto it = mod->fn.find(std::string_view(name));
     if (it != mod->fn.end()) { *out = it->second; return PSN_OK; }
     hipFunction_t f = nullptr;
     hipError_t e = hipErrorNotFound;
@@ -310,7 +346,7 @@ static int32_t get_fn(psn_module *mod, const char *name, hipFunction_t *out) {
         if (e == hipSuccess) break;
     }
     if (e != hipSuccess) return fail(PSN_E_MODULE, "kernel '%s' not found in module: hipError %d (%s)", name, (int)e, hipGetErrorString(e));
-    mod->fn.emplace(name, f);
+    mod->fn.emplace(std::string(name), f);
     *out = f;
     return PSN_OK;
 }
@@ -333,10 +369,8 @@ extern "C" int32_t psn_stream_create(psn_ctx *c, psn_stream **out) {
     if (!st) { (void)hipStreamDestroy(s); return fail(PSN_E_OOM, "host allocation failed"); }
     st->ctx = c;
     st->s = s;
-    st->ws = nullptr;
-    st->ws_bytes = 0;
-    st->ws_in_capture = false;
-    st->ws_graph_refs = std::make_shared<int>(0);
+    st->ws = std::make_shared<ws_state>();
+    st->ws->device = c->device;
     st->join_ev = nullptr;
     *out = st;
     return PSN_OK;
@@ -353,7 +387,16 @@ extern "C" int32_t psn_stream_destroy(psn_stream *s) {
     int32_t rc = bind(s->ctx);
     if (rc) return rc;
     (void)hipStreamSynchronize(s->s);
-    if (s->ws) (void)hipFree(s->ws);
+    {
+        std::lock_guard<std::mutex> lk(g_cap_mu);
+        if (s->ws->graph_refs > 0 || s->ws->capture_refs > 0) {
+            s->ws->orphaned = true;                       /* graphs still hold the address: the last of them frees it */
+        } else if (s->ws->p) {
+            (void)hipFree(s->ws->p);
+            s->ws->p = nullptr;
+            s->ws->bytes = 0;
+        }
+    }
     if (s->join_ev) (void)hipEventDestroy(s->join_ev);
     hipError_t e = hipStreamDestroy(s->s);
     delete s;
@@ -375,23 +418,43 @@ static int32_t refuse_while_capturing(psn_stream *s, const char *what) {
     return PSN_OK;
 }
 static int32_t ensure_workspace(psn_stream *s, int64_t bytes) {
-    if (s->ws_bytes >= (size_t)bytes) return PSN_OK;
+    ws_state &w = *s->ws;
+    if (w.bytes >= (size_t)bytes) return PSN_OK;
     bool cap = false;
     int32_t rc = is_capturing(s, &cap);
     if (rc) return rc;
     if (cap) return fail(PSN_E_INVALID_ARG, "activation workspace must grow to %lld bytes during capture: call psn_stream_reserve first", (long long)bytes);
-    if (s->ws_in_capture || *s->ws_graph_refs > 0)
-        return fail(PSN_E_INVALID_ARG, "activation workspace (%zu bytes) is referenced by a captured graph and cannot grow to %lld bytes: "
-                    "reserve the largest K x batch with psn_stream_reserve before the first capture", s->ws_bytes, (long long)bytes);
+    {
+        std::lock_guard<std::mutex> lk(g_cap_mu);
+        if (w.capture_refs > 0 || w.graph_refs > 0)
+            return fail(PSN_E_INVALID_ARG, "activation workspace (%zu bytes) is referenced by a captured graph and cannot grow to %lld bytes: "
+                        "reserve the largest K x batch with psn_stream_reserve before the first capture", w.bytes, (long long)bytes);
+    }
     /* earlier launches may still read the old workspace */
     HIP_TRY(hipStreamSynchronize(s->s));
-    if (s->ws) HIP_TRY(hipFree(s->ws));
-    s->ws = nullptr;
-    s->ws_bytes = 0;
+    if (w.p) HIP_TRY(hipFree(w.p));
+    w.p = nullptr;
+    w.bytes = 0;
     const size_t want = (size_t)align_up(bytes, 1 << 20);
-    hipError_t e = hipMalloc(&s->ws, want);
+    hipError_t e = hipMalloc(&w.p, want);
     if (e != hipSuccess) return hip_fail(e, "hipMalloc(workspace)");
-    s->ws_bytes = want;
+    w.bytes = want;
+    return PSN_OK;
+}
+/* Called by every launch path that hands the workspace address to a kernel: if the stream is being captured
+ * (as the origin of the capture or as a side stream forked into it), the capture is noted as holding the
+ * workspace, whichever stream later ends it. */
+static int32_t note_workspace_use(psn_stream *s) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    HIP_TRY(hipStreamGetCaptureInfo(s->s, &st, &id));
+    if (st == hipStreamCaptureStatusNone) return PSN_OK;
+    std::lock_guard<std::mutex> lk(g_cap_mu);
+    auto &v = g_cap_touched[id];
+    for (const auto &w : v)
+        if (w == s->ws) return PSN_OK;
+    v.push_back(s->ws);
+    ++s->ws->capture_refs;
     return PSN_OK;
 }
 extern "C" int32_t psn_stream_reserve(psn_stream *s, int64_t K, int32_t batch) {
@@ -421,7 +484,6 @@ extern "C" int32_t psn_graph_begin_capture(psn_stream *s) {
     int32_t rc = bind(s->ctx);
     if (rc) return rc;
     HIP_TRY(hipStreamBeginCapture(s->s, hipStreamCaptureModeThreadLocal));
-    s->ws_in_capture = false;
     return PSN_OK;
 }
 extern "C" int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out) {
@@ -430,22 +492,41 @@ extern "C" int32_t psn_graph_end_capture(psn_stream *s, psn_graph **out) {
     int32_t rc = bind(s->ctx);
     if (rc) return rc;
     hipGraph_t g = nullptr;
-    const bool holds_ws = s->ws_in_capture;
-    s->ws_in_capture = false;
-    HIP_TRY(hipStreamEndCapture(s->s, &g));
-    if (!g) return fail(PSN_E_HIP, "hipStreamEndCapture returned no graph (capture was invalidated)");
+    /* the workspaces this capture touched, on this stream or on side streams forked into it */
+    std::vector<std::shared_ptr<ws_state>> held;
+    {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        unsigned long long id = 0;
+        if (hipStreamGetCaptureInfo(s->s, &st, &id) == hipSuccess && st != hipStreamCaptureStatusNone) {
+            std::lock_guard<std::mutex> lk(g_cap_mu);
+            auto it = g_cap_touched.find(id);
+            if (it != g_cap_touched.end()) {
+                held.swap(it->second);
+                g_cap_touched.erase(it);
+            }
+        }
+    }
+    auto release_capture_refs = [&](bool to_graph) {
+        std::lock_guard<std::mutex> lk(g_cap_mu);
+        for (auto &w : held) {
+            --w->capture_refs;
+            if (to_graph) ++w->graph_refs;
+            else if (w->orphaned && w->graph_refs == 0 && w->capture_refs == 0 && w->p) { (void)hipFree(w->p); w->p = nullptr; w->bytes = 0; }
+        }
+    };
+    hipError_t e = hipStreamEndCapture(s->s, &g);
+    if (e != hipSuccess) { release_capture_refs(false); return hip_fail(e, "hipStreamEndCapture"); }
+    if (!g) { release_capture_refs(false); return fail(PSN_E_HIP, "hipStreamEndCapture returned no graph (capture was invalidated)"); }
     hipGraphExec_t ex = nullptr;
-    hipError_t e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
-    if (e != hipSuccess) { (void)hipGraphDestroy(g); return hip_fail(e, "hipGraphInstantiate"); }
+    e = hipGraphInstantiate(&ex, g, nullptr, nullptr, 0);
+    if (e != hipSuccess) { (void)hipGraphDestroy(g); release_capture_refs(false); return hip_fail(e, "hipGraphInstantiate"); }
     psn_graph *gr = new (std::nothrow) psn_graph();
-    if (!gr) { (void)hipGraphExecDestroy(ex); (void)hipGraphDestroy(g); return fail(PSN_E_OOM, "host allocation failed"); }
+    if (!gr) { (void)hipGraphExecDestroy(ex); (void)hipGraphDestroy(g); release_capture_refs(false); return fail(PSN_E_OOM, "host allocation failed"); }
     gr->ctx = s->ctx;
     gr->g = g;
     gr->exec = ex;
-    if (holds_ws) {
-        gr->ws_refs = s->ws_graph_refs;
-        ++*gr->ws_refs;
-    }
+    release_capture_refs(true);
+    gr->ws_held.swap(held);
     *out = gr;
     return PSN_OK;
 }
@@ -463,7 +544,14 @@ extern "C" int32_t psn_graph_destroy(psn_graph *g) {
     if (rc) return rc;
     (void)hipGraphExecDestroy(g->exec);
     (void)hipGraphDestroy(g->g);
-    if (g->ws_refs) --*g->ws_refs;
+    {
+        std::lock_guard<std::mutex> lk(g_cap_mu);
+        for (auto &w : g->ws_held) {
+            --w->graph_refs;
+            /* the stream that owned this workspace was destroyed while the graph lived: free it with the last graph */
+            if (w->orphaned && w->graph_refs == 0 && w->capture_refs == 0 && w->p) { (void)hipFree(w->p); w->p = nullptr; w->bytes = 0; }
+        }
+    }
     delete g;
     return PSN_OK;
 }
@@ -614,11 +702,37 @@ extern "C" int32_t psn_weight_upload(psn_ctx *c, int32_t qtype, int64_t N, int64
 
 /* ------------------------------------------------------------------ launches */
 
+/* The distinct kernels this thread has launched since psn_launch_log_clear(), in order of first launch,
+ * "name;name;..." (what a throughput record cites as the kernels that actually ran).  Names that no longer
+ * fit are dropped and the log ends in "...;". */
+static thread_local char g_launch_log[1024] = "";
+static thread_local size_t g_launch_log_len = 0;
+static void log_launch(const char *kernel) {
+    const size_t n = strlen(kernel);
+    for (const char *p = g_launch_log; (p = strstr(p, kernel)) != nullptr; p += n)
+        if ((p == g_launch_log || p[-1] == ';') && p[n] == ';') return;      /* already listed */
+    if (g_launch_log_len + n + 1 + 4 < sizeof g_launch_log) {
+        memcpy(g_launch_log + g_launch_log_len, kernel, n);
+        g_launch_log_len += n;
+        g_launch_log[g_launch_log_len++] = ';';
+        g_launch_log[g_launch_log_len] = 0;
+    } else if (g_launch_log_len + 4 < sizeof g_launch_log && (g_launch_log_len < 4 || memcmp(g_launch_log + g_launch_log_len - 4, "...;", 4) != 0)) {
+        memcpy(g_launch_log + g_launch_log_len, "...;", 5);
+        g_launch_log_len += 4;
+    }
+}
+extern "C" void psn_launch_log_clear(void) {
+    g_launch_log_len = 0;
+    g_launch_log[0] = 0;
+}
+extern "C" const char *psn_launch_log(void) { return g_launch_log; }
+
 static int32_t launch(psn_module *mod, psn_stream *s, const char *kernel, unsigned blocks, unsigned threads, unsigned lds,
                       void *args_struct) {
     hipFunction_t f;
     int32_t rc = get_fn(mod, kernel, &f);
     if (rc) return rc;
+    log_launch(kernel);
     void *params[] = {args_struct};
     hipError_t e = hipModuleLaunchKernel(f, blocks, 1, 1, threads, 1, 1, lds, s->s, params, nullptr);
     if (e != hipSuccess) return fail(PSN_E_HIP, "launch of %s <<<%u,%u,%u>>> failed: hipError %d (%s)", kernel, blocks, threads, lds, (int)e, hipGetErrorString(e));
@@ -1097,11 +1211,9 @@ extern "C" int32_t psn_qmatvec_multi(psn_module *mod, psn_stream *s, int32_t qty
     psn_actq_info li;
     if ((rc = psn_actq_layout(at, K, batch, &li))) return rc;
     if ((rc = ensure_workspace(s, li.bytes))) return rc;
-    bool cap = false;
-    if ((rc = is_capturing(s, &cap))) return rc;
-    if (cap) s->ws_in_capture = true;    /* the graph being recorded bakes the workspace address into its nodes */
-    if ((rc = quantize_into(mod, s, at, (const float *)x->p, s->ws, K, batch))) return rc;
-    return run_matvec(mod, s, qtype, scheme, sg, s->ws, K, batch, &plan);
+    if ((rc = note_workspace_use(s))) return rc;    /* a graph being recorded bakes the workspace address into its nodes */
+    if ((rc = quantize_into(mod, s, at, (const float *)x->p, s->ws->p, K, batch))) return rc;
+    return run_matvec(mod, s, qtype, scheme, sg, s->ws->p, K, batch, &plan);
 }
 
 extern "C" int32_t psn_qmatvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t scheme, const psn_buf *W,
@@ -1466,11 +1578,9 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
         if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
         if ((rc = bind(mod->ctx))) return rc;
         if ((rc = ensure_workspace(s, packed_bytes(N, K)))) return rc;
-        bool cap = false;
-        if ((rc = is_capturing(s, &cap))) return rc;
-        if (cap) s->ws_in_capture = true;
-        if ((rc = launch_unpack(mod, s, qtype, W->p, s->ws, N, K))) return rc;
-        return launch_dense(mod, s, s->ws, X, Y, M, N, K, bm, ksplit);
+        if ((rc = note_workspace_use(s))) return rc;
+        if ((rc = launch_unpack(mod, s, qtype, W->p, s->ws->p, N, K))) return rc;
+        return launch_dense(mod, s, s->ws->p, X, Y, M, N, K, bm, ksplit);
     }
     if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !(waves == 16 && bm == 128 && bn == 256 && qtype != PSN_Q6_K))
         return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family%s", fmt_name(qtype),
@@ -1540,7 +1650,12 @@ extern "C" int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t q
     bool cap = false;
     if ((rc = is_capturing(s, &cap))) return rc;
     const int64_t dense_ws = packed_bytes(N, K);
-    const bool dense_ok = s->ws_bytes >= (size_t)dense_ws || (!cap && *s->ws_graph_refs == 0);
+    bool ws_pinned;
+    {
+        std::lock_guard<std::mutex> lk(g_cap_mu);
+        ws_pinned = s->ws->graph_refs > 0 || s->ws->capture_refs > 0;
+    }
+    const bool dense_ok = s->ws->bytes >= (size_t)dense_ws || (!cap && !ws_pinned);
     if ((rc = prefill_plan_any(qtype, M, N, K, mod->ctx->compute_units, dense_ok, &bm, &bn, &sp, &wv))) return rc;
     return psn_qmatmul_prefill_tiled(mod, s, qtype, W, X, Y, M, N, K, bm, bn, sp, wv);
 }
@@ -1571,8 +1686,10 @@ static int32_t set_actq_out(const char *what, psn_module *mod, psn_buf *yq, int3
 }
 
 static int32_t launch_add_rmsnorm(psn_module *mod, psn_stream *s, float *x, const float *delta, const float *weight, float *y, float *x_out,
-                                  const psn_actq_out &qout, int64_t n, float eps) {
+                                  const psn_actq_out &qout, int64_t n, float eps, bool keep_x = false) {
     psn_norm_args a;
+    memset(&a, 0, sizeof a);
+    a.keep_x = keep_x ? 1 : 0;
     a.x = x;
     a.delta = delta;
     a.weight = weight;
@@ -1651,17 +1768,18 @@ extern "C" int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_
     psn_actq_info li;
     if ((rc = psn_actq_layout(at, K, 1, &li))) return rc;
     if ((rc = ensure_workspace(s, li.bytes))) return rc;
-    bool cap = false;
-    if ((rc = is_capturing(s, &cap))) return rc;
-    if (cap) s->ws_in_capture = true;
+    if ((rc = note_workspace_use(s))) return rc;
+    char *ws = (char *)s->ws->p;
     psn_actq_out qo;
-    qo.qs = (int8_t *)s->ws + li.off_qs;
-    qo.d = (float *)((char *)s->ws + li.off_d);
-    qo.s = (char *)s->ws + li.off_s;
+    qo.qs = (int8_t *)ws + li.off_qs;
+    qo.d = (float *)(ws + li.off_d);
+    qo.s = ws + li.off_s;
     qo.act_q8_K = at == PSN_Q8_K;
-    if ((rc = launch_add_rmsnorm(mod, s, (float *)x->p, nf.delta, nf.weight, nullptr, nf.h_out, qo, K, eps))) return rc;
+    qo.pad = 0;
+    /* like the fused launch, this path never writes x: the sum goes to h_out or nowhere */
+    if ((rc = launch_add_rmsnorm(mod, s, (float *)x->p, nf.delta, nf.weight, nullptr, nf.h_out, qo, K, eps, /*keep_x=*/true))) return rc;
     if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, 1, mod->ctx->compute_units, false, sg.N, sg.count, &plan))) return rc;
-    return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, s->ws, K, 1, &plan);
+    return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, ws, K, 1, &plan);
 }
 
 extern "C" int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q, psn_buf *k, const psn_buf *v, psn_buf *k_cache,

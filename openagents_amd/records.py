@@ -3,12 +3,21 @@ reference's `KernelThroughputRecord`
 (/root/reference/packages/tassadar-executor/src/kernel-optimization-parity.ts:26-59: targetModel,
 device, hardwareRef, opRef, kernelRef, graphDigest, tokensPerSecond), plus the `/health`-shaped
 object a Psionic server reports (/root/reference/apps/pylon/packages/runtime/src/cli.ts:1181 reads
-`execution_engine` / `backend`, :1206-1213 `default_model` / `model` / `models`).
+`execution_engine` / `backend`, :1206-1213 `default_model` / `model` / `models`) and the
+`PsionicWorkerAttachment` file `oa-node psionic attach` reads
+(/root/reference/crates/openagents-cloud-contract/src/lib.rs:1723-1745).
 
-    python -m openagents_amd.records [--out DIR] [--configs 1,3,4,5] [--samples 9]
+    python -m openagents_amd.records [--out DIR] [--configs 1,3,4,5] [--samples 9] [--read-sweep]
 
-writes one JSON file per record and `health.json` into DIR and prints a one-line summary per record.
-`bench.py` calls the same functions for the records it carries beside its headline.
+writes one JSON file per record, `health.json` and `psionic-workers.json` into DIR and prints a one-line
+summary per record.  `bench.py` calls the same functions for the records it writes beside its headline.
+
+The reference's acceptance rule looks at output parity before throughput and binds both to one
+`graphDigest` (kernel-optimization-parity.ts:118-136).  Every record therefore carries a `parity` object
+computed on the record's own weight bytes and activations.  The checker is passed in by the caller
+(`bench.py` hands in one built on the CPU oracle; this package never imports it); without one the record
+says `parity.status = "not_checked"` and lists the check under `not_measured`.  `kernelRef` is read back from
+the library's launch log (psn_launch_log), i.e. it names the kernels that actually ran.
 
 Every figure is measured on graph replays (the launches of one sample are one HIP graph), with HIP
 events on the launch stream; weights rotate over enough distinct device copies to defeat the 256 MB
@@ -29,7 +38,7 @@ import numpy as np
 
 from . import _ffi, quantize
 from ._ffi import ACT_Q8, Q4_0, Q4_K, Q6_K, Q8_0
-from .backend import HipBackend, act_type_for, matvec_plan, prefill_plan, row_bytes
+from .backend import HipBackend, act_type_for, prefill_plan, row_bytes
 
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
@@ -73,25 +82,53 @@ def time_graph(be: HipBackend, graph, launches_per_replay: int, samples: int = 9
     return out
 
 
-def record(be: HipBackend, op_ref: str, kernel_ref: str, digest: str, tokens_per_second: float, **extra) -> dict:
+PARITY_GATE = 1e-3
+PARITY_METRIC = "max|y-ref|/max|ref| against the CPU path on the same weight bytes and activations"
+NOT_CHECKED = {"status": "not_checked", "metric": PARITY_METRIC, "value": None, "gate": PARITY_GATE}
+
+
+def parity_of(got: np.ndarray, ref: np.ndarray, scheme: str, what: str) -> dict:
+    """The parity object of a record: got and ref are the same outputs from the device and from the checker."""
+    ref = np.asarray(ref, dtype=np.float64)
+    err = float(np.max(np.abs(np.asarray(got, dtype=np.float64) - ref)) / max(float(np.max(np.abs(ref))), 1e-30))
+    ok = bool(np.all(np.isfinite(got))) and err < PARITY_GATE
+    return {"status": "pass" if ok else "fail", "metric": PARITY_METRIC, "value": err, "gate": PARITY_GATE, "scheme": scheme, "checked": what}
+
+
+def roofline_of(bound: str, achieved: float) -> dict:
+    """bound "hbm": achieved GB/s against 8 TB/s; "mfma": achieved TFLOP/s against the fp16 dense peak."""
+    peak = HBM_PEAK_GBS if bound == "hbm" else MFMA_F16_PEAK_TFLOPS
+    return {"bound": bound, "peak": peak, "achieved": round(float(achieved), 1), "fraction": round(float(achieved) / peak, 4),
+            "unit": "GB/s" if bound == "hbm" else "TFLOP/s"}
+
+
+def launched_kernels(be: HipBackend, call) -> str:
+    """Runs `call` (one op's launches) and returns the kernels the library launched for it, in order, joined by ' + '."""
+    be.lib.psn_launch_log_clear()
+    call()
+    names = [n for n in be.lib.psn_launch_log().decode().split(";") if n]
+    return " + ".join(names)
+
+
+def record(be: HipBackend, op_ref: str, kernel_ref: str, digest: str, tokens_per_second: float, roofline: dict, parity: dict | None,
+           not_measured=(), **extra) -> dict:
     rec = {"targetModel": TARGET_MODEL, "device": DEVICE_CLASS, "hardwareRef": hardware_ref(be), "opRef": op_ref,
-           "kernelRef": kernel_ref, "graphDigest": digest, "tokensPerSecond": round(float(tokens_per_second), 2)}
+           "kernelRef": kernel_ref, "graphDigest": digest, "tokensPerSecond": round(float(tokens_per_second), 2),
+           "roofline": roofline, "parity": dict(parity) if parity else dict(NOT_CHECKED)}
     rec.update(extra)
+    rec["not_measured"] = list(not_measured) + ([] if parity else ["output parity (no checker was passed in)"])
     return rec
+
+
+def record_digest(rec: dict) -> str:
+    """SHA-256 over the fields that identify what was measured and how it came out (the evidence digest a
+    worker attachment cites)."""
+    keep = {k: rec[k] for k in ("targetModel", "device", "hardwareRef", "opRef", "kernelRef", "graphDigest", "tokensPerSecond", "roofline", "parity")}
+    return hashlib.sha256(json.dumps(keep, sort_keys=True).encode()).hexdigest()
 
 
 def seeded_weights(seed: int, n: int, k: int) -> np.ndarray:
     return np.random.default_rng(seed).standard_normal((n, k), dtype=np.float32) * np.float32(0.02)
-
-
-def matvec_kernel_name(qtype: int, ns, k: int, batch: int, cus: int, x_is_f32: bool = True) -> str:
-    p = matvec_plan(qtype, ACT_Q8, sum(ns), k, batch, cus, x_is_f32)
-    f = FMT_NAME[qtype]
-    if p.mfma:
-        return f"psn_quantize_q8_K + psn_mvm_{f}_q8_" + ("t8" if (k // 256) // p.mfma > 4 else "p4")
-    if p.stream:
-        return f"psn_mvs_{f}_q8_g{p.lanes_per_row}" + {1: "_lds", 2: "_xf"}[p.stage_lds] + f"_s{len(ns)}"
-    return f"psn_mv_{f}_q8_g{p.lanes_per_row}_r{p.rows_in_flight}_b{p.batch_tile}" + {0: "", 1: "_lds", 2: "_xf"}[p.stage_lds]
 
 
 def copies_for(nbytes: int, floor: int = 2) -> int:
@@ -103,19 +140,27 @@ def upload_copies(be: HipBackend, qtype: int, blocks: np.ndarray, n: int, k: int
     return [be.upload_weight(qtype, blocks, n, k) for _ in range(copies_for(blocks.nbytes))]
 
 
-def matvec_record(be: HipBackend, ws: list, blocks: np.ndarray, batch: int, op_ref: str, samples: int, seed: int) -> dict:
+def matvec_record(be: HipBackend, ws: list, blocks: np.ndarray, batch: int, op_ref: str, samples: int, seed: int, checker=None) -> dict:
     """One matrix (device copies `ws` of the host `blocks`), fp32 activations in, activation scheme Q8,
     fp32 out, `batch` columns."""
     qtype, n, k, copies = ws[0].qtype, ws[0].n, ws[0].k, len(ws)
-    x = be.upload(np.random.default_rng(seed).standard_normal((batch, k), dtype=np.float32))
+    x_host = np.random.default_rng(seed).standard_normal((batch, k), dtype=np.float32)
+    x = be.upload(x_host)
     y = be.alloc(batch * n * 4)
     be.reserve(k, batch)
+    kernel_ref = launched_kernels(be, lambda: be.quantized_matvec(ws[0], x, y, batch, ACT_Q8))
     be.begin_capture()
     for w in ws:
         be.quantized_matvec(w, x, y, batch, ACT_Q8)
     g = be.end_capture()
     st = stats(time_graph(be, g, copies, samples))
     be.destroy_graph(g)
+    parity = None
+    if checker is not None:
+        y.fill_zero()
+        be.quantized_matvec(ws[-1], x, y, batch, ACT_Q8)
+        parity = parity_of(y.download(np.float32, (batch, n)), checker.matvec(qtype, blocks, x_host, n, k), "Q8",
+                           f"all {batch} x {n} outputs")
     extra = {}
     if batch > 1:
         # the same projection fed with activations that are already quantized (what a fused producer hands over)
@@ -128,34 +173,34 @@ def matvec_record(be: HipBackend, ws: list, blocks: np.ndarray, batch: int, op_r
         be.destroy_graph(g)
     nbytes = n * row_bytes(qtype, k) + batch * 4 * (n + k)
     gbs = nbytes / st["median_us"] / 1e3
-    return record(be, op_ref, matvec_kernel_name(qtype, [n], k, batch, be.compute_units),
-                  graph_digest(f"{op_ref}:{FMT_NAME[qtype]}:n{n}:k{k}:b{batch}", blocks),
-                  batch * 1e6 / st["median_us"], shape={"N": n, "K": k, "batch": batch, "format": FMT_NAME[qtype]},
+    return record(be, op_ref, kernel_ref, graph_digest(f"{op_ref}:{FMT_NAME[qtype]}:n{n}:k{k}:b{batch}", blocks),
+                  batch * 1e6 / st["median_us"], roofline_of("hbm", gbs), parity,
+                  ["end-to-end model tokens/s (this record is one projection)", "host-side launch cost (graph replay)"],
+                  shape={"N": n, "K": k, "batch": batch, "format": FMT_NAME[qtype]},
                   timing=st, algorithmic_bytes=int(nbytes), GBps=round(gbs, 1), bound="hbm",
                   frac_of_roofline=round(gbs / HBM_PEAK_GBS, 4), weight_copies=copies, **extra,
-                  tokens_definition="activation columns through this one projection per second",
-                  not_measured=["end-to-end model tokens/s (this record is one projection)", "host-side launch cost (graph replay)"])
+                  tokens_definition="activation columns through this one projection per second")
 
 
-def config1(be: HipBackend, samples: int = 9, seed: int = 11, cpu: bool = True) -> list:
-    """Q8_0 4096x4096, batch 1: the reference's own CPU-runnable case, timed here on the GPU and (cpu=True)
-    on the host cores through the CPU oracle."""
+def config1(be: HipBackend, samples: int = 9, seed: int = 11, checker=None, cpu_path=None) -> list:
+    """Q8_0 4096x4096, batch 1: the reference's own CPU-runnable case, timed here on the GPU.  `cpu_path`, when
+    given, is the caller's CPU implementation `(qtype, blocks, x, n, k, threads) -> y` plus `.max_threads`; it is
+    timed on the host cores beside the GPU figure (one thread and all of them)."""
     n = k = 4096
     w = seeded_weights(seed, n, k)
     blocks = quantize.quantize_q8_0(w)
     ws = upload_copies(be, Q8_0, blocks, n, k)
-    rec = matvec_record(be, ws, blocks, 1, "matvec.q8_0.4096x4096.b1", samples, seed + 1)
+    rec = matvec_record(be, ws, blocks, 1, "matvec.q8_0.4096x4096.b1", samples, seed + 1, checker)
     for w in ws:
         w.buf.free()
-    if cpu:
-        import oracle
+    if cpu_path is not None:
         x = np.random.default_rng(seed + 1).standard_normal(k, dtype=np.float32)
         nbytes = rec["algorithmic_bytes"]
         cpu_rec = {}
-        for label, threads in (("threads_1", 1), ("threads_all", oracle.max_threads())):
+        for label, threads in (("threads_1", 1), ("threads_all", int(cpu_path.max_threads))):
             reps, t0 = 0, time.perf_counter()
             while time.perf_counter() - t0 < 1.0:
-                oracle.matvec(oracle.Q8_0, oracle.ACT_Q8, blocks, x, n, k, nthreads=threads)
+                cpu_path(Q8_0, blocks, x, n, k, threads)
                 reps += 1
             dt = (time.perf_counter() - t0) / reps
             cpu_rec[label] = {"threads": threads, "us": round(dt * 1e6, 1), "GBps": round(nbytes / dt / 1e9, 2)}
@@ -163,38 +208,40 @@ def config1(be: HipBackend, samples: int = 9, seed: int = 11, cpu: bool = True) 
     return [rec]
 
 
-def config3(be: HipBackend, samples: int = 9, seed: int = 31, weights=None) -> list:
+def config3(be: HipBackend, samples: int = 9, seed: int = 31, weights=None, checker=None) -> list:
     """Q4_K 4096->14336 and 14336->4096 at batch 1, 2, 4, 8.  `weights` = {(n, k): blocks} reuses matrices."""
     out = []
     for n, k in ((14336, 4096), (4096, 14336)):
         blocks = weights[(n, k)] if weights and (n, k) in weights else quantize.quantize_q4_K(seeded_weights(seed + n % 7, n, k))
         ws = upload_copies(be, Q4_K, blocks, n, k)
         for batch in (1, 2, 4, 8):
-            out.append(matvec_record(be, ws, blocks, batch, f"matvec.q4_K.{k}x{n}.b{batch}", samples, seed + batch))
+            out.append(matvec_record(be, ws, blocks, batch, f"matvec.q4_K.{k}x{n}.b{batch}", samples, seed + batch, checker))
         for w in ws:
             w.buf.free()
     return out
 
 
-def prefill_kernel_name(fmt: str, m: int, n: int, k: int, cus: int, qtype: int | None = None):
-    tm, tn, sp, wv = prefill_plan(m, n, k, cus, qtype)
-    name = {64: f"psn_prefill_{fmt}_skinny", 32: f"psn_prefill_{fmt}_wide", 128: f"psn_prefill_{fmt}_unpack + psn_prefill_dense_f16" + ("_m128" if tm == 128 else "")}.get(wv, f"psn_prefill_{fmt}_m{tm}_n{tn}" + {4: "", 16: "_ws"}.get(wv, ""))
-    return name, sp
-
-
-def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(64, 512, 2048)) -> list:
+def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(64, 512, 2048), checker=None, shapes=((14336, 4096), (4096, 14336)),
+            formats=(Q4_0, Q8_0)) -> list:
     """Quantized prefill matmul, Q4_0 and Q8_0, both shapes, M = 64 / 512 / 2048: twelve cells."""
     out = []
-    for qtype, quant in ((Q4_0, quantize.quantize_q4_0), (Q8_0, quantize.quantize_q8_0)):
+    for qtype in formats:
         fmt = FMT_NAME[qtype]
-        for n, k in ((14336, 4096), (4096, 14336)):
+
+        def quant(w, qtype=qtype):
+            return quantize.quantize(qtype, w)
+
+        for n, k in shapes:
             blocks = weights[(qtype, n, k)] if weights and (qtype, n, k) in weights else quant(seeded_weights(seed + n % 7, n, k))
             ws = upload_copies(be, qtype, blocks, n, k)
             copies = len(ws)
             digest = graph_digest(f"prefill:{fmt}:n{n}:k{k}", blocks)
             for m in ms:
-                x = be.upload(np.random.default_rng(seed + m).standard_normal((m, k), dtype=np.float32).astype(np.float16))
+                x_host = np.random.default_rng(seed + m).standard_normal((m, k), dtype=np.float32).astype(np.float16)
+                x = be.upload(x_host)
                 y = be.alloc(m * n * 4)
+                kname = launched_kernels(be, lambda: be.quantized_matmul(ws[0], x, y, m))
+                sp = prefill_plan(m, n, k, be.compute_units, qtype)[2]
                 be.begin_capture()
                 for w in ws:
                     be.quantized_matmul(w, x, y, m)
@@ -206,12 +253,25 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
                 t_us = st["median_us"]
                 bound_us = max(flops / (MFMA_F16_PEAK_TFLOPS * 1e6), nbytes / (HBM_PEAK_GBS * 1e3))
                 bound = "mfma" if flops / (MFMA_F16_PEAK_TFLOPS * 1e6) >= nbytes / (HBM_PEAK_GBS * 1e3) else "hbm"
-                kname, sp = prefill_kernel_name(fmt, m, n, k, be.compute_units, qtype)
+                parity = None
+                if checker is not None:
+                    y.fill_zero()
+                    be.quantized_matmul(ws[-1], x, y, m)
+                    got = y.download(np.float32, (m, n))
+                    # a sample of activation rows x weight rows (tile corners, edges, random interior) that the full result must match
+                    rng = np.random.default_rng(m + n)
+                    mi = np.unique(np.concatenate([[0, min(63, m - 1), min(64, m - 1), min(255, m - 1), m - 1], rng.integers(0, m, 43)]))
+                    ni = np.unique(np.concatenate([[0, 31, 32, 255, 256, n - 1], rng.integers(0, n, 122)]))
+                    parity = parity_of(got[np.ix_(mi, ni)], checker.prefill(qtype, blocks[ni], x_host[mi], len(ni), k), "fp16 x h(deq(W)), fp32 accumulate",
+                                       f"{len(mi)} activation rows x {len(ni)} weight rows of the full [{m}, {n}] product; all outputs finite: {bool(np.all(np.isfinite(got)))}")
+                    if not np.all(np.isfinite(got)):
+                        parity["status"] = "fail"
                 packed_extra = {}
                 if m >= 2048:
                     # the same projection with the dequantization hoisted out of the call (psn_prefill_pack once, then
                     # psn_qmatmul_prefill_packed): three packed copies rotate (2 bytes per weight each)
                     packs = [be.pack_for_prefill(w) for w in ws[:3]]
+                    packed_kernel = launched_kernels(be, lambda: be.quantized_matmul_packed(packs[0], x, y, m, n, k))
                     be.begin_capture()
                     for pk in packs:
                         be.quantized_matmul_packed(pk, x, y, m, n, k)
@@ -222,17 +282,17 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
                         pk.free()
                     packed_extra = {"timing_packed_weights": {**sp_, "TFLOPs": round(flops / sp_["median_us"] / 1e6, 1),
                                                               "frac_of_mfma_peak": round(flops / sp_["median_us"] / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
-                                                              "kernelRef": "psn_prefill_dense_f16 or psn_prefill_dense_f16_m128 (by shape)",
+                                                              "kernelRef": packed_kernel,
                                                               "note": "weights dequantized to fp16 fragments once beforehand (psn_prefill_pack, 2 bytes per weight resident)"}}
-                out.append(record(be, f"prefill.{fmt}.{k}x{n}.m{m}", kname, digest, m * 1e6 / t_us,
+                achieved = flops / t_us / 1e6 if bound == "mfma" else nbytes / t_us / 1e3
+                out.append(record(be, f"prefill.{fmt}.{k}x{n}.m{m}", kname, digest, m * 1e6 / t_us, roofline_of(bound, achieved), parity,
+                                  ["end-to-end prefill tokens/s (this record is one projection)", "host-side launch cost (graph replay)"],
                                   shape={"M": m, "N": n, "K": k, "format": fmt, "ksplit": sp}, timing=st,
                                   TFLOPs=round(flops / t_us / 1e6, 1), GBps=round(nbytes / t_us / 1e3, 1),
                                   algorithmic_bytes=int(nbytes), flops=int(flops), bound=bound,
                                   roofline_us=round(bound_us, 2), frac_of_roofline=round(bound_us / t_us, 4),
                                   frac_of_mfma_peak=round(flops / t_us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), weight_copies=copies,
-                                  tokens_definition="prompt rows through this one projection per second",
-                                  not_measured=["end-to-end prefill tokens/s (this record is one projection)",
-                                                "host-side launch cost (graph replay)"], **packed_extra))
+                                  tokens_definition="prompt rows through this one projection per second", **packed_extra))
                 x.free()
                 y.free()
             for w in ws:
@@ -240,7 +300,7 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
     return out
 
 
-def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, layers: int = 32) -> list:
+def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, layers: int = 32, checker=None) -> list:
     """The synthetic Llama-3-8B-shaped Q4_K decode step at batch 1, context `ctx`, Q6_K LM head."""
     from .decode import DecodeStep, LlamaShape, synthetic_weights
     shape = LlamaShape(n_layers=layers)
@@ -257,7 +317,10 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
     x0 = rng.standard_normal(shape.hidden, dtype=np.float32)
     step.x.upload(x0)
     setup_s = time.time() - t0
-    full, mv = step.capture(pos), step.capture(pos, matvecs_only=True)
+    be.lib.psn_launch_log_clear()
+    full = step.capture(pos)
+    launched = [n for n in be.lib.psn_launch_log().decode().split(";") if n]
+    mv = step.capture(pos, matvecs_only=True)
     st_full = stats(time_graph(be, full, 1, samples, replays=3))
     st_mv = stats(time_graph(be, mv, 1, samples, replays=3))
     step.x.upload(x0)
@@ -270,9 +333,15 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
     digest = graph_digest(f"decode-step:l{layers}:ctx{ctx}:h{shape.hidden}:ffn{shape.ffn}:v{shape.vocab}",
                           *[protos[name] for name in sorted(protos)])
     launches = step.launches_per_token
-    rec = record(be, "decode.step.q4_K.b1", f"psn decode-step graph ({launches} launches: psn_mvs_q4_K_q8_g*_xn_s*, psn_mvs_q4_K_q8_g*_lds_s1, "
-                 "psn_mvs_q6_K_q8_g16_xn_s1, psn_attn_partial_rope, psn_attn_combine, psn_swiglu, psn_rope_table)",
-                 digest, 1e6 / t_full, shape={"layers": layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,
+    parity = None
+    if checker is not None:
+        # the replay above left the logits of (x0, kv, pos) in place; the checker redoes the whole step on the CPU
+        parity = parity_of(logits, checker.decode_step(shape, protos, x0, kv, pos), "Q8",
+                           f"all {shape.vocab} logits of the {layers}-layer step at position {pos}")
+    distinct = sorted(set(launched) - {"..."})
+    rec = record(be, "decode.step.q4_K.b1", f"psn decode-step graph ({launches} launches: " + ", ".join(distinct) + ")",
+                 digest, 1e6 / t_full, roofline_of("hbm", mbytes / t_mv / 1e3), parity, ["sampling", "tokenizer", "host loop", "prompt prefill"],
+                 shape={"layers": layers, "hidden": shape.hidden, "heads": shape.n_heads, "kv_heads": shape.n_kv_heads,
                                               "head_dim": shape.head_dim, "ffn": shape.ffn, "vocab": shape.vocab, "context": ctx,
                                               "weights": "Q4_K projections, Q6_K LM head"},
                  timing=st_full, ms_per_token=round(t_full / 1e3, 4), matvec_ms=round(t_mv / 1e3, 4), glue_ms=round((t_full - t_mv) / 1e3, 4),
@@ -280,31 +349,58 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
                  bound="hbm", frac_of_roofline=round(mbytes / t_mv / 1e3 / HBM_PEAK_GBS, 4), launches_per_token=launches,
                  logits_finite=bool(np.all(np.isfinite(logits))), setup_s=round(setup_s, 1),
                  data="random-init weights (one unique layer copied to every layer's own allocation), fp16 N(0,1) KV cache",
-                 tokens_definition="decoded tokens per second at batch 1 (whole step, graph replay)",
-                 not_measured=["sampling", "tokenizer", "host loop", "prompt prefill"])
+                 roofline_note="matvec launches only (weights + fp32 vectors of one token) over the time of the matvecs-only graph",
+                 tokens_definition="decoded tokens per second at batch 1 (whole step, graph replay)")
     return [rec]
 
 
-def read_calibration(be: HipBackend, samples: int = 7) -> dict:
+CALIBRATION_SIZES = (("o_9.4MB", 9_437_184), ("qkv_14.2MB", 14_155_776), ("down_33MB", 33_030_144), ("gate_up_66MB", 66_060_288))
+
+
+def read_calibration(be: HipBackend, samples: int = 7, geometries=((256, 512, 0),)) -> dict:
     """What a kernel that only reads (no decode, one partial sum per thread) reaches on this device at the
-    byte counts of the four Llama-3-8B launches: the ceiling the streaming matvecs are compared with."""
+    byte counts of the four Llama-3-8B launches: what the streaming matvecs are compared with.  `geometries`:
+    (workgroups, threads, LDS ring depth per wave; 0 = loads into registers) to try; the fastest is reported per
+    size together with the geometry that reached it."""
     out = {}
-    for name, nbytes in (("o_9.4MB", 9_437_184), ("qkv_14.2MB", 14_155_776), ("down_33MB", 33_030_144), ("gate_up_66MB", 66_060_288)):
+    for name, nbytes in CALIBRATION_SIZES:
         copies = copies_for(nbytes)
         srcs = [be.alloc(nbytes) for _ in range(copies)]
         for s in srcs:
             s.fill_zero()
         sink = be.alloc(1 << 20)
-        be.begin_capture()
-        for s in srcs:
-            be.calibrate_read(s, nbytes, be.compute_units, 512, 0, sink)
-        g = be.end_capture()
-        st = stats(time_graph(be, g, copies, samples))
-        be.destroy_graph(g)
+        best, tried = None, {}
+        for blocks, threads, depth in geometries:
+            be.begin_capture()
+            for s in srcs:
+                be.calibrate_read(s, nbytes, blocks, threads, depth, sink)
+            g = be.end_capture()
+            st = stats(time_graph(be, g, copies, samples))
+            be.destroy_graph(g)
+            tried[f"{blocks}x{threads}" + (f"/lds{depth}" if depth else "")] = st["median_us"]
+            if best is None or st["median_us"] < best[0]["median_us"]:
+                best = (st, (blocks, threads, depth))
         for s in srcs:
             s.free()
-        out[name] = {"bytes": nbytes, **st, "GBps": round(nbytes / st["median_us"] / 1e3, 1)}
+        st, geo = best
+        out[name] = {"bytes": nbytes, **st, "GBps": round(nbytes / st["median_us"] / 1e3, 1),
+                     "geometry": {"blocks": geo[0], "threads": geo[1], "lds_depth": geo[2]}}
+        if len(tried) > 1:
+            out[name]["median_us_by_geometry"] = tried
     return out
+
+
+def read_sweep_geometries(cus: int = 256):
+    """Launch geometries of the read-only kernel worth comparing: one to eight workgroups per compute unit,
+    256 or 512 threads, loads into registers or through LDS rings of 2 / 4 / 8 KB per wave."""
+    geos = []
+    for per_cu in (1, 2, 4, 8):
+        for threads in (256, 512):
+            for depth in (0, 2, 4, 8):
+                if per_cu * threads > 2048 or per_cu * (threads // 64) * depth * 1024 > 160 * 1024:
+                    continue
+                geos.append((per_cu * cus, threads, depth))
+    return geos
 
 
 def health(be: HipBackend, models=(TARGET_MODEL,)) -> dict:
@@ -313,20 +409,49 @@ def health(be: HipBackend, models=(TARGET_MODEL,)) -> dict:
             "models": list(models), "device": hardware_ref(be), "abi_version": int(_ffi.load().psn_abi_version())}
 
 
+def worker_attachment(records: list, ready: bool = True, updated_at_ms: int | None = None, detail: str | None = None) -> dict:
+    """The `psionic-workers.json` object `oa-node psionic attach` consumes (PsionicWorkerAttachment{schema_version,
+    updated_at_ms, workers[{product_id, worker_id, worker_kind, ready, crashed, evidence_digest, detail}]},
+    /root/reference/crates/openagents-cloud-contract/src/lib.rs:1723-1745).  One worker: this backend serving the
+    target model; `evidence_digest` is the digest of the decode-step record when there is one, else of the first
+    record; `ready` additionally requires every parity verdict present in the records to be a pass."""
+    pick = next((r for r in records if r["opRef"].startswith("decode.step")), records[0] if records else None)
+    verdicts = [r["parity"]["status"] for r in records]
+    all_pass = all(v == "pass" for v in verdicts) if verdicts else False
+    text = detail or (f"{len(records)} throughput records; parity " + (", ".join(f"{v}: {verdicts.count(v)}" for v in sorted(set(verdicts))) or "none"))
+    return {"schema_version": 1, "updated_at_ms": int(updated_at_ms if updated_at_ms is not None else time.time() * 1000),
+            "workers": [{"product_id": f"psionic.hip.{TARGET_MODEL}", "worker_id": f"{records[0]['hardwareRef']}-0" if records else "hip-0",
+                         "worker_kind": "psionic-hip-gguf", "ready": bool(ready and all_pass), "crashed": False,
+                         "evidence_digest": record_digest(pick) if pick else None, "detail": text}]}
+
+
+def write_all(out_dir: str, recs: list, health_obj: dict) -> None:
+    os.makedirs(out_dir, exist_ok=True)
+    for r in recs:
+        with open(os.path.join(out_dir, r["opRef"] + ".json"), "w") as f:
+            json.dump(r, f, indent=1)
+    with open(os.path.join(out_dir, "health.json"), "w") as f:
+        json.dump(health_obj, f, indent=1)
+    with open(os.path.join(out_dir, "psionic-workers.json"), "w") as f:
+        json.dump(worker_attachment(recs), f, indent=1)
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--out", default="psn_records")
     ap.add_argument("--configs", default="1,3,4,5")
     ap.add_argument("--samples", type=int, default=9)
-    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--read-sweep", action="store_true", help="time the read-only kernel over launch geometries at the four launch sizes and exit")
     args = ap.parse_args(argv)
-    os.makedirs(args.out, exist_ok=True)
     be = HipBackend(0)
+    if args.read_sweep:
+        print(json.dumps(read_calibration(be, args.samples, read_sweep_geometries(be.compute_units)), indent=1))
+        return 0
     be.reserve_prefill(14336, 4096)      # the dense prefill family's workspace, before any graph refers to the stream's workspace
     recs = []
     todo = set(args.configs.split(","))
     if "1" in todo:
-        recs += config1(be, args.samples, cpu=not args.no_cpu)
+        recs += config1(be, args.samples)
     if "3" in todo:
         recs += config3(be, args.samples)
     if "4" in todo:
@@ -334,11 +459,8 @@ def main(argv=None):
     if "5" in todo:
         recs += config5(be, args.samples)
     for r in recs:
-        with open(os.path.join(args.out, r["opRef"] + ".json"), "w") as f:
-            json.dump(r, f, indent=1)
-        print(f"{r['opRef']:40s} {r['kernelRef'][:48]:48s} {r['timing']['median_us']:10.2f} us  frac {r['frac_of_roofline']:.3f}", flush=True)
-    with open(os.path.join(args.out, "health.json"), "w") as f:
-        json.dump(health(be), f, indent=1)
+        print(f"{r['opRef']:40s} {r['kernelRef'][:48]:48s} {r['timing']['median_us']:10.2f} us  frac {r['roofline']['fraction']:.3f}  parity {r['parity']['status']}", flush=True)
+    write_all(args.out, recs, health(be))
     return 0
 
 

@@ -66,3 +66,79 @@ def test_workspace_cannot_grow_once_a_graph_refers_to_it(orc):
         # no graph refers to the workspace any more: it may grow again
         be.quantized_matvec(wb, dxb, y, batch, _ffi.ACT_Q8)
         assert G.max_rel_err(y.download(np.float32, (batch, n)), orc.matvec(orc.Q6_K, orc.ACT_Q8, Wb, xb, n, k_big)) < 2e-5
+
+
+def test_side_stream_workspace_is_pinned_by_the_graph_that_the_origin_ends(orc):
+    """A batch-4 Q6_K matvec on a side stream forked into a capture quantizes into the SIDE stream's
+    workspace.  The graph ended on the origin stream must pin that workspace (growth on the side stream is
+    refused while the graph lives), a later capture begun on the side stream must not lift the pin, and
+    destroying the graph lifts it."""
+    with backend.HipBackend(0) as be:
+        n, k_small, k_big, batch = 8, 1024, 327680, 4
+        Ws, Wb = orc.quantize(orc.Q6_K, G.seeded_weights(975, n, k_small)), orc.quantize(orc.Q6_K, G.seeded_weights(976, n, k_big))
+        xs, xb = G.seeded_acts(977, batch, k_small), G.seeded_acts(978, batch, k_big)
+        ws, wb = be.upload_weight(orc.Q6_K, Ws, n, k_small), be.upload_weight(orc.Q6_K, Wb, n, k_big)
+        dxs, dxb, y, y_side = be.upload(xs), be.upload(xb), be.alloc(batch * n * 4), be.alloc(batch * n * 4)
+        side = be.new_stream()
+        with be.on_stream(side):
+            be.reserve(k_small, batch)
+        be.reserve(k_small, batch)
+        main = be.stream
+        be.begin_capture()
+        be.stream_wait(side, main)                           # fork
+        with be.on_stream(side):
+            be.quantized_matvec(ws, dxs, y_side, batch, _ffi.ACT_Q8)
+        be.quantized_matvec(ws, dxs, y, batch, _ffi.ACT_Q8)
+        be.stream_wait(main, side)                           # join
+        graph = be.end_capture()
+        ref = orc.matvec(orc.Q6_K, orc.ACT_Q8, Ws, xs, n, k_small)
+
+        def replay_ok():
+            y.fill_zero()
+            y_side.fill_zero()
+            be.launch_graph(graph)
+            return (G.max_rel_err(y.download(np.float32, (batch, n)), ref) < 2e-5 and
+                    G.max_rel_err(y_side.download(np.float32, (batch, n)), ref) < 2e-5)
+
+        assert replay_ok()
+        with be.on_stream(side):
+            with pytest.raises(backend.PsnError) as e:
+                be.quantized_matvec(wb, dxb, y_side, batch, _ffi.ACT_Q8)
+            assert e.value.code == _ffi.E_INVALID_ARG and "reserve" in str(e.value)
+            # an unrelated capture on the side stream comes and goes: the first graph still holds the workspace
+            be.begin_capture()
+            be.swiglu(dxs, dxs, y_side, 32)
+            be.destroy_graph(be.end_capture())
+            with pytest.raises(backend.PsnError) as e:
+                be.quantized_matvec(wb, dxb, y_side, batch, _ffi.ACT_Q8)
+            assert e.value.code == _ffi.E_INVALID_ARG
+        assert replay_ok()
+        be.destroy_graph(graph)
+        with be.on_stream(side):
+            be.quantized_matvec(wb, dxb, y_side, batch, _ffi.ACT_Q8)      # nothing refers to it any more: it may grow
+            be.sync()
+            assert G.max_rel_err(y_side.download(np.float32, (batch, n)), orc.matvec(orc.Q6_K, orc.ACT_Q8, Wb, xb, n, k_big)) < 2e-5
+        be.destroy_stream(side)
+
+
+def test_a_graph_outlives_the_stream_whose_workspace_it_holds(orc):
+    """Destroying a stream does not free a workspace that a live graph still points at: the graph keeps
+    replaying on another stream, and the memory goes with the graph."""
+    with backend.HipBackend(0) as be:
+        n, k, batch = 16, 2048, 4
+        W = orc.quantize(orc.Q6_K, G.seeded_weights(979, n, k))
+        x = G.seeded_acts(980, batch, k)
+        w, dx, y = be.upload_weight(orc.Q6_K, W, n, k), be.upload(x), be.alloc(batch * n * 4)
+        side = be.new_stream()
+        with be.on_stream(side):
+            be.reserve(k, batch)
+            be.begin_capture()
+            be.quantized_matvec(w, dx, y, batch, _ffi.ACT_Q8)
+            graph = be.end_capture()
+        be.destroy_stream(side)
+        ref = orc.matvec(orc.Q6_K, orc.ACT_Q8, W, x, n, k)
+        for _ in range(2):
+            y.fill_zero()
+            be.launch_graph(graph)
+            assert G.max_rel_err(y.download(np.float32, (batch, n)), ref) < 2e-5
+        be.destroy_graph(graph)

@@ -679,6 +679,34 @@ def test_norm_fused_projection_matches_oracle(hip, orc, qname, ns, k, with_delta
     hip.quantized_matvec_norm_multi(ws, xb, db, wb, None, y3, eps)
     for n, y, yy in zip(ns, ys, y3):
         assert np.array_equal(y.download(np.float32, (n,)), yy.download(np.float32, (n,)))
+    # ... which must not have written the sum anywhere: x and delta are still what was uploaded
+    assert np.array_equal(xb.download(np.float32, (k,)), x)
+    if with_delta:
+        assert np.array_equal(db.download(np.float32, (k,)), delta)
+
+
+@pytest.mark.parametrize("k", [4096, 14336, 5120])
+def test_norm_fused_projection_three_formats_share_x(hip, orc, k):
+    """q | k | v in three different formats take three calls on the same x and delta (a decoder passes h_out to
+    the first only).  On shapes that run as two launches (rows longer than 8192; Q6_K rows that are not whole
+    16-byte words) the norm kernel used to store x + delta back into x, so the second and third call saw
+    x + 2 delta, x + 3 delta."""
+    rng = np.random.default_rng(4500 + k)
+    x = rng.standard_normal(k, dtype=np.float32) * 2
+    delta = rng.standard_normal(k, dtype=np.float32)
+    wn = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    eps, n = 1e-5, 192
+    xb, db, wb, hb = hip.upload(x), hip.upload(delta), hip.upload(wn), hip.alloc(k * 4)
+    h_ref, xn_ref = norm_ref(x, delta, wn, eps)
+    for i, qname in enumerate(["Q4_K", "Q6_K", "Q5_K", "Q6_K"]):
+        qt = getattr(orc, qname)
+        b = weights(orc, qname, 4510 + i, n, k)
+        w, y = hip.upload_weight(qt, b, n, k), hip.alloc(n * 4)
+        say(f"norm-fused shared x: {qname} k={k} call {i}")
+        hip.quantized_matvec_norm_multi([w], xb, db, wb, hb if i == 0 else None, [y], eps)
+        assert G.max_rel_err(y.download(np.float32, (n,)), orc.matvec(qt, orc.ACT_Q8, b, xn_ref, n, k)) < 2e-4, (qname, i)
+        assert np.array_equal(xb.download(np.float32, (k,)), x), (qname, i)
+    assert np.array_equal(hb.download(np.float32, (k,)), h_ref)
 
 
 def test_norm_fused_projection_argument_errors(hip, orc):

@@ -150,7 +150,7 @@ def test_matvec_rejects_bad_shapes(orc):
     assert L.orc_matvec(orc.Q8_K, 0, vp(rows), vp(x), vp(y), 4, 256, 1, 1) == -1
 
 
-@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0"])
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_prefill_vs_fp64_of_fp16_rounded_weights(orc, qname):
     t = getattr(orc, qname)
     m, n, k = 9, 40, 1024

@@ -103,3 +103,11 @@ def test_native_dequantizer_argument_errors():
     assert lib.psn_error_name(lib.psn_dequantize_rows(_ffi.Q4_K, None, 2, 256, C.c_void_p(out.ctypes.data), out.size)) == b"PSN_E_INVALID_ARG"
     with pytest.raises(ValueError):
         quantize.dequantize(_ffi.Q4_K, np.zeros(100, np.uint8), 256)
+
+
+def test_absurd_thread_counts_are_clamped_not_fatal():
+    """A huge `threads` argument must neither spawn that many threads nor abort the process."""
+    w = np.random.default_rng(5).standard_normal((600, 256), dtype=np.float32)
+    a = quantize.quantize(_ffi.Q4_K, w, threads=1)
+    b = quantize.quantize(_ffi.Q4_K, w, threads=1 << 30)
+    assert np.array_equal(a, b)

@@ -57,6 +57,28 @@ def test_f32_scheme_and_graph_capture(hip, orc):
         hip.destroy_graph(graph)
 
 
+def test_repeated_calls_leave_free_device_memory_unchanged(hip, orc):
+    """After the first call of a shape (which looks its kernels up), further calls neither allocate nor free
+    device memory: hipMemGetInfo reads the same before and after."""
+    import ctypes as C
+    t, n, k, batch = orc.Q4_K, 512, 4096, 4
+    W = orc.quantize(t, G.seeded_weights(992, n, k))
+    w, xb, y = hip.upload_weight(t, W, n, k), hip.upload(G.seeded_acts(993, batch, k)), hip.alloc(batch * n * 4)
+    hip.quantized_matvec_noalloc(w, xb, y, batch, _ffi.ACT_Q8)
+    hip.sync()
+
+    def free_bytes():
+        f = C.c_int64()
+        assert hip.lib.psn_ctx_mem_info(hip.ctx, C.byref(f), None) == 0
+        return int(f.value)
+
+    before = free_bytes()
+    for _ in range(20):
+        hip.quantized_matvec_noalloc(w, xb, y, batch, _ffi.ACT_Q8)
+    hip.sync()
+    assert free_bytes() == before
+
+
 def test_inputs_beyond_the_static_scratch_are_rejected(hip, orc):
     limit = int(hip.lib.psn_noalloc_max_bytes())
     assert limit == 1 << 20
