@@ -95,6 +95,24 @@ class OracleChecker:
         """The timed CPU path of the config-1 record."""
         return self.orc.matvec(qtype, self.orc.ACT_Q8, blocks, x, n, k, nthreads=threads)
 
+    def decode_last_layer(self, shape, protos, got):
+        """Teacher-forced reference of the launches that end a step, from the device's own vectors: gate | up from the
+        residual `x` that entered the last layer's FFN norm, the logits from x + down (norm weights 1)."""
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        from decoderef import rmsnorm_ref
+        orc, s = self.orc, shape
+        n_unique = sum(1 for name in protos if name.endswith(".wq"))
+        p = f"layer{(s.n_layers - 1) % n_unique}."
+        ones, eps = np.ones(s.hidden, np.float32), np.float32(s.eps)
+        xn = rmsnorm_ref(got["x"], ones, eps)
+        out = {"gate": orc.matvec(orc.Q4_K, orc.ACT_Q8, protos[p + "w_gate"], xn, s.ffn, s.hidden).reshape(-1),
+               "up": orc.matvec(orc.Q4_K, orc.ACT_Q8, protos[p + "w_up"], xn, s.ffn, s.hidden).reshape(-1)}
+        uniq = protos["lm_head"].shape[0]
+        xf = rmsnorm_ref((got["x"] + got["down"]).astype(np.float32), ones, eps)
+        head = orc.matvec(orc.Q6_K, orc.ACT_Q8, protos["lm_head"], xf, uniq, s.hidden).reshape(-1)
+        out["logits"] = np.tile(head, -(-s.vocab // uniq))[:s.vocab]
+        return out
+
     def decode_step(self, shape, protos, x0, kv, pos):
         """Logits of one token at position `pos` of the synthetic model whose layers all hold the matrices in
         `protos` (norm weights 1, LM head = `lm_head` rows tiled to the vocabulary), every layer's K and V cache
@@ -197,8 +215,21 @@ def main(argv=None):
                     help="file that receives the full records, the per-launch table and the calibration")
     ap.add_argument("--vendor-gemm", action="store_true",
                     help="also time the vendor library's fp16 GEMM (torch.matmul) at the prefill shapes: a calibration of what "
-                         "fp16 MFMA sustains on this device, written to the records file; imports torch")
+                         "fp16 MFMA sustains on this device, written to the records file; runs in a child process of its own "
+                         "(torch brings its own HIP runtime) before this one touches the GPU")
+    ap.add_argument("--vendor-gemm-only", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args(argv)
+    if args.vendor_gemm_only:
+        print(json.dumps(vendor_gemm_calibration()))
+        return 0
+    vendor = None
+    if args.vendor_gemm:
+        import subprocess
+        p = subprocess.run([sys.executable, os.path.abspath(__file__), "--vendor-gemm-only"], capture_output=True, text=True, timeout=600)
+        try:
+            vendor = json.loads(p.stdout.strip().splitlines()[-1])
+        except (IndexError, ValueError):
+            vendor = {"error": (p.stderr or p.stdout)[-400:]}
     if args.gpus != 1:
         print("bench.py: this build drives one GPU; --gpus N with N > 1 is not supported "
               "(the path would shard by weight rows across GPUs, but nothing here launches a second rank)", file=sys.stderr)
@@ -371,7 +402,7 @@ def main(argv=None):
                "host": {"nproc": os.cpu_count(), "usable_threads": threads, "cpu_model": cpu_model()},
                "provenance": "this build's C restatement of the CPU quantized path (oracle/), not Psionic's binary"}
 
-    records, calibration, vendor = None, None, None
+    records, calibration = None, None
     if not args.no_records:
         for lw in weights:                                   # the headline's 3.9 GB of copies are no longer needed
             for ts in lw.values():
@@ -382,9 +413,6 @@ def main(argv=None):
         shared = {(_ffi.Q4_0, FFN, HIDDEN): layer["gate_up"][0], (_ffi.Q4_0, HIDDEN, FFN): layer["down"][0]}
         records = (R.config1(be, args.record_samples, checker=checker, cpu_path=checker) + R.config3(be, args.record_samples, checker=checker)
                    + R.config4(be, args.record_samples, weights=shared, checker=checker) + R.config5(be, args.record_samples, checker=checker))
-    if args.vendor_gemm:
-        vendor = vendor_gemm_calibration()
-
     head = {"value": round(value, 1), "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
             "launches_per_step": args.layers * len(LAUNCHES), "bytes_per_step": int(bytes_per_step), "roofline": roofline,
             "cpu_baseline": cpu, "parity": None if parity is None else {"value": float(f"{parity['value']:.3e}"), "gate": 1e-3, "status": parity["status"]},

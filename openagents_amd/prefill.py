@@ -85,11 +85,21 @@ def main(argv=None):
     ap.add_argument("--sample-clock", type=float, default=0.0, metavar="S", help="also run each cell for S seconds and report the shader clock under that load")
     ap.add_argument("--shapes", default="14336x4096,4096x14336", help="weight shapes as NxK, comma separated")
     ap.add_argument("--compare-plans", action="store_true", help="also time every explicit plan and name the fastest")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run four 256 MiB device-to-device copies: a transfer of known size that hardware-counter runs scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args(argv)
     fmts = {"q4_0": (Q4_0, quantize.quantize_q4_0), "q8_0": (Q8_0, quantize.quantize_q8_0), "q4_K": (Q4_K, quantize.quantize_q4_K),
             "q5_K": (Q5_K, quantize.quantize_q5_K), "q6_K": (Q6_K, quantize.quantize_q6_K)}
     be = HipBackend(0)
     rng = np.random.default_rng(args.seed)
+    if args.calibrate_copy:
+        nbytes = 256 << 20
+        src, dst = be.alloc(nbytes), be.alloc(nbytes)
+        for _ in range(4):
+            be.copy(dst, src, nbytes)
+        be.sync()
+        src.free()
+        dst.free()
     for fname in args.formats.split(","):
         qt, quant = fmts[fname]
         for n, k in (tuple(int(v) for v in t.split("x")) for t in args.shapes.split(",")):

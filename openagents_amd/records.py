@@ -333,11 +333,24 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
     digest = graph_digest(f"decode-step:l{layers}:ctx{ctx}:h{shape.hidden}:ffn{shape.ffn}:v{shape.vocab}",
                           *[protos[name] for name in sorted(protos)])
     launches = step.launches_per_token
-    parity = None
-    if checker is not None:
-        # the replay above left the logits of (x0, kv, pos) in place; the checker redoes the whole step on the CPU
-        parity = parity_of(logits, checker.decode_step(shape, protos, x0, kv, pos), "Q8",
-                           f"all {shape.vocab} logits of the {layers}-layer step at position {pos}")
+    parity, whole_step = None, None
+    if checker is not None and step.fused_norm:
+        # The replay above left the last layer's vectors in the step's buffers: x = the residual that entered the last
+        # layer's FFN norm, gate / up, down, and the logits.  The checker redoes, from the device's OWN inputs, the
+        # launches that produced gate | up and the logits (add + RMSNorm + quantize + matvec each).  A comparison of
+        # the whole 32-layer chain against a CPU run is reported beside it but is no verdict: an int8 activation that
+        # rounds the other way moves an output by ~2e-4, and the random-init network amplifies that from layer to layer
+        # (the CPU path fed an input perturbed by 1e-6 differs from itself by ~2e-2 in the logits).
+        got = {"x": step.x.download(np.float32, (shape.hidden,)), "down": step.down.download(np.float32, (shape.hidden,)),
+               "gate": step.gate.download(np.float32, (shape.ffn,)), "up": step.up.download(np.float32, (shape.ffn,)), "logits": logits}
+        ref = checker.decode_last_layer(shape, protos, got)
+        verdicts = [parity_of(got[name], ref[name], "Q8", "") for name in ("gate", "up", "logits")]
+        parity = max(verdicts, key=lambda v: (v["status"] != "pass", v["value"]))
+        parity["checked"] = (f"gate | up ({2 * shape.ffn} outputs) and all {shape.vocab} logits of the last of {layers} layers, each recomputed on the CPU "
+                             "from the input vectors the device itself produced (residual, down)")
+        whole = parity_of(logits, checker.decode_step(shape, protos, x0, kv, pos), "Q8", "")
+        whole_step = {"value": whole["value"], "note": "logits of the whole step against a CPU run of all layers from the same embedding: "
+                      "ill-conditioned (see above), reported, not gated"}
     distinct = sorted(set(launched) - {"..."})
     rec = record(be, "decode.step.q4_K.b1", f"psn decode-step graph ({launches} launches: " + ", ".join(distinct) + ")",
                  digest, 1e6 / t_full, roofline_of("hbm", mbytes / t_mv / 1e3), parity, ["sampling", "tokenizer", "host loop", "prompt prefill"],
@@ -349,6 +362,7 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
                  bound="hbm", frac_of_roofline=round(mbytes / t_mv / 1e3 / HBM_PEAK_GBS, 4), launches_per_token=launches,
                  logits_finite=bool(np.all(np.isfinite(logits))), setup_s=round(setup_s, 1),
                  data="random-init weights (one unique layer copied to every layer's own allocation), fp16 N(0,1) KV cache",
+                 whole_step_vs_cpu=whole_step,
                  roofline_note="matvec launches only (weights + fp32 vectors of one token) over the time of the matvecs-only graph",
                  tokens_definition="decoded tokens per second at batch 1 (whole step, graph replay)")
     return [rec]
