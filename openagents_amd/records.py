@@ -267,7 +267,7 @@ def config4(be: HipBackend, samples: int = 7, seed: int = 41, weights=None, ms=(
                     if not np.all(np.isfinite(got)):
                         parity["status"] = "fail"
                 packed_extra = {}
-                if m >= 2048:
+                if m >= 512:
                     # the same projection with the dequantization hoisted out of the call (psn_prefill_pack once, then
                     # psn_qmatmul_prefill_packed): three packed copies rotate (2 bytes per weight each)
                     packs = [be.pack_for_prefill(w) for w in ws[:3]]
