@@ -1320,7 +1320,7 @@ static const int k_prefill_wgs_per_cu[] = {3, 3, 2, 1, 1, 1};
  * consumer kernel of Q4_K and Q5_K (one round of workgroups, several rounds) */
 static const double k_q45_K_step_us[] = {0.76, 1.14, 1.33, 1.91, 1.71, 2.60};
 static const double k_q6_K_step_us[] = {0.95, 1.33, 1.51, 2.43, 1.96, 3.10};
-static const double k_kquant_ws_step_us[2] = {1.45, 3.4};
+static const double k_kquant_ws_step_us[2] = {1.58, 3.4};
 static const struct { int tile; int waves; double step_us; int per_cu; int fill; } k_prefill_alt[] = {{3, 16, 1.25, 1, 2}, {2, 16, 0.82, 1, 1}, {5, 32, 2.20, 1, 3}};
 
 /* zero fill of Y and the atomic adds of `sp` partial sums per element, plus a launch: with few ranges the adds overlap
@@ -1349,7 +1349,8 @@ static double dense_estimate(int64_t M, int64_t N, int64_t K, int32_t cus, bool 
             const double fill = (double)rest / cus;
             double t = unpack + (double)full * steps * k_dense_step_us[v][0] +
                        (rest ? steps * k_dense_step_us[v][fill >= 0.8 ? 0 : fill >= 0.6 ? 1 : 2] : 0.0) + 5.0;
-            if (sp > 1) t += ksplit_overhead_us(M, N, sp, v ? 8 : 4);
+            /* four contributors per element of a 128-row tile all finish together: their adds cost more than two do */
+            if (sp > 1) t += (v && sp == 4) ? (double)(M * N) * 4.0 * (1.0 / 3.0e6 + 4.0 / 2.0e6) + 4.0 : ksplit_overhead_us(M, N, sp, v ? 8 : 4);
             if (t < best) { best = t; *bm_out = bm; *ksplit_out = sp; }
         }
     }
@@ -1473,7 +1474,11 @@ static int32_t prefill_plan_any(int32_t qtype, int64_t M, int64_t N, int64_t K, 
     }
     if (allow_dense && M > 64) {
         int sp = 1, bm = 256;
-        if (dense_estimate(M, N, K, cus, true, &bm, &sp) < 0.95 * best) {   /* two more launches and a workspace: only for a clear gain */
+        /* two more launches and a workspace: only for a clear gain -- except for the K-quants on matrices of 16 M
+         * weights and more, whose in-loop kernels the estimates flatter (their fp32 decode competes with the MFMAs
+         * for issue slots): there the dense family wins ties */
+        const double margin = (qtype == PSN_Q4_0 || qtype == PSN_Q8_0 || N * K < ((int64_t)1 << 24)) ? 0.95 : 1.05;
+        if (dense_estimate(M, N, K, cus, true, &bm, &sp) < margin * best) {
             *tile_m = bm;
             *tile_n = 256;
             *ksplit = sp;
