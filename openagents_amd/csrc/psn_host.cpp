@@ -1363,6 +1363,17 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
                                             int32_t *waves) {
     return psn_qmatmul_prefill_plan_for(PSN_Q4_0, M, N, K, cus, tile_m, tile_n, ksplit, waves);
 }
+/* at most 64 rows (Q4_0, Q8_0, Q4_K, Q5_K): the weight-streaming kernel on 64 x 64 tiles; K is cut (atomic adds) only
+ * while the weight rows alone leave half of the compute units without a workgroup, down to two chunks per range */
+static void plan_weight_stream(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit, int32_t *waves) {
+    const int64_t nt = (N + 63) / 64, C = K / 256;
+    int sp = 1;
+    while (nt * sp * 2 <= cus && C / (sp * 2) >= 2 && (M * N) % 4 == 0) sp *= 2;
+    *tile_m = 64;
+    *tile_n = 64;
+    *ksplit = sp;
+    *waves = 64;
+}
 static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit, int32_t *waves,
                               double *t_best) {
     if (!tile_m || !tile_n || !ksplit || !waves) return fail(PSN_E_INVALID_ARG, "psn_qmatmul_prefill_plan: out is null");
@@ -1371,15 +1382,7 @@ static int32_t plan_q4_0_q8_0(int64_t M, int64_t N, int64_t K, int32_t cus, int3
     if (M <= 0 || N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "prefill: M=%lld N=%lld K=%lld", (long long)M, (long long)N, (long long)K);
     if (cus <= 0) cus = 256;
     if (M <= 64) {
-        /* at most 64 rows: the weight-streaming kernel on 64 x 64 tiles; K is cut (atomic adds) only when
-         * the weight rows alone leave most compute units without a workgroup */
-        const int64_t nt = (N + 63) / 64, C = K / 256;
-        int sp = 1;
-        while (nt * sp * 2 <= cus && C / (sp * 2) >= 4 && (M * N) % 4 == 0) sp *= 2;
-        *tile_m = 64;
-        *tile_n = 64;
-        *ksplit = sp;
-        *waves = 64;
+        plan_weight_stream(M, N, K, cus, tile_m, tile_n, ksplit, waves);
         return PSN_OK;
     }
     /* estimated time = waves of workgroups over the chip's slots x K steps per workgroup x step cost,
@@ -1469,6 +1472,9 @@ static int32_t prefill_plan_any(int32_t qtype, int64_t M, int64_t N, int64_t K, 
         if (rc) return rc;
         if (M <= 64) return PSN_OK;                              /* the weight-streaming kernel */
         if (qtype == PSN_Q8_0) best *= 1.15;                     /* the step costs above were measured on Q4_0; Q8_0 stages twice the bytes */
+    } else if (M <= 64 && qtype != PSN_Q6_K) {
+        plan_weight_stream(M, N, K, cus, tile_m, tile_n, ksplit, waves);
+        return PSN_OK;
     } else {
         best = prefill_plan_kquant(qtype, M, N, K, cus, tile_m, tile_n, ksplit, waves);
     }
@@ -1592,9 +1598,9 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
         if ((rc = launch_unpack(mod, s, qtype, W->p, s->ws->p, N, K))) return rc;
         return launch_dense(mod, s, s->ws->p, X, Y, M, N, K, bm, ksplit);
     }
-    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !(waves == 16 && bm == 128 && bn == 256 && qtype != PSN_Q6_K))
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !((waves == 64 || (waves == 16 && bm == 128 && bn == 256)) && qtype != PSN_Q6_K))
         return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family%s", fmt_name(qtype),
-                    qtype == PSN_Q6_K ? " only (waves = 4)" : " and the 128x256 producer / consumer kernel (waves = 16)");
+                    qtype == PSN_Q6_K ? " only (waves = 4)" : ", the 128x256 producer / consumer kernel (waves = 16) and the weight-streaming kernel for M <= 64 (waves = 64)");
     /* waves == 64 selects the skinny kernel (M <= 64, 64 x 64 tiles, deep LDS rings) */
     const bool skinny = waves == 64;
     if (skinny && (bm != 64 || bn != 64 || M > 64)) return fail(PSN_E_UNSUPPORTED, "prefill: the skinny kernel serves M <= 64 with a 64x64 tile");
@@ -1611,8 +1617,9 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
     /* the interleaved kernels carry their LDS as static arrays; the skinny kernel: rings of three X chunks
-     * (64 rows x 256 k fp16) and six (Q4_0) or three (Q8_0) raw weight chunks (64 rows), reused for the final 8 x 16 KB reduction */
-    const int skinny_rings = 3 * 32768 + (qtype == PSN_Q4_0 ? 6 * 64 * 144 : 3 * 64 * 272);
+     * (64 rows x 256 k fp16) and six (Q4_0, Q4_K), five (Q5_K) or three (Q8_0) raw weight chunks (64 rows), reused for the final
+     * 8 x 16 KB reduction */
+    const int skinny_rings = 3 * 32768 + (qtype == PSN_Q4_0 || qtype == PSN_Q4_K ? 6 * 64 * 144 : qtype == PSN_Q5_K ? 5 * 64 * 176 : 3 * 64 * 272);
     const int wide_rings = 3 * (32768 + 256 * (qtype == PSN_Q4_0 ? 36 : 68));   /* three stages of X (256 rows x 64 k) and of raw blocks (two per row) */
     const int lds = skinny ? (skinny_rings > 8 * 16384 ? skinny_rings : 8 * 16384) : wide ? wide_rings : waves == 16 ? 0 : 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);

@@ -128,8 +128,12 @@ struct PfQ8_0 {
 
 /* ---- K-quant weights (Q4_K, Q5_K, Q6_K): a chunk is one super-block.  The reference dequantizes in fp32
  *      with one rounding per operation (d * sc, then * q, then - dmin * m); the fp16 weight the MFMA sees is
- *      that fp32 value rounded once more, so the same operations are spelled out here (no fused
- *      multiply-add) and converted with round-to-nearest-even. ---- */
+ *      that fp32 value rounded once more.  d (fp16, 11 significant bits) * sc (6 bits) * q (<= 5 bits) has at most
+ *      22 significant bits, so both products are exact in fp32 and only the subtraction rounds: one fused
+ *      multiply-add d1 * q - m1 returns the same fp32 value bit for bit, and converting it to fp16 with
+ *      round-to-nearest-even is the second rounding (the compiler emits v_cvt_f32_ubyteN + v_fma_mix{lo,hi}_f16:
+ *      two instructions per weight).  Q6_K: d * scale (19 bits) * (q - 32) (5 bits, or the power of two 32) is
+ *      exact; written as fma(ds, q, -32 ds) the unsigned byte converts directly. ---- */
 PSN_DEV u32 pack_h2_rn(float a, float b) {
     const half2_t v = {(_Float16)a, (_Float16)b};
     return h2_bits(v);
@@ -143,8 +147,8 @@ PSN_DEV void pf_kq_scales(u32 s0, u32 s1, u32 s2, u32 (&sc)[2], u32 (&mn)[2]) {
 template <int I> PSN_DEV float pf_byte(const u32 (&v)[2]) { return (float)((v[I >> 2] >> (8 * (I & 3))) & 0xffu); }
 /* four unsigned byte values of q -> d1 * q - m1, two packed pairs */
 PSN_DEV void pf_affine4(u32 q, float d1, float m1, u32 &lo, u32 &hi) {
-    const float v0 = __fsub_rn(__fmul_rn(d1, (float)(q & 0xffu)), m1), v1 = __fsub_rn(__fmul_rn(d1, (float)((q >> 8) & 0xffu)), m1);
-    const float v2 = __fsub_rn(__fmul_rn(d1, (float)((q >> 16) & 0xffu)), m1), v3 = __fsub_rn(__fmul_rn(d1, (float)(q >> 24)), m1);
+    const float v0 = __builtin_fmaf(d1, (float)(q & 0xffu), -m1), v1 = __builtin_fmaf(d1, (float)((q >> 8) & 0xffu), -m1);
+    const float v2 = __builtin_fmaf(d1, (float)((q >> 16) & 0xffu), -m1), v3 = __builtin_fmaf(d1, (float)(q >> 24), -m1);
     lo = pack_h2_rn(v0, v1);
     hi = pack_h2_rn(v2, v3);
 }
@@ -234,15 +238,12 @@ struct PfQ6_K {
         constexpr int si = 8 * h + 2 * t;                       /* scale of elements l < 16; l >= 16: si + 1 */
         const float ds0 = __fmul_rn(d, (float)(int)(int8_t)((w[48 + (si >> 2)] >> (8 * (si & 3))) & 0xffu));
         const float ds1 = __fmul_rn(d, (float)(int)(int8_t)((w[48 + ((si + 1) >> 2)] >> (8 * ((si + 1) & 3))) & 0xffu));
+        const float dm0 = ds0 * 32.f, dm1 = ds1 * 32.f;
         UNROLL for (int i = 0; i < 8; ++i) {
             const u32 nib = (w[16 * h + 8 * (t & 1) + i] >> (4 * (t >> 1))) & 0x0f0f0f0fu;
             const u32 top = ((w[32 + 8 * h + i] >> (2 * t)) & 0x03030303u) << 4;
             const u32 q = nib | top;
-            const float ds = i < 4 ? ds0 : ds1;
-            const float v0 = __fmul_rn(ds, (float)((int)(q & 0xffu) - 32)), v1 = __fmul_rn(ds, (float)((int)((q >> 8) & 0xffu) - 32));
-            const float v2 = __fmul_rn(ds, (float)((int)((q >> 16) & 0xffu) - 32)), v3 = __fmul_rn(ds, (float)((int)(q >> 24) - 32));
-            o[2 * i] = pack_h2_rn(v0, v1);
-            o[2 * i + 1] = pack_h2_rn(v2, v3);
+            pf_affine4(q, i < 4 ? ds0 : ds1, i < 4 ? dm0 : dm1, o[2 * i], o[2 * i + 1]);
         }
     }
 };
@@ -625,7 +626,7 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
  * every iteration issues the same number of loads and the outstanding-load count is a constant. */
 template <typename WF> struct SkinnyRings {
     static constexpr int XR = 3;                                /* X chunks in the ring */
-    static constexpr int RS = WF::DW == 36 ? 6 : 3;             /* raw weight chunks in the ring */
+    static constexpr int RS = WF::BYTES == 144 ? 6 : WF::BYTES == 176 ? 5 : 3;   /* raw weight chunks in the ring: what 160 KB hold beside X */
     static constexpr int XBYTES = 4 * 64 * 128, RBYTES = 64 * WF::BYTES;
     static constexpr int BYTES = XR * XBYTES + RS * RBYTES;
 };
@@ -634,20 +635,29 @@ template <typename WF> struct SkinnyRings {
  * multiply the block before, then decode); 2: waves 5..7.  EVEN: the wave's block index is even -- the
  * block starts on a dword (scale in the low half of its first dword, quants two bytes in: aligned dwords
  * are read and shifted; LDS reads that straddle dwords are very slow); an odd block starts two bytes
- * later (scale in the high half of the dword before, quants aligned). */
+ * later (scale in the high half of the dword before, quants aligned).  Q4_K / Q5_K: the chunk is the row's
+ * super-block and the wave's "block" its sub-block `wave` -- even ones sit in the low nibbles, odd ones in the
+ * high nibbles of the same 32 bytes; sub-blocks 0..3 (LOADER 0) and 4..7 unpack their 6-bit scale and min
+ * from different bytes of the 12-byte field; every LDS read is an aligned dword. */
 template <typename WF, int LOADER, bool EVEN>
 PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, int n0, int c_begin, int nq, int rot,
                                  u32 xs_base, u32 raw_base, __attribute__((address_space(3))) char *lds_ptr, u32 lds0, float16_t (&acc)[2][2]) {
     typedef SkinnyRings<WF> R;
-    constexpr bool Q4 = WF::DW == 36;
+    constexpr bool KQ = WF::KQ;                             /* Q4_K / Q5_K: the chunk is one super-block per row, wave w owns its sub-block w */
+    constexpr bool Q4 = !KQ && WF::DW == 36;
+    constexpr bool Q5K = KQ && WF::DW == 44;
     constexpr int XR = R::XR, RS = R::RS, XBYTES = R::XBYTES, RBYTES = R::RBYTES;
-    constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9 or 17 */
+    constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9, 11 or 17 */
     constexpr int CX = 8;                                   /* X loads per X wave and chunk (32 KB over 4 waves) */
-    constexpr int CR = RINSTR / 4 + (LOADER == 1 ? RINSTR % 4 : 0);   /* raw loads per weight wave and chunk */
+    /* raw loads per weight wave and chunk: wave 4 takes the one load that does not divide over four waves; when
+     * three are left over (Q5_K) every wave issues the same number and wave 7 repeats the chunk's last load */
+    constexpr bool EVEN_SHARE = RINSTR % 4 != 1;
+    constexpr int CR = EVEN_SHARE ? (RINSTR + 3) / 4 : RINSTR / 4 + (LOADER == 1 ? 1 : 0);
     constexpr int DEPTH = LOADER == 0 ? XR : RS, PER = LOADER == 0 ? CX : CR;
-    constexpr int BB = WF::BYTES / 8;                       /* bytes of a GGUF block: 18 or 34 */
+    constexpr int BB = WF::BYTES / 8;                       /* Q4_0 / Q8_0: bytes of a GGUF block: 18 or 34 */
     constexpr int NP = Q4 ? 1 : 2;                          /* raw register sets per block: Q4_0 keeps both slices in the same bytes */
-    static_assert(RINSTR % 4 == 1, "wave 4 takes the one load that does not divide over four waves");
+    static_assert(WF::BYTES % 16 == 0 && RBYTES % 1024 == 0, "whole 16-byte words per row, whole load instructions per chunk");
+    static_assert(!KQ || WF::DW == 36 || WF::DW == 44, "Q4_K and Q5_K only: Q6_K super-blocks do not start on 16-byte words");
     const int M = a.M, N = a.N, K = a.K;
     auto chunk_of = [&](int q) { const int r = min(q, nq - 1) + rot; return c_begin + (r >= nq ? r - nq : r); };
     auto issue = [&](int q) {
@@ -664,7 +674,7 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
         } else {
             __attribute__((address_space(3))) char *dst = lds_ptr + (raw_base - lds0) + (q % RS) * RBYTES;
             UNROLL for (int u = 0; u < CR; ++u) {
-                const int i = (wave - 4) + 4 * u;               /* instruction index; wave 4's last one is index 8 or 16 */
+                const int i = min((wave - 4) + 4 * u, RINSTR - 1);   /* instruction index; wave 4's last one is index 8 or 16 */
                 const int word = i * 64 + lane, row = word / (WF::BYTES / 16), wd = word % (WF::BYTES / 16);
                 const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + (int64_t)c * WF::BYTES + wd * 16;
                 __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
@@ -677,17 +687,52 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
     const int h = lane >> 5;
     u32 xlane[2];
     UNROLL for (int sl = 0; sl < 2; ++sl) xlane[sl] = (u32)((wave >> 1) * 8192 + tile_off(lane & 31, 2 * (2 * (wave & 1) + sl) + h));
-    const u32 rlane = (u32)((lane & 31) * WF::BYTES + wave * BB), qlane = rlane + 8u * (u32)h;
+    /* K-quants: the row's super-block; its quants of sub-block `wave` (bytes 32 (wave / 2) .. + 31 of the nibble
+     * array, this lane's eight at 8h and 16 + 8h); Q5_K: the fifth bits of the same elements (qh, bit `wave`) */
+    const u32 rlane = KQ ? (u32)((lane & 31) * WF::BYTES) : (u32)((lane & 31) * WF::BYTES + wave * BB);
+    const u32 qlane = KQ ? rlane + (u32)((Q5K ? 48 : 16) + 32 * (wave >> 1) + 8 * h) : rlane + 8u * (u32)h;
+    const u32 hlane = rlane + (u32)(16 + 8 * h);
     constexpr int ROW32 = 32 * WF::BYTES;
 
-    struct unit { u32x4 xf[2][2]; u32 raw[NP][2][3], wd[2]; };
+    /* kq[j]: 0 = d | dmin << 16, 1..3 = the three scale dwords, 4..7 = quants (slice 0: two dwords, slice 1), 8..11 = qh likewise */
+    struct unit { u32x4 xf[2][2]; u32 raw[KQ ? 1 : NP][2][3], wd[2], kq[2][KQ ? 12 : 1]; };
     auto fetch = [&](u32 xst, u32 rst, unit &t) {
         const u32 xa0 = xst + xlane[0], xa1 = xst + xlane[1], rw = rst + rlane, rq = rst + qlane;
         t.xf[0][0] = lds_read128<0>(xa0);
         t.xf[0][1] = lds_read128<4096>(xa0);
         t.xf[1][0] = lds_read128<0>(xa1);
         t.xf[1][1] = lds_read128<4096>(xa1);
-        if constexpr (EVEN) {
+        if constexpr (KQ) {
+            const u32 rh = rst + hlane;
+            t.kq[0][0] = lds_read32o<0>(rw);
+            t.kq[1][0] = lds_read32o<ROW32>(rw);
+            t.kq[0][1] = lds_read32o<4>(rw);
+            t.kq[1][1] = lds_read32o<ROW32 + 4>(rw);
+            t.kq[0][2] = lds_read32o<8>(rw);
+            t.kq[1][2] = lds_read32o<ROW32 + 8>(rw);
+            if constexpr (LOADER != 0) {                                     /* sub-blocks 4..7: high bits in dwords 1, 2, low in 3 */
+                t.kq[0][3] = lds_read32o<12>(rw);
+                t.kq[1][3] = lds_read32o<ROW32 + 12>(rw);
+            }
+            t.kq[0][4] = lds_read32o<0>(rq);
+            t.kq[0][5] = lds_read32o<4>(rq);
+            t.kq[0][6] = lds_read32o<16>(rq);
+            t.kq[0][7] = lds_read32o<20>(rq);
+            t.kq[1][4] = lds_read32o<ROW32>(rq);
+            t.kq[1][5] = lds_read32o<ROW32 + 4>(rq);
+            t.kq[1][6] = lds_read32o<ROW32 + 16>(rq);
+            t.kq[1][7] = lds_read32o<ROW32 + 20>(rq);
+            if constexpr (Q5K) {
+                t.kq[0][8] = lds_read32o<0>(rh);
+                t.kq[0][9] = lds_read32o<4>(rh);
+                t.kq[0][10] = lds_read32o<16>(rh);
+                t.kq[0][11] = lds_read32o<20>(rh);
+                t.kq[1][8] = lds_read32o<ROW32>(rh);
+                t.kq[1][9] = lds_read32o<ROW32 + 4>(rh);
+                t.kq[1][10] = lds_read32o<ROW32 + 16>(rh);
+                t.kq[1][11] = lds_read32o<ROW32 + 20>(rh);
+            }
+        } else if constexpr (EVEN) {
             t.wd[0] = lds_read32o<0>(rw);                                    /* scale | first two quant bytes */
             t.wd[1] = lds_read32o<ROW32>(rw);
             UNROLL for (int p = 0; p < NP; ++p) {
@@ -714,14 +759,39 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
     auto arrived = [&](unit &t) {
         tie(t.xf[0]);
         tie(t.xf[1]);
-        UNROLL for (int j = 0; j < 2; ++j) {
+        if constexpr (KQ) {
+            UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int i = 0; i < (Q5K ? 12 : 8); ++i)
+                if (i != 3 || LOADER != 0) tie1(t.kq[j][i]);
+        } else UNROLL for (int j = 0; j < 2; ++j) {
             tie1(t.wd[j]);
             UNROLL for (int p = 0; p < NP; ++p) { tie1(t.raw[p][j][0]); tie1(t.raw[p][j][1]); if (EVEN) tie1(t.raw[p][j][2]); }
         }
     };
     /* MFMA operands of the block's two slices, column blocks j = 0, 1 */
     auto decode = [&](const unit &t, u32x4 (&wf)[2][2]) {
-        UNROLL for (int j = 0; j < 2; ++j) {
+        if constexpr (KQ) {
+            const int sh = 8 * (wave & 3);                  /* this sub-block's byte of the scale dwords */
+            UNROLL for (int j = 0; j < 2; ++j) {
+                u32 sc, mn;
+                if constexpr (LOADER == 0) {
+                    sc = (t.kq[j][1] >> sh) & 63u;
+                    mn = (t.kq[j][2] >> sh) & 63u;
+                } else {
+                    sc = ((t.kq[j][3] >> sh) & 0xfu) | (((t.kq[j][1] >> sh) >> 2) & 0x30u);
+                    mn = ((t.kq[j][3] >> (sh + 4)) & 0xfu) | (((t.kq[j][2] >> sh) >> 2) & 0x30u);
+                }
+                const float d1 = __fmul_rn(h2f_lo(t.kq[j][0]), (float)sc), m1 = __fmul_rn(h2f_hi(t.kq[j][0]), (float)mn);
+                UNROLL for (int sl = 0; sl < 2; ++sl) {
+                    u32 o[4];
+                    UNROLL for (int e = 0; e < 2; ++e) {
+                        u32 q = (EVEN ? t.kq[j][4 + 2 * sl + e] : t.kq[j][4 + 2 * sl + e] >> 4) & 0x0f0f0f0fu;
+                        if constexpr (Q5K) q |= ((t.kq[j][8 + 2 * sl + e] >> wave) & 0x01010101u) << 4;
+                        pf_affine4(q, d1, m1, o[2 * e], o[2 * e + 1]);
+                    }
+                    wf[sl][j] = (u32x4){o[0], o[1], o[2], o[3]};
+                }
+            }
+        } else UNROLL for (int j = 0; j < 2; ++j) {
             const half2_t w2 = bits_h2(t.wd[j]);
             const half2_t d2 = EVEN ? __builtin_shufflevector(w2, w2, 0, 0) : __builtin_shufflevector(w2, w2, 1, 1);
             u32 q[NP][2];
@@ -1345,6 +1415,8 @@ extern "C" __global__ void __launch_bounds__(256) psn_fill_zero(const psn_fill_a
 }
 PSN_PREFILL_KERNEL_SKINNY(q4_0, PfQ4_0)
 PSN_PREFILL_KERNEL_SKINNY(q8_0, PfQ8_0)
+PSN_PREFILL_KERNEL_SKINNY(q4_K, PfQ4_K)
+PSN_PREFILL_KERNEL_SKINNY(q5_K, PfQ5_K)
 #endif
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 2
 PSN_PREFILL_KERNEL_WIDE(q4_0, PfQ4_0)

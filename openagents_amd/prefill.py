@@ -33,8 +33,9 @@ from ._ffi import Q4_0, Q4_K, Q5_K, Q6_K, Q8_0
 from .backend import HipBackend, PsnError, prefill_plan, row_bytes
 
 # (tile_m, tile_n, ksplit, family): the explicit plans --compare-plans tries (family 4 = four waves, 16 = producer / consumer,
-# 32 = wide, 128 = dense)
-EXPLICIT_PLANS = [(64, 64, 2, 4), (64, 64, 4, 4), (64, 64, 8, 4), (64, 128, 2, 4), (64, 128, 4, 4), (64, 128, 8, 4), (256, 128, 2, 4), (256, 128, 4, 4), (256, 128, 8, 4),
+# 32 = wide, 64 = weight-streaming for M <= 64, 128 = dense)
+EXPLICIT_PLANS = [(64, 64, 1, 64), (64, 64, 2, 64), (64, 64, 4, 64), (64, 64, 8, 64),
+                  (64, 64, 2, 4), (64, 64, 4, 4), (64, 64, 8, 4), (64, 128, 2, 4), (64, 128, 4, 4), (64, 128, 8, 4), (256, 128, 2, 4), (256, 128, 4, 4), (256, 128, 8, 4),
                   (128, 128, 1, 4), (256, 128, 1, 4), (256, 256, 1, 4), (256, 256, 2, 4), (256, 256, 4, 4),
                   (128, 128, 1, 16), (128, 128, 2, 16), (128, 128, 4, 16), (128, 128, 8, 16),
                   (128, 256, 1, 16), (128, 256, 2, 16), (128, 256, 4, 16), (128, 256, 8, 16),
