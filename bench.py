@@ -210,7 +210,7 @@ def main(argv=None):
     ap.add_argument("--seed", type=int, default=1234)
     ap.add_argument("--calibrate-copy", action="store_true", help="also run four 256 MiB device-to-device copies (counter calibration)")
     ap.add_argument("--no-records", action="store_true", help="headline only: skip the records of the other configurations")
-    ap.add_argument("--record-samples", type=int, default=7)
+    ap.add_argument("--record-samples", type=int, default=21)
     ap.add_argument("--records-out", default=os.path.join("gpurun_out", "bench_records.json"),
                     help="file that receives the full records, the per-launch table and the calibration")
     ap.add_argument("--vendor-gemm", action="store_true",
