@@ -121,3 +121,14 @@ def test_read_sweep_geometries_fit_a_compute_unit():
         per_cu = blocks // 256
         assert blocks % 256 == 0 and threads in (256, 512) and per_cu * threads <= 2048
         assert per_cu * (threads // 64) * depth * 1024 <= 160 * 1024
+
+
+def test_measured_traffic_constants_are_the_ones_in_the_committed_profile():
+    """bench.py's `roofline.traffic` figures are pasted from a rocprofv3 counter summary: every constant must
+    still stand in that summary's table (a refreshed profile with an unrefreshed constant fails here), and the
+    file must name the kernel of the headline's dominant launch."""
+    text = open(os.path.join(ROOT, "profiles", "matvec_q4_0_llama3_8b_step.md")).read()
+    assert bench.MEASURED_TRAFFIC_BYTES, "no traffic constants"
+    for kernel, nbytes in bench.MEASURED_TRAFFIC_BYTES.items():
+        assert f"{nbytes:,}".replace(",", " ") in text, (kernel, nbytes)
+    assert "psn_mvs_q4_0_q8_g16_xf_s2" in text
