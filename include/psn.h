@@ -273,7 +273,7 @@ int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, i
 /* Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k]; X fp16 [M][K], Y fp32 [M][N], weight tiles are
  * dequantized to fp16 (h = round to nearest even) in LDS and fed to fp16 MFMA with fp32
  * accumulation.  qtype PSN_Q4_0 or PSN_Q8_0 (every kernel family below), PSN_Q4_K, PSN_Q5_K or PSN_Q6_K
- * (families 4 and 128, and for Q4_K / Q5_K family 16 on the 128x256 tile and family 64; planned by psn_qmatmul_prefill_plan_for;
+ * (families 4, 64 and 128, and for Q4_K / Q5_K family 16 on the 128x256 tile; planned by psn_qmatmul_prefill_plan_for;
  * their fp32 dequantization is restated operation by operation before the rounding to fp16).  Replaces the CUDA backend's quantized prefill
  * matmul op. */
 int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W,
@@ -288,8 +288,8 @@ int32_t psn_qmatmul_prefill(psn_module *mod, psn_stream *s, int32_t qtype, int32
  *   32  the wide kernel for large M (256x256 tiles only): four waves, each with all 256 rows x 64 columns
  *       in 256 accumulator registers; X and the raw GGUF bytes arrive in LDS rings by direct-to-LDS loads,
  *       a wave decodes the operand of its own columns one K slice ahead, interleaved with its MFMAs;
- *   64  the weight-streaming kernel for M <= 64 (64x64 tiles; Q4_0, Q8_0, Q4_K, Q5_K -- not Q6_K, whose 210-byte
- *       super-blocks do not start on 16-byte words): X and the raw GGUF bytes arrive in LDS rings by
+ *   64  the weight-streaming kernel for M <= 64 (64x64 tiles; every format, Q6_K only when K is a multiple of
+ *       2048 so that its rows are whole 16-byte words): X and the raw GGUF bytes arrive in LDS rings by
  *       direct-to-LDS loads, every wave decodes its own MFMA operand, one barrier per 256 of K;
  *  128  the dense family for large M (256x256 or 128x256 tiles, every format): one pass writes h(deq(W)) for the whole
  *       matrix as fp16 into the stream's workspace (ceil(N/256) * 256 * K * 2 bytes, see
@@ -300,7 +300,7 @@ int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int32_t comput
                                  int32_t *ksplit, int32_t *waves);
 /* The same for a given weight type: what psn_qmatmul_prefill runs when the dense family's workspace is
  * available (psn_qmatmul_prefill_plan answers for Q4_0 / Q8_0; the K-quants have families 4, 16 on the
- * 128x256 tile, 128, and -- Q4_K / Q5_K -- 64 for M <= 64).  While a stream is capturing, or while a captured graph refers to its workspace,
+ * 128x256 tile, 128, and 64 for M <= 64).  While a stream is capturing, or while a captured graph refers to its workspace,
  * the workspace cannot grow: psn_qmatmul_prefill then takes the best plan without family 128 unless
  * psn_prefill_reserve (or an earlier dense call of that size) has sized it. */
 int32_t psn_qmatmul_prefill_plan_for(int32_t qtype, int64_t M, int64_t N, int64_t K, int32_t compute_units, int32_t *tile_m,

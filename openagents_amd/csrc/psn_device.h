@@ -129,6 +129,7 @@ PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out
  * as memory traffic, and vmcnt / lgkmcnt waits are explicit (loads complete in issue order, so "at
  * most n younger loads outstanding" identifies what has landed). */
 typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
 
 /* wave-uniform n: wait until at most n vector-memory loads are outstanding */
 PSN_DEV void wait_vmcnt(int n) {
@@ -161,6 +162,11 @@ PSN_DEV u32 lds_read32(u32 addr) {
 template <int OFF> PSN_DEV u32 lds_read32o(u32 addr) {
     u32 v;
     asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
+    return v;
+}
+template <int OFF> PSN_DEV u32x2 lds_read64o(u32 addr) {          /* addr + OFF: a multiple of 8 */
+    u32x2 v;
+    asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
     return v;
 }
 PSN_DEV u32 lds_read_u16(u32 addr) {

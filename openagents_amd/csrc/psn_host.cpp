@@ -1363,7 +1363,7 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
                                             int32_t *waves) {
     return psn_qmatmul_prefill_plan_for(PSN_Q4_0, M, N, K, cus, tile_m, tile_n, ksplit, waves);
 }
-/* at most 64 rows (Q4_0, Q8_0, Q4_K, Q5_K): the weight-streaming kernel on 64 x 64 tiles; K is cut (atomic adds) only
+/* at most 64 rows (every format; Q6_K when its rows are whole 16-byte words): the weight-streaming kernel on 64 x 64 tiles; K is cut (atomic adds) only
  * while the weight rows alone leave half of the compute units without a workgroup, down to two chunks per range */
 static void plan_weight_stream(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit, int32_t *waves) {
     const int64_t nt = (N + 63) / 64, C = K / 256;
@@ -1472,7 +1472,7 @@ static int32_t prefill_plan_any(int32_t qtype, int64_t M, int64_t N, int64_t K, 
         if (rc) return rc;
         if (M <= 64) return PSN_OK;                              /* the weight-streaming kernel */
         if (qtype == PSN_Q8_0) best *= 1.15;                     /* the step costs above were measured on Q4_0; Q8_0 stages twice the bytes */
-    } else if (M <= 64 && qtype != PSN_Q6_K) {
+    } else if (M <= 64 && (qtype != PSN_Q6_K || K % 2048 == 0)) {
         plan_weight_stream(M, N, K, cus, tile_m, tile_n, ksplit, waves);
         return PSN_OK;
     } else {
@@ -1598,12 +1598,14 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
         if ((rc = launch_unpack(mod, s, qtype, W->p, s->ws->p, N, K))) return rc;
         return launch_dense(mod, s, s->ws->p, X, Y, M, N, K, bm, ksplit);
     }
-    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && !((waves == 64 || (waves == 16 && bm == 128 && bn == 256)) && qtype != PSN_Q6_K))
-        return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family%s", fmt_name(qtype),
-                    qtype == PSN_Q6_K ? " only (waves = 4)" : ", the 128x256 producer / consumer kernel (waves = 16) and the weight-streaming kernel for M <= 64 (waves = 64)");
+    if (qtype != PSN_Q4_0 && qtype != PSN_Q8_0 && waves != 4 && waves != 64 && !(waves == 16 && bm == 128 && bn == 256 && qtype != PSN_Q6_K))
+        return fail(PSN_E_UNSUPPORTED, "prefill: %s has the four-wave kernel family, the weight-streaming kernel for M <= 64 (waves = 64)%s", fmt_name(qtype),
+                    qtype == PSN_Q6_K ? "" : " and the 128x256 producer / consumer kernel (waves = 16)");
     /* waves == 64 selects the skinny kernel (M <= 64, 64 x 64 tiles, deep LDS rings) */
     const bool skinny = waves == 64;
     if (skinny && (bm != 64 || bn != 64 || M > 64)) return fail(PSN_E_UNSUPPORTED, "prefill: the skinny kernel serves M <= 64 with a 64x64 tile");
+    /* Q6_K super-blocks (210 bytes) are fetched as windows of aligned 16-byte words: the rows must start on one */
+    if (skinny && qtype == PSN_Q6_K && K % 2048) return fail(PSN_E_UNSUPPORTED, "prefill: the skinny Q6_K kernel needs K to be a multiple of 2048 (K=%lld)", (long long)K);
     /* waves == 32 selects the wide kernel: 256 x 256 tiles, four waves with 128 x 128 each, weights decoded
      * from raw bytes in LDS by the wave that multiplies them */
     const bool wide = waves == 32;
@@ -1617,9 +1619,9 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
     /* the interleaved kernels carry their LDS as static arrays; the skinny kernel: rings of three X chunks
-     * (64 rows x 256 k fp16) and six (Q4_0, Q4_K), five (Q5_K) or three (Q8_0) raw weight chunks (64 rows), reused for the final
+     * (64 rows x 256 k fp16) and six (Q4_0, Q4_K), five (Q5_K), four (Q6_K) or three (Q8_0) raw weight chunks (64 rows), reused for the final
      * 8 x 16 KB reduction */
-    const int skinny_rings = 3 * 32768 + (qtype == PSN_Q4_0 || qtype == PSN_Q4_K ? 6 * 64 * 144 : qtype == PSN_Q5_K ? 5 * 64 * 176 : 3 * 64 * 272);
+    const int skinny_rings = 3 * 32768 + (qtype == PSN_Q4_0 || qtype == PSN_Q4_K ? 6 * 64 * 144 : qtype == PSN_Q5_K ? 5 * 64 * 176 : qtype == PSN_Q6_K ? 4 * 64 * 240 : 3 * 64 * 272);
     const int wide_rings = 3 * (32768 + 256 * (qtype == PSN_Q4_0 ? 36 : 68));   /* three stages of X (256 rows x 64 k) and of raw blocks (two per row) */
     const int lds = skinny ? (skinny_rings > 8 * 16384 ? skinny_rings : 8 * 16384) : wide ? wide_rings : waves == 16 ? 0 : 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);

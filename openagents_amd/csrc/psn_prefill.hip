@@ -626,8 +626,14 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
  * every iteration issues the same number of loads and the outstanding-load count is a constant. */
 template <typename WF> struct SkinnyRings {
     static constexpr int XR = 3;                                /* X chunks in the ring */
-    static constexpr int RS = WF::BYTES == 144 ? 6 : WF::BYTES == 176 ? 5 : 3;   /* raw weight chunks in the ring: what 160 KB hold beside X */
-    static constexpr int XBYTES = 4 * 64 * 128, RBYTES = 64 * WF::BYTES;
+    /* bytes of a row's chunk in LDS.  Q6_K's 210-byte super-blocks start on 2-byte boundaries: what is loaded is the
+     * window of fourteen aligned 16-byte words that holds the super-block (rows must be whole 16-byte words, K a
+     * multiple of 2048; chunk c then starts (210 c) mod 16 bytes into its window, the same for every row), and a
+     * fifteenth word of padding: with 224 bytes between rows, every fourth row would share its LDS banks */
+    static constexpr int WORDS = (WF::BYTES + 14 + 15) / 16;     /* words that hold a chunk of a row whatever its alignment */
+    static constexpr int LROW = WF::BYTES % 16 == 0 ? WF::BYTES : (WORDS + 1) * 16;
+    static constexpr int RS = LROW == 144 ? 6 : LROW == 176 ? 5 : LROW == 240 ? 4 : 3;   /* raw weight chunks in the ring: what 160 KB hold beside X */
+    static constexpr int XBYTES = 4 * 64 * 128, RBYTES = 64 * LROW;
     static constexpr int BYTES = XR * XBYTES + RS * RBYTES;
 };
 
@@ -638,7 +644,9 @@ template <typename WF> struct SkinnyRings {
  * later (scale in the high half of the dword before, quants aligned).  Q4_K / Q5_K: the chunk is the row's
  * super-block and the wave's "block" its sub-block `wave` -- even ones sit in the low nibbles, odd ones in the
  * high nibbles of the same 32 bytes; sub-blocks 0..3 (LOADER 0) and 4..7 unpack their 6-bit scale and min
- * from different bytes of the 12-byte field; every LDS read is an aligned dword. */
+ * from different bytes of the 12-byte field; every LDS read is an aligned dword.  Q6_K: sub-block `wave` again
+ * (LOADER 0: the super-block's first half; EVEN: the first 32 of a 64-byte group of ql); its fields start on
+ * 2-byte boundaries, so three aligned dwords are read around each eight bytes and shifted with v_alignbyte. */
 template <typename WF, int LOADER, bool EVEN>
 PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, int n0, int c_begin, int nq, int rot,
                                  u32 xs_base, u32 raw_base, __attribute__((address_space(3))) char *lds_ptr, u32 lds0, float16_t (&acc)[2][2]) {
@@ -646,18 +654,19 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
     constexpr bool KQ = WF::KQ;                             /* Q4_K / Q5_K: the chunk is one super-block per row, wave w owns its sub-block w */
     constexpr bool Q4 = !KQ && WF::DW == 36;
     constexpr bool Q5K = KQ && WF::DW == 44;
-    constexpr int XR = R::XR, RS = R::RS, XBYTES = R::XBYTES, RBYTES = R::RBYTES;
-    constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9, 11 or 17 */
+    constexpr bool Q6K = KQ && WF::DW == 53;
+    constexpr int XR = R::XR, RS = R::RS, XBYTES = R::XBYTES, RBYTES = R::RBYTES, LROW = R::LROW;
+    constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9, 11, 15 or 17 */
     constexpr int CX = 8;                                   /* X loads per X wave and chunk (32 KB over 4 waves) */
     /* raw loads per weight wave and chunk: wave 4 takes the one load that does not divide over four waves; when
-     * three are left over (Q5_K) every wave issues the same number and wave 7 repeats the chunk's last load */
+     * three or two are left over (Q5_K, Q6_K) every wave issues the same number and the last waves repeat the chunk's
+     * last load */
     constexpr bool EVEN_SHARE = RINSTR % 4 != 1;
     constexpr int CR = EVEN_SHARE ? (RINSTR + 3) / 4 : RINSTR / 4 + (LOADER == 1 ? 1 : 0);
     constexpr int DEPTH = LOADER == 0 ? XR : RS, PER = LOADER == 0 ? CX : CR;
     constexpr int BB = WF::BYTES / 8;                       /* Q4_0 / Q8_0: bytes of a GGUF block: 18 or 34 */
     constexpr int NP = Q4 ? 1 : 2;                          /* raw register sets per block: Q4_0 keeps both slices in the same bytes */
-    static_assert(WF::BYTES % 16 == 0 && RBYTES % 1024 == 0, "whole 16-byte words per row, whole load instructions per chunk");
-    static_assert(!KQ || WF::DW == 36 || WF::DW == 44, "Q4_K and Q5_K only: Q6_K super-blocks do not start on 16-byte words");
+    static_assert(LROW % 16 == 0 && RBYTES % 1024 == 0, "whole 16-byte words per row, whole load instructions per chunk");
     const int M = a.M, N = a.N, K = a.K;
     auto chunk_of = [&](int q) { const int r = min(q, nq - 1) + rot; return c_begin + (r >= nq ? r - nq : r); };
     auto issue = [&](int q) {
@@ -675,8 +684,9 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
             __attribute__((address_space(3))) char *dst = lds_ptr + (raw_base - lds0) + (q % RS) * RBYTES;
             UNROLL for (int u = 0; u < CR; ++u) {
                 const int i = min((wave - 4) + 4 * u, RINSTR - 1);   /* instruction index; wave 4's last one is index 8 or 16 */
-                const int word = i * 64 + lane, row = word / (WF::BYTES / 16), wd = word % (WF::BYTES / 16);
-                const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + (int64_t)c * WF::BYTES + wd * 16;
+                const int word = i * 64 + lane, row = word / (LROW / 16), wd = Q6K ? min(word % (LROW / 16), R::WORDS - 1) : word % (LROW / 16);
+                const int64_t coff = Q6K ? (int64_t)((c * WF::BYTES) & ~15) : (int64_t)c * WF::BYTES;
+                const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + coff + wd * 16;
                 __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
             }
         }
@@ -689,48 +699,72 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
     UNROLL for (int sl = 0; sl < 2; ++sl) xlane[sl] = (u32)((wave >> 1) * 8192 + tile_off(lane & 31, 2 * (2 * (wave & 1) + sl) + h));
     /* K-quants: the row's super-block; its quants of sub-block `wave` (bytes 32 (wave / 2) .. + 31 of the nibble
      * array, this lane's eight at 8h and 16 + 8h); Q5_K: the fifth bits of the same elements (qh, bit `wave`) */
-    const u32 rlane = KQ ? (u32)((lane & 31) * WF::BYTES) : (u32)((lane & 31) * WF::BYTES + wave * BB);
-    const u32 qlane = KQ ? rlane + (u32)((Q5K ? 48 : 16) + 32 * (wave >> 1) + 8 * h) : rlane + 8u * (u32)h;
-    const u32 hlane = rlane + (u32)(16 + 8 * h);
-    constexpr int ROW32 = 32 * WF::BYTES;
+    /* Q6_K, sub-block `wave` = half wave / 4, quarter t = wave % 4 of the super-block: low bits in ql[64 half + 32 (t & 1)
+     * + l] (high nibble for t >= 2), bits 4..5 in qh[32 half + l] >> 2 t, int8 scales[8 half + 2 t + l / 16], d at 208 */
+    const u32 rlane = KQ ? (u32)((lane & 31) * LROW) : (u32)((lane & 31) * LROW + wave * BB);
+    const u32 qlane = Q6K ? rlane + (u32)(64 * (LOADER != 0) + 32 * !EVEN + 8 * h)
+                    : KQ  ? rlane + (u32)((Q5K ? 48 : 16) + 32 * (wave >> 1) + 8 * h) : rlane + 8u * (u32)h;
+    const u32 hlane = Q6K ? rlane + (u32)(128 + 32 * (LOADER != 0) + 8 * h) : rlane + (u32)(16 + 8 * h);
+    constexpr int ROW32 = 32 * LROW;
 
-    /* kq[j]: 0 = d | dmin << 16, 1..3 = the three scale dwords, 4..7 = quants (slice 0: two dwords, slice 1), 8..11 = qh likewise */
-    struct unit { u32x4 xf[2][2]; u32 raw[KQ ? 1 : NP][2][3], wd[2], kq[2][KQ ? 12 : 1]; };
-    auto fetch = [&](u32 xst, u32 rst, unit &t) {
+    /* Q4_K / Q5_K: kh[j] = d | dmin << 16 and the three scale dwords, kv[j][0..1] = quants of slice 0, 1 (two dwords each),
+     * kv[j][2..3] = qh likewise; Q6_K, kq[j]: 0..5 = the aligned dwords around ql (three per slice), 6..11 = around qh,
+     * 12 = the two scales, 13 = d */
+    struct unit { u32x4 xf[2][2]; u32 raw[KQ ? 1 : NP][2][3], wd[2], kq[2][Q6K ? 14 : 1]; u32x4 kh[2]; u32x2 kv[2][4]; };
+    /* `o`: Q6_K only, where in its 16-byte-aligned window this chunk's super-block starts (even, wave-uniform) */
+    auto fetch = [&](u32 xst, u32 rst, unit &t, u32 o) {
         const u32 xa0 = xst + xlane[0], xa1 = xst + xlane[1], rw = rst + rlane, rq = rst + qlane;
         t.xf[0][0] = lds_read128<0>(xa0);
         t.xf[0][1] = lds_read128<4096>(xa0);
         t.xf[1][0] = lds_read128<0>(xa1);
         t.xf[1][1] = lds_read128<4096>(xa1);
-        if constexpr (KQ) {
+        if constexpr (Q6K) {
+            /* every field starts o bytes into the record; o mod 4 is 0 or 2: aligned dwords are read and shifted in decode */
+            const u32 ob = o & ~3u, ql = rq + ob, qh = rst + hlane + ob;
+            const u32 sc = rw + (u32)(192 + 8 * (LOADER != 0)) + 2u * (u32)(wave & 3) + o, dd = rw + 208u + o;
+            t.kq[0][0] = lds_read32o<0>(ql);
+            t.kq[0][1] = lds_read32o<4>(ql);
+            t.kq[0][2] = lds_read32o<8>(ql);
+            t.kq[0][3] = lds_read32o<16>(ql);
+            t.kq[0][4] = lds_read32o<20>(ql);
+            t.kq[0][5] = lds_read32o<24>(ql);
+            t.kq[1][0] = lds_read32o<ROW32>(ql);
+            t.kq[1][1] = lds_read32o<ROW32 + 4>(ql);
+            t.kq[1][2] = lds_read32o<ROW32 + 8>(ql);
+            t.kq[1][3] = lds_read32o<ROW32 + 16>(ql);
+            t.kq[1][4] = lds_read32o<ROW32 + 20>(ql);
+            t.kq[1][5] = lds_read32o<ROW32 + 24>(ql);
+            t.kq[0][6] = lds_read32o<0>(qh);
+            t.kq[0][7] = lds_read32o<4>(qh);
+            t.kq[0][8] = lds_read32o<8>(qh);
+            t.kq[0][9] = lds_read32o<16>(qh);
+            t.kq[0][10] = lds_read32o<20>(qh);
+            t.kq[0][11] = lds_read32o<24>(qh);
+            t.kq[1][6] = lds_read32o<ROW32>(qh);
+            t.kq[1][7] = lds_read32o<ROW32 + 4>(qh);
+            t.kq[1][8] = lds_read32o<ROW32 + 8>(qh);
+            t.kq[1][9] = lds_read32o<ROW32 + 16>(qh);
+            t.kq[1][10] = lds_read32o<ROW32 + 20>(qh);
+            t.kq[1][11] = lds_read32o<ROW32 + 24>(qh);
+            t.kq[0][12] = lds_read_u16(sc);
+            t.kq[1][12] = lds_read_u16(sc + (u32)ROW32);
+            t.kq[0][13] = lds_read_u16(dd);
+            t.kq[1][13] = lds_read_u16(dd + (u32)ROW32);
+        } else if constexpr (KQ) {
+            /* a 32-bit read of 32 rows hits each LDS bank four times (rows are whole 16-byte words apart) and takes as long
+             * as a conflict-free 128-bit one: the header word (d, dmin, scales) is read whole, the quants 64 bits at a time */
             const u32 rh = rst + hlane;
-            t.kq[0][0] = lds_read32o<0>(rw);
-            t.kq[1][0] = lds_read32o<ROW32>(rw);
-            t.kq[0][1] = lds_read32o<4>(rw);
-            t.kq[1][1] = lds_read32o<ROW32 + 4>(rw);
-            t.kq[0][2] = lds_read32o<8>(rw);
-            t.kq[1][2] = lds_read32o<ROW32 + 8>(rw);
-            if constexpr (LOADER != 0) {                                     /* sub-blocks 4..7: high bits in dwords 1, 2, low in 3 */
-                t.kq[0][3] = lds_read32o<12>(rw);
-                t.kq[1][3] = lds_read32o<ROW32 + 12>(rw);
-            }
-            t.kq[0][4] = lds_read32o<0>(rq);
-            t.kq[0][5] = lds_read32o<4>(rq);
-            t.kq[0][6] = lds_read32o<16>(rq);
-            t.kq[0][7] = lds_read32o<20>(rq);
-            t.kq[1][4] = lds_read32o<ROW32>(rq);
-            t.kq[1][5] = lds_read32o<ROW32 + 4>(rq);
-            t.kq[1][6] = lds_read32o<ROW32 + 16>(rq);
-            t.kq[1][7] = lds_read32o<ROW32 + 20>(rq);
+            t.kh[0] = lds_read128<0>(rw);
+            t.kh[1] = lds_read128<ROW32>(rw);
+            t.kv[0][0] = lds_read64o<0>(rq);
+            t.kv[0][1] = lds_read64o<16>(rq);
+            t.kv[1][0] = lds_read64o<ROW32>(rq);
+            t.kv[1][1] = lds_read64o<ROW32 + 16>(rq);
             if constexpr (Q5K) {
-                t.kq[0][8] = lds_read32o<0>(rh);
-                t.kq[0][9] = lds_read32o<4>(rh);
-                t.kq[0][10] = lds_read32o<16>(rh);
-                t.kq[0][11] = lds_read32o<20>(rh);
-                t.kq[1][8] = lds_read32o<ROW32>(rh);
-                t.kq[1][9] = lds_read32o<ROW32 + 4>(rh);
-                t.kq[1][10] = lds_read32o<ROW32 + 16>(rh);
-                t.kq[1][11] = lds_read32o<ROW32 + 20>(rh);
+                t.kv[0][2] = lds_read64o<0>(rh);
+                t.kv[0][3] = lds_read64o<16>(rh);
+                t.kv[1][2] = lds_read64o<ROW32>(rh);
+                t.kv[1][3] = lds_read64o<ROW32 + 16>(rh);
             }
         } else if constexpr (EVEN) {
             t.wd[0] = lds_read32o<0>(rw);                                    /* scale | first two quant bytes */
@@ -759,33 +793,52 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
     auto arrived = [&](unit &t) {
         tie(t.xf[0]);
         tie(t.xf[1]);
-        if constexpr (KQ) {
-            UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int i = 0; i < (Q5K ? 12 : 8); ++i)
-                if (i != 3 || LOADER != 0) tie1(t.kq[j][i]);
+        if constexpr (Q6K) {
+            UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int i = 0; i < 14; ++i) tie1(t.kq[j][i]);
+        } else if constexpr (KQ) {
+            tie(t.kh);
+            UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int i = 0; i < (Q5K ? 4 : 2); ++i) asm volatile("" : "+v"(t.kv[j][i]));
         } else UNROLL for (int j = 0; j < 2; ++j) {
             tie1(t.wd[j]);
             UNROLL for (int p = 0; p < NP; ++p) { tie1(t.raw[p][j][0]); tie1(t.raw[p][j][1]); if (EVEN) tie1(t.raw[p][j][2]); }
         }
     };
     /* MFMA operands of the block's two slices, column blocks j = 0, 1 */
-    auto decode = [&](const unit &t, u32x4 (&wf)[2][2]) {
-        if constexpr (KQ) {
+    auto decode = [&](const unit &t, u32x4 (&wf)[2][2], u32 o) {
+        if constexpr (Q6K) {
+            const u32 sh = o & 2u;                          /* byte shift of every field against its aligned dwords */
+            const int tq = wave & 3;
+            UNROLL for (int j = 0; j < 2; ++j) {
+                const float d = h2f_lo(t.kq[j][13]);
+                UNROLL for (int sl = 0; sl < 2; ++sl) {
+                    const float ds = __fmul_rn(d, (float)(int)(int8_t)((t.kq[j][12] >> (8 * sl)) & 0xffu)), dm = ds * 32.f;
+                    u32 o4[4];
+                    UNROLL for (int e = 0; e < 2; ++e) {
+                        const u32 lo = __builtin_amdgcn_alignbyte(t.kq[j][3 * sl + e + 1], t.kq[j][3 * sl + e], sh);
+                        const u32 hi = __builtin_amdgcn_alignbyte(t.kq[j][6 + 3 * sl + e + 1], t.kq[j][6 + 3 * sl + e], sh);
+                        const u32 q = ((lo >> (4 * (tq >> 1))) & 0x0f0f0f0fu) | (((hi >> (2 * tq)) & 0x03030303u) << 4);
+                        pf_affine4(q, ds, dm, o4[2 * e], o4[2 * e + 1]);
+                    }
+                    wf[sl][j] = (u32x4){o4[0], o4[1], o4[2], o4[3]};
+                }
+            }
+        } else if constexpr (KQ) {
             const int sh = 8 * (wave & 3);                  /* this sub-block's byte of the scale dwords */
             UNROLL for (int j = 0; j < 2; ++j) {
                 u32 sc, mn;
                 if constexpr (LOADER == 0) {
-                    sc = (t.kq[j][1] >> sh) & 63u;
-                    mn = (t.kq[j][2] >> sh) & 63u;
+                    sc = (t.kh[j][1] >> sh) & 63u;
+                    mn = (t.kh[j][2] >> sh) & 63u;
                 } else {
-                    sc = ((t.kq[j][3] >> sh) & 0xfu) | (((t.kq[j][1] >> sh) >> 2) & 0x30u);
-                    mn = ((t.kq[j][3] >> (sh + 4)) & 0xfu) | (((t.kq[j][2] >> sh) >> 2) & 0x30u);
+                    sc = ((t.kh[j][3] >> sh) & 0xfu) | (((t.kh[j][1] >> sh) >> 2) & 0x30u);
+                    mn = ((t.kh[j][3] >> (sh + 4)) & 0xfu) | (((t.kh[j][2] >> sh) >> 2) & 0x30u);
                 }
-                const float d1 = __fmul_rn(h2f_lo(t.kq[j][0]), (float)sc), m1 = __fmul_rn(h2f_hi(t.kq[j][0]), (float)mn);
+                const float d1 = __fmul_rn(h2f_lo(t.kh[j][0]), (float)sc), m1 = __fmul_rn(h2f_hi(t.kh[j][0]), (float)mn);
                 UNROLL for (int sl = 0; sl < 2; ++sl) {
                     u32 o[4];
                     UNROLL for (int e = 0; e < 2; ++e) {
-                        u32 q = (EVEN ? t.kq[j][4 + 2 * sl + e] : t.kq[j][4 + 2 * sl + e] >> 4) & 0x0f0f0f0fu;
-                        if constexpr (Q5K) q |= ((t.kq[j][8 + 2 * sl + e] >> wave) & 0x01010101u) << 4;
+                        u32 q = (EVEN ? t.kv[j][sl][e] : t.kv[j][sl][e] >> 4) & 0x0f0f0f0fu;
+                        if constexpr (Q5K) q |= ((t.kv[j][2 + sl][e] >> wave) & 0x01010101u) << 4;
                         pf_affine4(q, d1, m1, o[2 * e], o[2 * e + 1]);
                     }
                     wf[sl][j] = (u32x4){o[0], o[1], o[2], o[3]};
@@ -825,12 +878,13 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
     for (int q = 0; q < nq; ++q) {
         issue(q + DEPTH - 1);
         unit t;
-        fetch(xs_base + (u32)((q % XR) * XBYTES), raw_base + (u32)((q % RS) * RBYTES), t);
+        const u32 o = Q6K ? (u32)((chunk_of(q) * WF::BYTES) & 15) : 0u;
+        fetch(xs_base + (u32)((q % XR) * XBYTES), raw_base + (u32)((q % RS) * RBYTES), t, o);
         if constexpr (LOADER == 0) {
             u32x4 wf[2][2];
             lds_wait();
             arrived(t);
-            decode(t, wf);
+            decode(t, wf, o);
             __builtin_amdgcn_sched_barrier(0);
             multiply(t.xf, wf);
         } else {
@@ -838,7 +892,7 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
             __builtin_amdgcn_sched_barrier(0);
             lds_wait();
             arrived(t);
-            decode(t, wp);
+            decode(t, wp, o);
             UNROLL for (int sl = 0; sl < 2; ++sl) UNROLL for (int i = 0; i < 2; ++i) xp[sl][i] = t.xf[sl][i];
         }
         /* my share of chunk q+1: everything but the loads of the youngest DEPTH-2 iterations */
@@ -1417,6 +1471,7 @@ PSN_PREFILL_KERNEL_SKINNY(q4_0, PfQ4_0)
 PSN_PREFILL_KERNEL_SKINNY(q8_0, PfQ8_0)
 PSN_PREFILL_KERNEL_SKINNY(q4_K, PfQ4_K)
 PSN_PREFILL_KERNEL_SKINNY(q5_K, PfQ5_K)
+PSN_PREFILL_KERNEL_SKINNY(q6_K, PfQ6_K)
 #endif
 #if !defined(PSN_BUILD_ONLY) || PSN_BUILD_PF == 2
 PSN_PREFILL_KERNEL_WIDE(q4_0, PfQ4_0)

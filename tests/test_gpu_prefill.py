@@ -94,19 +94,26 @@ def test_k_quant_prefill_default_plan_and_refusals(hip, orc, qname):
         say(f"  max_rel_err={err:.3e}")
         assert err < PARITY_TOL
     X = G.seeded_acts(842, 64, k).astype(np.float16)
-    # Q6_K super-blocks (210 bytes) do not start on 16-byte words: no weight-streaming kernel for it
-    for tile in ((64, 64, 1, 64),) * (qname == "Q6_K") + ((128, 128, 1, 16), (256, 256, 1, 32)):
+    for tile in ((128, 128, 1, 16), (256, 256, 1, 32)):
         with pytest.raises(backend.PsnError) as e:
             hip.matmul_host(t, W, X, n, k, tile)
         assert e.value.code == _ffi.E_UNSUPPORTED
 
 
-@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K"])
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_skinny_kernel_ragged_shapes(hip, orc, qname):
     """The M <= 64 kernel (waves code 64): every combination of ragged m and n, K ranges of one to many
-    256-wide chunks (one chunk: the load rings are deeper than the whole range), with and without K split."""
+    256-wide chunks (one chunk: the load rings are deeper than the whole range), with and without K split.
+    Q6_K rows must be whole 16-byte words (K a multiple of 2048); its eight chunks per 2048 start at all eight
+    possible offsets inside their aligned windows."""
     t = getattr(orc, qname)
-    for m, n, k in ((1, 70, 256), (37, 300, 768), (64, 130, 1280), (50, 516, 4096), (64, 64, 14336)):
+    shapes = ((1, 70, 256), (37, 300, 768), (64, 130, 1280), (50, 516, 4096), (64, 64, 14336))
+    if qname == "Q6_K":
+        shapes = ((1, 70, 2048), (37, 300, 4096), (64, 130, 6144), (50, 516, 4096), (64, 64, 14336))
+        with pytest.raises(backend.PsnError) as e:
+            hip.matmul_host(t, weights(orc, qname, 859, 70, 768), G.seeded_acts(1, 4, 768).astype(np.float16), 70, 768, (64, 64, 1, 64))
+        assert e.value.code == _ffi.E_UNSUPPORTED
+    for m, n, k in shapes:
         say(f"skinny {qname} m={m} n={n} k={k}")
         W = weights(orc, qname, 860, n, k)
         X = G.seeded_acts(861 + m, m, k).astype(np.float16)
@@ -141,7 +148,7 @@ def test_prefill_m1_matches_matvec_f32_scheme(hip, orc, qname):
 
 
 @pytest.mark.parametrize("n,k", [(14336, 4096), (4096, 14336)])
-@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K"])
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
 def test_prefill_baseline_shapes_m64(hip, orc, qname, n, k):
     say(f"prefill {qname} m=64 n={n} k={k} (full oracle)")
     t = getattr(orc, qname)
@@ -228,7 +235,7 @@ def test_prefill_errors(hip, orc):
     assert e.value.code == _ffi.E_INVALID_ARG
     wk = hip.upload_weight(orc.Q6_K, weights(orc, "Q6_K", 851, n, k), n, k)
     with pytest.raises(backend.PsnError) as e:
-        hip.quantized_matmul(wk, x, y, 4, tile=(64, 64, 1, 64))   # no weight-streaming kernel for Q6_K
+        hip.quantized_matmul(wk, x, y, 4, tile=(64, 64, 1, 64))   # Q6_K rows of K = 512 are not whole 16-byte words
     assert e.value.code == _ffi.E_UNSUPPORTED
     hip.quantized_matmul(w, x, y, 4)
     hip.sync()

@@ -207,7 +207,7 @@ def test_prefill_plans_take_the_dense_family_only_for_large_m():
             tm, tn, sp, wv = backend.prefill_plan(4096, n, k, 256, qt)
             assert tm in (128, 256) and (tn, wv) == (256, 128) and sp in (1, 2, 4), (qt, n, k)
             for m in (1, 16, 64):
-                # 64 rows and fewer: the weight-streaming kernel, except for Q6_K (no 16-byte-aligned super-blocks)
-                assert backend.prefill_plan(m, n, k, 256, qt)[3] == (4 if qt == _ffi.Q6_K else 64)
+                assert backend.prefill_plan(m, n, k, 256, qt)[3] == 64     # 64 rows and fewer: the weight-streaming kernel
+    assert backend.prefill_plan(64, 4096, 4096 + 256, 256, _ffi.Q6_K)[3] == 4   # Q6_K rows that are not whole 16-byte words
     lib = _ffi.load()
     assert lib.psn_error_name(lib.psn_prefill_reserve(None, 4096, 4096)) == b"PSN_E_INVALID_ARG"
