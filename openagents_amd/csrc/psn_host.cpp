@@ -1619,9 +1619,9 @@ extern "C" int32_t psn_qmatmul_prefill_tiled(psn_module *mod, psn_stream *s, int
     if (ksplit < 1 || ksplit > 64) return fail(PSN_E_UNSUPPORTED, "prefill: ksplit=%d outside 1..64", ksplit);
     if (ksplit > 1 && (M * N) % 4 != 0) return fail(PSN_E_UNSUPPORTED, "prefill: splitting K needs M*N to be a multiple of 4");
     /* the interleaved kernels carry their LDS as static arrays; the skinny kernel: rings of three X chunks
-     * (64 rows x 256 k fp16) and six (Q4_0, Q4_K), five (Q5_K), four (Q6_K) or three (Q8_0) raw weight chunks (64 rows), reused for the final
+     * (64 rows x 256 k fp16) and six (Q4_0, Q4_K), five (Q5_K), four (Q6_K) or three (Q8_0) raw weight chunks (64 rows, padded: SkinnyRings), reused for the final
      * 8 x 16 KB reduction */
-    const int skinny_rings = 3 * 32768 + (qtype == PSN_Q4_0 || qtype == PSN_Q4_K ? 6 * 64 * 144 : qtype == PSN_Q5_K ? 5 * 64 * 176 : qtype == PSN_Q6_K ? 4 * 64 * 240 : 3 * 64 * 272);
+    const int skinny_rings = 3 * 32768 + (qtype == PSN_Q4_0 || qtype == PSN_Q4_K ? 6 * 64 * 144 : qtype == PSN_Q5_K ? 5 * 64 * 176 : qtype == PSN_Q6_K ? 4 * 64 * 240 : 3 * 64 * 304);
     const int wide_rings = 3 * (32768 + 256 * (qtype == PSN_Q4_0 ? 36 : 68));   /* three stages of X (256 rows x 64 k) and of raw blocks (two per row) */
     const int lds = skinny ? (skinny_rings > 8 * 16384 ? skinny_rings : 8 * 16384) : wide ? wide_rings : waves == 16 ? 0 : 2 * (bm + bn) * 128;
     if (lds > mod->ctx->max_lds) return fail(PSN_E_UNSUPPORTED, "prefill: tile %dx%d needs %d bytes of LDS, device offers %d", bm, bn, lds, mod->ctx->max_lds);

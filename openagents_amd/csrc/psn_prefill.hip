@@ -626,13 +626,22 @@ PSN_DEV void prefill_body_ws(const psn_prefill_args &a) {
  * every iteration issues the same number of loads and the outstanding-load count is a constant. */
 template <typename WF> struct SkinnyRings {
     static constexpr int XR = 3;                                /* X chunks in the ring */
-    /* bytes of a row's chunk in LDS.  Q6_K's 210-byte super-blocks start on 2-byte boundaries: what is loaded is the
-     * window of fourteen aligned 16-byte words that holds the super-block (rows must be whole 16-byte words, K a
-     * multiple of 2048; chunk c then starts (210 c) mod 16 bytes into its window, the same for every row), and a
-     * fifteenth word of padding: with 224 bytes between rows, every fourth row would share its LDS banks */
-    static constexpr int WORDS = (WF::BYTES + 14 + 15) / 16;     /* words that hold a chunk of a row whatever its alignment */
-    static constexpr int LROW = WF::BYTES % 16 == 0 ? WF::BYTES : (WORDS + 1) * 16;
-    static constexpr int RS = LROW == 144 ? 6 : LROW == 176 ? 5 : LROW == 240 ? 4 : 3;   /* raw weight chunks in the ring: what 160 KB hold beside X */
+    /* DATA: the 16-byte words that hold a row's chunk.  Q6_K's 210-byte super-blocks start on 2-byte boundaries: what is
+     * loaded is the window of fourteen aligned words that holds the super-block (rows must be whole 16-byte words, K a
+     * multiple of 2048; chunk c then starts (210 c) mod 16 bytes into its window, the same for every row).
+     * LROW: bytes between rows in LDS.  A wave reads the same 32-bit field of 32 different rows at a time; rows lie whole
+     * 16-byte words apart, so those reads can reach only eight of the 32 banks (a four-way conflict) -- unless the rows
+     * are ROTated against each other: row n is fetched from 4 rho(n) bytes before its chunk, rho(n) = (n >> RSH) & 3 (one
+     * more word per row takes the bytes pushed out at the end; the bytes in front belong to the chunk or the row before).
+     * With 304 (Q8_0) or 240 (Q6_K) bytes between rows all 32 rows then hit different banks.  Q4_K / Q5_K read whole
+     * aligned words instead; Q4_0 stays unrotated (measured: with 160 bytes between rows its conflicts halve and the
+     * kernel gets 10 % slower -- the fetches that no longer start on 16-byte words and the extra word cost more than
+     * its few 32-bit reads per chunk). */
+    static constexpr int DATA = (WF::BYTES % 16 == 0 ? WF::BYTES : WF::BYTES + 14 + 15) / 16;
+    static constexpr bool ROT = DATA == 17 || DATA == 14;
+    static constexpr int LROW = !ROT ? WF::BYTES : DATA == 17 ? 304 : 240;
+    static constexpr int RSH = 3;
+    static constexpr int RS = LROW <= 160 ? 6 : LROW == 176 ? 5 : LROW == 240 ? 4 : 3;   /* raw weight chunks in the ring: what 160 KB hold beside X */
     static constexpr int XBYTES = 4 * 64 * 128, RBYTES = 64 * LROW;
     static constexpr int BYTES = XR * XBYTES + RS * RBYTES;
 };
@@ -648,7 +657,7 @@ template <typename WF> struct SkinnyRings {
  * (LOADER 0: the super-block's first half; EVEN: the first 32 of a 64-byte group of ql); its fields start on
  * 2-byte boundaries, so three aligned dwords are read around each eight bytes and shifted with v_alignbyte. */
 template <typename WF, int LOADER, bool EVEN>
-PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, int n0, int c_begin, int nq, int rot,
+PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, int n0, int c_begin, int nq, int rot, bool rotate_rows,
                                  u32 xs_base, u32 raw_base, __attribute__((address_space(3))) char *lds_ptr, u32 lds0, float16_t (&acc)[2][2]) {
     typedef SkinnyRings<WF> R;
     constexpr bool KQ = WF::KQ;                             /* Q4_K / Q5_K: the chunk is one super-block per row, wave w owns its sub-block w */
@@ -656,7 +665,7 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
     constexpr bool Q5K = KQ && WF::DW == 44;
     constexpr bool Q6K = KQ && WF::DW == 53;
     constexpr int XR = R::XR, RS = R::RS, XBYTES = R::XBYTES, RBYTES = R::RBYTES, LROW = R::LROW;
-    constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9, 11, 15 or 17 */
+    constexpr int RINSTR = RBYTES / 1024;                   /* wave-wide load instructions per raw chunk: 9, 10, 11, 15 or 19 */
     constexpr int CX = 8;                                   /* X loads per X wave and chunk (32 KB over 4 waves) */
     /* raw loads per weight wave and chunk: wave 4 takes the one load that does not divide over four waves; when
      * three or two are left over (Q5_K, Q6_K) every wave issues the same number and the last waves repeat the chunk's
@@ -683,10 +692,13 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
         } else {
             __attribute__((address_space(3))) char *dst = lds_ptr + (raw_base - lds0) + (q % RS) * RBYTES;
             UNROLL for (int u = 0; u < CR; ++u) {
-                const int i = min((wave - 4) + 4 * u, RINSTR - 1);   /* instruction index; wave 4's last one is index 8 or 16 */
-                const int word = i * 64 + lane, row = word / (LROW / 16), wd = Q6K ? min(word % (LROW / 16), R::WORDS - 1) : word % (LROW / 16);
+                const int i = min((wave - 4) + 4 * u, RINSTR - 1);   /* instruction index (the last waves repeat the chunk's last load when the count does not divide) */
+                const int word = i * 64 + lane, row = word / (LROW / 16);
+                const int rho = R::ROT && rotate_rows ? ((row & 31) >> R::RSH) & 3 : 0;
+                /* words past the row's data (and past the one that takes the rotated-out bytes) repeat its last one */
+                const int wd = min(word % (LROW / 16), R::DATA - 1 + (rho > 0));
                 const int64_t coff = Q6K ? (int64_t)((c * WF::BYTES) & ~15) : (int64_t)c * WF::BYTES;
-                const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + coff + wd * 16;
+                const uint8_t *src = a.W + (int64_t)min(n0 + row, N - 1) * a.row_bytes + coff + wd * 16 - 4 * rho;
                 __builtin_amdgcn_global_load_lds((const void *)src, (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
             }
         }
@@ -701,7 +713,8 @@ PSN_DEV void prefill_skinny_loop(const psn_prefill_args &a, int wave, int lane, 
      * array, this lane's eight at 8h and 16 + 8h); Q5_K: the fifth bits of the same elements (qh, bit `wave`) */
     /* Q6_K, sub-block `wave` = half wave / 4, quarter t = wave % 4 of the super-block: low bits in ql[64 half + 32 (t & 1)
      * + l] (high nibble for t >= 2), bits 4..5 in qh[32 half + l] >> 2 t, int8 scales[8 half + 2 t + l / 16], d at 208 */
-    const u32 rlane = KQ ? (u32)((lane & 31) * LROW) : (u32)((lane & 31) * LROW + wave * BB);
+    const u32 rho_lane = R::ROT && rotate_rows ? (u32)(((lane & 31) >> R::RSH) & 3) : 0u;
+    const u32 rlane = (KQ ? (u32)((lane & 31) * LROW) : (u32)((lane & 31) * LROW + wave * BB)) + 4u * rho_lane;
     const u32 qlane = Q6K ? rlane + (u32)(64 * (LOADER != 0) + 32 * !EVEN + 8 * h)
                     : KQ  ? rlane + (u32)((Q5K ? 48 : 16) + 32 * (wave >> 1) + 8 * h) : rlane + 8u * (u32)h;
     const u32 hlane = Q6K ? rlane + (u32)(128 + 32 * (LOADER != 0) + 8 * h) : rlane + (u32)(16 + 8 * h);
@@ -929,7 +942,10 @@ PSN_DEV void prefill_skinny_body(const psn_prefill_args &a) {
 
     float16_t acc[2][2];
     UNROLL for (int i = 0; i < 2; ++i) UNROLL for (int j = 0; j < 2; ++j) UNROLL for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-#define PSN_SKINNY_LOOP(LOADER, EVEN) prefill_skinny_loop<WF, LOADER, EVEN>(a, wave, lane, n0, c_begin, nq, rot, xs_base, raw_base, lds_ptr, lds0, acc)
+    /* the last tile's rows stay unrotated: the word that takes a rotated row's last bytes reaches up to twelve bytes
+     * past the row, which for the matrix's last row is past the buffer */
+    const bool rotate_rows = tile_n != nt - 1;
+#define PSN_SKINNY_LOOP(LOADER, EVEN) prefill_skinny_loop<WF, LOADER, EVEN>(a, wave, lane, n0, c_begin, nq, rot, rotate_rows, xs_base, raw_base, lds_ptr, lds0, acc)
     if (wave < 4) {
         if ((wave & 1) == 0) PSN_SKINNY_LOOP(0, true);
         else PSN_SKINNY_LOOP(0, false);
