@@ -1368,7 +1368,7 @@ extern "C" int32_t psn_qmatmul_prefill_plan(int64_t M, int64_t N, int64_t K, int
 static void plan_weight_stream(int64_t M, int64_t N, int64_t K, int32_t cus, int32_t *tile_m, int32_t *tile_n, int32_t *ksplit, int32_t *waves) {
     const int64_t nt = (N + 63) / 64, C = K / 256;
     int sp = 1;
-    while (nt * sp * 2 <= cus && C / (sp * 2) >= 2 && (M * N) % 4 == 0) sp *= 2;
+    while (sp < 8 && nt * sp * 2 <= cus && C / (sp * 2) >= 2 && (M * N) % 4 == 0) sp *= 2;
     *tile_m = 64;
     *tile_n = 64;
     *ksplit = sp;

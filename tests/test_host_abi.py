@@ -103,6 +103,34 @@ def test_matvec_plans_are_consistent_over_many_shapes(lib):
                             assert batch == 1 and p.stage_lds in (1, 2) and k // 256 <= p.lanes_per_row, p.as_dict()
 
 
+def test_prefill_plans_are_consistent_over_many_shapes(lib):
+    """Host arithmetic only: every prefill plan over a grid of shapes is one psn_qmatmul_prefill_tiled accepts --
+    a known tile, a family the format has, a K split that leaves whole chunks per range and an atomically addable Y."""
+    tiles = {(64, 64), (64, 128), (128, 128), (128, 256), (256, 128), (256, 256)}
+    for qt in (_ffi.Q4_0, _ffi.Q8_0, _ffi.Q4_K, _ffi.Q5_K, _ffi.Q6_K):
+        for k in (256, 512, 1024, 2048, 2304, 4096, 5120, 8192, 11008, 14336):
+            for n in (1, 17, 64, 130, 1000, 1024, 4096, 6144, 14336):
+                for m in (1, 7, 64, 65, 128, 200, 512, 777, 2048, 4096):
+                    tm, tn, sp, wv = backend.prefill_plan(m, n, k, 256, qt)
+                    tag = (qt, m, n, k, tm, tn, sp, wv)
+                    assert (tm, tn) in tiles and sp in (1, 2, 4, 8), tag
+                    if sp > 1:
+                        assert (m * n) % 4 == 0 and k // 256 >= 2 * sp, tag
+                    if m <= 64 and (qt != _ffi.Q6_K or k % 2048 == 0):
+                        assert wv == 64 and (tm, tn) == (64, 64), tag           # the weight-streaming kernel
+                    else:
+                        assert wv != 64, tag
+                    if wv == 128:
+                        assert m > 64 and tn == 256 and tm in (128, 256) and sp <= 4, tag
+                    elif wv == 32:
+                        assert qt in (_ffi.Q4_0, _ffi.Q8_0) and (tm, tn) == (256, 256), tag
+                    elif wv == 16:
+                        assert (tm, tn) in {(64, 64), (64, 128), (128, 128), (128, 256)}, tag
+                        assert qt in (_ffi.Q4_0, _ffi.Q8_0) or (qt != _ffi.Q6_K and (tm, tn) == (128, 256)), tag
+                    else:
+                        assert wv in (4, 64), tag
+
+
 def test_null_handles_are_rejected_without_a_device(lib):
     assert lib.psn_stream_sync(None) == _ffi.E_INVALID_ARG
     assert lib.psn_buf_free(None) == _ffi.E_INVALID_ARG
