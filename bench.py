@@ -153,7 +153,7 @@ class OracleChecker:
 def compact_configs(records):
     """One figure per configuration for the headline line: fraction of the roofline that bounds it."""
     out = {"c1_q8_0_4096": None, "c3_q4_K_b1248": {}, "c4_m64_512_2048": {}, "c5": None}
-    bad = 0
+    bad, lm_head = 0, None
     for r in records or []:
         op, frac = r["opRef"], r["roofline"]["fraction"]
         bad += r["parity"]["status"] != "pass"
@@ -164,8 +164,12 @@ def compact_configs(records):
             out["c3_q4_K_b1248"].setdefault(parts[2], []).append(frac)
         elif op.startswith("prefill."):
             out["c4_m64_512_2048"].setdefault(parts[1] + "." + parts[2], []).append(frac)
+        elif op.startswith("matvec.q6_K"):
+            lm_head = frac
         elif op.startswith("decode.step"):
             out["c5"] = {"tok_s": r["tokensPerSecond"], "matvec_share": r.get("matvec_share"), "matvec_frac": frac}
+    if lm_head is not None and out["c5"] is not None:
+        out["c5"]["lm_head_q6_K_frac"] = lm_head
     out["parity_not_pass"] = bad
     return out
 

@@ -36,6 +36,7 @@ def canned_records():
                                      R.roofline_of(bound, a), None))
     recs.append(R.record(be, "decode.step.q4_K.b1", "psn decode-step graph (226 launches: " + ", ".join(f"psn_kernel_with_a_long_name_{i}" for i in range(12)) + ")",
                          "a" * 64, 602.27, R.roofline_of("hbm", 3929.2), ok, ["sampling"], matvec_share=0.6693))
+    recs.append(R.record(be, "matvec.q6_K.4096x128256.b1", "psn_mvs_q6_K_q8_g16_xf_s1", "b" * 64, 1.2e4, R.roofline_of("hbm", 5400.0), ok))
     return recs
 
 
@@ -68,7 +69,7 @@ def test_headline_line_is_short_and_complete():
     assert c["c1_q8_0_4096"] == recs[0]["roofline"]["fraction"]
     assert [len(v) for v in c["c3_q4_K_b1248"].values()] == [4, 4]
     assert len(c["c4_m64_512_2048"]) == 4 and all(len(v) == 3 for v in c["c4_m64_512_2048"].values())
-    assert c["c5"]["tok_s"] == 602.27 and c["c5"]["matvec_share"] == 0.6693
+    assert c["c5"]["tok_s"] == 602.27 and c["c5"]["matvec_share"] == 0.6693 and c["c5"]["lm_head_q6_K_frac"] == 0.675
     assert c["parity_not_pass"] == 12                     # the twelve canned prefill records carry no verdict
     # without records (headline only) and without the CPU leg the line is still well formed
     head = canned_head()

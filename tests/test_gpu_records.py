@@ -67,9 +67,12 @@ def test_small_batch_record_names_both_launches(hip, orc):
 
 def test_decode_step_record_and_worker_attachment(hip, orc):
     checker = bench.OracleChecker()
-    (rec,) = R.config5(hip, 2, ctx=256, layers=2, checker=checker)
+    rec, head = R.config5(hip, 2, ctx=256, layers=2, checker=checker)
     print(f"record {rec['opRef']}: {rec['kernelRef']} parity={rec['parity']['value']:.2e}", flush=True)
     check(hip, rec)
+    print(f"record {head['opRef']}: {head['kernelRef']} parity={head['parity']['value']:.2e}", flush=True)
+    check(hip, head)                                         # the Q6_K LM head on its own
+    assert head["opRef"].startswith("matvec.q6_K.4096x128256") and "q6_K" in head["kernelRef"]
     assert rec["launches_per_token"] >= 2 * 7 + 2 and 0 < rec["matvec_share"] <= 1
     assert any(k.startswith("psn_attn") for k in kernels_of(rec)) and any("q6_K" in k for k in kernels_of(rec))
     att = R.worker_attachment([rec], updated_at_ms=5)
