@@ -169,6 +169,12 @@ template <int OFF> PSN_DEV u32x2 lds_read64o(u32 addr) {          /* addr + OFF:
     asm volatile("ds_read_b64 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF) : "memory");
     return v;
 }
+/* two dwords at addr + 4 * D0 and addr + 4 * D1 (addr a multiple of 4, not necessarily of 8) */
+template <int D0, int D1> PSN_DEV u32x2 lds_read2_b32(u32 addr) {
+    u32x2 v;
+    asm volatile("ds_read2_b32 %0, %1 offset0:%2 offset1:%3" : "=v"(v) : "v"(addr), "n"(D0), "n"(D1) : "memory");
+    return v;
+}
 PSN_DEV u32 lds_read_u16(u32 addr) {
     u32 v;
     asm volatile("ds_read_u16 %0, %1" : "=v"(v) : "v"(addr) : "memory");

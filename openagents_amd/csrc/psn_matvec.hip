@@ -980,13 +980,29 @@ template <> PSN_DEV void stream_load_chunk<FmtQ4_0>(u32 addr, u32 (&w)[FmtQ4_0::
 template <> PSN_DEV void stream_load_chunk<FmtQ4_K>(u32 addr, u32 (&w)[FmtQ4_K::DW]) { stream_read_words<9>(addr, w); }
 template <> PSN_DEV void stream_load_chunk<FmtQ5_K>(u32 addr, u32 (&w)[FmtQ5_K::DW]) { stream_read_words<11>(addr, w); }
 template <> PSN_DEV void stream_load_chunk<FmtQ8_0>(u32 addr, u32 (&w)[FmtQ8_0::DW]) { stream_read_words<17>(addr, w); }
-/* Q6_K super-blocks are 210 bytes: a chunk starts on an even byte, not on a 16-byte word (gfx950 reads
- * LDS at any alignment); 13 words cover bytes 0..207, the fp16 d sits in the last two */
+/* Q6_K super-blocks are 210 bytes: a lane's chunk starts on an even byte, two bytes past a dword for every other
+ * lane.  LDS reads that are not naturally aligned work and stall the LDS pipe (SQ_LDS_UNALIGNED_STALL: two thirds of
+ * this kernel's cycles when the chunk was read as thirteen 16-byte words at its own address), so the 53 dwords are
+ * read at the aligned address in front of the chunk, two per instruction, and shifted into place. */
+template <int I> PSN_DEV void lds_read_pairs(u32 addr, u32x2 (&v)[26]) {
+    if constexpr (I < 26) {
+        v[I] = lds_read2_b32<2 * I, 2 * I + 1>(addr);
+        lds_read_pairs<I + 1>(addr, v);
+    }
+}
 template <> PSN_DEV void stream_load_chunk<FmtQ6_K>(u32 addr, u32 (&w)[FmtQ6_K::DW]) {
-    u32 d = lds_read_u16(addr + 208u);
-    stream_read_words<13>(addr, w);
-    tie1(d);
-    w[52] = d;
+    const u32 sh = addr & 2u, a4 = addr - sh;
+    u32x2 v[26];
+    lds_read_pairs<0>(a4, v);
+    u32 last = lds_read32o<208>(a4);
+    lds_wait();
+    UNROLL for (int i = 0; i < 26; ++i) asm volatile("" : "+v"(v[i]));
+    tie1(last);
+    UNROLL for (int k = 0; k < 52; ++k) {
+        const u32 lo = v[k >> 1][k & 1], hi = k + 1 < 52 ? v[(k + 1) >> 1][(k + 1) & 1] : last;
+        w[k] = __builtin_amdgcn_alignbyte(hi, lo, sh);
+    }
+    w[52] = __builtin_amdgcn_alignbyte(0u, last, sh) & 0xffffu;   /* the fp16 d: bytes 208, 209 of the chunk */
 }
 
 /* Scheme F32: weights dequantized to fp32 in registers, fp32 FMA against the fp32 activations.
