@@ -102,10 +102,14 @@ PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out
     /* >= scanning downwards leaves the lowest index among equal magnitudes */
     _Pragma("unroll") for (int i = 3; i >= 0; --i) if (fabsf(e[i]) >= amax) { amax = fabsf(e[i]); first = i; }
     const float wmax = group_max<64>(amax);
-    const int cand = (amax == wmax) ? lane * 4 + first : 1 << 20;
-    const int idx = group_min_i<64>(cand);
-    const float mine = e[idx & 3];
-    const float vmax = __shfl(mine, idx >> 2, 64);
+    /* the first element of largest magnitude: the lowest lane that holds the maximum (a ballot and a scalar
+     * find-first instead of a second wave-wide reduction), and in it the lowest index (`first`) */
+    float mine = e[0];
+    _Pragma("unroll") for (int i = 1; i < 4; ++i) mine = first == i ? e[i] : mine;
+    const unsigned long long holders = __builtin_amdgcn_ballot_w64(amax == wmax);
+    const int src = holders ? __builtin_ctzll(holders) : 0;          /* no holder: a NaN among the inputs */
+    const float vmax = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), src));
+    (void)lane;
     packed = 0;
     int s4 = 0;
     d_out = 0.f;
