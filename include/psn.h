@@ -268,6 +268,13 @@ int32_t psn_qmatvec_planned(psn_module *mod, psn_stream *s, int32_t qtype, int32
 int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_buf *src, int64_t bytes, int32_t blocks, int32_t threads,
                            int32_t lds_depth, int32_t every_workgroup, psn_buf *out);
 
+/* No counterpart in the reference: a check of this device's arithmetic.  The activation quantizers take their
+ * IEEE divisions (amax / 127, 1 / d, -127 / max, 1 / iscale) by a reciprocal approximation corrected with fused
+ * multiply-adds; the launch compares those shortcuts with true division for every float between 2^-100 and 2^100
+ * in magnitude, both signs, and leaves eight 64-bit mismatch counters in `out` (64 bytes; all zero on gfx950).
+ * Outside that range the quantizers divide the long way. */
+int32_t psn_selftest_arith(psn_module *mod, psn_stream *s, psn_buf *out);
+
 /* ---- prefill matmul ----------------------------------------------------------------------- */
 
 /* Y[m][n] = sum_k h(deq(W)[n][k]) * X[m][k]; X fp16 [M][K], Y fp32 [M][N], weight tiles are

@@ -88,6 +88,7 @@ SIGNATURES = {
     "psn_qmatvec_q8_multi": (_i32, [_vp, _vp, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32]),
     "psn_qmatvec_planned": (_i32, [_vp, _vp, _i32, _i32, _i32, _pp, _vp, _pp, C.POINTER(_i64), _i64, _i32, C.POINTER(MatvecPlan)]),
     "psn_calibrate_read": (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _i32, _vp]),
+    "psn_selftest_arith": (_i32, [_vp, _vp, _vp]),
     "psn_qmatmul_prefill": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _i64, _i64, _i64]),
     "psn_qmatmul_prefill_plan": (_i32, [_i64, _i64, _i64, _i32, C.POINTER(_i32), C.POINTER(_i32), C.POINTER(_i32), C.POINTER(_i32)]),
     "psn_qmatmul_prefill_plan_for": (_i32, [_i32, _i64, _i64, _i64, _i32, C.POINTER(_i32), C.POINTER(_i32), C.POINTER(_i32), C.POINTER(_i32)]),

@@ -291,6 +291,15 @@ class HipBackend:
         _check(self.lib.psn_calibrate_read(self.module, self.stream, src.handle, nbytes, blocks, threads, lds_depth, int(every_workgroup), self._h(out)))
 
     # -- decode-step glue --------------------------------------------------------------------
+    def selftest_arith(self) -> list:
+        """Mismatch counts of the quantizers' division shortcuts against IEEE division over every float they are used
+        on (see psn_selftest_arith): eight zeros on a device whose arithmetic the library was written for."""
+        out = self.alloc(64)
+        _check(self.lib.psn_selftest_arith(self.module, self.stream, out.handle))
+        counts = [int(v) for v in out.download(np.uint64, (8,))]
+        out.free()
+        return counts
+
     def add_rmsnorm(self, x: DeviceBuffer, delta, weight: DeviceBuffer, y: DeviceBuffer, n: int, eps: float = 1e-5):
         _check(self.lib.psn_add_rmsnorm(self.module, self.stream, x.handle, delta.handle if delta is not None else None,
                                         weight.handle, y.handle, n, eps))

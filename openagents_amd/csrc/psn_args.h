@@ -87,6 +87,13 @@ struct psn_calib_args {
     int32_t every_wg;     /* 1: every workgroup reads the whole range; 0: the workgroups share it */
 };
 
+/* psn_selftest_arith: float bit patterns lo .. hi (positive), one mismatch counter per checked identity */
+struct psn_selftest_args {
+    uint32_t lo, hi;
+    unsigned long long *bad;   /* [PSN_SELFTEST_COUNTERS] */
+};
+#define PSN_SELFTEST_COUNTERS 8
+
 /* decode-step glue kernels (psn_decode.hip) */
 /* optional quantized output of an elementwise kernel: the three fields of the activation layout for
  * one row of n elements (qs null = not wanted); act_q8_K selects Q8_K (else Q8_0) */

@@ -52,3 +52,32 @@ extern "C" __global__ void __launch_bounds__(1024) psn_calib_read_lds(const psn_
     }
     if (lane == 0 && a.out) a.out[(int64_t)blockIdx.x * (blockDim.x >> 6) + wib] = r;
 }
+
+/* The activation quantizers replace IEEE divisions by rcp_rn / div_rn (psn_device.h).  This kernel walks every
+ * float x with bit pattern lo .. hi and counts, per identity, the values for which the shortcut and the compiler's
+ * division differ in any bit:
+ *   0  rcp_rn(x)  vs  1 / x              1  rcp_rn(-x)  vs  1 / -x
+ *   2  div_rn(-127, x, rcp_rn(x))  vs  -127 / x      3  the same for -x
+ *   4  div_rn(x, 127, RN(1/127))  vs  x / 127        5  rcp_rn(x / 127)  vs  1 / (x / 127)
+ *   6  rcp_rn(-127 / x)  vs  1 / (-127 / x)          7  the same for -x
+ * (5 - 7: the reciprocals the quantizers take of their own quotients.) */
+extern "C" __global__ void __launch_bounds__(256) psn_selftest_arith(const psn_selftest_args a) {
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    unsigned c[PSN_SELFTEST_COUNTERS];
+    _Pragma("unroll") for (int i = 0; i < PSN_SELFTEST_COUNTERS; ++i) c[i] = 0;
+    auto differ = [](float p, float q) { return __float_as_uint(p) != __float_as_uint(q) ? 1u : 0u; };
+    for (unsigned long long b = a.lo + (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; b <= a.hi; b += stride) {
+        const float x = __uint_as_float((u32)b);
+        c[0] += differ(rcp_rn(x), 1.f / x);
+        c[1] += differ(rcp_rn(-x), 1.f / -x);
+        c[2] += differ(div_rn(-127.f, x, rcp_rn(x)), -127.f / x);
+        c[3] += differ(div_rn(-127.f, -x, rcp_rn(-x)), -127.f / -x);
+        const float d = x / 127.f;
+        c[4] += differ(div_rn(x, 127.f, 1.f / 127.f), d);
+        c[5] += differ(rcp_rn(d), 1.f / d);
+        const float sp = -127.f / x, sn = -127.f / -x;
+        c[6] += differ(rcp_rn(sp), 1.f / sp);
+        c[7] += differ(rcp_rn(sn), 1.f / sn);
+    }
+    _Pragma("unroll") for (int i = 0; i < PSN_SELFTEST_COUNTERS; ++i) if (c[i]) atomicAdd(&a.bad[i], (unsigned long long)c[i]);
+}

@@ -63,6 +63,19 @@ PSN_DEV float group_max(float v) {
     if (G >= 64) v = fmaxf(v, __shfl_xor(v, 32, 64));
     return v;
 }
+/* the same for values that are neither negative nor NaN: their bit patterns order like the values, and an unsigned
+ * maximum needs no canonicalization of its operands (one instruction per step instead of three) */
+template <int G>
+PSN_DEV float group_max_nonneg(float v) {
+    u32 b = __float_as_uint(v);
+    if (G >= 2) b = max(b, (u32)dpp_i<0xB1>((int)b));
+    if (G >= 4) b = max(b, (u32)dpp_i<0x4E>((int)b));
+    if (G >= 8) b = max(b, (u32)dpp_i<0x141>((int)b));
+    if (G >= 16) b = max(b, (u32)dpp_i<0x140>((int)b));
+    if (G >= 32) b = max(b, (u32)__builtin_amdgcn_ds_swizzle((int)b, 0x401F));
+    if (G >= 64) b = max(b, (u32)__shfl_xor((int)b, 32, 64));
+    return __uint_as_float(b);
+}
 template <int G>
 PSN_DEV int group_min_i(int v) {
     if (G >= 2) v = min(v, dpp_i<0xB1>(v));
@@ -80,15 +93,48 @@ PSN_DEV int group_min_i(int v) {
 /* Q8_0: the four elements a lane owns of a 32-element block shared by 8 adjacent lanes.
  * d = amax/127, q = round-half-away(x/d); returns the packed int8x4, the fp16-rounded scale
  * (widened) and the block's sum of q. */
+/* IEEE-754 quotients in three or four instructions instead of the compiler's eleven.  v_rcp_f32 is accurate to one
+ * ulp; one Newton step on it, r + r (1 - b r) in two fused multiply-adds, returns the correctly rounded 1 / b, and
+ * a quotient a / b follows from a r corrected by its own remainder.  This is arithmetic of THIS device's v_rcp_f32:
+ * psn_selftest_arith (psn_calib.hip) compares the shortcuts with the compiler's IEEE division for every float of
+ * the range they are used on, 2^-100 ... 2^100 in magnitude, both signs, and found no difference; outside
+ * fast_div_range the callers divide the long way. */
+PSN_DEV float rcp_rn(float b) {
+    const float r = __builtin_amdgcn_rcpf(b);
+    return __builtin_fmaf(__builtin_fmaf(-b, r, 1.f), r, r);
+}
+/* a / b with r = rcp_rn(b), or for a constant b its rounded reciprocal */
+PSN_DEV float div_rn(float a, float b, float r) {
+    const float q = a * r;
+    return __builtin_fmaf(__builtin_fmaf(-q, b, a), r, q);
+}
+PSN_DEV bool fast_div_range(float magnitude) { return magnitude >= 0x1p-90f && magnitude <= 0x1p90f; }
+
+/* roundf (halves away from zero) of |t| < 2^22 as a conversion that truncates: t + copysign(c, t) with c the
+ * largest float below 0.5 lands on the right side of every integer (with 0.5 itself, 0.5 - 2^-25 would round up
+ * to 1).  Checked against roundf for every float below 4096 in magnitude (tests/test_oracle_formats.py restates
+ * the check for the range the quantizers produce). */
+PSN_DEV int round_half_away(float t) { return (int)(t + __builtin_copysignf(__uint_as_float(0x3effffffu), t)); }
+/* the low bytes of four ints as one dword */
+PSN_DEV u32 pack_bytes4(int q0, int q1, int q2, int q3) {
+    const u32 lo = __builtin_amdgcn_perm((u32)q1, (u32)q0, 0x0c0c0400u), hi = __builtin_amdgcn_perm((u32)q3, (u32)q2, 0x0c0c0400u);
+    return (hi << 16) | lo;
+}
 PSN_DEV void q8_0_quant4(const float4 v, u32 &packed, float &d_out, int &sum) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = group_max<8>(amax);
-    const float d = amax / 127.f;
-    const float id = d != 0.f ? 1.f / d : 0.f;
-    const int q0 = (int)roundf(v.x * id), q1 = (int)roundf(v.y * id);
-    const int q2 = (int)roundf(v.z * id), q3 = (int)roundf(v.w * id);
+    amax = group_max_nonneg<8>(amax);
+    float d, id;
+    if (fast_div_range(amax)) {                    /* amax / 127 stays inside the checked range of rcp_rn */
+        d = div_rn(amax, 127.f, 1.f / 127.f);
+        id = rcp_rn(d);
+    } else {
+        d = amax / 127.f;
+        id = d != 0.f ? 1.f / d : 0.f;
+    }
+    const int q0 = round_half_away(v.x * id), q1 = round_half_away(v.y * id);
+    const int q2 = round_half_away(v.z * id), q3 = round_half_away(v.w * id);
     sum = group_sum_i<8>(q0 + q1 + q2 + q3);
-    packed = (u32)(q0 & 0xff) | ((u32)(q1 & 0xff) << 8) | ((u32)(q2 & 0xff) << 16) | ((u32)q3 << 24);
+    packed = pack_bytes4(q0, q1, q2, q3);
     d_out = (float)(f16)d;            /* what a reader of the fp16 field would see */
 }
 
@@ -101,7 +147,7 @@ PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out
     int first = 4;
     /* >= scanning downwards leaves the lowest index among equal magnitudes */
     _Pragma("unroll") for (int i = 3; i >= 0; --i) if (fabsf(e[i]) >= amax) { amax = fabsf(e[i]); first = i; }
-    const float wmax = group_max<64>(amax);
+    const float wmax = group_max_nonneg<64>(amax);
     /* the first element of largest magnitude: the lowest lane that holds the maximum (a ballot and a scalar
      * find-first instead of a second wave-wide reduction), and in it the lowest index (`first`) */
     float mine = e[0];
@@ -114,14 +160,16 @@ PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out
     int s4 = 0;
     d_out = 0.f;
     if (wmax != 0.f) {
-        const float iscale = -127.f / vmax;
+        const bool fast = fast_div_range(wmax);    /* wave-uniform */
+        const float iscale = fast ? div_rn(-127.f, vmax, rcp_rn(vmax)) : -127.f / vmax;
+        int q[4];
         _Pragma("unroll") for (int i = 0; i < 4; ++i) {
-            int q = (int)__builtin_rintf(iscale * e[i]);
-            q = q > 127 ? 127 : q;
-            s4 += q;
-            packed |= (u32)(q & 0xff) << (8 * i);
+            q[i] = (int)__builtin_rintf(iscale * e[i]);
+            q[i] = q[i] > 127 ? 127 : q[i];
+            s4 += q[i];
         }
-        d_out = 1.f / iscale;
+        packed = pack_bytes4(q[0], q[1], q[2], q[3]);
+        d_out = fast ? rcp_rn(iscale) : 1.f / iscale;
     }
     s16 = group_sum_i<4>(s4);
 }

@@ -1285,6 +1285,25 @@ extern "C" int32_t psn_calibrate_read(psn_module *mod, psn_stream *s, const psn_
     return launch(mod, s, lds_depth ? "psn_calib_read_lds" : "psn_calib_read", (unsigned)blocks, (unsigned)threads, (unsigned)lds, &a);
 }
 
+extern "C" int32_t psn_selftest_arith(psn_module *mod, psn_stream *s, psn_buf *out) {
+    if (!mod || !s || !out) return fail(PSN_E_INVALID_ARG, "psn_selftest_arith: null handle");
+    if (s->ctx != mod->ctx || out->ctx != mod->ctx) return fail(PSN_E_INVALID_ARG, "psn_selftest_arith: handles belong to different contexts");
+    if (out->bytes < PSN_SELFTEST_COUNTERS * sizeof(unsigned long long))
+        return fail(PSN_E_INVALID_ARG, "psn_selftest_arith: out holds %zu bytes, need %zu", out->bytes, PSN_SELFTEST_COUNTERS * sizeof(unsigned long long));
+    int32_t rc = bind(mod->ctx);
+    if (rc) return rc;
+    psn_fill_args f;
+    f.p = (uint32_t *)out->p;
+    f.n16 = PSN_SELFTEST_COUNTERS * sizeof(unsigned long long) / 16;
+    if ((rc = launch(mod, s, "psn_fill_zero", 1, 256, 0, &f))) return rc;
+    psn_selftest_args a;
+    const float lo = 0x1p-100f, hi = 0x1p100f;
+    memcpy(&a.lo, &lo, 4);
+    memcpy(&a.hi, &hi, 4);
+    a.bad = (unsigned long long *)out->p;
+    return launch(mod, s, "psn_selftest_arith", 4096, 256, 0, &a);
+}
+
 /* ------------------------------------------------------------------ prefill */
 
 static const int k_prefill_tiles[][2] = {{64, 64}, {64, 128}, {128, 128}, {128, 256}, {256, 128}, {256, 256}};

@@ -312,3 +312,40 @@ def test_requantizing_dequantized_rows_is_stable(orc, qname):
     y1 = orc.dequantize(t, orc.quantize(t, w), 512)
     y2 = orc.dequantize(t, orc.quantize(t, y1), 512)
     assert np.sqrt(np.mean((y2 - y1) ** 2)) <= 0.02 * np.sqrt(np.mean(y1 ** 2))
+
+
+def test_truncating_round_half_away_matches_roundf_over_the_quantizers_range():
+    """The device quantizers round halves away from zero as (int)(t + copysign(c, t)) with c the largest float below
+    0.5 (one addition and a truncating conversion instead of roundf).  Every float from 0.25 up to 130 in magnitude --
+    the quotients x / d of a Q8_0 block reach 127 -- and a sample below: the same integer as round-half-away computed
+    exactly in float64."""
+    c = np.float32(np.frombuffer(np.uint32(0x3EFFFFFF).tobytes(), dtype=np.float32)[0])
+    lo, hi = np.float32(0.25).view(np.uint32), np.float32(130.0).view(np.uint32)
+    step = 1 << 24
+    for start in range(int(lo), int(hi) + 1, step):
+        bits = np.arange(start, min(start + step, int(hi) + 1), dtype=np.uint32)
+        for sign in (np.float32(1), np.float32(-1)):
+            t = bits.view(np.float32) * sign
+            fast = np.trunc(t + np.copysign(c, t)).astype(np.int32)           # float32 addition, as on the device
+            t64 = t.astype(np.float64)
+            ref = (np.sign(t64) * np.floor(np.abs(t64) + 0.5)).astype(np.int32)
+            assert np.array_equal(fast, ref)
+    small = np.linspace(0, 0.25, 100001, dtype=np.float32)
+    assert not np.any(np.trunc(small + c)) and not np.any(np.trunc(-small - c))
+    # the one value that defeats adding 0.5 itself: the largest float below one half
+    t = np.float32(0.5) - np.float32(2.0 ** -25)
+    assert np.trunc(t + np.float32(0.5)) == 1 and np.trunc(t + c) == 0
+
+
+def test_division_by_127_as_two_fused_multiply_adds_is_exact():
+    """x / 127 as q + fma(-q, 127, x) * r with q = x * r, r = RN(1 / 127): compared in exact rational arithmetic with the
+    correctly rounded quotient on a dense sample (the device self-test covers every float; float64 fma is emulated
+    exactly here because x, q and 127 are float32: the products fit in 53 bits)."""
+    rng = np.random.default_rng(7)
+    r = np.float32(1.0) / np.float32(127.0)
+    bits = rng.integers(np.float32(2.0 ** -90).view(np.uint32), np.float32(2.0 ** 90).view(np.uint32), 2_000_000, dtype=np.uint32)
+    x = bits.view(np.float32)
+    q = (x * r).astype(np.float32)
+    rem = (x.astype(np.float64) - q.astype(np.float64) * 127.0).astype(np.float32)     # exact product, one rounding: an fma
+    fast = (rem.astype(np.float64) * np.float64(r) + q.astype(np.float64)).astype(np.float32)
+    assert np.array_equal(fast, x / np.float32(127.0))
