@@ -811,7 +811,7 @@ static int32_t stream_plan_check(int32_t qtype, int32_t scheme, int64_t K, int32
     if (C > g) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs rows of at most lanes_per_row chunks (K <= %d)", g * 256);
     if (plan->stage_lds < 1 || plan->stage_lds > 3) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs stage_lds 1, 2 or 3");
     if (plan->stage_lds == 3 && (g > 32 || count > 3)) return fail(PSN_E_UNSUPPORTED, "plan: the norm-fused kernels exist for rows of at most 32 chunks and three matrices");
-    if (plan->threads != 256 && plan->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", plan->threads);
+    if (plan->threads < 256 || plan->threads > 512 || plan->threads % 64) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 .. 512, whole waves)", plan->threads);
     if (ring < 1 || ring > 8) return fail(PSN_E_UNSUPPORTED, "plan: stream=%d (passes in flight per wave, 1..8)", ring);
     for (int i = 0; n_rows && i < count; ++i)
         if (n_rows[i] % rows) return fail(PSN_E_UNSUPPORTED, "plan: streaming needs every matrix to hold a multiple of %d rows", rows);
@@ -904,15 +904,16 @@ static int32_t make_plan(int32_t qtype, int32_t scheme, int64_t N, int64_t K, in
         q.lanes_per_row = gs;
         q.stream = 1;
         /* One pass per wave while the chip holds that many waves in one workgroup per compute unit
-         * (four waves, then eight); beyond that, four-wave workgroups, as many as stay resident, and the
-         * waves loop.  fp32 activations pass through registers on their way into LDS: 256 threads hold
-         * K <= 8192.  (Measured on MI355X: 1536 passes run 6.4 us with 192 x 512 threads, 7.0 us with
-         * 384 x 256.) */
+         * (four waves up to eight, so that every compute unit gets a workgroup); beyond that, four-wave
+         * workgroups, as many as stay resident, and the waves loop.  fp32 activations pass through
+         * registers on their way into LDS: 256 threads hold K <= 8192.  (Measured on MI355X: 1536 passes
+         * run 6.0 us with 256 x 384 threads, 6.4 us with 192 x 512, 7.0 us with 384 x 256.) */
         const int64_t npass = N / rows;
         /* (Between eight and sixteen passes per compute unit, e.g. one 14336 x 4096 matrix: eight-wave workgroups, one
          * per compute unit, whose waves loop twice, measured 9.0-9.7 us against 10.5-11.4 us for three four-wave workgroups.) */
         const bool two_rounds = npass > 8 * (int64_t)cus && npass <= 16 * (int64_t)cus;
-        q.threads = (npass > 4 * (int64_t)cus && npass <= 8 * (int64_t)cus) || two_rounds || (p.stage_lds == 2 && K > 8192) ? 512 : 256;
+        q.threads = two_rounds || (p.stage_lds == 2 && K > 8192) ? 512
+                    : npass > 4 * (int64_t)cus && npass <= 8 * (int64_t)cus ? 64 * (int32_t)((npass + cus - 1) / cus) : 256;
         int64_t lds = 0;
         q.blocks = 1;
         if (whole && stream_plan_check(qtype, scheme, K, batch, &q, n_rows, count, 160 * 1024, &lds) == PSN_OK) {
@@ -1012,7 +1013,9 @@ static int32_t plan_is_valid(const psn_matvec_plan *p, int32_t qtype, int32_t sc
     const int g = p->lanes_per_row, r = p->rows_in_flight, nb = p->batch_tile;
     if (!(g == 8 || g == 16 || g == 32 || g == 64)) return fail(PSN_E_UNSUPPORTED, "plan: lanes_per_row=%d", g);
     if (nb < batch || !(nb == 1 || nb == 2 || nb == 4 || nb == 8)) return fail(PSN_E_UNSUPPORTED, "plan: batch_tile=%d for batch %d", nb, batch);
-    if (p->threads != 256 && p->threads != 512) return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512)", p->threads);
+    /* the streaming kernels index by the wave count they are given; the others are written for four or eight waves */
+    if (p->stream && p->mfma == 0 ? (p->threads < 256 || p->threads > 512 || p->threads % 64) : (p->threads != 256 && p->threads != 512))
+        return fail(PSN_E_UNSUPPORTED, "plan: threads=%d (256 or 512; streaming kernels: 256 .. 512 in whole waves)", p->threads);
     if (r != 1) return fail(PSN_E_UNSUPPORTED, "plan: no kernel for rows_in_flight=%d batch_tile=%d scheme=%d", r, nb, scheme);
     if (p->blocks < 1 || p->blocks > (1 << 20)) return fail(PSN_E_UNSUPPORTED, "plan: blocks=%d", p->blocks);
     int32_t lds = 0;
@@ -1788,7 +1791,7 @@ extern "C" int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_
         psn_matvec_plan q = plan;
         q.stage_lds = 3;
         int64_t lds = 0;
-        if (K > 4096 && q.threads == 256) q.threads = 512;       /* x, delta and the weights: four 16-byte registers each per thread */
+        if (K > 4096 && q.threads < 512) q.threads = 512;        /* x, delta and the weights: four 16-byte registers each per thread */
         if (stream_plan_check(qtype, PSN_ACT_Q8, K, 1, &q, sg.N, sg.count, mod->ctx->max_lds, &lds) == PSN_OK) {
             if (q.threads != plan.threads) {
                 const int64_t rows = 64 / q.lanes_per_row, npass = sg.total / rows, wpb = q.threads / 64;

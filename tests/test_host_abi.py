@@ -70,7 +70,8 @@ def test_matvec_plan_is_host_arithmetic(lib):
                     p = backend.matvec_plan(qt, scheme, n, k, batch)
                     assert p.lanes_per_row in (8, 16, 32, 64) and p.rows_in_flight == 1
                     assert p.batch_tile >= batch and p.batch_tile in (1, 2, 4, 8)
-                    assert 1 <= p.blocks <= 256 * 16 and p.threads in (256, 512)
+                    assert 1 <= p.blocks <= 256 * 16
+                    assert p.threads in (256, 512) or (p.stream and not p.mfma and p.threads in (320, 384, 448))
                     assert p.mfma in (0, 1, 2, 4, 8) and (p.mfma == 0 or (batch >= 2 and scheme == _ffi.ACT_Q8 and qt in (_ffi.Q4_K, _ffi.Q5_K)))
     for args, code in (((_ffi.Q4_0, 1, 0, 4096, 1), _ffi.E_SHAPE), ((_ffi.Q4_0, 1, 16, 4096 + 32, 1), _ffi.E_SHAPE),
                        ((_ffi.Q4_0, 1, 16, 4096, 9), _ffi.E_SHAPE), ((_ffi.Q8_K, 1, 16, 4096, 1), _ffi.E_UNSUPPORTED),
@@ -89,7 +90,9 @@ def test_matvec_plans_are_consistent_over_many_shapes(lib):
                 for batch in (1, 2, 3, 5, 8):
                     for x_is_f32 in (False, True):
                         p = backend.matvec_plan(qt, _ffi.ACT_Q8, n, k, batch, 256, x_is_f32)
-                        assert p.threads in (256, 512) and 1 <= p.blocks <= 1 << 20, p.as_dict()
+                        assert 1 <= p.blocks <= 1 << 20, p.as_dict()
+                        # four or eight waves; the batch-1 streaming kernels also take five to seven
+                        assert p.threads in (256, 512) or (p.stream and not p.mfma and p.threads in (320, 384, 448)), p.as_dict()
                         if p.mfma:
                             c, waves = k // 256, p.threads // 64
                             assert qt in (_ffi.Q4_K, _ffi.Q5_K) and batch >= 2 and n % 16 == 0, p.as_dict()
@@ -101,6 +104,13 @@ def test_matvec_plans_are_consistent_over_many_shapes(lib):
                             assert lds <= 160 * 1024, p.as_dict()
                         elif p.stream:
                             assert batch == 1 and p.stage_lds in (1, 2) and k // 256 <= p.lanes_per_row, p.as_dict()
+                            npass = n // (64 // p.lanes_per_row)
+                            if 4 * 256 < npass <= 8 * 256 and p.threads < 512:
+                                # one pass per wave, one workgroup on every compute unit
+                                assert p.blocks == 256 and p.blocks * (p.threads // 64) >= npass, p.as_dict()
+    # Llama-3-8B's fused q/k/v projection: 6144 rows of sixteen chunks, four rows a pass -> 1536 passes = 256 x 6 waves
+    p = backend.matvec_plan(_ffi.Q4_0, _ffi.ACT_Q8, 6144, 4096, 1, 256, True)
+    assert (p.stream > 0, p.threads, p.blocks) == (True, 384, 256), p.as_dict()
 
 
 def test_prefill_plans_are_consistent_over_many_shapes(lib):
