@@ -39,8 +39,8 @@ MAX_LINE_CHARS = 2000
 # 256 MiB device-to-device copy (the copies are what --calibrate-copy adds).  Keyed by the kernel the figure was
 # taken on: when the library picks another kernel for the launch, `traffic` is null instead of a stale number.
 # The figures and the commands are in profiles/matvec_q4_0_llama3_8b_step.md.
-MEASURED_TRAFFIC_BYTES = {"psn_mvs_q4_0_q8_g16_xf_s2": 66_512_700, "psn_mvs_q4_0_q8_g16_xf_s3": 14_517_000,
-                          "psn_mvs_q4_0_q8_g16_xf_s1": 9_781_300, "psn_mvs_q4_0_q8_g64_xf_s1": 33_708_900}
+MEASURED_TRAFFIC_BYTES = {"psn_mvs_q4_0_q8_g16_xf_s2": 66_491_100, "psn_mvs_q4_0_q8_g16_xf_s3": 14_512_800,
+                          "psn_mvs_q4_0_q8_g16_xf_s1": 9_782_300, "psn_mvs_q4_0_q8_g64_xf_s1": 33_703_700}
 HIDDEN, KV, FFN, LAYERS = 4096, 1024, 14336, 32
 BPW_Q4_0 = 18.0 / 32.0
 
