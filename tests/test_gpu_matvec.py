@@ -440,7 +440,8 @@ def test_streaming_kernels_every_variant(hip, orc, qname):
             if k // 256 > g:
                 continue
             for stage in (1, 2):
-                for threads, blocks, ring in ((256, 2, 1), (512, 1, 2), (512, 3, 3), (256, 5, 4)):
+                # (five to seven waves per workgroup: the plans that give every compute unit one pass per wave)
+                for threads, blocks, ring in ((256, 2, 1), (512, 1, 2), (512, 3, 3), (256, 5, 4), (384, 2, 2), (320, 1, 1), (448, 3, 2)):
                     p = _ffi.MatvecPlan()
                     p.lanes_per_row, p.rows_in_flight, p.batch_tile, p.stage_lds, p.blocks, p.threads, p.stream = g, 1, 1, stage, blocks, threads, ring
                     say(f"stream {qname} k={k} ns={ns} {p.as_dict()}")
@@ -458,7 +459,7 @@ def test_streaming_kernels_every_variant(hip, orc, qname):
                         err = G.max_rel_err(y.download(np.float32, (1, n)), ref)
                         assert err < PARITY_TOL, (p.as_dict(), k, n, err)
     say(f"stream {qname}: {ran} variants ran, {refused} refused")
-    assert ran >= (20 if qname == "Q6_K" else 40)
+    assert ran >= (35 if qname == "Q6_K" else 70)
 
 
 # ------------------------------------------------------------------ small-batch int8-MFMA kernels
@@ -580,6 +581,13 @@ def test_streaming_plan_is_refused_where_it_cannot_run(hip, orc):
     with pytest.raises(backend.PsnError) as e:
         hip.quantized_matvec_planned(w4, x, y, 1, _ffi.ACT_Q8, p)
     assert e.value.code == _ffi.E_UNSUPPORTED
+    # workgroups are whole waves, four to eight of them; only the streaming kernels take five to seven
+    w80 = hip.upload_weight(orc.Q4_0, weights(orc, "Q4_0", 912, 80, k), 80, k)
+    for stream, threads in ((1, 352), (1, 192), (1, 576), (0, 384)):
+        p.stream, p.threads = stream, threads
+        with pytest.raises(backend.PsnError) as e:
+            hip.quantized_matvec_planned(w80, x, y, 1, _ffi.ACT_Q8, p)
+        assert e.value.code == _ffi.E_UNSUPPORTED and "threads" in str(e.value), (stream, threads, str(e.value))
 
 
 def test_two_branch_graph_of_independent_launches(hip, orc):
