@@ -174,6 +174,83 @@ PSN_DEV void q8_K_quant_wave(const float4 v, int lane, u32 &packed, float &d_out
     s16 = group_sum_i<4>(s4);
 }
 
+/* Q8_K with sixteen lanes to a super-block, four super-blocks to a wave: lane l15 of the sixteen holds the 16-byte
+ * words l15, 16 + l15, 32 + l15, 48 + l15 of the block (v[0..3]), i.e. elements (16 i + l15) * 4 + e.  All
+ * reductions stay inside a 16-lane DPP row (no trip through the LDS crossbar), and a wave runs through one
+ * dependent chain for four blocks instead of four chains.  Same results as q8_K_quant_wave: packed[i] are the
+ * int8 of v[i], d_out the block's scale, s16[i] the sum over the 16-element group that word 16 i + l15 belongs to
+ * (valid in every lane of its quad).  A block of zeros gives zeros. */
+PSN_DEV u32 row16_max_u(u32 b) {
+    b = max(b, (u32)dpp_i<0xB1>((int)b));
+    b = max(b, (u32)dpp_i<0x4E>((int)b));
+    b = max(b, (u32)dpp_i<0x141>((int)b));
+    return max(b, (u32)dpp_i<0x140>((int)b));
+}
+PSN_DEV u32 row16_min_u(u32 b) {
+    b = min(b, (u32)dpp_i<0xB1>((int)b));
+    b = min(b, (u32)dpp_i<0x4E>((int)b));
+    b = min(b, (u32)dpp_i<0x141>((int)b));
+    return min(b, (u32)dpp_i<0x140>((int)b));
+}
+PSN_DEV u32 row16_or(u32 b) {
+    b |= (u32)dpp_i<0xB1>((int)b);
+    b |= (u32)dpp_i<0x4E>((int)b);
+    b |= (u32)dpp_i<0x141>((int)b);
+    return b | (u32)dpp_i<0x140>((int)b);
+}
+PSN_DEV void q8_K_quant_row16(const float4 (&v)[4], int lane, u32 (&packed)[4], float &d_out, int (&s16)[4]) {
+    float e[16];
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) { e[4 * i] = v[i].x; e[4 * i + 1] = v[i].y; e[4 * i + 2] = v[i].z; e[4 * i + 3] = v[i].w; }
+    /* the lane's element of largest magnitude, the earlier one on ties (its own elements are in index order):
+     * a tournament that carries the signed value along */
+    float ab[16], sg[16];
+    _Pragma("unroll") for (int p = 0; p < 16; ++p) { ab[p] = fabsf(e[p]); sg[p] = e[p]; }
+    _Pragma("unroll") for (int w = 1; w < 16; w *= 2)
+        _Pragma("unroll") for (int p = 0; p < 16; p += 2 * w) {
+            const bool later = ab[p + w] > ab[p];
+            sg[p] = later ? sg[p + w] : sg[p];
+            ab[p] = later ? ab[p + w] : ab[p];
+        }
+    const float amax = ab[0], mine = sg[0];
+    const float gmax = __uint_as_float(row16_max_u(__float_as_uint(amax)));
+    const bool zero = gmax == 0.f;
+    /* the block's first element of largest magnitude.  One lane of the sixteen holds the maximum, except on exact
+     * ties between lanes: then the element indices decide (a second and third reduction, taken by the whole wave) */
+    const bool holds = amax == gmax && !zero;
+    const unsigned long long holders = __builtin_amdgcn_ballot_w64(holds);
+    bool tie = false;
+    _Pragma("unroll") for (int g = 0; g < 4; ++g) {
+        const unsigned b = (unsigned)(holders >> (16 * g)) & 0xffffu;
+        tie = tie || (b & (b - 1u)) != 0u;
+    }
+    float vmax;
+    if (!tie) {                                             /* wave-uniform */
+        vmax = __uint_as_float(row16_or(holds ? __float_as_uint(mine) : 0u));
+    } else {
+        u32 pos = 0xffffffffu;                              /* index of the lane's `mine` inside the block */
+        _Pragma("unroll") for (int p = 15; p >= 0; --p)
+            if (fabsf(e[p]) == amax) pos = (u32)(((p >> 2) * 16 + (lane & 15)) * 4 + (p & 3));
+        pos = holds ? pos : 0xffffffffu;
+        const u32 first = row16_min_u(pos);
+        vmax = __uint_as_float(row16_or(holds && pos == first ? __float_as_uint(mine) : 0u));
+    }
+    const float vm = zero ? 1.f : vmax;
+    const bool fast = __builtin_amdgcn_ballot_w64(!(zero || fast_div_range(gmax))) == 0ull;   /* every block of the wave */
+    const float iscale = fast ? div_rn(-127.f, vm, rcp_rn(vm)) : -127.f / vm;
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {
+        int q[4], s4 = 0;
+        _Pragma("unroll") for (int k = 0; k < 4; ++k) {
+            q[k] = (int)__builtin_rintf(iscale * e[4 * i + k]);
+            q[k] = q[k] > 127 ? 127 : q[k];
+            s4 += q[k];
+        }
+        packed[i] = pack_bytes4(q[0], q[1], q[2], q[3]);
+        s16[i] = group_sum_i<4>(s4);
+    }
+    const float d = fast ? rcp_rn(iscale) : 1.f / iscale;
+    d_out = zero ? 0.f : d;
+}
+
 /* ---- hand-scheduled memory access ------------------------------------------------------------
  * Kernels that keep several direct-to-LDS loads in flight place every wait themselves: the compiler's
  * wait insertion cannot tell ring buffers in dynamic LDS apart and would drain ALL outstanding loads

@@ -743,10 +743,14 @@ struct StreamStager {
             const int idx = threadIdx.x + i * nthreads;
             return idx < C * 64 ? idx : -1;
         } else {
-            const int sb = (threadIdx.x >> 6) + i * (nthreads >> 6);
-            return sb < C ? sb * 64 + (int)(threadIdx.x & 63) : -1;
+            const int sb = q8_K_block(i);
+            return sb < C ? sb * 64 + (i & 3) * 16 + (int)(threadIdx.x & 15) : -1;
         }
     }
+    /* Q8_K: sixteen lanes share a super-block and a wave works on four at a time -- slots 0..3 hold the four
+     * quarters of the lane's block in the first round (blocks 0 .. 4 waves - 1 of the vector), slots 4..7 those
+     * of the second round */
+    PSN_DEV int q8_K_block(int i) const { return (i >> 2) * (nthreads >> 4) + (int)(threadIdx.x >> 4); }
 
     PSN_DEV void issue(const psn_matvec_args &a, int d_per_col, int s_per_col) {
         C = a.K >> 8;
@@ -785,10 +789,9 @@ struct StreamStager {
                     if (idx < total4) t[i] = global_read128(x4 + idx);
                 }
             } else {
-                const int wpb = nthreads >> 6, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
                 UNROLL for (int i = 0; i < SLOTS; ++i) {
-                    const int sb = wid + i * wpb;
-                    if (sb < C) t[i] = global_read128(x4 + sb * 64 + lane);
+                    const int idx = f32_word(i);
+                    if (idx >= 0) t[i] = global_read128(x4 + idx);
                 }
             }
         }
@@ -860,17 +863,25 @@ struct StreamStager {
                 }
             }
         } else {
-            const int wpb = nthreads >> 6, wid = threadIdx.x >> 6;
-            UNROLL for (int k = 0; k < SLOTS; ++k) {
-                const int sb = wid + k * wpb;
-                if (sb < C) {                                      /* wave-uniform */
-                    u32 packed;
+            const int l15 = lane & 15;
+            UNROLL for (int r = 0; r < SLOTS / 4; ++r) {
+                const int sb = q8_K_block(4 * r);
+                /* wave-uniform: does the wave's first block of this round exist?  (XSRC 3 holds one round) */
+                if ((XSRC != 3 || r == 0) && __builtin_amdgcn_readfirstlane(sb) < C) {
+                    float4 v[4];
+                    UNROLL for (int i = 0; i < 4; ++i)
+                        v[i] = make_float4(__uint_as_float(t[4 * r + i].x), __uint_as_float(t[4 * r + i].y), __uint_as_float(t[4 * r + i].z), __uint_as_float(t[4 * r + i].w));
+                    u32 packed[4];
                     float d;
-                    int s16;
-                    q8_K_quant_wave(make_float4(__uint_as_float(t[k].x), __uint_as_float(t[k].y), __uint_as_float(t[k].z), __uint_as_float(t[k].w)), lane, packed, d, s16);
-                    lds_write32(qs_addr + (u32)(sb * 272 + lane * 4), packed);
-                    if ((lane & 3) == 0) lds_write16(s_addr + (u32)(sb * 16 + (lane >> 2)) * 2u, (u32)s16 & 0xffffu);
-                    if (lane == 0) lds_write32(d_addr + (u32)sb * 4u, __float_as_uint(d));
+                    int s16[4];
+                    q8_K_quant_row16(v, lane, packed, d, s16);
+                    if (sb < C) {
+                        UNROLL for (int i = 0; i < 4; ++i) {
+                            lds_write32(qs_addr + (u32)(sb * 272 + (i * 16 + l15) * 4), packed[i]);
+                            if ((lane & 3) == 0) lds_write16(s_addr + (u32)(sb * 16 + i * 4 + (l15 >> 2)) * 2u, (u32)s16[i] & 0xffffu);
+                        }
+                        if (l15 == 0) lds_write32(d_addr + (u32)sb * 4u, __float_as_uint(d));
+                    }
                 }
             }
         }

@@ -735,6 +735,49 @@ def test_norm_fused_projection_argument_errors(hip, orc):
     assert e.value.name == "PSN_E_INVALID_ARG"
 
 
+@pytest.mark.parametrize("qname", ["Q4_0", "Q4_K", "Q5_K", "Q6_K"])
+@pytest.mark.parametrize("k,n", [(4096, 1024), (14336, 512), (2048, 1024)])
+def test_streaming_kernels_quantize_awkward_activations_like_the_quantize_kernel(hip, orc, qname, k, n):
+    """The streaming kernels quantize fp32 activations while they stage them (Q8_K: sixteen lanes to a block,
+    four blocks to a wave).  Blocks that take the quantizer's rare paths -- all zeros, the largest magnitude held
+    twice in one lane, in two lanes of one quarter, in two quarters and with opposite signs, a maximum too small
+    or too large for the reciprocal shortcuts -- must give the very floats that quantizing with the stand-alone
+    kernel and running the same matvec on its output gives, and match the oracle."""
+    t = getattr(orc, qname)
+    x = G.seeded_acts(7000 + k, 1, k)
+    x[0, 0:256] = 0                                         # a zero block
+    x[0, 256:512] *= 0.1
+    x[0, 256 + 9] = x[0, 256 + 10] = 2.5                    # twice in one 16-byte word (one lane)
+    x[0, 512:768] *= 0.1
+    x[0, 512 + 4 * 3] = -2.0                                # two lanes of the first quarter
+    x[0, 512 + 4 * 11 + 2] = 2.0
+    x[0, 768:1024] *= 0.1
+    x[0, 768 + 64 * 2 + 4 * 5 + 1] = 1.75                   # third quarter first in memory ...
+    x[0, 768 + 64 * 3 + 4 * 5 + 1] = -1.75                  # ... same lane, fourth quarter
+    x[0, 768 + 64 * 1 + 4 * 14] = -1.75                     # and an earlier element in another lane: this one wins
+    x[0, 1024:1280] *= 1e-36                                # below the range of the reciprocal shortcuts
+    x[0, 1280:1536] *= 1e30 if qname != "Q4_0" else 100.0   # above it (Q8_0 blocks keep their scale in fp16: stay inside it)
+    x[0, k - 256:k] *= 0.1
+    x[0, k - 1] = -4.0                                      # the last element of the vector
+    x[0, k - 256] = 4.0                                     # ties with the first of its block
+    W = weights(orc, qname, 7100 + k, n, k)
+    ref = orc.matvec(t, orc.ACT_Q8, W, x, n, k)
+    w = hip.upload_weight(t, W, n, k)
+    xb = hip.upload(x)
+    plan = backend.matvec_plan(t, _ffi.ACT_Q8, n, k, 1, hip.compute_units, True)
+    say(f"awkward activations {qname} k={k} n={n} {plan.as_dict()}")
+    assert plan.stream and plan.stage_lds == 2              # the kernel under test
+    y1 = hip.upload(np.full((1, n), np.nan, np.float32))
+    hip.quantized_matvec(w, xb, y1, 1, _ffi.ACT_Q8)
+    xq = hip.quantize_activations(xb, k, 1, backend.act_type_for(t))
+    y2 = hip.upload(np.full((1, n), np.nan, np.float32))
+    hip.quantized_matvec_q8(w, xq, y2, 1)
+    got1, got2 = y1.download(np.float32, (1, n)), y2.download(np.float32, (1, n))
+    assert np.array_equal(got1.view(np.uint32), got2.view(np.uint32))
+    # the huge block dominates the sums: relative to the largest output
+    assert np.all(np.isfinite(got1)) and G.max_rel_err(got1, ref) < PARITY_TOL
+
+
 def test_default_plans_over_seeded_random_shapes(hip, orc):
     """Whatever the planner picks for shapes nobody tuned for (odd row counts, one to 56 chunks per row,
     every batch, both schemes, fp32 and pre-quantized input) must match the oracle."""
