@@ -203,12 +203,14 @@ struct Stager {
                     }
                 }
             } else {
-                const int nsb = a.batch * C, wpb = nthreads >> 6, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+                /* sixteen lanes to a super-block, four blocks to a wave and round: slots 0..3 hold the four quarters
+                 * of the lane's block in the first round, slots 4..7 those of the second */
+                const int nsb = a.batch * C, wpb = nthreads >> 6, l15 = threadIdx.x & 15;
                 in_regs = nsb <= SLOTS * wpb;
                 if (in_regs) {
                     UNROLL for (int i = 0; i < SLOTS; ++i) {
-                        const int sb = wid + i * wpb;
-                        if (sb < nsb) { const float4 v = x4[sb * 64 + lane]; t[i] = make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)); }
+                        const int sb = (i >> 2) * (wpb * 4) + (int)(threadIdx.x >> 4);
+                        if (sb < nsb) { const float4 v = x4[sb * 64 + (i & 3) * 16 + l15]; t[i] = make_uint4(__float_as_uint(v.x), __float_as_uint(v.y), __float_as_uint(v.z), __float_as_uint(v.w)); }
                     }
                 }
             }
@@ -267,23 +269,38 @@ struct Stager {
                         for (int i = threadIdx.x; i < total4; i += nthreads) one(i, x4[i]);
                     }
                 } else {
-                    const int nsb = a.batch * C, wpb = nthreads >> 6, wid = threadIdx.x >> 6;
-                    auto one = [&](int sb, const float4 v) {
-                        u32 packed;
+                    const int nsb = a.batch * C, wpb = nthreads >> 6, l15 = lane & 15;
+                    /* the wave's four blocks of one round: sb is this lane's, v its four quarters (zeros past the end) */
+                    auto four = [&](int sb, const float4 (&v)[4]) {
+                        u32 packed[4];
                         float d;
-                        int s16;
-                        q8_K_quant_wave(v, lane, packed, d, s16);
-                        l_qs[sb * 68 + lane] = packed;
-                        if ((lane & 3) == 0) l_s[sb * 16 + (lane >> 2)] = (ST)s16;
-                        if (lane == 0) l_d[sb] = d;
+                        int s16[4];
+                        q8_K_quant_row16(v, lane, packed, d, s16);
+                        if (sb < nsb) {
+                            UNROLL for (int i = 0; i < 4; ++i) {
+                                l_qs[sb * 68 + i * 16 + l15] = packed[i];
+                                if ((lane & 3) == 0) l_s[sb * 16 + i * 4 + (l15 >> 2)] = (ST)s16[i];
+                            }
+                            if (l15 == 0) l_d[sb] = d;
+                        }
                     };
                     if (in_regs) {
-                        UNROLL for (int k = 0; k < SLOTS; ++k) {
-                            const int sb = wid + k * wpb;
-                            if (sb < nsb) one(sb, make_float4(__uint_as_float(t[k].x), __uint_as_float(t[k].y), __uint_as_float(t[k].z), __uint_as_float(t[k].w)));
+                        UNROLL for (int r = 0; r < SLOTS / 4; ++r) {
+                            const int sb = r * (wpb * 4) + (int)(threadIdx.x >> 4);
+                            if (__builtin_amdgcn_readfirstlane(sb) < nsb) {       /* wave-uniform: the round's first block exists */
+                                float4 v[4];
+                                UNROLL for (int i = 0; i < 4; ++i)
+                                    v[i] = make_float4(__uint_as_float(t[4 * r + i].x), __uint_as_float(t[4 * r + i].y), __uint_as_float(t[4 * r + i].z), __uint_as_float(t[4 * r + i].w));
+                                four(sb, v);
+                            }
                         }
                     } else {
-                        for (int sb = wid; sb < nsb; sb += wpb) one(sb, x4[sb * 64 + lane]);
+                        for (int base = (int)(threadIdx.x >> 6) * 4; base < nsb; base += wpb * 4) {
+                            const int sb = base + (lane >> 4);
+                            float4 v[4];
+                            UNROLL for (int i = 0; i < 4; ++i) v[i] = sb < nsb ? x4[sb * 64 + i * 16 + l15] : make_float4(0.f, 0.f, 0.f, 0.f);
+                            four(sb, v);
+                        }
                     }
                 }
             }
