@@ -373,6 +373,20 @@ int32_t psn_swiglu_q8(psn_module *mod, psn_stream *s, const psn_buf *gate, const
 int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, int32_t count,
                                const psn_buf *const *W, const psn_buf *x, const psn_buf *delta, const psn_buf *norm_weight,
                                psn_buf *h_out, psn_buf *const *y_f32, const int64_t *N, int64_t K, float eps);
+/* The same launch for a feed-forward block's gate | up pair with SwiGLU applied to the two products before they
+ * leave the kernel:
+ *     h = x + delta;  n = q8(h * rsqrt(mean(h^2) + eps) * norm_weight);  act_f32[i] = silu(W_gate[i] . n) * (W_up[i] . n)
+ * (N rows each, act_f32 holds N floats) -- the floats psn_qmatvec_norm_multi + psn_swiglu return, without the
+ * SwiGLU launch and without the two N-vectors in between: a wave multiplies the same rows of both matrices one
+ * after the other and keeps the first product in a register.  The down projection then takes act_f32 through
+ * psn_qmatvec, which quantizes while it stages.  Only shapes the fused streaming kernels serve (batch 1, rows
+ * of at most 8192, N a multiple of the rows per pass): psn_qmatvec_norm_swiglu_check says beforehand, by host
+ * arithmetic alone, whether a shape is one of them (PSN_OK) or the three separate calls are needed
+ * (PSN_E_UNSUPPORTED).  No counterpart in the reference's CPU path, which runs the steps one by one. */
+int32_t psn_qmatvec_norm_swiglu(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W_gate,
+                                const psn_buf *W_up, const psn_buf *x, const psn_buf *delta, const psn_buf *norm_weight,
+                                psn_buf *h_out, psn_buf *act_f32, int64_t N, int64_t K, float eps);
+int32_t psn_qmatvec_norm_swiglu_check(int32_t qtype, int64_t N, int64_t K, int32_t compute_units);
 int32_t psn_attention_decode_q8(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
                                 psn_buf *workspace, psn_buf *out, psn_buf *out_q, int32_t act_type, int32_t n_heads,
                                 int32_t n_kv_heads, int32_t head_dim, int32_t n_ctx);

@@ -104,6 +104,8 @@ SIGNATURES = {
     "psn_add_rmsnorm_q8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64, C.c_float]),
     "psn_swiglu_q8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i64]),
     "psn_qmatvec_norm_multi": (_i32, [_vp, _vp, _i32, _i32, _i32, _pp, _vp, _vp, _vp, _vp, _pp, C.POINTER(_i64), _i64, C.c_float]),
+    "psn_qmatvec_norm_swiglu": (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, C.c_float]),
+    "psn_qmatvec_norm_swiglu_check": (_i32, [_i32, _i64, _i64, _i32]),
     "psn_attention_decode_q8": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32]),
     "psn_rope_table": (_i32, [_vp, _vp, _vp, _i32, _i32, C.c_float]),
     "psn_attention_decode_rope": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp]),

@@ -281,6 +281,18 @@ class HipBackend:
         _check(self.lib.psn_qmatvec_norm_multi(self.module, self.stream, w0.qtype, LAYOUT_GGUF, n, W, x.handle, self._h(delta), norm_weight.handle,
                                                self._h(h_out), Y, N, w0.k, eps))
 
+    def quantized_matvec_norm_swiglu(self, w_gate: QuantizedTensor, w_up: QuantizedTensor, x: DeviceBuffer, delta, norm_weight: DeviceBuffer,
+                                     h_out, act: DeviceBuffer, eps: float = 1e-5):
+        """act = silu(w_gate . n) * (w_up . n) with n = q8(rmsnorm(x + delta) * norm_weight), one launch (psn_qmatvec_norm_swiglu)."""
+        if (w_gate.qtype, w_gate.n, w_gate.k) != (w_up.qtype, w_up.n, w_up.k):
+            raise ValueError("gate and up projections must share format and shape")
+        _check(self.lib.psn_qmatvec_norm_swiglu(self.module, self.stream, w_gate.qtype, LAYOUT_GGUF, w_gate.buf.handle, w_up.buf.handle, x.handle,
+                                                self._h(delta), norm_weight.handle, self._h(h_out), act.handle, w_gate.n, w_gate.k, eps))
+
+    def norm_swiglu_supported(self, qtype: int, n: int, k: int) -> bool:
+        """Whether psn_qmatvec_norm_swiglu serves this shape on this device (host arithmetic)."""
+        return int(self.lib.psn_qmatvec_norm_swiglu_check(qtype, n, k, self.compute_units)) == 0
+
     def quantized_matvec_planned(self, ws, x: DeviceBuffer, ys, batch: int, scheme: int, plan: MatvecPlan):
         w0, n, W, Y, N = self._pack(ws, ys)
         _check(self.lib.psn_qmatvec_planned(self.module, self.stream, w0.qtype, scheme, n, W, x.handle, Y, N, w0.k, batch, C.byref(plan)))

@@ -1050,6 +1050,7 @@ struct norm_fusion {
     const float *delta, *weight;
     float *h_out;
     float eps;
+    bool pair;      /* two matrices, a gate and an up projection: the launch stores silu(W0 x) * (W1 x) into y[0] */
 };
 
 static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t scheme, const seg_list &sg, const void *x,
@@ -1110,8 +1111,10 @@ static int32_t run_matvec(psn_module *mod, psn_stream *s, int32_t qtype, int32_t
         }
         a.ring = ring;
         (void)rows;
+        if (norm && norm->pair && (plan->stage_lds != 3 || sg.count != 2 || sg.N[0] != sg.N[1] || g > 32))
+            return fail(PSN_E_UNSUPPORTED, "plan: the SwiGLU-fused launch takes two matrices of equal height on the norm-fused streaming kernels");
         snprintf(name, sizeof name, "psn_mvs_%s_q8_g%d_%s_s%d", fmt_name(qtype), g,
-                 plan->stage_lds == 3 ? "xn" : plan->stage_lds == 2 ? "xf" : "lds", sg.count);
+                 plan->stage_lds == 3 ? (norm->pair ? "xnp" : "xn") : plan->stage_lds == 2 ? "xf" : "lds", sg.count);
         return launch(mod, s, name, (unsigned)plan->blocks, (unsigned)plan->threads, (unsigned)total, &a);
     }
     if (scheme == PSN_ACT_Q8 && plan->stage_lds == 2) {
@@ -1789,7 +1792,7 @@ extern "C" int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_
     psn_matvec_plan plan;
     if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, 1, mod->ctx->compute_units, true, sg.N, sg.count, &plan))) return rc;
     if ((rc = bind(mod->ctx))) return rc;
-    norm_fusion nf = {delta ? (const float *)delta->p : nullptr, (const float *)norm_weight->p, h_out ? (float *)h_out->p : nullptr, eps};
+    norm_fusion nf = {delta ? (const float *)delta->p : nullptr, (const float *)norm_weight->p, h_out ? (float *)h_out->p : nullptr, eps, false};
     if (plan.stream && plan.stage_lds == 2) {
         psn_matvec_plan q = plan;
         q.stage_lds = 3;
@@ -1824,6 +1827,58 @@ extern "C" int32_t psn_qmatvec_norm_multi(psn_module *mod, psn_stream *s, int32_
     if ((rc = launch_add_rmsnorm(mod, s, (float *)x->p, nf.delta, nf.weight, nullptr, nf.h_out, qo, K, eps, /*keep_x=*/true))) return rc;
     if ((rc = make_plan(qtype, PSN_ACT_Q8, sg.total, K, 1, mod->ctx->compute_units, false, sg.N, sg.count, &plan))) return rc;
     return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, ws, K, 1, &plan);
+}
+
+/* the plan of the SwiGLU-fused gate | up launch, or an error where no fused kernel serves the shape */
+static int32_t norm_swiglu_plan(int32_t qtype, int64_t N, int64_t K, int32_t cus, int max_lds, psn_matvec_plan *out) {
+    if (N <= 0 || K <= 0 || K % 256) return fail(PSN_E_SHAPE, "psn_qmatvec_norm_swiglu: N=%lld K=%lld", (long long)N, (long long)K);
+    const int64_t rows[2] = {N, N};
+    psn_matvec_plan plan;
+    int32_t rc = make_plan(qtype, PSN_ACT_Q8, 2 * N, K, 1, cus, true, rows, 2, &plan);
+    if (rc) return rc;
+    if (!plan.stream || plan.stage_lds != 2 || plan.lanes_per_row > 32)
+        return fail(PSN_E_UNSUPPORTED, "psn_qmatvec_norm_swiglu: no fused kernel for N=%lld K=%lld of this format (rows of at most 8192, whole passes)",
+                    (long long)N, (long long)K);
+    plan.stage_lds = 3;
+    if (K > 4096 && plan.threads < 512) {
+        plan.threads = 512;
+        plan.blocks = (plan.blocks + 1) / 2;
+    }
+    int64_t lds = 0;
+    if ((rc = stream_plan_check(qtype, PSN_ACT_Q8, K, 1, &plan, rows, 2, max_lds, &lds))) return rc;
+    *out = plan;
+    return PSN_OK;
+}
+
+extern "C" int32_t psn_qmatvec_norm_swiglu_check(int32_t qtype, int64_t N, int64_t K, int32_t cus) {
+    psn_matvec_plan plan;
+    return norm_swiglu_plan(qtype, N, K, cus > 0 ? cus : 256, 160 * 1024, &plan);
+}
+
+extern "C" int32_t psn_qmatvec_norm_swiglu(psn_module *mod, psn_stream *s, int32_t qtype, int32_t layout, const psn_buf *W_gate,
+                                           const psn_buf *W_up, const psn_buf *x, const psn_buf *delta, const psn_buf *norm_weight,
+                                           psn_buf *h_out, psn_buf *act_f32, int64_t N, int64_t K, float eps) {
+    const char *what = "psn_qmatvec_norm_swiglu";
+    if (layout != PSN_LAYOUT_GGUF) return fail(PSN_E_UNSUPPORTED, "matvec: layout %d", layout);
+    if (!norm_weight || !W_gate || !W_up || !act_f32) return fail(PSN_E_INVALID_ARG, "%s: null handle", what);
+    const psn_buf *W[2] = {W_gate, W_up};
+    psn_buf *y[2] = {act_f32, act_f32};
+    const int64_t rows[2] = {N, N};
+    seg_list sg;
+    int32_t rc = gather_segments(what, mod, s, qtype, PSN_ACT_Q8, 2, W, x, y, rows, K, 1, &sg);
+    if (rc) return rc;
+    if ((rc = check_x_f32(what, x, K, 1)) || (rc = need(norm_weight, K * 4, what, "norm_weight")) ||
+        (delta && (rc = need(delta, K * 4, what, "delta"))) || (h_out && (rc = need(h_out, K * 4, what, "h_out"))))
+        return rc;
+    if (norm_weight->ctx != mod->ctx || (delta && delta->ctx != mod->ctx) || (h_out && h_out->ctx != mod->ctx))
+        return fail(PSN_E_INVALID_ARG, "%s: handles belong to different contexts", what);
+    if (h_out && (h_out->p == x->p || (delta && h_out->p == delta->p)))
+        return fail(PSN_E_INVALID_ARG, "%s: h_out must not alias x or delta (every workgroup reads them while one writes h_out)", what);
+    psn_matvec_plan plan;
+    if ((rc = norm_swiglu_plan(qtype, N, K, mod->ctx->compute_units, mod->ctx->max_lds, &plan))) return rc;
+    if ((rc = bind(mod->ctx))) return rc;
+    norm_fusion nf = {delta ? (const float *)delta->p : nullptr, (const float *)norm_weight->p, h_out ? (float *)h_out->p : nullptr, eps, true};
+    return run_matvec(mod, s, qtype, PSN_ACT_Q8, sg, x->p, K, 1, &plan, &nf);
 }
 
 extern "C" int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q, psn_buf *k, const psn_buf *v, psn_buf *k_cache,

@@ -905,8 +905,12 @@ struct StreamStager {
     }
 };
 
-template <typename F, int G, int XSRC, int NSEG>
+/* PAIR (two matrices of equal height, a gate and an up projection): the launch stores silu(W0 x) * (W1 x) into
+ * y[0] instead of the two products.  A wave then works in units of two passes -- the same S rows of W0, then of
+ * W1 -- keeps the first dot product in a register and stores one value per row. */
+template <typename F, int G, int XSRC, int NSEG, bool PAIR = false>
 PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
+    static_assert(!PAIR || NSEG == 2, "a pair is two matrices");
     typedef typename F::ActSum ST;
     constexpr int S = 64 / G;                                /* rows per pass; every matrix holds a multiple of S rows */
     extern __shared__ uint4 psn_smem[];
@@ -972,6 +976,51 @@ PSN_DEV void mv_q8_stream(const psn_matvec_args &a) {
         }
     };
 
+    if constexpr (PAIR) {
+        /* Units: unit u = passes u and nunits + u (rows u S .. of either matrix).  Whole rounds go wave by wave
+         * like the passes below; the units of the last, partial round are dealt block by block (unit r of it to
+         * block r % blocks, wave r / blocks), so that the compute units, each holding blocks a whole number of
+         * compute units apart, end up with equal shares. */
+        const int nunits = npass >> 1, full = nunits / stride, rem0 = full * stride;
+        const int extra = wib * a.blocks + (int)blockIdx.x;
+        const int mine = full + (rem0 + extra < nunits ? 1 : 0);          /* units of this wave */
+        auto pass_of = [&](int i) {                                       /* the wave's i-th pass, i < 2 * mine */
+            const int k = i >> 1, u = k < full ? p0 + k * stride : rem0 + extra;
+            return (i & 1) ? nunits + u : u;
+        };
+        const int mypasses = 2 * mine;
+        int issued = 0;
+        for (; issued < ring && issued < mypasses; ++issued) issue(pass_of(issued), issued);
+        u32 qs_addr, d_addr, s_addr;
+        st.finish(a, issued * nloads, lds0, qs_addr, d_addr, s_addr);
+        lds_barrier();
+        u32 xr[F::XR];
+        UNROLL for (int i = 0; i < F::XR; ++i) xr[i] = 0;
+        if (j < C) stream_load_x<ST, F::XR>(qs_addr, d_addr, s_addr, j, xr);
+        int b = 0;
+        float gate = 0.f;
+        for (int i = 0; i < mypasses; ++i) {
+            wait_vmcnt((issued - i - 1) * nloads);
+            u32 w[F::DW];
+            UNROLL for (int q = 0; q < F::DW; ++q) w[q] = 0;
+            if (j < C) stream_load_chunk<F>(ring_base + (u32)(b * wbuf + slot * rb + j * F::BYTES), w);
+            else lds_wait();
+            if (issued < mypasses) {
+                issue(pass_of(issued), b);
+                ++issued;
+            }
+            b = b + 1 == ring ? 0 : b + 1;
+            float acc = (j < C) ? F::dot(w, xr) : 0.f;
+            acc = group_sum<G>(acc);
+            if (i & 1) {
+                /* the expression of psn_swiglu, so that the fused launch returns its very floats */
+                if (j == 0) Y0[(pass_of(i) - nunits) * S + slot] = gate / (1.f + __expf(-gate)) * acc;
+            } else {
+                gate = acc;
+            }
+        }
+        return;
+    }
     /* everything the ring holds goes in flight at once */
     int issued = 0;                                          /* passes issued so far */
     for (; issued < ring && p0 + issued * stride < npass; ++issued) issue(p0 + issued * stride, issued);
@@ -1129,7 +1178,13 @@ PSN_DEV void mv_f32(const psn_matvec_args &a) {
     extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_xn_s##NSEG(const psn_matvec_args a) {  \
         mv_q8_stream<F, G, 3, NSEG>(a);                                                                   \
     }
-#define PSN_STREAM_NORM_G(fmt, F, G) PSN_STREAM_NORM_KERNEL(fmt, F, G, 1) PSN_STREAM_NORM_KERNEL(fmt, F, G, 2) PSN_STREAM_NORM_KERNEL(fmt, F, G, 3)
+/* ... and, for a gate | up pair, with SwiGLU applied to the two products (_xnp) */
+#define PSN_STREAM_PAIR_KERNEL(fmt, F, G)                                                                 \
+    extern "C" __global__ void __launch_bounds__(512) psn_mvs_##fmt##_q8_g##G##_xnp_s2(const psn_matvec_args a) {      \
+        mv_q8_stream<F, G, 3, 2, true>(a);                                                                \
+    }
+#define PSN_STREAM_NORM_G(fmt, F, G) PSN_STREAM_NORM_KERNEL(fmt, F, G, 1) PSN_STREAM_NORM_KERNEL(fmt, F, G, 2) PSN_STREAM_NORM_KERNEL(fmt, F, G, 3) \
+    PSN_STREAM_PAIR_KERNEL(fmt, F, G)
 #define PSN_STREAM_G(fmt, F, G) PSN_STREAM_KERNEL(fmt, F, G, 1) PSN_STREAM_KERNEL(fmt, F, G, 2) PSN_STREAM_KERNEL(fmt, F, G, 3) PSN_STREAM_KERNEL(fmt, F, G, 4)
 #define PSN_STREAM_ALL(fmt, F) PSN_STREAM_G(fmt, F, 8) PSN_STREAM_G(fmt, F, 16) PSN_STREAM_G(fmt, F, 32) PSN_STREAM_G(fmt, F, 64) \
     PSN_STREAM_NORM_G(fmt, F, 8) PSN_STREAM_NORM_G(fmt, F, 16) PSN_STREAM_NORM_G(fmt, F, 32)

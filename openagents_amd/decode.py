@@ -84,16 +84,21 @@ class DecodeStep:
     """Owns the activations, KV caches and scratch of one sequence and enqueues one token step."""
 
     def __init__(self, be: HipBackend, shape: LlamaShape, weights: ModelWeights, max_ctx: int, scheme: int = ACT_Q8,
-                 fused_quant: bool = True, fused_norm: bool = True):
+                 fused_quant: bool = True, fused_norm: bool = True, fused_swiglu: bool = True):
         """fused_quant (scheme Q8): the norm, attention and SwiGLU kernels emit their result already
         quantized, and the matvecs read it with the pre-quantized entry points; otherwise every matvec
         quantizes its fp32 input itself.  fused_norm (with fused_quant): the residual add and the RMSNorm
         run inside the projection that consumes them (psn_qmatvec_norm_multi), the residual stream
-        alternating between two buffers."""
+        alternating between two buffers.  fused_swiglu (with fused_norm): layers whose gate and up projections
+        share a format the fused kernels serve get SwiGLU applied inside the gate|up launch
+        (psn_qmatvec_norm_swiglu) and a down projection that quantizes its fp32 input while staging it -- six
+        launches instead of seven."""
         self.be, self.shape, self.w, self.max_ctx, self.scheme = be, shape, weights, max_ctx, scheme
         self.fused = fused_quant and scheme == ACT_Q8
         self.fused_norm = self.fused and fused_norm
         s = shape
+        self.fused_swiglu = [self.fused_norm and fused_swiglu and lw.w_gate.qtype == lw.w_up.qtype
+                             and be.norm_swiglu_supported(lw.w_gate.qtype, s.ffn, s.hidden) for lw in weights.layers]
         if s.n_heads * s.head_dim != s.hidden:
             raise ValueError("n_heads * head_dim must equal hidden")
         f32 = 4
@@ -144,7 +149,7 @@ class DecodeStep:
     def launches_per_token(self) -> int:
         """Every launch of one step, counting one extra per additional format among q|k|v and gate|up."""
         extra = sum(n - 1 for n in self.qkv_launches) + sum(n - 1 for n in self.gate_up_launches)
-        return len(self.w.layers) * self.launches_per_layer + self.launches_outside_layers + extra
+        return len(self.w.layers) * self.launches_per_layer + self.launches_outside_layers + extra - sum(self.fused_swiglu)
 
     def _norm_multi(self, ws, x, delta, norm, h_out, ys):
         """ys = ws . q(rmsnorm(x + delta) * norm): one launch per weight format, each redoing the add and the norm
@@ -154,7 +159,8 @@ class DecodeStep:
 
     def _enqueue_norm_fused(self, pos: int):
         """Seven launches per layer: q|k|v (with add + norm), attention partial, combine, o, gate|up (with
-        add + norm), SwiGLU, down.  The residual stream moves self.x -> self.x2 -> self.x within a layer."""
+        add + norm), SwiGLU, down -- six where SwiGLU runs inside the gate|up launch.  The residual stream moves
+        self.x -> self.x2 -> self.x within a layer."""
         be, s = self.be, self.shape
         be.rope_table(self.rope_tab, s.head_dim, pos, s.rope_theta)
         for li, lw in enumerate(self.w.layers):
@@ -162,9 +168,13 @@ class DecodeStep:
             be.attention_decode_rope(self.q, self.k, self.v, self.k_cache[li], self.v_cache[li], self.attn_ws, None, self.xq_attn,
                                      act_type_for(lw.wo.qtype), s.n_heads, s.n_kv_heads, s.head_dim, pos, self.rope_tab)
             be.quantized_matvec_q8(lw.wo, self.xq_attn, self.o, 1)
-            self._norm_multi([lw.w_gate, lw.w_up], self.x2, self.o, lw.ffn_norm, self.x, [self.gate, self.up])
-            be.swiglu_q8(self.gate, self.up, None, self.xq_f, act_type_for(lw.w_down.qtype), s.ffn)
-            be.quantized_matvec_q8(lw.w_down, self.xq_f, self.down, 1)
+            if self.fused_swiglu[li]:
+                be.quantized_matvec_norm_swiglu(lw.w_gate, lw.w_up, self.x2, self.o, lw.ffn_norm, self.x, self.act, s.eps)
+                be.quantized_matvec(lw.w_down, self.act, self.down, 1, ACT_Q8)
+            else:
+                self._norm_multi([lw.w_gate, lw.w_up], self.x2, self.o, lw.ffn_norm, self.x, [self.gate, self.up])
+                be.swiglu_q8(self.gate, self.up, None, self.xq_f, act_type_for(lw.w_down.qtype), s.ffn)
+                be.quantized_matvec_q8(lw.w_down, self.xq_f, self.down, 1)
         be.quantized_matvec_norm_multi([self.w.lm_head], self.x, self.down, self.w.final_norm, None, [self.logits], s.eps)
 
     def _enqueue_fused(self, pos: int, matvecs_only: bool):
@@ -418,6 +428,7 @@ def main(argv=None):
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--unfused", action="store_true", help="every matvec quantizes its own fp32 input")
     ap.add_argument("--separate-norm", action="store_true", help="RMSNorm as its own launch instead of inside the consuming projection")
+    ap.add_argument("--separate-swiglu", action="store_true", help="SwiGLU as its own launch instead of inside the gate|up projection")
     ap.add_argument("--gguf", help="decode greedily from this llama-architecture model file instead of timing the synthetic step")
     ap.add_argument("--prompt", default="1", help="with --gguf: comma-separated prompt token ids (no tokenizer is part of this library)")
     ap.add_argument("--new", type=int, default=16, help="with --gguf: tokens to generate")
@@ -429,7 +440,7 @@ def main(argv=None):
         load_s = time.time() - t0
         prompt = [int(t) for t in args.prompt.split(",")]
         step = DecodeStep(be, model.shape, model.weights, min(args.ctx, max(len(prompt) + args.new, 1)),
-                          fused_quant=not args.unfused, fused_norm=not args.separate_norm)
+                          fused_quant=not args.unfused, fused_norm=not args.separate_norm, fused_swiglu=not args.separate_swiglu)
         t0 = time.time()
         tokens, logits = greedy_tokens(model, step, prompt, args.new)
         wall = time.time() - t0
@@ -448,7 +459,7 @@ def main(argv=None):
     shape = LlamaShape(n_layers=args.layers)
     t0 = time.time()
     weights = synthetic_weights(be, shape, args.seed)
-    step = DecodeStep(be, shape, weights, args.ctx, fused_quant=not args.unfused, fused_norm=not args.separate_norm)
+    step = DecodeStep(be, shape, weights, args.ctx, fused_quant=not args.unfused, fused_norm=not args.separate_norm, fused_swiglu=not args.separate_swiglu)
     rng = np.random.default_rng(args.seed + 1)
     pos = args.ctx - 1
     kv = rng.standard_normal((pos, shape.kv_dim), dtype=np.float32).astype(np.float16)

@@ -339,7 +339,8 @@ def test_model_file_with_mixed_formats_decodes_like_the_reference(hip, orc, tmp_
     step = DecodeStep(hip, s, model.weights, ctx)
     assert step.fused_norm
     assert step.qkv_launches == [2, 1, 2] and step.gate_up_launches == [1, 2, 1]
-    assert step.launches_per_token == 3 * 7 + 2 + 3
+    assert step.fused_swiglu == [True, False, True]                    # layer 1's gate and up differ in format
+    assert step.launches_per_token == 3 * 7 + 2 + 3 - 2
     with pytest.raises(ValueError):
         DecodeStep(hip, s, model.weights, ctx, fused_norm=False)       # one quantized copy cannot serve Q8_0 and Q8_K readers
 

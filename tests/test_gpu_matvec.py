@@ -693,6 +693,79 @@ def test_norm_fused_projection_matches_oracle(hip, orc, qname, ns, k, with_delta
         assert np.array_equal(db.download(np.float32, (k,)), delta)
 
 
+@pytest.mark.parametrize("qname,n,k", [
+    ("Q4_K", 14336, 4096),                   # Llama-3-8B's feed-forward block: 3584 units on 768 workgroups, a partial last round
+    ("Q4_0", 14336, 4096),
+    ("Q5_K", 1024, 2048),
+    ("Q6_K", 2048, 2048),
+    ("Q8_0", 512, 1024),
+    ("Q4_K", 1016, 512),                     # two chunks per row, eight rows a pass, 127 units
+    ("Q4_K", 4096, 8192),                    # 512-thread staging
+])
+@pytest.mark.parametrize("with_delta", [True, False])
+def test_swiglu_fused_gate_up_returns_the_floats_of_the_three_launches(hip, orc, qname, n, k, with_delta):
+    """psn_qmatvec_norm_swiglu against psn_qmatvec_norm_multi + psn_swiglu on the same inputs: the same dot
+    products in the same order and the same SwiGLU expression, so the same floats bit for bit; and against
+    the oracle's products through numpy's SwiGLU."""
+    qt = getattr(orc, qname)
+    rng = np.random.default_rng(4700 + k + n)
+    x = rng.standard_normal(k, dtype=np.float32) * 2
+    delta = rng.standard_normal(k, dtype=np.float32) if with_delta else None
+    wn = (1 + 0.1 * rng.standard_normal(k)).astype(np.float32)
+    eps = 1e-5
+    bg, bu = weights(orc, qname, 4800, n, k), weights(orc, qname, 4801, n, k)
+    wg, wu = hip.upload_weight(qt, bg, n, k), hip.upload_weight(qt, bu, n, k)
+    xb, wb = hip.upload(x), hip.upload(wn)
+    db = hip.upload(delta) if with_delta else None
+    assert hip.norm_swiglu_supported(qt, n, k)
+    say(f"swiglu-fused {qname} n={n} k={k} delta={with_delta}")
+    hb, act = hip.upload(np.full(k, np.nan, np.float32)), hip.upload(np.full(n, np.nan, np.float32))
+    hip.quantized_matvec_norm_swiglu(wg, wu, xb, db, wb, hb, act, eps)
+    got = act.download(np.float32, (n,))
+    h_ref, xn_ref = norm_ref(x, delta, wn, eps)
+    assert np.array_equal(hb.download(np.float32, (k,)), h_ref)
+    assert np.array_equal(xb.download(np.float32, (k,)), x)
+    # the three launches
+    yg, yu, out = hip.alloc(n * 4), hip.alloc(n * 4), hip.alloc(n * 4)
+    hip.quantized_matvec_norm_multi([wg, wu], xb, db, wb, None, [yg, yu], eps)
+    hip.swiglu(yg, yu, out, n)
+    want = out.download(np.float32, (n,))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # the oracle
+    g = orc.matvec(qt, orc.ACT_Q8, bg, xn_ref, n, k).reshape(-1).astype(np.float64)
+    u = orc.matvec(qt, orc.ACT_Q8, bu, xn_ref, n, k).reshape(-1).astype(np.float64)
+    ref = g / (1.0 + np.exp(-g)) * u
+    assert np.all(np.isfinite(got)) and G.max_rel_err(got.reshape(1, -1), ref.reshape(1, -1)) < 5e-4, (qname, n, k)
+    # without h_out
+    act2 = hip.alloc(n * 4)
+    hip.quantized_matvec_norm_swiglu(wg, wu, xb, db, wb, None, act2, eps)
+    assert np.array_equal(act2.download(np.float32, (n,)), got)
+
+
+def test_swiglu_fused_gate_up_refusals(hip, orc):
+    """Shapes the fused kernels do not serve are refused before anything is launched, and the check function
+    says so beforehand; argument errors surface as codes."""
+    k = 4096
+    assert not hip.norm_swiglu_supported(orc.Q4_K, 4096, 14336)      # rows longer than 8192
+    assert not hip.norm_swiglu_supported(orc.Q4_K, 1026, k)          # not whole passes
+    assert not hip.norm_swiglu_supported(orc.Q6_K, 1024, 2304)       # Q6_K rows that are not whole 16-byte words
+    assert hip.norm_swiglu_supported(orc.Q4_K, 14336, k)
+    w = hip.upload_weight(orc.Q4_K, weights(orc, "Q4_K", 4900, 1026, k), 1026, k)
+    x, wn, act = hip.upload(np.ones(k, np.float32)), hip.upload(np.ones(k, np.float32)), hip.alloc(1026 * 4)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_norm_swiglu(w, w, x, None, wn, None, act)
+    assert e.value.code == _ffi.E_UNSUPPORTED
+    w2 = hip.upload_weight(orc.Q4_K, weights(orc, "Q4_K", 4901, 1024, k), 1024, k)
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_norm_swiglu(w2, w2, x, None, wn, None, hip.alloc(1024 * 2))   # act too short
+    assert e.value.name == "PSN_E_INVALID_ARG"
+    with pytest.raises(backend.PsnError) as e:
+        hip.quantized_matvec_norm_swiglu(w2, w2, x, None, wn, x, hip.alloc(1024 * 4))      # h_out aliases x
+    assert e.value.name == "PSN_E_INVALID_ARG"
+    with pytest.raises(ValueError):
+        hip.quantized_matvec_norm_swiglu(w2, w, x, None, wn, None, act)                    # shapes differ
+
+
 @pytest.mark.parametrize("k", [4096, 14336, 5120])
 def test_norm_fused_projection_three_formats_share_x(hip, orc, k):
     """q | k | v in three different formats take three calls on the same x and delta (a decoder passes h_out to

@@ -113,6 +113,18 @@ def test_matvec_plans_are_consistent_over_many_shapes(lib):
     assert (p.stream > 0, p.threads, p.blocks) == (True, 384, 256), p.as_dict()
 
 
+def test_swiglu_fused_launch_check_is_host_arithmetic(lib):
+    """psn_qmatvec_norm_swiglu_check: which gate|up shapes the SwiGLU-fused launch serves, without a device."""
+    chk = lambda qt, n, k: int(lib.psn_qmatvec_norm_swiglu_check(qt, n, k, 256))
+    for qt in (_ffi.Q4_0, _ffi.Q8_0, _ffi.Q4_K, _ffi.Q5_K, _ffi.Q6_K):
+        assert chk(qt, 14336, 4096) == 0 and chk(qt, 1024, 2048) == 0
+        assert chk(qt, 4096, 14336) == _ffi.E_UNSUPPORTED              # rows longer than the fused staging holds
+        assert chk(qt, 1026, 4096) == _ffi.E_UNSUPPORTED               # not whole passes
+        assert chk(qt, 0, 4096) == _ffi.E_SHAPE and chk(qt, 1024, 4100) == _ffi.E_SHAPE
+    assert chk(_ffi.Q6_K, 1024, 2304) == _ffi.E_UNSUPPORTED            # 210-byte blocks: rows of whole 16-byte words only
+    assert chk(_ffi.Q8_K, 1024, 4096) != 0                             # not a weight format
+
+
 def test_prefill_plans_are_consistent_over_many_shapes(lib):
     """Host arithmetic only: every prefill plan over a grid of shapes is one psn_qmatmul_prefill_tiled accepts --
     a known tile, a family the format has, a K split that leaves whole chunks per range and an atomically addable Y."""
