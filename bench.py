@@ -96,8 +96,9 @@ class OracleChecker:
         return self.orc.matvec(qtype, self.orc.ACT_Q8, blocks, x, n, k, nthreads=threads)
 
     def decode_last_layer(self, shape, protos, got):
-        """Teacher-forced reference of the launches that end a step, from the device's own vectors: gate | up from the
-        residual `x` that entered the last layer's FFN norm, the logits from x + down (norm weights 1)."""
+        """Teacher-forced reference of the launches that end a step, from the device's own vectors: gate | up (or, where
+        the device applied SwiGLU inside that launch, silu(gate) * up and the down projection of the device's own
+        `act`) from the residual `x` that entered the last layer's FFN norm, the logits from x + down (norm weights 1)."""
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         from decoderef import rmsnorm_ref
         orc, s = self.orc, shape
@@ -107,6 +108,11 @@ class OracleChecker:
         xn = rmsnorm_ref(got["x"], ones, eps)
         out = {"gate": orc.matvec(orc.Q4_K, orc.ACT_Q8, protos[p + "w_gate"], xn, s.ffn, s.hidden).reshape(-1),
                "up": orc.matvec(orc.Q4_K, orc.ACT_Q8, protos[p + "w_up"], xn, s.ffn, s.hidden).reshape(-1)}
+        if "act" in got:
+            # SwiGLU ran inside the gate | up launch: its output, and the down projection of the device's own output
+            g, u = out["gate"].astype(np.float64), out["up"].astype(np.float64)
+            out["act"] = (g / (1.0 + np.exp(-g)) * u).astype(np.float32)
+            out["down"] = orc.matvec(orc.Q4_K, orc.ACT_Q8, protos[p + "w_down"], got["act"], s.hidden, s.ffn).reshape(-1)
         uniq = protos["lm_head"].shape[0]
         xf = rmsnorm_ref((got["x"] + got["down"]).astype(np.float32), ones, eps)
         head = orc.matvec(orc.Q6_K, orc.ACT_Q8, protos["lm_head"], xf, uniq, s.hidden).reshape(-1)

@@ -345,18 +345,24 @@ def config5(be: HipBackend, samples: int = 7, seed: int = 0, ctx: int = 2048, la
     parity, whole_step = None, None
     if checker is not None and step.fused_norm:
         # The replay above left the last layer's vectors in the step's buffers: x = the residual that entered the last
-        # layer's FFN norm, gate / up, down, and the logits.  The checker redoes, from the device's OWN inputs, the
-        # launches that produced gate | up and the logits (add + RMSNorm + quantize + matvec each).  A comparison of
+        # layer's FFN norm, gate / up (or silu(gate) * up), down, and the logits.  The checker redoes, from the device's OWN
+        # inputs, the launches that produced them (add + RMSNorm + quantize + matvec each).  A comparison of
         # the whole 32-layer chain against a CPU run is reported beside it but is no verdict: an int8 activation that
         # rounds the other way moves an output by ~2e-4, and the random-init network amplifies that from layer to layer
         # (the CPU path fed an input perturbed by 1e-6 differs from itself by ~2e-2 in the logits).
-        got = {"x": step.x.download(np.float32, (shape.hidden,)), "down": step.down.download(np.float32, (shape.hidden,)),
-               "gate": step.gate.download(np.float32, (shape.ffn,)), "up": step.up.download(np.float32, (shape.ffn,)), "logits": logits}
+        got = {"x": step.x.download(np.float32, (shape.hidden,)), "down": step.down.download(np.float32, (shape.hidden,)), "logits": logits}
+        if step.fused_swiglu[-1]:
+            # SwiGLU ran inside the gate | up launch: gate and up never reach memory, silu(gate) * up does
+            got["act"] = step.act.download(np.float32, (shape.ffn,))
+            names, what = ("act", "down", "logits"), f"silu(gate) * up ({shape.ffn} outputs), down ({shape.hidden})"
+        else:
+            got["gate"], got["up"] = step.gate.download(np.float32, (shape.ffn,)), step.up.download(np.float32, (shape.ffn,))
+            names, what = ("gate", "up", "logits"), f"gate | up ({2 * shape.ffn} outputs)"
         ref = checker.decode_last_layer(shape, protos, got)
-        verdicts = [parity_of(got[name], ref[name], "Q8", "") for name in ("gate", "up", "logits")]
+        verdicts = [parity_of(got[name], ref[name], "Q8", "") for name in names]
         parity = max(verdicts, key=lambda v: (v["status"] != "pass", v["value"]))
-        parity["checked"] = (f"gate | up ({2 * shape.ffn} outputs) and all {shape.vocab} logits of the last of {layers} layers, each recomputed on the CPU "
-                             "from the input vectors the device itself produced (residual, down)")
+        parity["checked"] = (f"{what} and all {shape.vocab} logits of the last of {layers} layers, each recomputed on the CPU "
+                             "from the input vectors the device itself produced (residual, act, down)")
         whole = parity_of(logits, checker.decode_step(shape, protos, x0, kv, pos), "Q8", "")
         whole_step = {"value": whole["value"], "note": "logits of the whole step against a CPU run of all layers from the same embedding: "
                       "ill-conditioned (see above), reported, not gated"}

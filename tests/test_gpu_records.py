@@ -73,7 +73,7 @@ def test_decode_step_record_and_worker_attachment(hip, orc):
     print(f"record {head['opRef']}: {head['kernelRef']} parity={head['parity']['value']:.2e}", flush=True)
     check(hip, head)                                         # the Q6_K LM head on its own
     assert head["opRef"].startswith("matvec.q6_K.4096x128256") and "q6_K" in head["kernelRef"]
-    assert rec["launches_per_token"] >= 2 * 7 + 2 and 0 < rec["matvec_share"] <= 1
+    assert rec["launches_per_token"] == 2 * 6 + 2 and "xnp" in rec["kernelRef"] and 0 < rec["matvec_share"] <= 1   # SwiGLU inside gate|up
     assert any(k.startswith("psn_attn") for k in kernels_of(rec)) and any("q6_K" in k for k in kernels_of(rec))
     att = R.worker_attachment([rec], updated_at_ms=5)
     assert att["workers"][0]["ready"] is True and att["workers"][0]["evidence_digest"] == R.record_digest(rec)
