@@ -114,7 +114,14 @@ PSN_DEV bool fast_div_range(float magnitude) { return magnitude >= 0x1p-90f && m
  * largest float below 0.5 lands on the right side of every integer (with 0.5 itself, 0.5 - 2^-25 would round up
  * to 1).  Checked against roundf for every float below 4096 in magnitude (tests/test_oracle_formats.py restates
  * the check for the range the quantizers produce). */
-PSN_DEV int round_half_away(float t) { return (int)(t + __builtin_copysignf(__uint_as_float(0x3effffffu), t)); }
+PSN_DEV int round_half_away(float t) {
+    /* t is a rounded product: the addition must not be fused with the multiplication that made it (a fused
+     * multiply-add sees the exact product, which can lie on the other side of a half-integer than t does; the
+     * compiler contracts across the inlined call, and HIP's __fadd_rn / __fmul_rn do not stop it).  The empty asm
+     * makes t opaque: the product is rounded to a register before the half is added. */
+    asm volatile("" : "+v"(t));
+    return (int)(t + __builtin_copysignf(__uint_as_float(0x3effffffu), t));
+}
 /* the low bytes of four ints as one dword */
 PSN_DEV u32 pack_bytes4(int q0, int q1, int q2, int q3) {
     const u32 lo = __builtin_amdgcn_perm((u32)q1, (u32)q0, 0x0c0c0400u), hi = __builtin_amdgcn_perm((u32)q3, (u32)q2, 0x0c0c0400u);

@@ -57,6 +57,55 @@ def test_quantize_q8_0_bit_exact(hip, orc, k, batch):
         assert np.array_equal(s[b], ref_q.reshape(-1, 32).astype(np.int32).sum(axis=1))
 
 
+def _half_integer_products(amax):
+    """fp32 values x with |x| <= amax whose product with id = 1 / (amax / 127) rounds to a half-integer m + 1/2 from
+    just below it: roundf of the rounded product is m + 1, but adding the rounding constant to the exact product (what
+    a fused multiply-add does) can land below m + 1.  A quantizer that rounds in fewer steps than the reference gets
+    these wrong by one."""
+    A = np.float32(amax)
+    idv = np.float32(np.float32(1.0) / np.float32(A / np.float32(127.0)))
+    c = np.uint32(0x3effffff).view(np.float32)
+    out = []
+    base = ((np.arange(1, 127, dtype=np.float64) + 0.5) / np.float64(idv)).astype(np.float32)
+    for k in range(-6, 7):
+        x = base.copy()
+        for _ in range(abs(k)):
+            x = np.nextafter(x, np.float32(np.inf if k > 0 else -np.inf))
+        t = (x * idv).astype(np.float32)
+        ref = np.floor(t.astype(np.float64) + 0.5)
+        fused = (x.astype(np.float64) * np.float64(idv) + np.float64(c)).astype(np.float32)
+        out.extend(float(v) for v in x[(np.trunc(fused.astype(np.float64)) != ref) & (x <= A)])
+    return out
+
+
+def test_quantize_q8_0_rounds_the_rounded_product(hip, orc):
+    """q = roundf(RN(x * id)): the product is rounded to fp32 before the half is added.  Inputs chosen so that one
+    fused step would differ (see _half_integer_products), both signs, next to ordinary values."""
+    blocks = []
+    for amax in (100.0, 3.7, 1.234567, 77.7, 0.9, 12.5, 640.0):
+        hard = _half_integer_products(amax)
+        hard = hard + [-v for v in hard]
+        for i in range(0, len(hard), 30):
+            blk = np.zeros(32, np.float32)
+            blk[0] = amax
+            part = hard[i:i + 30]
+            blk[1:1 + len(part)] = part
+            blk[31] = -amax / 3
+            blocks.append(blk)
+    assert len(blocks) >= 4
+    while len(blocks) % 8:
+        blocks.append(blocks[-1])                       # whole 256-element chunks
+    x = np.concatenate(blocks)[None, :]
+    k = x.shape[1]
+    say(f"quantize_q8_0 half-integer products: {len(blocks)} blocks")
+    xq = hip.quantize_activations(hip.upload(x), k, 1, _ffi.Q8_0)
+    li = backend.actq_layout(_ffi.Q8_0, k, 1)
+    qs = xq.download(np.int8, (1, k), li.off_qs)
+    ref_q = orc.quantize(orc.Q8_0, x[0]).reshape(k // 32, 34)[:, 2:].copy().view(np.int8).reshape(-1)
+    differ = np.flatnonzero(qs[0] != ref_q)
+    assert differ.size == 0, [(int(i), float(x[0, i]), int(qs[0, i]), int(ref_q[i])) for i in differ[:8]]
+
+
 @pytest.mark.parametrize("k,batch", [(256, 1), (4096, 1), (14336, 3), (4096, 8)])
 def test_quantize_q8_K_bit_exact(hip, orc, k, batch):
     say(f"quantize_q8_K k={k} batch={batch}")

@@ -90,6 +90,33 @@ def test_q8_0_round_half_away_and_zero_block(orc):
     assert not z.any()
 
 
+def test_q8_0_rounds_the_rounded_product_not_the_exact_one(orc):
+    """q = roundf(RN(x * id)): the reference rounds the product to fp32 before it rounds to an integer.  Inputs whose
+    rounded product is a half-integer m + 1/2 reached from below: roundf gives m + 1, while rounding the exact
+    product (or adding the half inside one fused multiply-add) gives m.  The oracle must do the former; the formula
+    is evaluated here step by step in float32."""
+    hits = 0
+    for amax in (100.0, 3.7, 1.234567, 77.7, 0.9, 12.5, 640.0):
+        A = np.float32(amax)
+        d = np.float32(A / np.float32(127.0))
+        idv = np.float32(np.float32(1.0) / d)
+        base = ((np.arange(1, 127, dtype=np.float64) + 0.5) / np.float64(idv)).astype(np.float32)
+        for k in range(-6, 7):
+            x = base.copy()
+            for _ in range(abs(k)):
+                x = np.nextafter(x, np.float32(np.inf if k > 0 else -np.inf))
+            t = (x * idv).astype(np.float32)                                    # the rounded product
+            two_step = np.floor(t.astype(np.float64) + 0.5)
+            one_step = np.floor(x.astype(np.float64) * np.float64(idv) + 0.5)   # rounding the exact product
+            for xi, want in zip(x[(two_step != one_step) & (x <= A)], two_step[(two_step != one_step) & (x <= A)]):
+                blk = np.zeros(32, np.float32)
+                blk[0], blk[1], blk[2] = A, xi, -xi
+                q = orc.quantize(orc.Q8_0, blk)[2:].view(np.int8)
+                assert (int(q[0]), int(q[1]), int(q[2])) == (127, int(want), -int(want)), (amax, float(xi))
+                hits += 1
+    assert hits >= 8
+
+
 def test_q8_0_closed_form_and_error_bound(orc):
     x = G.seeded_acts(11, 1, 4096)[0]
     blk = orc.quantize(orc.Q8_0, x).reshape(1, -1)
