@@ -106,6 +106,36 @@ def test_quantize_q8_0_rounds_the_rounded_product(hip, orc):
     assert differ.size == 0, [(int(i), float(x[0, i]), int(qs[0, i]), int(ref_q[i])) for i in differ[:8]]
 
 
+def test_quantizers_match_the_oracle_on_many_random_blocks(hip, orc):
+    """Both device quantizers against the oracle over 16 M random elements each: block scales from 2^-12 to 2^11, a
+    third of the vectors snapped to a 1/8 grid (exact ties, equal magnitudes).  Every byte, scale and sum."""
+    rng = np.random.default_rng(123)
+    k = 1 << 20
+    for it in range(16):
+        x = rng.standard_normal(k, dtype=np.float32).reshape(-1, 32) * np.exp2(rng.integers(-12, 12, k // 32)).astype(np.float32)[:, None]
+        x = x.reshape(-1)
+        if it % 3 == 1:
+            x = np.round(x * 8) / 8
+        x = x.astype(np.float32)[None, :]
+        xb = hip.upload(x)
+        say(f"quantizer sweep #{it}")
+        xq = hip.quantize_activations(xb, k, 1, _ffi.Q8_0)
+        li = backend.actq_layout(_ffi.Q8_0, k, 1)
+        ref = orc.quantize(orc.Q8_0, x[0]).reshape(k // 32, 34)
+        assert np.array_equal(xq.download(np.int8, (1, k), li.off_qs)[0], ref[:, 2:].copy().view(np.int8).reshape(-1))
+        ref_d = ref[:, :2].copy().view(np.float16).astype(np.float32).reshape(-1)
+        assert np.array_equal(xq.download(np.float32, (1, k // 32), li.off_d)[0].view(np.uint32), ref_d.view(np.uint32))
+        xq.free()
+        xq = hip.quantize_activations(xb, k, 1, _ffi.Q8_K)
+        li = backend.actq_layout(_ffi.Q8_K, k, 1)
+        rd, rq, rbs = G.parse_q8_K(orc.quantize(orc.Q8_K, x[0]), k)
+        assert np.array_equal(xq.download(np.int8, (1, k), li.off_qs)[0], rq.reshape(-1).astype(np.int8))
+        assert np.array_equal(xq.download(np.float32, (1, k // 256), li.off_d)[0].astype(np.float64), rd)
+        assert np.array_equal(xq.download(np.int16, (1, k // 16), li.off_s)[0], rbs.reshape(-1).astype(np.int16))
+        xq.free()
+        xb.free()
+
+
 @pytest.mark.parametrize("k,batch", [(256, 1), (4096, 1), (14336, 3), (4096, 8)])
 def test_quantize_q8_K_bit_exact(hip, orc, k, batch):
     say(f"quantize_q8_K k={k} batch={batch}")
