@@ -353,6 +353,32 @@ def test_packed_weights_multiply_like_the_dense_family(hip, orc, qname):
     assert e.value.name == "PSN_E_SHAPE"
 
 
+@pytest.mark.parametrize("qname", ["Q4_0", "Q8_0", "Q4_K", "Q5_K", "Q6_K"])
+def test_packed_fragments_hold_the_reference_fp16_values_bit_for_bit(hip, orc, qname):
+    """psn_prefill_pack writes h(deq(W)): every weight as the fp16 rounding of the value the reference's
+    dequantizer returns, in fragment order [row / 32][k / 16][half][row % 32][8].  Read back and compared
+    bit for bit (up to the sign of a zero) with numpy.float16 of the oracle's dequantization -- rows scaled over twelve binades so that
+    block scales, mins and fp16 roundings of every size occur, and a ragged last row panel."""
+    t = getattr(orc, qname)
+    n, k = 200, 2048
+    rng = np.random.default_rng(8100)
+    w = rng.standard_normal((n, k), dtype=np.float32) * np.exp2(rng.integers(-8, 4, (n, k // 32))).astype(np.float32).repeat(32, axis=1)
+    blocks = orc.quantize(t, w)
+    wt = hip.upload_weight(t, blocks, n, k)
+    packed = hip.pack_for_prefill(wt)
+    npanel = -(-n // 32)
+    raw = packed.download(np.uint16, (packed.nbytes // 2,))[:npanel * (k // 16) * 64 * 8].reshape(npanel, k // 16, 2, 32, 8)
+    # [panel][kslice][half][row % 32][j] -> [row][k]
+    got = raw.transpose(0, 3, 1, 2, 4).reshape(npanel * 32, k)[:n]
+    want = orc.dequantize(t, blocks, k).reshape(n, k).astype(np.float16).view(np.uint16)
+    # a zero keeps no sign: the reference's d * sc * (q - 32) is -0 where d * sc is negative and q = 32, the
+    # kernels' fused form d sc q - 32 d sc returns +0 (Q6_K; the other formats agree in the sign of zero too)
+    zero = (want & 0x7fff) == 0
+    got, want = np.where(zero, got & 0x7fff, got), np.where(zero, want & 0x7fff, want)
+    differ = np.argwhere(got != want)
+    assert differ.size == 0, [(int(r), int(c), hex(int(got[r, c])), hex(int(want[r, c]))) for r, c in differ[:6]]
+
+
 def test_prefill_refuses_operands_beyond_32_bit_offsets(hip, orc):
     """Several families address X and W with 32-bit byte offsets: shapes that would overflow them are
     refused by the host before any buffer is looked at."""
