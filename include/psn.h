@@ -344,7 +344,8 @@ int32_t psn_add_rmsnorm(psn_module *mod, psn_stream *s, psn_buf *x, const psn_bu
 int32_t psn_rope_kv_store(psn_module *mod, psn_stream *s, psn_buf *q, psn_buf *k, const psn_buf *v, psn_buf *k_cache,
                           psn_buf *v_cache, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim, int32_t pos, float theta_base);
 /* softmax(q K^T / sqrt(head_dim)) V over cache positions 0 .. n_ctx-1, grouped-query (n_heads a multiple
- * of n_kv_heads, at most 8 per group), head_dim 128; workspace holds n_heads * ceil(n_ctx/64) * 130 floats */
+ * of n_kv_heads, at most 8 per group), head_dim 128; workspace holds n_heads * ceil(n_ctx/64) * 130 floats
+ * (beyond 4096 positions the kernels use fewer, longer splits and only the front of it) */
 int32_t psn_attention_decode(psn_module *mod, psn_stream *s, const psn_buf *q, const psn_buf *k_cache, const psn_buf *v_cache,
                              psn_buf *workspace, psn_buf *out, int32_t n_heads, int32_t n_kv_heads, int32_t head_dim,
                              int32_t n_ctx);

@@ -133,7 +133,7 @@ struct psn_attn_args {
     float *out;           /* [n_heads][128] (may be null when only the quantized one is wanted) */
     int32_t n_heads, n_kv_heads, n_ctx, n_splits;
     float scale;
-    int32_t pad;
+    int32_t chunks;       /* psn_attn_partial(_rope)_long: 64-position chunks per split (the other kernels: one) */
     struct psn_actq_out qout;
     /* fused rotary + cache append (psn_attn_partial_rope): q and k_new are the raw projections of the
      * token at position n_ctx - 1; the kernel rotates them itself and stores k_new / v_new in the caches */

@@ -289,9 +289,283 @@ PSN_DEV void attn_partial_body(const psn_attn_args &a) {
     if (lane == 0) { dst[D] = m; dst[D + 1] = sum; }
 }
 
+/* Long contexts: a split is a.chunks chunks of 64 positions, walked sixteen positions at a time (row 4 j + quarter of
+ * a step in lane quarter `quarter`, j = 0 .. 3) with the next step's K and V rows already requested while the
+ * current ones are multiplied, and a running (max, sum, output) per lane quarter in the manner of a streaming
+ * softmax: the cross-lane sums and the partial store, which the kernel above pays per 64 positions, are paid once
+ * per split, and a workgroup's loads overlap its arithmetic.  Same partial format, same combine kernel. */
+template <bool ROPE>
+PSN_DEV void attn_partial_long_body(const psn_attn_args &a) {
+    constexpr int D = 128;
+    __shared__ float qs[8][D];
+    __shared__ uint4 knew_row[16];
+    const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int quarter = lane >> 4, sub = lane & 15;
+    const int kvh = blockIdx.x % a.n_kv_heads, split = blockIdx.x / a.n_kv_heads;
+    const int group = a.n_heads / a.n_kv_heads;
+    const int head = kvh * group + g;
+    const int pos_last = a.n_ctx - 1;
+    const int p_begin = split * a.chunks * 64;                   /* < n_ctx: the host launches no empty split */
+    const int p_end = min(p_begin + a.chunks * 64, a.n_ctx);     /* one past the split's last valid position */
+    const int nsteps = (p_end - p_begin + 15) >> 4;
+    const bool own = ROPE && pos_last >= p_begin && pos_last < p_end;   /* uniform: the split that holds the token's position */
+    const int64_t row16 = (int64_t)a.n_kv_heads * (D / 8);       /* 16-byte words between positions */
+    const uint4 *kb = reinterpret_cast<const uint4 *>(a.k_cache) + (int64_t)kvh * (D / 8) + sub;
+    const uint4 *vb = reinterpret_cast<const uint4 *>(a.v_cache) + (int64_t)kvh * (D / 8) + sub;
+    auto fetch = [&](int it, uint4 (&k)[4], uint4 (&v)[4]) {
+        UNROLL for (int j = 0; j < 4; ++j) {
+            const int p = min(p_begin + 16 * it + 4 * j + quarter, p_end - 1);
+            k[j] = kb[(int64_t)p * row16];
+            v[j] = vb[(int64_t)p * row16];
+        }
+    };
+    uint4 ka[4], va[4], kbuf[4], vbuf[4];
+    fetch(0, ka, va);
+    uint4 vnew = make_uint4(0, 0, 0, 0);
+    if constexpr (ROPE) {
+        const float2 tc = *reinterpret_cast<const float2 *>(a.rope_table + 2 * lane);
+        const float cs = tc.x, sn = tc.y;
+        float r0, r1;
+        const float2 qv = *reinterpret_cast<const float2 *>(a.q + head * D + 2 * lane);
+        rope_pair(qv.x, qv.y, cs, sn, r0, r1);
+        qs[g][2 * lane] = r0;
+        qs[g][2 * lane + 1] = r1;
+        if (g == 0 && own) {
+            const float2 kv = *reinterpret_cast<const float2 *>(a.k_new + kvh * D + 2 * lane);
+            float k0, k1;
+            rope_pair(kv.x, kv.y, cs, sn, k0, k1);
+            const u32 packed = pack_h2(k0, k1);
+            reinterpret_cast<u32 *>(knew_row)[lane] = packed;
+            reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.k_cache_w) + ((int64_t)pos_last * a.n_kv_heads + kvh) * D)[lane] = packed;
+        }
+        const float4 x0 = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub), x1 = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub + 4);
+        vnew.x = pack_h2(x0.x, x0.y); vnew.y = pack_h2(x0.z, x0.w); vnew.z = pack_h2(x1.x, x1.y); vnew.w = pack_h2(x1.z, x1.w);
+        if (own && g == 0 && quarter == 0)
+            reinterpret_cast<uint4 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos_last * a.n_kv_heads + kvh) * D)[sub] = vnew;
+    } else {
+        qs[g][lane] = a.q[head * D + lane];
+        qs[g][lane + 64] = a.q[head * D + lane + 64];
+    }
+    __syncthreads();
+    uint4 knew = make_uint4(0, 0, 0, 0);
+    if (own) knew = knew_row[sub];
+    const float4 qa = *reinterpret_cast<const float4 *>(&qs[g][8 * sub]), qb = *reinterpret_cast<const float4 *>(&qs[g][8 * sub + 4]);
+    float m_run = -INFINITY, l_run = 0.f;
+    float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    auto step = [&](int it, uint4 (&k)[4], uint4 (&v)[4]) {
+        float sc[4];
+        float m_new = m_run;
+        UNROLL for (int j = 0; j < 4; ++j) {
+            const int p = p_begin + 16 * it + 4 * j + quarter;
+            if (own) {
+                /* the token's own row is not in the cache yet (its key comes from LDS, its value from the fresh
+                 * projection, both rounded to fp16 like a cached row); rows behind it were loaded from the row at its
+                 * position, which nothing has written: they get weight 0, but 0 * (a stale Inf / NaN pattern) would
+                 * still poison the sum, so their values are replaced as well */
+                const bool mine = p == pos_last, behind = p >= pos_last;
+                k[j].x = mine ? knew.x : k[j].x; k[j].y = mine ? knew.y : k[j].y; k[j].z = mine ? knew.z : k[j].z; k[j].w = mine ? knew.w : k[j].w;
+                v[j].x = behind ? vnew.x : v[j].x; v[j].y = behind ? vnew.y : v[j].y; v[j].z = behind ? vnew.z : v[j].z; v[j].w = behind ? vnew.w : v[j].w;
+            }
+            const u32 kw[4] = {k[j].x, k[j].y, k[j].z, k[j].w};
+            float s = h2f_lo(kw[0]) * qa.x + h2f_hi(kw[0]) * qa.y + h2f_lo(kw[1]) * qa.z + h2f_hi(kw[1]) * qa.w;
+            s += h2f_lo(kw[2]) * qb.x + h2f_hi(kw[2]) * qb.y + h2f_lo(kw[3]) * qb.z + h2f_hi(kw[3]) * qb.w;
+            s = group_sum<16>(s);
+            sc[j] = p < p_end ? s * a.scale : -INFINITY;
+            m_new = fmaxf(m_new, sc[j]);
+        }
+        /* a quarter that has seen no valid row yet keeps max = -inf: subtract 0 then, every weight is exp(-inf) = 0 */
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float r = __expf(m_run - m_use);
+        l_run *= r;
+        UNROLL for (int t = 0; t < 8; ++t) o[t] *= r;
+        UNROLL for (int j = 0; j < 4; ++j) {
+            const float w = __expf(sc[j] - m_use);
+            l_run += w;
+            const u32 vw[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+            UNROLL for (int t = 0; t < 4; ++t) {
+                o[2 * t] += w * h2f_lo(vw[t]);
+                o[2 * t + 1] += w * h2f_hi(vw[t]);
+            }
+        }
+        m_run = m_new;
+    };
+    for (int it = 0; it < nsteps; it += 2) {
+        if (it + 1 < nsteps) fetch(it + 1, kbuf, vbuf);
+        step(it, ka, va);
+        if (it + 1 < nsteps) {
+            if (it + 2 < nsteps) fetch(it + 2, ka, va);
+            step(it + 1, kbuf, vbuf);
+        }
+    }
+    /* the four quarters' running states meet: common maximum (row p_begin is valid, so it is finite), rescaled sums */
+    const float m = quarters_max(m_run);
+    const float f = __expf(m_run - m);
+    const float sum = quarters_sum(l_run * f);
+    UNROLL for (int t = 0; t < 8; ++t) o[t] = quarters_sum(o[t] * f);
+    float *dst = a.partial + ((int64_t)head * a.n_splits + split) * (D + 2);
+    if (quarter == 0) {
+        UNROLL for (int t = 0; t < 4; ++t) *reinterpret_cast<float2 *>(dst + 8 * sub + 2 * t) = make_float2(o[2 * t], o[2 * t + 1]);
+    }
+    if (lane == 0) { dst[D] = m; dst[D + 1] = sum; }
+}
+
+/* The same for groups of exactly four query heads per kv head, with the roles turned: a wave takes sixteen of a
+ * step's 64 positions for all four heads instead of all 64 for one head.  Every K and V row is then fetched by
+ * one wave only (a quarter of the requests, four times the distinct bytes in flight per compute unit, which is
+ * what bounds a long context), converted to fp32 once and used four times.  The four waves' running states meet
+ * through LDS at the end of the split. */
+template <bool ROPE>
+PSN_DEV void attn_partial_long4_body(const psn_attn_args &a) {
+    constexpr int D = 128, H = 4;
+    __shared__ float qs[H][D];
+    __shared__ uint4 knew_row[16];
+    __shared__ float part_o[4][H][D];
+    __shared__ float part_ml[4][H][2];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int quarter = lane >> 4, sub = lane & 15;
+    const int kvh = blockIdx.x % a.n_kv_heads, split = blockIdx.x / a.n_kv_heads;
+    const int pos_last = a.n_ctx - 1;
+    const int p_begin = split * a.chunks * 64;
+    const int p_end = min(p_begin + a.chunks * 64, a.n_ctx);
+    const int nsteps = (p_end - p_begin + 63) >> 6;
+    const bool own = ROPE && pos_last >= p_begin && pos_last < p_end;
+    const int64_t row16 = (int64_t)a.n_kv_heads * (D / 8);
+    const uint4 *kb = reinterpret_cast<const uint4 *>(a.k_cache) + (int64_t)kvh * (D / 8) + sub;
+    const uint4 *vb = reinterpret_cast<const uint4 *>(a.v_cache) + (int64_t)kvh * (D / 8) + sub;
+    auto fetch = [&](int it, uint4 (&k)[4], uint4 (&v)[4]) {
+        UNROLL for (int j = 0; j < 4; ++j) {
+            const int p = min(p_begin + 64 * it + 16 * w + 4 * j + quarter, p_end - 1);
+            k[j] = kb[(int64_t)p * row16];
+            v[j] = vb[(int64_t)p * row16];
+        }
+    };
+    uint4 ka[4], va[4], kbuf[4], vbuf[4];
+    fetch(0, ka, va);
+    uint4 vnew = make_uint4(0, 0, 0, 0);
+    if constexpr (ROPE) {
+        /* wave w rotates query head w of the group; wave 0 of the split that owns the token's position the new key */
+        const float2 tc = *reinterpret_cast<const float2 *>(a.rope_table + 2 * lane);
+        const float cs = tc.x, sn = tc.y;
+        float r0, r1;
+        const float2 qv = *reinterpret_cast<const float2 *>(a.q + (kvh * H + w) * D + 2 * lane);
+        rope_pair(qv.x, qv.y, cs, sn, r0, r1);
+        qs[w][2 * lane] = r0;
+        qs[w][2 * lane + 1] = r1;
+        if (w == 0 && own) {
+            const float2 kv = *reinterpret_cast<const float2 *>(a.k_new + kvh * D + 2 * lane);
+            float k0, k1;
+            rope_pair(kv.x, kv.y, cs, sn, k0, k1);
+            const u32 packed = pack_h2(k0, k1);
+            reinterpret_cast<u32 *>(knew_row)[lane] = packed;
+            reinterpret_cast<u32 *>(reinterpret_cast<f16 *>(a.k_cache_w) + ((int64_t)pos_last * a.n_kv_heads + kvh) * D)[lane] = packed;
+        }
+        const float4 x0 = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub), x1 = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub + 4);
+        vnew.x = pack_h2(x0.x, x0.y); vnew.y = pack_h2(x0.z, x0.w); vnew.z = pack_h2(x1.x, x1.y); vnew.w = pack_h2(x1.z, x1.w);
+        if (own && w == 0 && quarter == 0)
+            reinterpret_cast<uint4 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos_last * a.n_kv_heads + kvh) * D)[sub] = vnew;
+    } else {
+        qs[w][lane] = a.q[(kvh * H + w) * D + lane];
+        qs[w][lane + 64] = a.q[(kvh * H + w) * D + lane + 64];
+    }
+    __syncthreads();
+    uint4 knew = make_uint4(0, 0, 0, 0);
+    if (own) knew = knew_row[sub];
+    float q[H][8];
+    UNROLL for (int h = 0; h < H; ++h) {
+        const float4 lo = *reinterpret_cast<const float4 *>(&qs[h][8 * sub]), hi = *reinterpret_cast<const float4 *>(&qs[h][8 * sub + 4]);
+        q[h][0] = lo.x; q[h][1] = lo.y; q[h][2] = lo.z; q[h][3] = lo.w; q[h][4] = hi.x; q[h][5] = hi.y; q[h][6] = hi.z; q[h][7] = hi.w;
+    }
+    float m_run[H], l_run[H], o[H][8];
+    UNROLL for (int h = 0; h < H; ++h) {
+        m_run[h] = -INFINITY;
+        l_run[h] = 0.f;
+        UNROLL for (int t = 0; t < 8; ++t) o[h][t] = 0.f;
+    }
+    auto step = [&](int it, uint4 (&k)[4], uint4 (&v)[4]) {
+        float sc[H][4];
+        UNROLL for (int j = 0; j < 4; ++j) {
+            const int p = p_begin + 64 * it + 16 * w + 4 * j + quarter;
+            if (own) {                                           /* see attn_partial_long_body */
+                const bool mine = p == pos_last, behind = p >= pos_last;
+                k[j].x = mine ? knew.x : k[j].x; k[j].y = mine ? knew.y : k[j].y; k[j].z = mine ? knew.z : k[j].z; k[j].w = mine ? knew.w : k[j].w;
+                v[j].x = behind ? vnew.x : v[j].x; v[j].y = behind ? vnew.y : v[j].y; v[j].z = behind ? vnew.z : v[j].z; v[j].w = behind ? vnew.w : v[j].w;
+            }
+            const u32 kw[4] = {k[j].x, k[j].y, k[j].z, k[j].w};
+            float kf[8];
+            UNROLL for (int t = 0; t < 4; ++t) { kf[2 * t] = h2f_lo(kw[t]); kf[2 * t + 1] = h2f_hi(kw[t]); }
+            UNROLL for (int h = 0; h < H; ++h) {
+                /* the order of the one-head kernels: two sums of four products */
+                float s = kf[0] * q[h][0] + kf[1] * q[h][1] + kf[2] * q[h][2] + kf[3] * q[h][3];
+                s += kf[4] * q[h][4] + kf[5] * q[h][5] + kf[6] * q[h][6] + kf[7] * q[h][7];
+                s = group_sum<16>(s);
+                sc[h][j] = p < p_end ? s * a.scale : -INFINITY;
+            }
+        }
+        float m_use[H];
+        UNROLL for (int h = 0; h < H; ++h) {
+            const float m_new = fmaxf(fmaxf(m_run[h], fmaxf(sc[h][0], sc[h][1])), fmaxf(sc[h][2], sc[h][3]));
+            m_use[h] = m_new == -INFINITY ? 0.f : m_new;
+            const float r = __expf(m_run[h] - m_use[h]);
+            l_run[h] *= r;
+            UNROLL for (int t = 0; t < 8; ++t) o[h][t] *= r;
+            m_run[h] = m_new;
+        }
+        UNROLL for (int j = 0; j < 4; ++j) {
+            const u32 vw[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+            float vf[8];
+            UNROLL for (int t = 0; t < 4; ++t) { vf[2 * t] = h2f_lo(vw[t]); vf[2 * t + 1] = h2f_hi(vw[t]); }
+            UNROLL for (int h = 0; h < H; ++h) {
+                const float wt = __expf(sc[h][j] - m_use[h]);
+                l_run[h] += wt;
+                UNROLL for (int t = 0; t < 8; ++t) o[h][t] += wt * vf[t];
+            }
+        }
+    };
+    for (int it = 0; it < nsteps; it += 2) {
+        if (it + 1 < nsteps) fetch(it + 1, kbuf, vbuf);
+        step(it, ka, va);
+        if (it + 1 < nsteps) {
+            if (it + 2 < nsteps) fetch(it + 2, ka, va);
+            step(it + 1, kbuf, vbuf);
+        }
+    }
+    /* quarters meet inside the wave, waves through LDS (a wave that saw no valid position contributes weight 0) */
+    UNROLL for (int h = 0; h < H; ++h) {
+        const float m = quarters_max(m_run[h]);
+        const float mu = m == -INFINITY ? 0.f : m;
+        const float f = __expf(m_run[h] - mu);
+        const float l = quarters_sum(l_run[h] * f);
+        UNROLL for (int t = 0; t < 8; ++t) o[h][t] = quarters_sum(o[h][t] * f);
+        if (quarter == 0) {
+            UNROLL for (int t = 0; t < 8; ++t) part_o[w][h][8 * sub + t] = o[h][t];
+        }
+        if (lane == 0) { part_ml[w][h][0] = m; part_ml[w][h][1] = l; }
+    }
+    __syncthreads();
+    {
+        const int h = w;                                         /* wave w finishes head w */
+        float mw[4], M = -INFINITY;
+        UNROLL for (int i = 0; i < 4; ++i) { mw[i] = part_ml[i][h][0]; M = fmaxf(M, mw[i]); }
+        float L = 0.f, o0 = 0.f, o1 = 0.f;
+        UNROLL for (int i = 0; i < 4; ++i) {
+            const float f = __expf(mw[i] - M);                   /* M is finite: wave 0 saw position p_begin */
+            L += part_ml[i][h][1] * f;
+            o0 += part_o[i][h][2 * lane] * f;
+            o1 += part_o[i][h][2 * lane + 1] * f;
+        }
+        float *dst = a.partial + ((int64_t)(kvh * H + h) * a.n_splits + split) * (D + 2);
+        *reinterpret_cast<float2 *>(dst + 2 * lane) = make_float2(o0, o1);
+        if (lane == 0) { dst[D] = M; dst[D + 1] = L; }
+    }
+}
+
 extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_attn_args a) { attn_partial_body<false>(a); }
 /* the same with the rotary embedding of q and k and the KV-cache append of the new token folded in */
 extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_rope(const psn_attn_args a) { attn_partial_body<true>(a); }
+extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_long(const psn_attn_args a) { attn_partial_long_body<false>(a); }
+extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_rope_long(const psn_attn_args a) { attn_partial_long_body<true>(a); }
+extern "C" __global__ void __launch_bounds__(256) psn_attn_partial_long4(const psn_attn_args a) { attn_partial_long4_body<false>(a); }
+extern "C" __global__ void __launch_bounds__(256) psn_attn_partial_rope_long4(const psn_attn_args a) { attn_partial_long4_body<true>(a); }
 
 /* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One wave per head, two heads per
  * workgroup; a lane owns two output dims.  The splits are taken 32 at a time and everything a wave needs

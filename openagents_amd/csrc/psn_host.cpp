@@ -1974,7 +1974,17 @@ static int32_t attention_impl(psn_module *mod, psn_stream *s, const psn_buf *q, 
     a.n_heads = n_heads;
     a.n_kv_heads = n_kv_heads;
     a.n_ctx = n_ctx;
-    a.n_splits = splits;
+    /* Up to 4096 positions: one workgroup per 64-position chunk and kv head (at 2048 positions that is one
+     * workgroup per compute unit of an MI355X).  Beyond: splits of several chunks, about two workgroups per compute unit,
+     * walked by the kernel that overlaps its loads with its arithmetic (measured on MI355X at 8192 .. 131072
+     * positions).  The workspace is sized for one split per chunk either way. */
+    const bool long_ctx = splits > 64;
+    int32_t want = 2 * mod->ctx->compute_units / n_kv_heads;      /* splits per kv head: about two workgroups per compute unit */
+    want = want < 16 ? 16 : want > 512 ? 512 : want;
+    const int32_t chunks = long_ctx ? (splits + want - 1) / want : 1;
+    const int32_t nsplits = (splits + chunks - 1) / chunks;
+    a.n_splits = nsplits;
+    a.chunks = chunks;
     a.scale = 0.08838834764831845f;                 /* 1/sqrt(128) */
     if (rope) {
         if (rope->k_new->ctx != mod->ctx || rope->v_new->ctx != mod->ctx || rope->table->ctx != mod->ctx)
@@ -1989,8 +1999,11 @@ static int32_t attention_impl(psn_module *mod, psn_stream *s, const psn_buf *q, 
         a.rope_table = (const float *)rope->table->p;
     }
     const int32_t group = n_heads / n_kv_heads;
-    if ((rc = launch(mod, s, rope ? "psn_attn_partial_rope" : "psn_attn_partial", (unsigned)(n_kv_heads * splits),
-                     (unsigned)(64 * group), 0, &a)))
+    /* (groups of four query heads have a long-context kernel of their own, in which a wave serves all four) */
+    const char *partial = long_ctx ? (group == 4 ? (rope ? "psn_attn_partial_rope_long4" : "psn_attn_partial_long4")
+                                                 : (rope ? "psn_attn_partial_rope_long" : "psn_attn_partial_long"))
+                                   : (rope ? "psn_attn_partial_rope" : "psn_attn_partial");
+    if ((rc = launch(mod, s, partial, (unsigned)(n_kv_heads * nsplits), (unsigned)(64 * group), 0, &a)))
         return rc;
     return launch(mod, s, "psn_attn_combine", (unsigned)((n_heads + 1) / 2), 128, 0, &a);
 }

@@ -27,7 +27,7 @@ from dataclasses import dataclass, field
 
 import numpy as np
 
-from ._ffi import ACT_Q8, Q4_K, Q6_K
+from ._ffi import ACT_Q8, Q4_K, Q6_K, Q8_K as Q8_K_ACT
 from . import gguf as _gguf
 from .backend import DeviceBuffer, HipBackend, QuantizedTensor, act_type_for, actq_layout, row_bytes
 
@@ -419,6 +419,42 @@ def greedy_tokens(model: GGUFModel, step: "DecodeStep", prompt, n_new: int):
     return tokens, logits
 
 
+def attention_sweep(be: HipBackend, contexts, samples: int = 9, n_heads: int = 32, n_kv_heads: int = 8, head_dim: int = 128):
+    """Time psn_attention_decode_rope (two launches) for a token at the last position of each context length, over
+    enough distinct KV caches that no launch finds its rows in a cache: microseconds per call and the rate at which
+    the K and V rows (fp16) are read."""
+    from . import records as R
+    rng = np.random.default_rng(0)
+    row = n_kv_heads * head_dim
+    q, k, v = (be.upload(rng.standard_normal(n, dtype=np.float32)) for n in (n_heads * head_dim, row, row))
+    out_q = be.alloc(int(actq_layout(Q8_K_ACT, n_heads * head_dim, 1).bytes))
+    tab = be.alloc(head_dim * 4)
+    rows = []
+    for ctx in contexts:
+        nbytes = ctx * row * 2
+        copies = max(2, min(8, int(700e6 // (2 * nbytes)) + 1))
+        block = rng.standard_normal((min(ctx, 4096), row), dtype=np.float32).astype(np.float16)
+        caches = []
+        for _ in range(2 * copies):
+            buf = be.alloc(nbytes)
+            for off in range(0, ctx, block.shape[0]):
+                buf.upload(block[:min(block.shape[0], ctx - off)], off * row * 2)
+            caches.append(buf)
+        ws = be.alloc(n_heads * ((ctx + 63) // 64) * 130 * 4)
+        be.rope_table(tab, head_dim, ctx - 1, 500000.0)
+        be.begin_capture()
+        for i in range(copies):
+            be.attention_decode_rope(q, k, v, caches[2 * i], caches[2 * i + 1], ws, None, out_q, Q8_K_ACT, n_heads, n_kv_heads, head_dim, ctx - 1, tab)
+        g = be.end_capture()
+        st = R.stats(R.time_graph(be, g, copies, samples))
+        be.destroy_graph(g)
+        rows.append({"context": ctx, "us": round(st["median_us"], 2), "kv_MB": round(2 * nbytes / 1e6, 1),
+                     "kv_TBps": round(2 * nbytes / st["median_us"] / 1e6, 2), "heads": f"{n_heads}/{n_kv_heads}"})
+        for b in caches + [ws]:
+            b.free()
+    return rows
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
     ap.add_argument("--layers", type=int, default=32)
@@ -432,8 +468,13 @@ def main(argv=None):
     ap.add_argument("--gguf", help="decode greedily from this llama-architecture model file instead of timing the synthetic step")
     ap.add_argument("--prompt", default="1", help="with --gguf: comma-separated prompt token ids (no tokenizer is part of this library)")
     ap.add_argument("--new", type=int, default=16, help="with --gguf: tokens to generate")
+    ap.add_argument("--attention-sweep", help="comma-separated context lengths: time the attention of one layer (rotary, cache append, "
+                                              "split kernel, combine) at each and exit")
     args = ap.parse_args(argv)
     be = HipBackend(0)
+    if args.attention_sweep:
+        print(json.dumps({"attention_sweep": attention_sweep(be, [int(c) for c in args.attention_sweep.split(",")], args.steps)}))
+        return 0
     if args.gguf:
         t0 = time.time()
         model = load_gguf_model(be, args.gguf)

@@ -74,6 +74,65 @@ def test_attention_decode(hip, nh, nkv):
         assert G.max_rel_err(got, attention_ref(q, kc, vc, nh, nkv, d, n_ctx)) < 2e-5
 
 
+@pytest.mark.parametrize("nh,nkv", [(32, 8), (8, 1), (4, 2)])
+def test_attention_decode_long_contexts(hip, nh, nkv):
+    """Beyond 4096 positions the splits hold several 64-position chunks and a workgroup walks its split sixteen
+    positions at a time with a running maximum: contexts that end a split early, in the middle of a chunk, one
+    position into a chunk, and a one-row last split; scores spread widely (K scaled) so that the running maximum
+    moves and the rescaling matters."""
+    rng = np.random.default_rng(903)
+    d = 128
+    for n_ctx in (4097, 4160, 5000, 8192, 8193, 12345, 20000):
+        say(f"long attention heads={nh}/{nkv} ctx={n_ctx}")
+        q = rng.standard_normal(nh * d, dtype=np.float32)
+        kc = (rng.standard_normal((n_ctx, nkv * d), dtype=np.float32) * (1 + 2 * rng.random((n_ctx, 1), dtype=np.float32))).astype(np.float16)
+        vc = rng.standard_normal((n_ctx, nkv * d), dtype=np.float32).astype(np.float16)
+        ws = hip.alloc(nh * ((n_ctx + 63) // 64) * 130 * 4)
+        out = hip.alloc(nh * d * 4)
+        hip.attention_decode(hip.upload(q), hip.upload(kc), hip.upload(vc), ws, out, nh, nkv, d, n_ctx)
+        got = out.download(np.float32, (nh * d,))
+        assert np.all(np.isfinite(got)) and G.max_rel_err(got, attention_ref(q, kc, vc, nh, nkv, d, n_ctx)) < 2e-5, n_ctx
+
+
+@pytest.mark.parametrize("nh,nkv", [(32, 8), (16, 2)])              # four heads to a kv head: a wave serves all four; otherwise one each
+@pytest.mark.parametrize("pos", [4096, 4159, 4160, 6000, 8191, 9999])
+def test_rope_fused_long_context_attention(hip, pos, nh, nkv):
+    """The long-context kernel with the rotary embedding and the cache append folded in: against the three
+    separate launches (rotary + append, attention, combine) on a cache whose rows at and behind the token's
+    position hold NaN patterns, which must not reach the output; appended rows and untouched rows as in the
+    short-context test."""
+    rng = np.random.default_rng(960 + pos)
+    d = 128
+    ctx = pos + 70
+    q = rng.standard_normal(nh * d, dtype=np.float32)
+    k = rng.standard_normal(nkv * d, dtype=np.float32)
+    v = rng.standard_normal(nkv * d, dtype=np.float32)
+    kc0 = rng.standard_normal((ctx, nkv * d), dtype=np.float32).astype(np.float16)
+    vc0 = rng.standard_normal((ctx, nkv * d), dtype=np.float32).astype(np.float16)
+    ws = hip.alloc(nh * ((ctx + 63) // 64) * 130 * 4)
+    qb, kb, vb = hip.upload(q), hip.upload(k), hip.upload(v)
+    kc, vc = hip.upload(kc0), hip.upload(vc0)
+    ref = hip.alloc(nh * d * 4)
+    hip.rope_kv_store(qb, kb, vb, kc, vc, nh, nkv, d, pos, 500000.0)
+    hip.attention_decode(qb, kc, vc, ws, ref, nh, nkv, d, pos + 1)
+    poisoned_k, poisoned_v = kc0.copy(), vc0.copy()
+    poisoned_k.view(np.uint16)[pos:] = 0x7E00
+    poisoned_v.view(np.uint16)[pos:] = 0x7E00
+    kc2, vc2 = hip.upload(poisoned_k), hip.upload(poisoned_v)
+    out = hip.alloc(nh * d * 4)
+    tab = hip.alloc(d * 4)
+    hip.rope_table(tab, d, pos, 500000.0)
+    say(f"long rope-fused attention pos={pos}")
+    hip.attention_decode_rope(hip.upload(q), hip.upload(k), hip.upload(v), kc2, vc2, ws, out, None, _ffi.Q8_K, nh, nkv, d, pos, tab)
+    got = out.download(np.float32, (nh * d,))
+    assert np.all(np.isfinite(got)) and G.max_rel_err(got, ref.download(np.float32, (nh * d,))) < 2e-5
+    k_two, k_three = kc2.download(np.float16, (ctx, nkv * d)), kc.download(np.float16, (ctx, nkv * d))
+    assert np.array_equal(k_two[:pos].view(np.uint16), k_three[:pos].view(np.uint16))
+    assert np.max(np.abs(k_two[pos].astype(np.float32) - k_three[pos].astype(np.float32))) <= 2e-3
+    assert np.array_equal(vc2.download(np.float16, (ctx, nkv * d))[:pos + 1].view(np.uint16), vc.download(np.float16, (ctx, nkv * d))[:pos + 1].view(np.uint16))
+    assert np.all(k_two[pos + 1:].view(np.uint16) == 0x7E00)                 # rows behind the position are left alone
+
+
 def test_attention_over_changing_shapes_on_one_stream(hip):
     """Head layouts beyond the parametrized ones (odd groups, one kv head per query head, a single
     position), interleaved on one stream and each run twice: against the fp64 restatement, and the
