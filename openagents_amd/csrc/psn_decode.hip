@@ -409,19 +409,20 @@ PSN_DEV void attn_partial_long_body(const psn_attn_args &a) {
     if (lane == 0) { dst[D] = m; dst[D + 1] = sum; }
 }
 
-/* The same for groups of exactly four query heads per kv head, with the roles turned: a wave takes sixteen of a
- * step's 64 positions for all four heads instead of all 64 for one head.  Every K and V row is then fetched by
+/* The same for groups of four or eight query heads per kv head, with the roles turned: a wave takes sixteen of a
+ * step's 64 positions for four heads (HB blocks of four heads, four waves each) instead of all 64 for one head.  Every K and V row is then fetched by
  * one wave only (a quarter of the requests, four times the distinct bytes in flight per compute unit, which is
  * what bounds a long context), converted to fp32 once and used four times.  The four waves' running states meet
  * through LDS at the end of the split. */
-template <bool ROPE>
+template <bool ROPE, int HB>
 PSN_DEV void attn_partial_long4_body(const psn_attn_args &a) {
-    constexpr int D = 128, H = 4;
-    __shared__ float qs[H][D];
+    constexpr int D = 128, H = 4, GROUP = H * HB;
+    __shared__ float qs[GROUP][D];
     __shared__ uint4 knew_row[16];
-    __shared__ float part_o[4][H][D];
-    __shared__ float part_ml[4][H][2];
-    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    __shared__ float part_o[HB][4][H][D];
+    __shared__ float part_ml[HB][4][H][2];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int w = wave & 3, hb = wave >> 2;                      /* position quarter of a step, block of four heads */
     const int quarter = lane >> 4, sub = lane & 15;
     const int kvh = blockIdx.x % a.n_kv_heads, split = blockIdx.x / a.n_kv_heads;
     const int pos_last = a.n_ctx - 1;
@@ -443,15 +444,15 @@ PSN_DEV void attn_partial_long4_body(const psn_attn_args &a) {
     fetch(0, ka, va);
     uint4 vnew = make_uint4(0, 0, 0, 0);
     if constexpr (ROPE) {
-        /* wave w rotates query head w of the group; wave 0 of the split that owns the token's position the new key */
+        /* wave i rotates query head i of the group; wave 0 of the split that owns the token's position the new key */
         const float2 tc = *reinterpret_cast<const float2 *>(a.rope_table + 2 * lane);
         const float cs = tc.x, sn = tc.y;
         float r0, r1;
-        const float2 qv = *reinterpret_cast<const float2 *>(a.q + (kvh * H + w) * D + 2 * lane);
+        const float2 qv = *reinterpret_cast<const float2 *>(a.q + (kvh * GROUP + wave) * D + 2 * lane);
         rope_pair(qv.x, qv.y, cs, sn, r0, r1);
-        qs[w][2 * lane] = r0;
-        qs[w][2 * lane + 1] = r1;
-        if (w == 0 && own) {
+        qs[wave][2 * lane] = r0;
+        qs[wave][2 * lane + 1] = r1;
+        if (wave == 0 && own) {
             const float2 kv = *reinterpret_cast<const float2 *>(a.k_new + kvh * D + 2 * lane);
             float k0, k1;
             rope_pair(kv.x, kv.y, cs, sn, k0, k1);
@@ -461,18 +462,18 @@ PSN_DEV void attn_partial_long4_body(const psn_attn_args &a) {
         }
         const float4 x0 = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub), x1 = *reinterpret_cast<const float4 *>(a.v_new + kvh * D + 8 * sub + 4);
         vnew.x = pack_h2(x0.x, x0.y); vnew.y = pack_h2(x0.z, x0.w); vnew.z = pack_h2(x1.x, x1.y); vnew.w = pack_h2(x1.z, x1.w);
-        if (own && w == 0 && quarter == 0)
+        if (own && wave == 0 && quarter == 0)
             reinterpret_cast<uint4 *>(reinterpret_cast<f16 *>(a.v_cache_w) + ((int64_t)pos_last * a.n_kv_heads + kvh) * D)[sub] = vnew;
     } else {
-        qs[w][lane] = a.q[(kvh * H + w) * D + lane];
-        qs[w][lane + 64] = a.q[(kvh * H + w) * D + lane + 64];
+        qs[wave][lane] = a.q[(kvh * GROUP + wave) * D + lane];
+        qs[wave][lane + 64] = a.q[(kvh * GROUP + wave) * D + lane + 64];
     }
     __syncthreads();
     uint4 knew = make_uint4(0, 0, 0, 0);
     if (own) knew = knew_row[sub];
     float q[H][8];
     UNROLL for (int h = 0; h < H; ++h) {
-        const float4 lo = *reinterpret_cast<const float4 *>(&qs[h][8 * sub]), hi = *reinterpret_cast<const float4 *>(&qs[h][8 * sub + 4]);
+        const float4 lo = *reinterpret_cast<const float4 *>(&qs[hb * H + h][8 * sub]), hi = *reinterpret_cast<const float4 *>(&qs[hb * H + h][8 * sub + 4]);
         q[h][0] = lo.x; q[h][1] = lo.y; q[h][2] = lo.z; q[h][3] = lo.w; q[h][4] = hi.x; q[h][5] = hi.y; q[h][6] = hi.z; q[h][7] = hi.w;
     }
     float m_run[H], l_run[H], o[H][8];
@@ -537,23 +538,23 @@ PSN_DEV void attn_partial_long4_body(const psn_attn_args &a) {
         const float l = quarters_sum(l_run[h] * f);
         UNROLL for (int t = 0; t < 8; ++t) o[h][t] = quarters_sum(o[h][t] * f);
         if (quarter == 0) {
-            UNROLL for (int t = 0; t < 8; ++t) part_o[w][h][8 * sub + t] = o[h][t];
+            UNROLL for (int t = 0; t < 8; ++t) part_o[hb][w][h][8 * sub + t] = o[h][t];
         }
-        if (lane == 0) { part_ml[w][h][0] = m; part_ml[w][h][1] = l; }
+        if (lane == 0) { part_ml[hb][w][h][0] = m; part_ml[hb][w][h][1] = l; }
     }
     __syncthreads();
     {
-        const int h = w;                                         /* wave w finishes head w */
+        const int h = w;                                         /* wave (hb, w) finishes head w of its block */
         float mw[4], M = -INFINITY;
-        UNROLL for (int i = 0; i < 4; ++i) { mw[i] = part_ml[i][h][0]; M = fmaxf(M, mw[i]); }
+        UNROLL for (int i = 0; i < 4; ++i) { mw[i] = part_ml[hb][i][h][0]; M = fmaxf(M, mw[i]); }
         float L = 0.f, o0 = 0.f, o1 = 0.f;
         UNROLL for (int i = 0; i < 4; ++i) {
             const float f = __expf(mw[i] - M);                   /* M is finite: wave 0 saw position p_begin */
-            L += part_ml[i][h][1] * f;
-            o0 += part_o[i][h][2 * lane] * f;
-            o1 += part_o[i][h][2 * lane + 1] * f;
+            L += part_ml[hb][i][h][1] * f;
+            o0 += part_o[hb][i][h][2 * lane] * f;
+            o1 += part_o[hb][i][h][2 * lane + 1] * f;
         }
-        float *dst = a.partial + ((int64_t)(kvh * H + h) * a.n_splits + split) * (D + 2);
+        float *dst = a.partial + ((int64_t)(kvh * GROUP + hb * H + h) * a.n_splits + split) * (D + 2);
         *reinterpret_cast<float2 *>(dst + 2 * lane) = make_float2(o0, o1);
         if (lane == 0) { dst[D] = M; dst[D + 1] = L; }
     }
@@ -564,8 +565,10 @@ extern "C" __global__ void __launch_bounds__(512) psn_attn_partial(const psn_att
 extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_rope(const psn_attn_args a) { attn_partial_body<true>(a); }
 extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_long(const psn_attn_args a) { attn_partial_long_body<false>(a); }
 extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_rope_long(const psn_attn_args a) { attn_partial_long_body<true>(a); }
-extern "C" __global__ void __launch_bounds__(256) psn_attn_partial_long4(const psn_attn_args a) { attn_partial_long4_body<false>(a); }
-extern "C" __global__ void __launch_bounds__(256) psn_attn_partial_rope_long4(const psn_attn_args a) { attn_partial_long4_body<true>(a); }
+extern "C" __global__ void __launch_bounds__(256) psn_attn_partial_long4(const psn_attn_args a) { attn_partial_long4_body<false, 1>(a); }
+extern "C" __global__ void __launch_bounds__(256) psn_attn_partial_rope_long4(const psn_attn_args a) { attn_partial_long4_body<true, 1>(a); }
+extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_long8(const psn_attn_args a) { attn_partial_long4_body<false, 2>(a); }
+extern "C" __global__ void __launch_bounds__(512) psn_attn_partial_rope_long8(const psn_attn_args a) { attn_partial_long4_body<true, 2>(a); }
 
 /* out[head][d] = sum_s o_s[d] e^(m_s - M) / sum_s l_s e^(m_s - M).  One wave per head, two heads per
  * workgroup; a lane owns two output dims.  The splits are taken 32 at a time and everything a wave needs

@@ -1999,9 +1999,10 @@ static int32_t attention_impl(psn_module *mod, psn_stream *s, const psn_buf *q, 
         a.rope_table = (const float *)rope->table->p;
     }
     const int32_t group = n_heads / n_kv_heads;
-    /* (groups of four query heads have a long-context kernel of their own, in which a wave serves all four) */
-    const char *partial = long_ctx ? (group == 4 ? (rope ? "psn_attn_partial_rope_long4" : "psn_attn_partial_long4")
-                                                 : (rope ? "psn_attn_partial_rope_long" : "psn_attn_partial_long"))
+    /* (groups of four and eight query heads have long-context kernels of their own, in which a wave serves four heads) */
+    const char *partial = long_ctx ? (group == 4   ? (rope ? "psn_attn_partial_rope_long4" : "psn_attn_partial_long4")
+                                      : group == 8 ? (rope ? "psn_attn_partial_rope_long8" : "psn_attn_partial_long8")
+                                                   : (rope ? "psn_attn_partial_rope_long" : "psn_attn_partial_long"))
                                    : (rope ? "psn_attn_partial_rope" : "psn_attn_partial");
     if ((rc = launch(mod, s, partial, (unsigned)(n_kv_heads * nsplits), (unsigned)(64 * group), 0, &a)))
         return rc;

@@ -94,7 +94,7 @@ def test_attention_decode_long_contexts(hip, nh, nkv):
         assert np.all(np.isfinite(got)) and G.max_rel_err(got, attention_ref(q, kc, vc, nh, nkv, d, n_ctx)) < 2e-5, n_ctx
 
 
-@pytest.mark.parametrize("nh,nkv", [(32, 8), (16, 2)])              # four heads to a kv head: a wave serves all four; otherwise one each
+@pytest.mark.parametrize("nh,nkv", [(32, 8), (16, 2), (8, 4)])      # groups of four and eight: a wave serves four heads; otherwise one each
 @pytest.mark.parametrize("pos", [4096, 4159, 4160, 6000, 8191, 9999])
 def test_rope_fused_long_context_attention(hip, pos, nh, nkv):
     """The long-context kernel with the rotary embedding and the cache append folded in: against the three
