@@ -79,3 +79,35 @@ def test_decode_step_record_and_worker_attachment(hip, orc):
     assert att["workers"][0]["ready"] is True and att["workers"][0]["evidence_digest"] == R.record_digest(rec)
     h = R.health(hip)
     assert h["execution_engine"] == "psionic" and h["backend"] == "hip" and h["models"] == [h["default_model"]]
+
+
+def test_wide_model_shape_against_the_cpu_path(hip, orc):
+    """A 70B-class layer shape (hidden 8192, 64 query / 8 kv heads, FFN 28672): the norm-fused projections stage
+    8192 values with eight-wave workgroups, the SwiGLU pair kernel runs at K = 8192, the down projection's rows
+    (112 chunks) are too long for the streaming kernels, the attention group is eight heads.  Two layers from a
+    512-token cache; the last layer's launches are recomputed on the CPU from the device's own inputs."""
+    from openagents_amd.decode import DecodeStep, LlamaShape, synthetic_weights
+    shape = LlamaShape(hidden=8192, n_heads=64, n_kv_heads=8, ffn=28672, vocab=4096, n_layers=2)
+    protos = {}
+    weights = synthetic_weights(hip, shape, 3, head_rows_unique=4096, keep_host=protos)
+    ctx = 512
+    step = DecodeStep(hip, shape, weights, ctx)
+    assert step.fused_norm and step.fused_swiglu == [True, True]
+    rng = np.random.default_rng(4)
+    pos = ctx - 1
+    kv = rng.standard_normal((pos, shape.kv_dim), dtype=np.float32).astype(np.float16)
+    for li in range(shape.n_layers):
+        step.k_cache[li].upload(kv)
+        step.v_cache[li].upload(kv)
+    step.x.upload(rng.standard_normal(shape.hidden, dtype=np.float32))
+    print("wide shape: enqueue", flush=True)
+    step.enqueue(pos)
+    hip.sync()
+    got = {"x": step.x.download(np.float32, (shape.hidden,)), "down": step.down.download(np.float32, (shape.hidden,)),
+           "act": step.act.download(np.float32, (shape.ffn,)), "logits": step.logits.download(np.float32, (shape.vocab,))}
+    assert all(np.all(np.isfinite(v)) for v in got.values())
+    ref = bench.OracleChecker().decode_last_layer(shape, protos, got)
+    for name in ("act", "down", "logits"):
+        verdict = R.parity_of(got[name], ref[name], "Q8", name)
+        print(f"wide shape {name}: {verdict['value']:.2e}", flush=True)
+        assert verdict["status"] == "pass", (name, verdict)
